@@ -1,0 +1,127 @@
+// Shared helpers of the gfx950 kernels: element types, wave64 reductions, argument checks.
+//
+// Every entry point is extern "C", takes raw device pointers and a hipStream_t, validates
+// its arguments on the host before it launches anything, and returns 0 on success. On failure
+// it returns non-zero and lmsf_last_error() gives the reason; nothing is launched then.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#define LMSF_WAVE 64
+
+// dtype codes shared with the Python side
+enum { LMSF_F32 = 0, LMSF_BF16 = 1 };
+
+typedef uint16_t bf16_t;  // raw bfloat16 bits
+
+void lmsf_set_error(const char* fmt, ...);
+
+#define LMSF_CHECK(cond, ...)            \
+  do {                                   \
+    if (!(cond)) {                       \
+      lmsf_set_error(__VA_ARGS__);       \
+      return 1;                          \
+    }                                    \
+  } while (0)
+
+#define LMSF_LAUNCH_CHECK(name)                                             \
+  do {                                                                      \
+    hipError_t e_ = hipGetLastError();                                      \
+    if (e_ != hipSuccess) {                                                 \
+      lmsf_set_error("%s: launch failed: %s", name, hipGetErrorString(e_)); \
+      return 2;                                                             \
+    }                                                                       \
+  } while (0)
+
+// ---------------------------------------------------------------- element conversion
+
+__device__ __forceinline__ float bf16_to_f32(bf16_t v) { return __uint_as_float(((uint32_t)v) << 16); }
+
+// round to nearest even; NaN stays NaN
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (bf16_t)(u >> 16);
+}
+
+template <typename T> __device__ __forceinline__ float to_f32(T v);
+template <> __device__ __forceinline__ float to_f32<float>(float v) { return v; }
+template <> __device__ __forceinline__ float to_f32<bf16_t>(bf16_t v) { return bf16_to_f32(v); }
+
+template <typename T> __device__ __forceinline__ T from_f32(float v);
+template <> __device__ __forceinline__ float from_f32<float>(float v) { return v; }
+template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float v) { return f32_to_bf16(v); }
+
+// 16-byte vectors: 4 floats or 8 bfloat16
+template <typename T> struct Vec16;
+template <> struct Vec16<float> {
+  static constexpr int N = 4;
+  float4 v;
+  __device__ __forceinline__ void load(const float* p) { v = *reinterpret_cast<const float4*>(p); }
+  __device__ __forceinline__ void store(float* p) const { *reinterpret_cast<float4*>(p) = v; }
+  __device__ __forceinline__ float get(int i) const { return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w; }
+  __device__ __forceinline__ void set(int i, float f) {
+    if (i == 0) v.x = f; else if (i == 1) v.y = f; else if (i == 2) v.z = f; else v.w = f;
+  }
+};
+template <> struct Vec16<bf16_t> {
+  static constexpr int N = 8;
+  uint4 v;
+  __device__ __forceinline__ void load(const bf16_t* p) { v = *reinterpret_cast<const uint4*>(p); }
+  __device__ __forceinline__ void store(bf16_t* p) const { *reinterpret_cast<uint4*>(p) = v; }
+  __device__ __forceinline__ float get(int i) const {
+    uint32_t w = (i >> 1) == 0 ? v.x : (i >> 1) == 1 ? v.y : (i >> 1) == 2 ? v.z : v.w;
+    return __uint_as_float((i & 1) ? (w & 0xffff0000u) : (w << 16));
+  }
+  __device__ __forceinline__ void set(int i, float f) {
+    uint32_t b = f32_to_bf16(f);
+    uint32_t* w = (i >> 1) == 0 ? &v.x : (i >> 1) == 1 ? &v.y : (i >> 1) == 2 ? &v.z : &v.w;
+    *w = (i & 1) ? ((*w & 0x0000ffffu) | (b << 16)) : ((*w & 0xffff0000u) | b);
+  }
+};
+
+// ---------------------------------------------------------------- wave64 and block reductions
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = LMSF_WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, LMSF_WAVE);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = LMSF_WAVE / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, LMSF_WAVE));
+  return v;
+}
+
+// Sum over a block of up to 1024 threads (a multiple of 64); every thread gets the result.
+// ``red`` is LDS scratch of at least 16 floats. Safe to call repeatedly with the same scratch.
+__device__ __forceinline__ float block_sum(float v, float* red) {
+  v = wave_sum(v);
+  const int nw = (blockDim.x + LMSF_WAVE - 1) / LMSF_WAVE;
+  if (nw == 1) return v;
+  const int w = threadIdx.x / LMSF_WAVE, l = threadIdx.x % LMSF_WAVE;
+  __syncthreads();
+  if (l == 0) red[w] = v;
+  __syncthreads();
+  float r = 0.f;
+  for (int i = 0; i < nw; ++i) r += red[i];
+  return r;
+}
+__device__ __forceinline__ float block_max(float v, float* red) {
+  v = wave_max(v);
+  const int nw = (blockDim.x + LMSF_WAVE - 1) / LMSF_WAVE;
+  if (nw == 1) return v;
+  const int w = threadIdx.x / LMSF_WAVE, l = threadIdx.x % LMSF_WAVE;
+  __syncthreads();
+  if (l == 0) red[w] = v;
+  __syncthreads();
+  float r = red[0];
+  for (int i = 1; i < nw; ++i) r = fmaxf(r, red[i]);
+  return r;
+}
+
+static inline bool lmsf_aligned16(const void* p) { return (((uintptr_t)p) & 15u) == 0; }
+static inline int lmsf_elem_size(int dtype) { return dtype == LMSF_F32 ? 4 : 2; }

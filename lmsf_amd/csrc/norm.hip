@@ -1,0 +1,89 @@
+// RMSNorm, with the residual addition fused in.
+//
+//   r = branch + residual          (float32; either operand may be absent)
+//   residual <- r                  (kept in float32, written only when both are present)
+//   out = r * rsqrt(mean(r^2) + eps) * (w + weight_offset)
+//
+// The reference has the two forms as separate kernels (vllm/kernels/layernorm_kernels.cu:13-38
+// rms_norm_kernel, :41-68 fused_add_rms_norm_kernel), rounds the residual to the model's dtype
+// and rounds the normalised value before the weight multiply. Here the residual stream stays in
+// float32 and the row is rounded once, at the store.
+//
+// One workgroup per output row. ``rows`` (optional) gathers: output row i is computed from input
+// row rows[i], and the residual is then left untouched.
+#include "common.h"
+
+template <typename TB, typename TO, typename TW>
+__global__ __launch_bounds__(1024) void add_rms_norm_kernel(
+    const TB* __restrict__ branch, float* __restrict__ residual, const TW* __restrict__ weight,
+    TO* __restrict__ out, const int* __restrict__ rows, int H, float eps, float weight_offset) {
+  __shared__ float red[16];
+  const int r = blockIdx.x;
+  const long src = rows ? (long)rows[r] : (long)r;
+  const TB* b = branch ? branch + src * H : nullptr;
+  float* res = residual ? residual + src * H : nullptr;
+  const bool write_res = (b != nullptr) && (res != nullptr) && (rows == nullptr);
+  // When the sum cannot be written back to the residual (gather, or no residual), the second
+  // pass recomputes it from the inputs.
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    float x = 0.f;
+    if (b) x += to_f32<TB>(b[i]);
+    if (res) x += res[i];
+    if (write_res) res[i] = x;
+    ss += x * x;
+  }
+  ss = block_sum(ss, red);
+  const float inv = rsqrtf(ss / (float)H + eps);
+  TO* o = out + (long)r * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    float x;
+    if (write_res) {
+      x = res[i];
+    } else {
+      x = 0.f;
+      if (b) x += to_f32<TB>(b[i]);
+      if (res) x += res[i];
+    }
+    o[i] = from_f32<TO>(x * inv * (to_f32<TW>(weight[i]) + weight_offset));
+  }
+}
+
+template <typename TB, typename TO, typename TW>
+static void launch_norm(const void* branch, float* residual, const void* weight, void* out, const int* rows,
+                        int n_out, int H, float eps, float woff, hipStream_t stream) {
+  int threads = ((H + 3) / 4 + 63) / 64 * 64;
+  if (threads > 1024) threads = 1024;
+  if (threads < 64) threads = 64;
+  hipLaunchKernelGGL((add_rms_norm_kernel<TB, TO, TW>), dim3(n_out), dim3(threads), 0, stream,
+                     (const TB*)branch, residual, (const TW*)weight, (TO*)out, rows, H, eps, woff);
+}
+
+// branch [n_in, H] of branch_dtype or null; residual [n_in, H] float32 or null (not both null);
+// weight [H]; out [n_out, H]; rows int32 [n_out] or null (then n_out rows are rows 0..n_out-1).
+extern "C" int lmsf_add_rms_norm(const void* branch, int branch_dtype, float* residual, const void* weight,
+                                 int weight_dtype, void* out, int out_dtype, const int* rows, int n_out, int H,
+                                 float eps, float weight_offset, hipStream_t stream) {
+  LMSF_CHECK(branch != nullptr || residual != nullptr, "add_rms_norm: neither branch nor residual given");
+  LMSF_CHECK(weight != nullptr && out != nullptr, "add_rms_norm: null weight or out");
+  LMSF_CHECK(H > 0 && n_out >= 0, "add_rms_norm: bad sizes n_out=%d H=%d", n_out, H);
+  LMSF_CHECK(eps > 0.f, "add_rms_norm: eps must be > 0");
+  LMSF_CHECK((branch_dtype == LMSF_F32 || branch_dtype == LMSF_BF16) &&
+                 (weight_dtype == LMSF_F32 || weight_dtype == LMSF_BF16) &&
+                 (out_dtype == LMSF_F32 || out_dtype == LMSF_BF16),
+             "add_rms_norm: unknown dtype code");
+  if (n_out == 0) return 0;
+  const int key = branch_dtype * 4 + out_dtype * 2 + weight_dtype;
+  switch (key) {
+    case 0: launch_norm<float, float, float>(branch, residual, weight, out, rows, n_out, H, eps, weight_offset, stream); break;
+    case 1: launch_norm<float, float, bf16_t>(branch, residual, weight, out, rows, n_out, H, eps, weight_offset, stream); break;
+    case 2: launch_norm<float, bf16_t, float>(branch, residual, weight, out, rows, n_out, H, eps, weight_offset, stream); break;
+    case 3: launch_norm<float, bf16_t, bf16_t>(branch, residual, weight, out, rows, n_out, H, eps, weight_offset, stream); break;
+    case 4: launch_norm<bf16_t, float, float>(branch, residual, weight, out, rows, n_out, H, eps, weight_offset, stream); break;
+    case 5: launch_norm<bf16_t, float, bf16_t>(branch, residual, weight, out, rows, n_out, H, eps, weight_offset, stream); break;
+    case 6: launch_norm<bf16_t, bf16_t, float>(branch, residual, weight, out, rows, n_out, H, eps, weight_offset, stream); break;
+    default: launch_norm<bf16_t, bf16_t, bf16_t>(branch, residual, weight, out, rows, n_out, H, eps, weight_offset, stream); break;
+  }
+  LMSF_LAUNCH_CHECK("add_rms_norm");
+  return 0;
+}

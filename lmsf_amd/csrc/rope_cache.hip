@@ -1,0 +1,108 @@
+// Rotary position embedding fused with the write of K and V into the paged cache.
+//
+// Rotation (vllm/kernels/pos_encoding_kernels.cu:12-77): for every head of q and k and every
+// pair index i < rot/2,  x' = x cos - y sin,  y' = y cos + x sin, with (x, y) = elements
+// (i, i + rot/2) in NeoX style or (2i, 2i+1) in GPT-J style, and cos/sin read from the row of the
+// table that the token's position selects. The reference computes in the model's dtype from a
+// table in that dtype; here the table is float32 [max_pos, rot] = [cos(rot/2) | sin(rot/2)] and the
+// arithmetic is float32, rounded once at the store.
+//
+// Cache write (vllm/kernels/cache_kernels.cu:190-232): the token's rotated k and its v go to slot
+// s = page * page_size + offset; a negative slot is skipped. Page layout here is
+// [page, kv_head, offset, d] for both K and V (the reference uses [page, head, d/x, offset, x] and
+// [page, head, d, offset]; only the slot arithmetic is shared).
+//
+// q, k, v point at the first column of their parts inside one row-strided buffer (the fused QKV
+// output); row_stride is in elements. Either half may be switched off: table == null leaves q and
+// k unrotated, slots == null writes no cache. One workgroup per token.
+#include "common.h"
+
+template <typename T>
+__global__ __launch_bounds__(256) void rope_cache_write_kernel(
+    T* __restrict__ q, T* __restrict__ k, const T* __restrict__ v, long row_stride, const int* __restrict__ positions,
+    const float* __restrict__ table, int rot, int neox, const int* __restrict__ slots, T* __restrict__ k_pages,
+    T* __restrict__ v_pages, int nh, int nkv, int d, int ps) {
+  const long t = blockIdx.x;
+  const int half = rot / 2;
+  const float* cs = table ? table + (long)positions[t] * rot : nullptr;
+  long kdst = -1;  // element offset of (page, head 0, offset, 0)
+  long head_step = (long)ps * d;
+  if (slots) {
+    const int s = slots[t];
+    if (s >= 0) kdst = ((long)(s / ps) * nkv * ps + (s % ps)) * d;
+  }
+  if (cs && q) {
+    T* qt = q + t * row_stride;
+    for (int idx = threadIdx.x; idx < nh * half; idx += blockDim.x) {
+      const int h = idx / half, i = idx % half;
+      const int xi = neox ? i : 2 * i, yi = neox ? i + half : 2 * i + 1;
+      const float c = cs[i], s = cs[half + i];
+      const float x = to_f32<T>(qt[h * d + xi]), y = to_f32<T>(qt[h * d + yi]);
+      qt[h * d + xi] = from_f32<T>(x * c - y * s);
+      qt[h * d + yi] = from_f32<T>(y * c + x * s);
+    }
+  }
+  if (k) {
+    T* kt = k + t * row_stride;
+    if (cs) {
+      for (int idx = threadIdx.x; idx < nkv * half; idx += blockDim.x) {
+        const int h = idx / half, i = idx % half;
+        const int xi = neox ? i : 2 * i, yi = neox ? i + half : 2 * i + 1;
+        const float c = cs[i], s = cs[half + i];
+        const float x = to_f32<T>(kt[h * d + xi]), y = to_f32<T>(kt[h * d + yi]);
+        const T xr = from_f32<T>(x * c - y * s), yr = from_f32<T>(y * c + x * s);
+        kt[h * d + xi] = xr;
+        kt[h * d + yi] = yr;
+        if (kdst >= 0) {
+          k_pages[kdst + h * head_step + xi] = xr;
+          k_pages[kdst + h * head_step + yi] = yr;
+        }
+      }
+    }
+    if (kdst >= 0) {
+      // the part of k that the rotation did not touch (all of it without a table)
+      const int lo = cs ? rot : 0, tail = d - lo;
+      for (int idx = threadIdx.x; idx < nkv * tail; idx += blockDim.x) {
+        const int h = idx / tail, i = lo + idx % tail;
+        k_pages[kdst + h * head_step + i] = kt[h * d + i];
+      }
+    }
+  }
+  if (v && kdst >= 0) {
+    const T* vt = v + t * row_stride;
+    for (int idx = threadIdx.x; idx < nkv * d; idx += blockDim.x) {
+      const int h = idx / d, i = idx % d;
+      v_pages[kdst + h * head_step + i] = vt[h * d + i];
+    }
+  }
+}
+
+extern "C" int lmsf_rope_cache_write(void* q, void* k, const void* v, int dtype, int n_tokens, long row_stride,
+                                     const int* positions, const float* table, int rot, int neox, int max_pos,
+                                     const int* slots, void* k_pages, void* v_pages, long num_pages, int nh, int nkv,
+                                     int d, int ps, hipStream_t stream) {
+  LMSF_CHECK(dtype == LMSF_F32 || dtype == LMSF_BF16, "rope_cache_write: unknown dtype code %d", dtype);
+  LMSF_CHECK(n_tokens >= 0 && nh >= 0 && nkv >= 0 && d > 0, "rope_cache_write: bad sizes");
+  LMSF_CHECK(row_stride >= 0, "rope_cache_write: bad row stride");
+  if (table) {
+    LMSF_CHECK(positions != nullptr, "rope_cache_write: rotation needs positions");
+    LMSF_CHECK(rot > 0 && rot % 2 == 0 && rot <= d, "rope_cache_write: rotary_dim %d must be even and <= head_dim %d",
+               rot, d);
+    LMSF_CHECK(max_pos > 0, "rope_cache_write: empty table");
+  }
+  if (slots) {
+    LMSF_CHECK(k && v && k_pages && v_pages, "rope_cache_write: cache write needs k, v and both page tensors");
+    LMSF_CHECK(ps > 0 && num_pages > 0, "rope_cache_write: bad page geometry");
+  }
+  if (n_tokens == 0) return 0;
+  if (dtype == LMSF_F32)
+    hipLaunchKernelGGL((rope_cache_write_kernel<float>), dim3(n_tokens), dim3(256), 0, stream, (float*)q, (float*)k,
+                       (const float*)v, row_stride, positions, table, rot, neox, slots, (float*)k_pages,
+                       (float*)v_pages, nh, nkv, d, ps);
+  else
+    hipLaunchKernelGGL((rope_cache_write_kernel<bf16_t>), dim3(n_tokens), dim3(256), 0, stream, (bf16_t*)q,
+                       (bf16_t*)k, (const bf16_t*)v, row_stride, positions, table, rot, neox, slots, (bf16_t*)k_pages,
+                       (bf16_t*)v_pages, nh, nkv, d, ps);
+  LMSF_LAUNCH_CHECK("rope_cache_write");
+  return 0;
+}

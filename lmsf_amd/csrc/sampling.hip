@@ -1,0 +1,243 @@
+// Sampling from float32 logits: greedy, temperature, top-k, top-p, min-p, and the penalties.
+//
+// Pipeline of the reference (core/src/model_executor/layers/sampler.rs:839-971): penalties, divide
+// by the temperature, top-k/top-p, min-p, float32 softmax, then argmax for greedy rows and
+// argmax(probs / q) with q ~ Exp(1) for random rows (:326-361). The reference sorts the whole
+// vocabulary for top-k/top-p (:139-210). Here one workgroup per row finds the two cut values by
+// bisection on the order-preserving integer image of the floats, without a sort, and draws with the
+// same exponential race written as argmax(x_i - log(-log u_i)), u_i from a counter-based generator
+// keyed by (seed of the request, number of the draw, vocabulary index): the token does not depend
+// on what else is in the batch.
+//
+// Cut rules (ties at a cut value are kept together):
+//   top-k : keep x >= k-th largest value                         (sampler.rs:170-178)
+//   top-p : keep x whose mass of strictly larger values is < p   (sampler.rs:180-197: ascending
+//           cumulative sums <= 1 - p are removed, the largest always stays)
+//   min-p : keep x with prob >= min_p * max prob, i.e. x >= max + log(min_p)   (sampler.rs:305-325)
+#include "common.h"
+
+#include <math.h>
+
+#define SAMP_THREADS 1024
+
+__device__ __forceinline__ uint32_t order_key(float f) {
+  const uint32_t b = __float_as_uint(f);
+  return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+
+// Philox4x32-10; returns the first of the four output words.
+__device__ __forceinline__ uint32_t philox_first(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0,
+                                                 uint32_t k1) {
+#pragma unroll
+  for (int r = 0; r < 10; ++r) {
+    const uint32_t hi0 = __umulhi(0xD2511F53u, c0), lo0 = 0xD2511F53u * c0;
+    const uint32_t hi1 = __umulhi(0xCD9E8D57u, c2), lo1 = 0xCD9E8D57u * c2;
+    const uint32_t n0 = hi1 ^ c1 ^ k0, n1 = lo1, n2 = hi0 ^ c3 ^ k1, n3 = lo0;
+    c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+  return c0;
+}
+
+__device__ __forceinline__ float gumbel_noise(uint64_t seed, uint32_t draw, uint32_t index) {
+  const uint32_t r = philox_first(index, draw, 0u, 0u, (uint32_t)seed, (uint32_t)(seed >> 32));
+  const float u = ((float)(r >> 8) + 0.5f) * (1.0f / 16777216.0f);  // in (0, 1)
+  return -logf(-logf(u));
+}
+
+__device__ __forceinline__ unsigned long long block_sum_u64(unsigned long long v, unsigned long long* red) {
+#pragma unroll
+  for (int o = LMSF_WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, LMSF_WAVE);
+  const int nw = blockDim.x / LMSF_WAVE;
+  const int w = threadIdx.x / LMSF_WAVE, l = threadIdx.x % LMSF_WAVE;
+  __syncthreads();
+  if (l == 0) red[w] = v;
+  __syncthreads();
+  unsigned long long r = 0;
+  for (int i = 0; i < nw; ++i) r += red[i];
+  return r;
+}
+
+// Largest (value, lowest index) over the block; every thread gets the index.
+__device__ __forceinline__ int block_argmax(float v, int idx, float* redv, int* redi) {
+#pragma unroll
+  for (int o = LMSF_WAVE / 2; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(v, o, LMSF_WAVE);
+    const int oi = __shfl_xor(idx, o, LMSF_WAVE);
+    if (ov > v || (ov == v && oi < idx)) { v = ov; idx = oi; }
+  }
+  const int nw = blockDim.x / LMSF_WAVE;
+  const int w = threadIdx.x / LMSF_WAVE, l = threadIdx.x % LMSF_WAVE;
+  __syncthreads();
+  if (l == 0) { redv[w] = v; redi[w] = idx; }
+  __syncthreads();
+  float bv = redv[0];
+  int bi = redi[0];
+  for (int i = 1; i < nw; ++i)
+    if (redv[i] > bv || (redv[i] == bv && redi[i] < bi)) { bv = redv[i]; bi = redi[i]; }
+  return bi;
+}
+
+// One workgroup per row. temperature < 1e-5 means greedy (core/src/common/sampling_params.rs:156-163).
+__global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(
+    const float* __restrict__ logits, long ld, int V, const float* __restrict__ temperature,
+    const int* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ min_p,
+    const unsigned long long* __restrict__ seeds, const unsigned int* __restrict__ draws, int* __restrict__ out) {
+  __shared__ float redf[16];
+  __shared__ int redi[16];
+  __shared__ unsigned long long redu[16];
+  const int r = blockIdx.x, tid = threadIdx.x;
+  const float* row = logits + (long)r * ld;
+  const float T = temperature ? temperature[r] : 0.f;
+  const bool greedy = T < 1e-5f;
+
+  if (greedy) {
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int i = tid; i < V; i += SAMP_THREADS) {
+      const float x = row[i];
+      if (x > bv) { bv = x; bi = i; }  // ascending i per thread: the first maximum wins
+    }
+    const int best = block_argmax(bv, bi, redf, redi);
+    if (tid == 0) out[r] = best < V ? best : 0;
+    return;
+  }
+
+  const float invT = 1.0f / T;
+  float mx = -INFINITY;
+  for (int i = tid; i < V; i += SAMP_THREADS) mx = fmaxf(mx, row[i] * invT);
+  mx = block_max(mx, redf);
+
+  uint32_t cut = 0u;  // keep order_key(x) >= cut
+  const int k = top_k ? top_k[r] : -1;
+  if (k > 0 && k < V) {
+    uint32_t cur = 0u;
+    for (int bit = 31; bit >= 0; --bit) {
+      const uint32_t cand = cur | (1u << bit);
+      unsigned long long cnt = 0;
+      for (int i = tid; i < V; i += SAMP_THREADS) cnt += order_key(row[i] * invT) >= cand ? 1u : 0u;
+      cnt = block_sum_u64(cnt, redu);
+      if (cnt >= (unsigned long long)k) cur = cand;
+    }
+    cut = cur;
+  }
+  const float p = top_p ? top_p[r] : 1.0f;
+  if (p < 1.0f) {
+    float z = 0.f;
+    for (int i = tid; i < V; i += SAMP_THREADS) {
+      const float x = row[i] * invT;
+      if (order_key(x) >= cut) z += expf(x - mx);
+    }
+    z = block_sum(z, redf);
+    const float target = p * z;
+    uint32_t cur = 0u;
+    for (int bit = 31; bit >= 0; --bit) {
+      const uint32_t cand = cur | (1u << bit);
+      float mass = 0.f;
+      for (int i = tid; i < V; i += SAMP_THREADS) {
+        const float x = row[i] * invT;
+        const uint32_t key = order_key(x);
+        if (key >= cand && key >= cut) mass += expf(x - mx);
+      }
+      mass = block_sum(mass, redf);
+      if (mass >= target) cur = cand;
+    }
+    if (cur > cut) cut = cur;
+  }
+  const float mp = min_p ? min_p[r] : 0.f;
+  if (mp > 0.f) {
+    const uint32_t c = order_key(mx + logf(mp));
+    if (c > cut) cut = c;
+  }
+  // the maximum is always kept, whatever rounding did to the cuts
+  const uint32_t kmax = order_key(mx);
+  if (cut > kmax) cut = kmax;
+
+  const unsigned long long seed = seeds ? seeds[r] : 0ull;
+  const unsigned int draw = draws ? draws[r] : 0u;
+  float bv = -INFINITY;
+  int bi = 0x7fffffff;
+  for (int i = tid; i < V; i += SAMP_THREADS) {
+    const float x = row[i] * invT;
+    if (order_key(x) < cut) continue;
+    const float y = x + gumbel_noise(seed, draw, (uint32_t)i);
+    if (y > bv) { bv = y; bi = i; }
+  }
+  const int best = block_argmax(bv, bi, redf, redi);
+  if (tid == 0) out[r] = best < V ? best : 0;
+}
+
+// logits [R, V] float32 with row stride ld. temperature/top_k/top_p/min_p/seeds/draws are per-row
+// device arrays; any of them may be null (greedy, no cut, seed 0, draw 0).
+extern "C" int lmsf_sample(const float* logits, long ld, int R, int V, const float* temperature, const int* top_k,
+                           const float* top_p, const float* min_p, const unsigned long long* seeds,
+                           const unsigned int* draws, int* out, hipStream_t stream) {
+  LMSF_CHECK(logits && out, "sample: null pointer");
+  LMSF_CHECK(R >= 0 && V > 0 && ld >= V, "sample: bad sizes R=%d V=%d ld=%ld", R, V, ld);
+  if (R == 0) return 0;
+  hipLaunchKernelGGL(sample_kernel, dim3(R), dim3(SAMP_THREADS), 0, stream, logits, ld, V, temperature, top_k, top_p,
+                     min_p, seeds, draws, out);
+  LMSF_LAUNCH_CHECK("sample");
+  return 0;
+}
+
+// ---------------------------------------------------------------- penalties
+// counts[r, v] = (times v occurs in the output tokens of row r) | PROMPT_BIT if v occurs in the
+// prompt. tokens is the concatenation over rows of [prompt tokens, output tokens];
+// offsets[r] .. offsets[r+1] is row r's range and prompt_lens[r] how many of them are prompt.
+#define PROMPT_BIT 0x40000000
+
+__global__ __launch_bounds__(256) void penalty_count_kernel(const int* __restrict__ tokens,
+                                                            const int* __restrict__ offsets,
+                                                            const int* __restrict__ prompt_lens,
+                                                            int* __restrict__ counts, int V) {
+  const int r = blockIdx.x;
+  const int b = offsets[r], e = offsets[r + 1], np = prompt_lens[r];
+  int* c = counts + (long)r * V;
+  for (int i = b + threadIdx.x; i < e; i += blockDim.x) {
+    const int tok = tokens[i];
+    if (tok < 0 || tok >= V) continue;
+    if (i - b < np)
+      atomicOr(&c[tok], PROMPT_BIT);
+    else
+      atomicAdd(&c[tok], 1);
+  }
+}
+
+// core/src/model_executor/layers/sampler.rs:48-137: seen tokens: x > 0 ? x / rep : x * rep;
+// then x -= frequency * output count; then x -= presence * [output count > 0].
+__global__ __launch_bounds__(256) void penalty_apply_kernel(float* __restrict__ logits, long ld,
+                                                            const int* __restrict__ counts, int V,
+                                                            const float* __restrict__ presence,
+                                                            const float* __restrict__ frequency,
+                                                            const float* __restrict__ repetition) {
+  const int r = blockIdx.x;
+  const int i = blockIdx.y * blockDim.x + threadIdx.x;
+  if (i >= V) return;
+  const int c = counts[(long)r * V + i];
+  if (c == 0) return;
+  const int n_out = c & (PROMPT_BIT - 1);
+  float x = logits[(long)r * ld + i];
+  const float rep = repetition[r];
+  x = x > 0.f ? x / rep : x * rep;
+  x -= frequency[r] * (float)n_out;
+  if (n_out > 0) x -= presence[r];
+  logits[(long)r * ld + i] = x;
+}
+
+// counts must be an int32 [R, V] buffer filled with zeros before the call.
+extern "C" int lmsf_apply_penalties(float* logits, long ld, int R, int V, const int* tokens, const int* offsets,
+                                    const int* prompt_lens, int* counts, const float* presence,
+                                    const float* frequency, const float* repetition, hipStream_t stream) {
+  LMSF_CHECK(logits && tokens && offsets && prompt_lens && counts && presence && frequency && repetition,
+             "apply_penalties: null pointer");
+  LMSF_CHECK(R >= 0 && V > 0 && ld >= V, "apply_penalties: bad sizes R=%d V=%d ld=%ld", R, V, ld);
+  LMSF_CHECK((V + 255) / 256 <= 65535, "apply_penalties: vocabulary too large");
+  if (R == 0) return 0;
+  hipLaunchKernelGGL(penalty_count_kernel, dim3(R), dim3(256), 0, stream, tokens, offsets, prompt_lens, counts, V);
+  hipLaunchKernelGGL(penalty_apply_kernel, dim3(R, (V + 255) / 256), dim3(256), 0, stream, logits, ld, counts, V,
+                     presence, frequency, repetition);
+  LMSF_LAUNCH_CHECK("apply_penalties");
+  return 0;
+}

@@ -1,0 +1,148 @@
+"""Builds what a model folder needs to run steps: configuration, model, weights, cache, executor.
+
+This is the common base of the engine (scheduler + sampler on top) and of trace replay (nothing
+on top). Reference: Worker::from + Worker::init_cache (core/src/worker/model_worker.rs:34-126) and
+the sizing of the cache from free device memory (:128-162).
+"""
+import os
+from dataclasses import dataclass
+from typing import Any, Optional, Sequence
+
+import torch
+
+from .. import models as _models  # noqa: F401  (registers the architectures)
+from ..cache.storage import CacheStorage, plan_groups
+from ..config.model_config import ArchConfig
+from ..config.registry import Architecture, get_architecture, load_model_config
+from ..models.decoder import DecoderModel
+from ..parts.base import Runtime
+from ..weights.loader import load_weights, load_weights_from_generator
+from ..weights.random_init import random_tensor
+from .executor import ModelExecutor
+
+_DTYPES = {"float32": torch.float32, "float": torch.float32, "bfloat16": torch.bfloat16,
+           "float16": torch.bfloat16, "half": torch.bfloat16}
+
+
+def resolve_dtype(name: Optional[str], config: ArchConfig) -> torch.dtype:
+    """--dtype overrides config.json's torch_dtype (core/src/common/config.rs:181-186). float16
+    checkpoints run in bfloat16: the kernels have two element types, float32 and bfloat16."""
+    key = name if name not in (None, "auto") else config.torch_dtype
+    if key not in _DTYPES:
+        raise ValueError("dtype %r is not supported (float32, bfloat16)" % (key,))
+    return _DTYPES[key]
+
+
+@dataclass
+class EngineCore:
+    arch: Architecture
+    config: ArchConfig
+    rt: Runtime
+    model: DecoderModel
+    storage: CacheStorage
+    executor: ModelExecutor
+    max_model_len: int
+    block_size: int
+
+
+def _default_ops():
+    from ..ops import get_ops
+    return get_ops()
+
+
+def build_model(arch: Architecture, config: ArchConfig, rt: Runtime, model_dir: Optional[str],
+                load_format: str = "auto", seed: int = 0) -> DecoderModel:
+    model = DecoderModel(arch.build_spec(config), rt)
+    if load_format == "random":
+        std = 0.02
+        store = torch.float32 if rt.dtype == torch.float32 else torch.bfloat16
+        load_weights_from_generator(model.parts(),
+                                    lambda name, decl: random_tensor(name, decl, seed, std, store, rt.device))
+    elif load_format == "auto":
+        if model_dir is None:
+            raise ValueError("a model folder is needed unless load_format is 'random'")
+        load_weights(model.parts(), model_dir, rt.device, rt.dtype, tolerated=arch.tolerated_tensors)
+    else:
+        raise ValueError("load_format %r unknown (auto, random)" % load_format)
+    return model
+
+
+def profile_num_pages(model: DecoderModel, rt: Runtime, block_size: int, gpu_memory_utilization: float,
+                      max_num_batched_tokens: int, max_num_seqs: int, max_model_len: int) -> Sequence[int]:
+    """Pages per cache group from the device memory that is free after the weights are loaded:
+    (total * utilization - used - room for one step's activations) / bytes per page
+    (core/src/worker/model_worker.rs:146-154). Groups that keep every key share the budget in
+    proportion to their page size in bytes; a window group gets what its window can ever hold."""
+    groups, _ = plan_groups(model.cache_requirements(), block_size)
+    if not groups:
+        return []
+    es = 4 if rt.dtype == torch.float32 else 2
+    free, total = torch.cuda.mem_get_info(rt.device)
+    spec = model.spec
+    widest = max((p.weight.shape[0] for p in model.parts() if getattr(p, "weight", None) is not None
+                  and p.weight.dim() == 2 and p.weight.shape[0] != spec.vocab_size), default=spec.hidden_size)
+    act = max_num_batched_tokens * (spec.hidden_size * 4 * 2 + widest * es * 3) \
+        + max_num_seqs * spec.vocab_size * 4 * 3 + (512 << 20)
+    budget = int(total * gpu_memory_utilization) - (total - free) - act
+    counts = [0] * len(groups)
+    for gi, g in enumerate(groups):
+        if g.spec.window is not None:
+            per_seq = (g.spec.window + max_num_batched_tokens) // block_size + 2
+            counts[gi] = per_seq * max_num_seqs
+            budget -= counts[gi] * g.bytes_per_page(es)
+    full = [gi for gi, g in enumerate(groups) if g.spec.window is None]
+    if full:
+        per_page_all = sum(groups[gi].bytes_per_page(es) for gi in full)
+        n = max(0, budget // per_page_all)
+        n = min(n, max_num_seqs * (-(-max_model_len // block_size)) + 1)   # more can never be used
+        for gi in full:
+            counts[gi] = int(n)
+    return counts
+
+
+def load_engine_core(model_dir: Optional[str], dtype: Optional[str] = None, block_size: int = 16,
+                     max_model_len: Optional[int] = None, num_pages: Optional[int] = None,
+                     gpu_memory_utilization: float = 0.9, max_num_seqs: int = 256,
+                     max_num_batched_tokens: Optional[int] = None, device: str = "cuda:0",
+                     ops: Any = None, load_format: str = "auto", seed: int = 0,
+                     config: Optional[ArchConfig] = None) -> EngineCore:
+    """``num_pages``: pages of every cache group (tests, replay); None sizes the pools from free memory."""
+    if config is None:
+        if model_dir is None:
+            raise ValueError("need a model folder or a configuration")
+        arch, config = load_model_config(model_dir)
+    else:
+        arch = get_architecture(config.architecture)
+    derived = config.max_position_embeddings
+    if max_model_len is None:
+        max_model_len = derived
+    elif max_model_len > derived:
+        # core/src/common/config.rs:146-153
+        raise ValueError("max_model_len %d is greater than the model's context length %d (config.json)"
+                         % (max_model_len, derived))
+    if not (0 < gpu_memory_utilization <= 1.0):
+        raise ValueError("gpu_memory_utilization must be in (0, 1], got %r" % gpu_memory_utilization)  # config.rs:245-250
+    if block_size <= 0:
+        raise ValueError("block_size must be > 0")
+    run_dtype = resolve_dtype(dtype, config)
+    dev = torch.device(device)
+    if ops is None:
+        ops = _default_ops()
+    rt = Runtime(ops=ops, device=dev, dtype=run_dtype, max_positions=max_model_len)
+    model = build_model(arch, config, rt, model_dir, load_format, seed)
+    groups, _ = plan_groups(model.cache_requirements(), block_size)
+    if max_num_batched_tokens is None:
+        max_num_batched_tokens = max(max_model_len, 2048)   # config.rs:301-307
+    if num_pages is None:
+        counts = profile_num_pages(model, rt, block_size, gpu_memory_utilization, max_num_batched_tokens,
+                                   max_num_seqs, max_model_len)
+        if any(c * block_size < max_model_len for c, g in zip(counts, groups) if g.spec.window is None):
+            # core/src/worker/model_worker.rs:115-118
+            raise RuntimeError("the cache has room for %d tokens, fewer than max_model_len %d; raise "
+                               "gpu_memory_utilization or lower max_model_len"
+                               % (min(counts) * block_size, max_model_len))
+    else:
+        counts = [int(num_pages)] * len(groups)
+    storage = CacheStorage(model, rt, block_size, counts, num_state_slots=max_num_seqs)
+    executor = ModelExecutor(model, storage, rt, max_model_len)
+    return EngineCore(arch, config, rt, model, storage, executor, max_model_len, block_size)

@@ -1,0 +1,189 @@
+"""The step function: runs a batch of (request, its next tokens) from the cache and returns the
+logits at the wanted places.
+
+The reference's Worker::execute_model (core/src/worker/model_worker.rs:213-264) prepares either a
+prompt batch or a decode batch, runs the model and samples inside the worker. Here the step only
+produces logits: it takes pages for the new tokens, builds the flat batch, runs the model once over
+exactly the tokens it was given, and commits them to the cache. Sampling is a separate call, so that
+trace replay can take the logits.
+"""
+from typing import Dict, Hashable, List, Optional, Sequence, Tuple
+
+import torch
+
+from ..cache.manager import CacheManager, OutOfPages
+from ..cache.storage import CacheStorage
+from ..parts.base import Runtime
+from .batch import GroupView, StepContext, StepEntry
+
+
+class StepError(ValueError):
+    """A step that cannot be run as given (unknown token id, too long a request, bad ``want``)."""
+
+
+def _align4(n: int) -> int:
+    return (n + 3) // 4 * 4
+
+
+class ModelExecutor:
+    def __init__(self, model, storage: CacheStorage, rt: Runtime, max_model_len: int):
+        self.model = model
+        self.storage = storage
+        self.manager: CacheManager = storage.manager
+        self.rt = rt
+        self.max_model_len = int(max_model_len)
+        if self.max_model_len > rt.max_positions:
+            raise ValueError("max_model_len %d exceeds the positions the parts were built for (%d)"
+                             % (self.max_model_len, rt.max_positions))
+        self.vocab_size = model.spec.vocab_size
+        self._pinned: Optional[torch.Tensor] = None
+
+    # ------------------------------------------------------------------ the step
+
+    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """Run one batch. Returns float32 logits [R, V] on the device, rows in the order of the entries
+        and of each entry's ``want``. Raises OutOfPages (and takes nothing) if the cache cannot hold
+        the new tokens."""
+        entries = [e for e in entries if len(e.tokens) > 0]
+        self._validate(entries)
+        if not entries:
+            return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.rt.device)
+        mgr = self.manager
+        added: List[Hashable] = []
+        appended: List[Hashable] = []
+        starts: List[int] = []
+        try:
+            for e in entries:
+                if not mgr.has_request(e.request_id):
+                    mgr.add_request(e.request_id)
+                    added.append(e.request_id)
+                starts.append(mgr.append(e.request_id, len(e.tokens)))
+                appended.append(e.request_id)
+        except OutOfPages:
+            for rid in appended:
+                mgr.rollback(rid)
+            for rid in added:
+                mgr.free_request(rid)
+            raise
+        ctx = self._build_context(entries, starts)
+        logits = self.model.forward(ctx)
+        for e in entries:
+            mgr.commit(e.request_id)
+        return logits
+
+    def release(self, request_id: Hashable) -> None:
+        """The request is finished: its pages and state slot go back."""
+        if self.manager.has_request(request_id):
+            self.manager.free_request(request_id)
+
+    # ------------------------------------------------------------------ helpers
+
+    def _validate(self, entries: Sequence[StepEntry]) -> None:
+        seen = set()
+        for e in entries:
+            if e.request_id in seen:
+                raise StepError("request %r appears twice in one step" % (e.request_id,))
+            seen.add(e.request_id)
+            n = len(e.tokens)
+            for t in e.tokens:
+                if not (0 <= int(t) < self.vocab_size):
+                    raise StepError("request %r: token id %r outside the vocabulary of %d"
+                                    % (e.request_id, t, self.vocab_size))
+            for w in e.want:
+                if not (0 <= int(w) < n):
+                    raise StepError("request %r: wanted place %r outside its %d tokens" % (e.request_id, w, n))
+            held = self.manager.num_tokens(e.request_id) if self.manager.has_request(e.request_id) else 0
+            if held + n > self.max_model_len:
+                raise StepError("request %r would hold %d tokens, more than max_model_len %d"
+                                % (e.request_id, held + n, self.max_model_len))
+
+    def _build_context(self, entries: Sequence[StepEntry], starts: Sequence[int]) -> StepContext:
+        mgr = self.manager
+        S = len(entries)
+        lens = [len(e.tokens) for e in entries]
+        N = sum(lens)
+        seg_starts = [0]
+        for n in lens:
+            seg_starts.append(seg_starts[-1] + n)
+        token_ids: List[int] = []
+        positions: List[int] = []
+        seg_of: List[int] = []
+        logit_rows: List[int] = []
+        state_slots: List[int] = []
+        for s, (e, st) in enumerate(zip(entries, starts)):
+            token_ids.extend(int(t) for t in e.tokens)
+            positions.extend(range(st, st + lens[s]))
+            seg_of.extend([s] * lens[s])
+            logit_rows.extend(seg_starts[s] + int(w) for w in e.want)
+            state_slots.append(mgr.request(e.request_id).state_slot)
+        G = len(mgr.groups)
+        group_slots: List[List[int]] = []
+        group_tables: List[List[List[int]]] = []
+        widths: List[int] = []
+        for gi in range(G):
+            sl: List[int] = []
+            tables = []
+            for e, st, n in zip(entries, starts, lens):
+                sl.extend(mgr.slot_mapping(e.request_id, gi, st, n))
+                tables.append([p if p >= 0 else 0 for p in mgr.block_table(e.request_id, gi)])
+            group_slots.append(sl)
+            group_tables.append(tables)
+            widths.append(max(1, max(len(t) for t in tables)))
+        # one pinned staging buffer, one copy to the device, views into it
+        R = len(logit_rows)
+        sections = [("token_ids", N), ("positions", N), ("seg_of", N), ("seg_starts", S + 1), ("seg_first", S),
+                    ("state_slots", S), ("logit_rows", R)]
+        for gi in range(G):
+            sections.append(("slots%d" % gi, N))
+            sections.append(("tables%d" % gi, S * widths[gi]))
+        offsets: Dict[str, Tuple[int, int]] = {}
+        total = 0
+        for name, n in sections:
+            offsets[name] = (total, n)
+            total += _align4(n)
+        total = max(total, 4)
+        if self._pinned is None or self._pinned.numel() < total:
+            self._pinned = torch.empty(max(total, 4096), dtype=torch.int32,
+                                       pin_memory=self.rt.device.type == "cuda")
+        host = self._pinned[:total]
+
+        def put(name: str, values: Sequence[int]):
+            o, n = offsets[name]
+            if n:
+                host[o:o + n] = torch.tensor(values, dtype=torch.int32)
+
+        put("token_ids", token_ids)
+        put("positions", positions)
+        put("seg_of", seg_of)
+        put("seg_starts", seg_starts)
+        put("seg_first", list(starts))
+        put("state_slots", state_slots)
+        put("logit_rows", logit_rows)
+        for gi in range(G):
+            put("slots%d" % gi, group_slots[gi])
+            flat: List[int] = []
+            for t in group_tables[gi]:
+                flat.extend(t + [0] * (widths[gi] - len(t)))
+            put("tables%d" % gi, flat)
+        if self.rt.device.type == "cuda":
+            # the staging buffer is reused by the next step: wait for earlier copies out of it
+            dev = torch.empty(total, dtype=torch.int32, device=self.rt.device)
+            dev.copy_(host, non_blocking=False)
+        else:
+            dev = host.clone()
+
+        def view(name: str) -> torch.Tensor:
+            o, n = offsets[name]
+            return dev[o:o + n]
+
+        groups = [GroupView(slots=view("slots%d" % gi),
+                            block_tables=view("tables%d" % gi).view(S, widths[gi]),
+                            page_size=mgr.groups[gi].page_size) for gi in range(G)]
+        return StepContext(
+            n_tokens=N, n_segments=S, token_ids=view("token_ids"), positions=view("positions"),
+            seg_of_token=view("seg_of"), seg_starts=view("seg_starts"), seg_first_pos=view("seg_first"),
+            state_slots=view("state_slots"), logit_rows=view("logit_rows"), n_logit_rows=R, groups=groups,
+            host_seg_starts=seg_starts, host_seg_lens=lens, host_seg_first_pos=list(starts),
+            host_state_slots=state_slots, request_ids=[e.request_id for e in entries],
+            max_seg_len=max(lens), max_context=max(st + n for st, n in zip(starts, lens)),
+            all_single=all(n == 1 for n in lens))

@@ -1,0 +1,303 @@
+"""The kernels as Python calls on torch tensors.
+
+Every method checks on the host that shapes, dtypes, devices and contiguity match what the
+kernel and its grid assume, then passes raw device pointers and the current HIP stream to
+the library. Nothing here computes on the CPU and nothing falls back to a library routine
+except where the matrix products say so (``linear``).
+"""
+import ctypes
+from typing import Optional
+
+import torch
+
+from . import library
+
+F32 = 0
+BF16 = 1
+
+
+def _code(dtype: torch.dtype) -> int:
+    if dtype == torch.float32:
+        return F32
+    if dtype == torch.bfloat16:
+        return BF16
+    raise TypeError("kernels take float32 or bfloat16 tensors, got %s" % dtype)
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else ctypes.c_void_p(t.data_ptr())
+
+
+class HipOps:
+    """Kernel calls of the product path. One instance per process is enough."""
+
+    name = "hip"
+
+    def __init__(self):
+        if not torch.cuda.is_available():
+            raise library.KernelLibraryError(
+                "lmsf_amd needs a GPU: torch.cuda.is_available() is False and there is no CPU path")
+        self.lib = library.load_library()
+        buf = ctypes.create_string_buffer(256)
+        if self.lib.lmsf_device_arch(buf, 256) != 0:
+            raise library.KernelLibraryError(library.last_error(self.lib))
+        self.device_arch = buf.value.decode()
+        if not self.device_arch.startswith("gfx950"):
+            raise library.KernelLibraryError(
+                "the kernels are built for gfx950 only; this device reports %r" % self.device_arch)
+        self._bad_flag = None
+        self.use_library_gemm = True   # bfloat16 matrix products of many rows go to the BLAS library
+
+    # ------------------------------------------------------------------ helpers
+
+    def _stream(self):
+        return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def _check(self, rc: int):
+        if rc != 0:
+            raise RuntimeError("lmsf_amd kernel error: " + library.last_error(self.lib))
+
+    @staticmethod
+    def _dev(*tensors):
+        for t in tensors:
+            if t is not None and not t.is_cuda:
+                raise ValueError("kernel operand is not on the GPU")
+
+    @staticmethod
+    def _i32(t: Optional[torch.Tensor], name: str, numel: Optional[int] = None):
+        if t is None:
+            return
+        if t.dtype != torch.int32 or not t.is_contiguous():
+            raise ValueError("%s must be a contiguous int32 tensor" % name)
+        if numel is not None and t.numel() < numel:
+            raise ValueError("%s holds %d elements, %d needed" % (name, t.numel(), numel))
+
+    # ------------------------------------------------------------------ embedding
+
+    def embedding(self, ids: torch.Tensor, table: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+        """float32 [N, H] rows of ``table`` [V, H] selected by int32 ``ids`` [N], times ``scale``."""
+        self._dev(ids, table)
+        self._i32(ids, "ids")
+        if table.dim() != 2 or not table.is_contiguous():
+            raise ValueError("embedding table must be contiguous [V, H]")
+        n, (V, H) = ids.numel(), table.shape
+        out = torch.empty((n, H), dtype=torch.float32, device=table.device)
+        if self._bad_flag is None or self._bad_flag.device != table.device:
+            self._bad_flag = torch.zeros(1, dtype=torch.int32, device=table.device)
+        self._check(self.lib.lmsf_embedding(_ptr(ids), _ptr(table), _code(table.dtype), _ptr(out), n, H, V,
+                                            float(scale), _ptr(self._bad_flag), self._stream()))
+        return out
+
+    def bad_token_seen(self) -> bool:
+        """True if an embedding call since the last query met an id outside the vocabulary."""
+        if self._bad_flag is None:
+            return False
+        bad = bool(self._bad_flag.item())
+        if bad:
+            self._bad_flag.zero_()
+        return bad
+
+    # ------------------------------------------------------------------ norm
+
+    def add_rms_norm(self, branch: Optional[torch.Tensor], residual: Optional[torch.Tensor], weight: torch.Tensor,
+                     eps: float, out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None,
+                     weight_offset: float = 0.0) -> torch.Tensor:
+        """out = rms_norm(branch + residual) * (weight + weight_offset).
+
+        ``residual`` (float32 [N, H]) is updated to the sum in place when both operands are given
+        and ``rows`` is None. ``rows`` (int32 [R]) selects input rows; the output then has R rows.
+        """
+        self._dev(branch, residual, weight, rows)
+        ref = branch if branch is not None else residual
+        if ref is None:
+            raise ValueError("add_rms_norm needs a branch or a residual")
+        if ref.dim() != 2 or not ref.is_contiguous():
+            raise ValueError("add_rms_norm operands must be contiguous [N, H]")
+        N, H = ref.shape
+        if branch is not None and residual is not None and branch.shape != residual.shape:
+            raise ValueError("branch %s and residual %s differ in shape" % (tuple(branch.shape), tuple(residual.shape)))
+        if residual is not None and (residual.dtype != torch.float32 or not residual.is_contiguous()):
+            raise ValueError("the residual stream must be contiguous float32")
+        if weight.shape != (H,) or not weight.is_contiguous():
+            raise ValueError("norm weight must be [%d], got %s" % (H, tuple(weight.shape)))
+        self._i32(rows, "rows")
+        n_out = N if rows is None else rows.numel()
+        out = torch.empty((n_out, H), dtype=out_dtype, device=ref.device)
+        self._check(self.lib.lmsf_add_rms_norm(
+            _ptr(branch), _code(branch.dtype) if branch is not None else F32, _ptr(residual), _ptr(weight),
+            _code(weight.dtype), _ptr(out), _code(out_dtype), _ptr(rows), n_out, H, float(eps),
+            float(weight_offset), self._stream()))
+        return out
+
+    # ------------------------------------------------------------------ rotary + cache write
+
+    def rope_cache_write(self, qkv: torch.Tensor, nh: int, nkv: int, d: int, positions: Optional[torch.Tensor],
+                         table: Optional[torch.Tensor], rot_dim: int, neox: bool, slots: Optional[torch.Tensor],
+                         k_pages: Optional[torch.Tensor], v_pages: Optional[torch.Tensor]) -> None:
+        """Rotate the q and k heads of the fused ``qkv`` [N, (nh + 2 nkv) d] in place and store k, v in
+        the pages at ``slots``. ``table`` None: no rotation. ``slots`` None: no cache write."""
+        self._dev(qkv, positions, table, slots, k_pages, v_pages)
+        if qkv.dim() != 2 or qkv.stride(1) != 1 or qkv.shape[1] != (nh + 2 * nkv) * d:
+            raise ValueError("qkv must be [N, %d] with unit column stride, got %s" % ((nh + 2 * nkv) * d,
+                                                                                      tuple(qkv.shape)))
+        N = qkv.shape[0]
+        es = qkv.element_size()
+        max_pos = 0
+        if table is not None:
+            if table.dtype != torch.float32 or table.dim() != 2 or table.shape[1] != rot_dim or not table.is_contiguous():
+                raise ValueError("rotary table must be contiguous float32 [max_pos, %d]" % rot_dim)
+            self._i32(positions, "positions", N)
+            if positions is None:
+                raise ValueError("rotation needs positions")
+            max_pos = table.shape[0]
+        num_pages, ps = 0, 1
+        if slots is not None:
+            self._i32(slots, "slots", N)
+            for name, pg in (("k_pages", k_pages), ("v_pages", v_pages)):
+                if pg is None or pg.dim() != 4 or pg.shape[1] != nkv or pg.shape[3] != d or not pg.is_contiguous() \
+                        or pg.dtype != qkv.dtype:
+                    raise ValueError("%s must be contiguous [pages, %d, page_size, %d] of %s" % (name, nkv, d, qkv.dtype))
+            if k_pages.shape != v_pages.shape:
+                raise ValueError("k_pages and v_pages differ in shape")
+            num_pages, ps = k_pages.shape[0], k_pages.shape[2]
+        base = qkv.data_ptr()
+        q = ctypes.c_void_p(base)
+        k = ctypes.c_void_p(base + nh * d * es)
+        v = ctypes.c_void_p(base + (nh + nkv) * d * es)
+        self._check(self.lib.lmsf_rope_cache_write(
+            q, k, v, _code(qkv.dtype), N, qkv.stride(0), _ptr(positions), _ptr(table), rot_dim, 1 if neox else 0,
+            max_pos, _ptr(slots), _ptr(k_pages), _ptr(v_pages), num_pages, nh, nkv, d, ps, self._stream()))
+
+    # ------------------------------------------------------------------ attention
+
+    def paged_attention(self, q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
+                        block_tables: torch.Tensor, seg: torch.Tensor, pos: torch.Tensor, nh: int, nkv: int, d: int,
+                        scale: float, window: int = 0, batch=None) -> torch.Tensor:
+        """Attention of every query token over the cached keys of its request.
+
+        ``q`` is [N, >= nh*d] with unit column stride (it may be the fused QKV buffer, of which the
+        first nh*d columns are read). ``block_tables`` int32 [S, W]; ``seg``, ``pos`` int32 [N].
+        ``batch`` carries host-side facts about the step for the choice of kernel.
+        Returns [N, nh*d] in q's dtype.
+        """
+        self._dev(q, k_pages, v_pages, block_tables, seg, pos)
+        if q.dim() != 2 or q.stride(1) != 1 or q.shape[1] < nh * d:
+            raise ValueError("q must be [N, >= %d] with unit column stride" % (nh * d))
+        N = q.shape[0]
+        for name, pg in (("k_pages", k_pages), ("v_pages", v_pages)):
+            if pg.dim() != 4 or pg.shape[1] != nkv or pg.shape[3] != d or not pg.is_contiguous() or pg.dtype != q.dtype:
+                raise ValueError("%s must be contiguous [pages, %d, page_size, %d] of %s" % (name, nkv, d, q.dtype))
+        if k_pages.shape != v_pages.shape:
+            raise ValueError("k_pages and v_pages differ in shape")
+        if block_tables.dim() != 2:
+            raise ValueError("block_tables must be [segments, width]")
+        self._i32(block_tables, "block_tables")
+        self._i32(seg, "seg", N)
+        self._i32(pos, "pos", N)
+        out = torch.empty((N, nh * d), dtype=q.dtype, device=q.device)
+        num_pages, ps = k_pages.shape[0], k_pages.shape[2]
+        self._check(self.lib.lmsf_paged_attention_generic(
+            _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pages), _ptr(v_pages), num_pages,
+            _ptr(block_tables), block_tables.shape[1], _ptr(seg), _ptr(pos), N, nh, nkv, d, ps, float(scale),
+            int(window or 0), _code(q.dtype), self._stream()))
+        return out
+
+    # ------------------------------------------------------------------ feed-forward
+
+    def gated_act(self, gu: torch.Tensor, kind: str = "silu") -> torch.Tensor:
+        """act(gu[:, :I]) * gu[:, I:] for gu [N, 2I]; kind "silu" or "gelu"."""
+        self._dev(gu)
+        if gu.dim() != 2 or gu.stride(1) != 1 or gu.shape[1] % 2 != 0:
+            raise ValueError("gated_act input must be [N, 2I] with unit column stride")
+        kinds = {"silu": 0, "gelu": 1}
+        if kind not in kinds:
+            raise ValueError("unknown activation %r (known: %s)" % (kind, ", ".join(kinds)))
+        N, I = gu.shape[0], gu.shape[1] // 2
+        out = torch.empty((N, I), dtype=gu.dtype, device=gu.device)
+        self._check(self.lib.lmsf_gated_act(_ptr(gu), _ptr(out), _code(gu.dtype), N, I, gu.stride(0), kinds[kind],
+                                            self._stream()))
+        return out
+
+    # ------------------------------------------------------------------ matrix products
+
+    def linear(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
+               out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+        """y = x weight^T (+ bias); x [M, K], weight [N, K]; y [M, N] in ``out_dtype`` (default x's).
+
+        float32 operands always run the float32 multiply-add kernel. bfloat16 products with bfloat16
+        output and many rows go to the BLAS library, as the reference's do
+        (core/src/model_executor/layers/linear.rs:44-106 calls cuBLASLt); the rest run here.
+        """
+        self._dev(x, weight, bias)
+        if x.dim() != 2 or weight.dim() != 2 or x.shape[1] != weight.shape[1]:
+            raise ValueError("linear: x %s and weight %s do not match" % (tuple(x.shape), tuple(weight.shape)))
+        if x.stride(1) != 1 or weight.stride(1) != 1:
+            raise ValueError("linear: operands need unit column stride")
+        M, K = x.shape
+        N = weight.shape[0]
+        if bias is not None and (bias.shape != (N,) or bias.dtype != weight.dtype or not bias.is_contiguous()):
+            raise ValueError("linear: bias must be [%d] of the weight's dtype" % N)
+        out_dtype = out_dtype or x.dtype
+        if (self.use_library_gemm and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
+                and out_dtype == torch.bfloat16 and M > 64):
+            return torch.nn.functional.linear(x, weight, bias)
+        y = torch.empty((M, N), dtype=out_dtype, device=x.device)
+        self._check(self.lib.lmsf_gemm_plain(_ptr(x), _code(x.dtype), x.stride(0), _ptr(weight), _code(weight.dtype),
+                                             weight.stride(0), _ptr(bias), _ptr(y), _code(out_dtype), y.stride(0),
+                                             M, N, K, self._stream()))
+        return y
+
+    # ------------------------------------------------------------------ sampling
+
+    def sample(self, logits: torch.Tensor, temperature: Optional[torch.Tensor] = None,
+               top_k: Optional[torch.Tensor] = None, top_p: Optional[torch.Tensor] = None,
+               min_p: Optional[torch.Tensor] = None, seeds: Optional[torch.Tensor] = None,
+               draws: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """One token per row of float32 ``logits`` [R, V]; int32 [R]. All parameters are per-row device
+        tensors: temperature/top_p/min_p float32, top_k int32, seeds int64, draws int32."""
+        self._dev(logits, temperature, top_k, top_p, min_p, seeds, draws)
+        if logits.dim() != 2 or logits.dtype != torch.float32 or logits.stride(1) != 1:
+            raise ValueError("sample: logits must be float32 [R, V] with unit column stride")
+        R, V = logits.shape
+        for name, t, dt in (("temperature", temperature, torch.float32), ("top_k", top_k, torch.int32),
+                            ("top_p", top_p, torch.float32), ("min_p", min_p, torch.float32),
+                            ("seeds", seeds, torch.int64), ("draws", draws, torch.int32)):
+            if t is not None and (t.dtype != dt or t.numel() != R or not t.is_contiguous()):
+                raise ValueError("sample: %s must be a contiguous %s tensor of %d elements" % (name, dt, R))
+        out = torch.empty((R,), dtype=torch.int32, device=logits.device)
+        self._check(self.lib.lmsf_sample(_ptr(logits), logits.stride(0), R, V, _ptr(temperature), _ptr(top_k),
+                                         _ptr(top_p), _ptr(min_p), _ptr(seeds), _ptr(draws), _ptr(out),
+                                         self._stream()))
+        return out
+
+    def apply_penalties(self, logits: torch.Tensor, tokens: torch.Tensor, offsets: torch.Tensor,
+                        prompt_lens: torch.Tensor, presence: torch.Tensor, frequency: torch.Tensor,
+                        repetition: torch.Tensor) -> None:
+        """Presence, frequency and repetition penalties on float32 ``logits`` [R, V], in place.
+        ``tokens`` int32: each row's prompt then output tokens, concatenated; ``offsets`` int32 [R+1];
+        ``prompt_lens`` int32 [R]; the penalties float32 [R]."""
+        self._dev(logits, tokens, offsets, prompt_lens, presence, frequency, repetition)
+        if logits.dim() != 2 or logits.dtype != torch.float32 or logits.stride(1) != 1:
+            raise ValueError("apply_penalties: logits must be float32 [R, V] with unit column stride")
+        R, V = logits.shape
+        self._i32(tokens, "tokens")
+        self._i32(offsets, "offsets", R + 1)
+        self._i32(prompt_lens, "prompt_lens", R)
+        for name, t in (("presence", presence), ("frequency", frequency), ("repetition", repetition)):
+            if t.dtype != torch.float32 or t.numel() != R or not t.is_contiguous():
+                raise ValueError("apply_penalties: %s must be contiguous float32 [%d]" % (name, R))
+        counts = torch.zeros((R, V), dtype=torch.int32, device=logits.device)
+        self._check(self.lib.lmsf_apply_penalties(_ptr(logits), logits.stride(0), R, V, _ptr(tokens), _ptr(offsets),
+                                                  _ptr(prompt_lens), _ptr(counts), _ptr(presence), _ptr(frequency),
+                                                  _ptr(repetition), self._stream()))
+
+
+_default_ops: Optional[HipOps] = None
+
+
+def get_ops() -> HipOps:
+    """The process-wide kernel object; raises if the GPU or the library is missing."""
+    global _default_ops
+    if _default_ops is None:
+        _default_ops = HipOps()
+    return _default_ops

@@ -1,0 +1,66 @@
+"""Linear layers, with the fusion of several checkpoint matrices into one product.
+
+y = x W^T (+ b), W stored [out, in]. The reference fuses q, k, v into one weight of
+(nh + 2 nkv) d rows (core/src/model_executor/layers/linear.rs:499-728, row offsets :573-583) and
+gate, up into one of 2 I rows (:325-497, offsets :364-366) by copying the checkpoint tensors into
+row slices of a zeroed buffer at load time; the same is done here, for weights and biases alike.
+"""
+from typing import Callable, Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+from .base import Part, Runtime, TensorDecl
+
+
+class FusedLinear(Part):
+    """One matrix product whose weight rows are the concatenation of several checkpoint tensors.
+
+    ``sources`` is a list of (checkpoint sub-name, rows): the tensor ``prefix.sub-name.weight`` has
+    shape [rows, in_features] and, with ``bias``, ``prefix.sub-name.bias`` has [rows]."""
+
+    def __init__(self, prefix: str, rt: Runtime, in_features: int, sources: Sequence[Tuple[str, int]],
+                 bias: bool = False):
+        super().__init__(prefix, rt)
+        if not sources:
+            raise ValueError("FusedLinear needs at least one source")
+        self.in_features = int(in_features)
+        self.sources = [(str(n), int(r)) for n, r in sources]
+        self.out_features = sum(r for _, r in self.sources)
+        self.has_bias = bool(bias)
+        self.weight: Optional[torch.Tensor] = None
+        self.bias: Optional[torch.Tensor] = None
+
+    def _name(self, sub: str, what: str) -> str:
+        return "%s.%s.%s" % (self.prefix, sub, what) if self.prefix else "%s.%s" % (sub, what)
+
+    def checkpoint_tensors(self) -> Dict[str, TensorDecl]:
+        out = {}
+        for sub, rows in self.sources:
+            out[self._name(sub, "weight")] = TensorDecl((rows, self.in_features))
+            if self.has_bias:
+                out[self._name(sub, "bias")] = TensorDecl((rows,))
+        return out
+
+    @staticmethod
+    def _cat(ts: List[torch.Tensor]) -> torch.Tensor:
+        if len(ts) == 1:
+            return ts[0].contiguous()
+        if any(t.dtype == torch.float32 for t in ts):
+            ts = [t.to(torch.float32) for t in ts]
+        return torch.cat(ts, dim=0).contiguous()
+
+    def load_weights(self, fetch: Callable[[str], torch.Tensor]) -> None:
+        self.weight = self._cat([fetch(self._name(sub, "weight")) for sub, _ in self.sources])
+        if self.has_bias:
+            b = self._cat([fetch(self._name(sub, "bias")) for sub, _ in self.sources])
+            self.bias = b.to(self.weight.dtype)
+
+    def forward(self, x: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+        return self.rt.ops.linear(x, self.weight, self.bias, out_dtype=out_dtype)
+
+
+class Linear(FusedLinear):
+    """A single checkpoint matrix ``prefix.name.weight`` [out_features, in_features]."""
+
+    def __init__(self, prefix: str, rt: Runtime, name: str, in_features: int, out_features: int, bias: bool = False):
+        super().__init__(prefix, rt, in_features, [(name, out_features)], bias)
