@@ -22,6 +22,15 @@ class Architecture:
 
 
 _ARCHITECTURES: Dict[str, Architecture] = {}
+_builtin_loaded = False
+
+
+def _load_builtin() -> None:
+    """Import the package's own architectures once, so that they are registered before a lookup."""
+    global _builtin_loaded
+    if not _builtin_loaded:
+        _builtin_loaded = True
+        from .. import models  # noqa: F401
 
 
 def register_architecture(name: str, model_type: str, config_class: type,
@@ -39,10 +48,12 @@ def unregister_architecture(name: str) -> None:
 
 
 def registered_architectures() -> Tuple[str, ...]:
+    _load_builtin()
     return tuple(sorted(_ARCHITECTURES))
 
 
 def get_architecture(name: str) -> Architecture:
+    _load_builtin()
     try:
         return _ARCHITECTURES[name]
     except KeyError:
@@ -53,6 +64,7 @@ def get_architecture(name: str) -> Architecture:
 def resolve_architecture(config_dict: Dict[str, Any]) -> Architecture:
     """The architecture that a config.json names: "architectures"[0], else "model_type"
     (case-insensitive, as the reference's strum enum, model_factory.rs:44-50)."""
+    _load_builtin()
     archs = config_dict.get("architectures")
     if isinstance(archs, (list, tuple)) and archs:
         return get_architecture(str(archs[0]))

@@ -1,0 +1,87 @@
+"""Trace replay: feeds given token ids through the model step by step and writes logits.
+
+It samples nothing and has no forward pass, cache or loader of its own: it drives the model,
+step function, cache manager and kernels that generation uses. The reference has nothing like
+it (its closest is the hand-driven step loop of example/examples/llm_engine_example.rs:65-151).
+
+    trace_run --model DIR --dtype bfloat16|float32 --out DIR --max-tokens N
+
+Steps come on standard input, one JSON object a line:
+
+    {"step": 0, "entries": [{"id": "a", "tokens": [5, 17, 3], "want": [0, 2]}], "end": []}
+
+``entries`` gives each request's next tokens and the places among them whose logits are wanted;
+all entries of a step run as one batch. ``end`` lists requests that are finished after the step;
+their pages go back to the pool. If anything is wanted the step writes ``<out>/<step>.f32``:
+little-endian float32 [wanted, vocab], in the order of the entries and of ``want``. After every
+step a line ``done <step>`` is printed and flushed.
+"""
+import argparse
+import json
+import os
+import sys
+import tempfile
+import time
+
+PAGE_SIZE = 16
+
+
+def _say(msg: str) -> None:
+    sys.stderr.write("[trace_run] %s\n" % msg)
+    sys.stderr.flush()
+
+
+def _usable_home() -> None:
+    """Libraries may want to write below HOME; with an empty or unwritable one, point it at a temporary folder."""
+    home = os.environ.get("HOME", "")
+    if not home or not os.path.isdir(home) or not os.access(home, os.W_OK):
+        os.environ["HOME"] = tempfile.mkdtemp(prefix="lmsf_home_")
+
+
+def main(argv=None) -> int:
+    ap = argparse.ArgumentParser(prog="trace_run", description=__doc__.split("\n\n")[0])
+    ap.add_argument("--model", required=True, help="folder with config.json and model.safetensors")
+    ap.add_argument("--dtype", required=True, choices=["bfloat16", "float32"])
+    ap.add_argument("--out", required=True, help="folder the logits files are written to")
+    ap.add_argument("--max-tokens", type=int, required=True,
+                    help="most tokens that live requests hold at any time; the cache pool is made for this many")
+    ap.add_argument("--device", default="cuda:0")
+    args = ap.parse_args(argv)
+    if args.max_tokens <= 0:
+        ap.error("--max-tokens must be > 0")
+    _usable_home()
+    os.makedirs(args.out, exist_ok=True)
+    t0 = time.time()
+    _say("starting (first import of torch can take a minute or two)")
+    import numpy as np
+    import torch  # noqa: F401
+
+    from lmsf_amd.engine import StepEntry, load_engine_core
+
+    _say("torch ready after %.0f s; loading kernels and %s" % (time.time() - t0, args.model))
+    num_pages = -(-args.max_tokens // PAGE_SIZE)
+    core = load_engine_core(args.model, dtype=args.dtype, block_size=PAGE_SIZE, num_pages=num_pages,
+                            max_num_seqs=64, device=args.device)
+    _say("model %s ready after %.0f s: %s, %d pages of %d tokens" % (
+        core.arch.name, time.time() - t0, args.dtype, num_pages, PAGE_SIZE))
+    executor = core.executor
+    for line in sys.stdin:
+        line = line.strip()
+        if not line:
+            continue
+        obj = json.loads(line)
+        step = obj["step"]
+        entries = [StepEntry(e["id"], e["tokens"], e.get("want", [])) for e in obj.get("entries", [])]
+        logits = executor.step(entries)
+        if logits.shape[0] > 0:
+            arr = logits.detach().to("cpu").numpy().astype("<f4", copy=False)
+            arr.tofile(os.path.join(args.out, "%s.f32" % step))
+        for rid in obj.get("end", []):
+            executor.release(rid)
+        sys.stdout.write("done %s\n" % step)
+        sys.stdout.flush()
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,315 @@
+"""Each HIP kernel alone against its plain torch reference (tests/torch_ops.py), at sizes other
+than the engine's tiny models: head sizes in steps of 16, odd numbers of heads and groups,
+widths and vocabularies that are no power of two, float32 and bfloat16."""
+import math
+
+import pytest
+import torch
+
+from torch_ops import TorchOps
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from lmsf_amd.ops import get_ops
+    return get_ops()
+
+
+@pytest.fixture(scope="module")
+def ref():
+    return TorchOps()
+
+
+def dev(t):
+    return t.to("cuda:0")
+
+
+def tol(dtype):
+    return dict(atol=2e-5, rtol=2e-5) if dtype == torch.float32 else dict(atol=2e-2, rtol=2e-2)
+
+
+def test_library_is_loaded(ops):
+    from lmsf_amd.ops import library_path
+    assert library_path() and library_path().endswith("liblmsf_hip.so")
+    assert ops.device_arch.startswith("gfx950")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("V,H,N", [(331, 80, 7), (1000, 4096, 33), (50, 17, 1)])
+def test_embedding(ops, ref, dtype, V, H, N):
+    g = torch.Generator().manual_seed(V + H)
+    table = dev(torch.randn(V, H, generator=g).to(dtype))
+    ids = dev(torch.randint(0, V, (N,), generator=g, dtype=torch.int32))
+    out = ops.embedding(ids, table, 1.5)
+    assert out.dtype == torch.float32
+    assert torch.equal(out, ref.embedding(ids, table, 1.5))
+
+
+def test_embedding_flags_bad_id(ops):
+    table = dev(torch.randn(10, 8))
+    out = ops.embedding(dev(torch.tensor([3, 11, -1], dtype=torch.int32)), table)
+    assert ops.bad_token_seen()
+    assert not ops.bad_token_seen()
+    assert torch.equal(out[1], torch.zeros(8, device="cuda:0")) and torch.equal(out[0], table[3])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("N,H", [(5, 80), (3, 4096), (2, 5000), (9, 17)])
+def test_add_rms_norm(ops, ref, dtype, N, H):
+    g = torch.Generator().manual_seed(N * H)
+    branch = dev((torch.randn(N, H, generator=g) * 3).to(dtype))
+    res = dev(torch.randn(N, H, generator=g))
+    w = dev(torch.randn(H, generator=g).to(dtype))
+    for eps, off in ((1e-5, 0.0), (1e-6, 1.0)):
+        r1, r2 = res.clone(), res.clone()
+        a = ops.add_rms_norm(branch, r1, w, eps, dtype, weight_offset=off)
+        b = ref.add_rms_norm(branch, r2, w, eps, dtype, weight_offset=off)
+        assert torch.allclose(r1, r2, atol=1e-6, rtol=1e-6)
+        assert torch.allclose(a.float(), b.float(), **tol(dtype))
+    # norm of the stream alone, of a branch alone, and gathered rows
+    a = ops.add_rms_norm(None, res.clone(), w, 1e-5, dtype)
+    assert torch.allclose(a.float(), ref.add_rms_norm(None, res.clone(), w, 1e-5, dtype).float(), **tol(dtype))
+    a = ops.add_rms_norm(branch, None, w, 1e-5, dtype)
+    assert torch.allclose(a.float(), ref.add_rms_norm(branch, None, w, 1e-5, dtype).float(), **tol(dtype))
+    rows = dev(torch.tensor([N - 1, 0], dtype=torch.int32))
+    r1 = res.clone()
+    a = ops.add_rms_norm(branch, r1, w, 1e-5, dtype, rows=rows)
+    assert torch.equal(r1, res)          # a gather leaves the stream alone
+    assert torch.allclose(a.float(), ref.add_rms_norm(branch, res.clone(), w, 1e-5, dtype, rows=rows).float(),
+                          **tol(dtype))
+    # float32 weight with bfloat16 activations
+    if dtype == torch.bfloat16:
+        a = ops.add_rms_norm(branch, res.clone(), w.float(), 1e-5, dtype)
+        assert torch.allclose(a.float(), ref.add_rms_norm(branch, res.clone(), w.float(), 1e-5, dtype).float(),
+                              **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,d,rot,neox,ps", [(5, 5, 48, 48, True, 16), (6, 2, 64, 32, False, 8),
+                                                 (8, 1, 128, 128, True, 16), (3, 3, 16, 16, True, 4)])
+def test_rope_cache_write(ops, ref, dtype, nh, nkv, d, rot, neox, ps):
+    g = torch.Generator().manual_seed(nh * d)
+    N, max_pos, pages = 11, 64, 9
+    qkv = dev(torch.randn(N, (nh + 2 * nkv) * d, generator=g).to(dtype))
+    pos = dev(torch.randint(0, max_pos, (N,), generator=g, dtype=torch.int32))
+    ang = torch.arange(max_pos, dtype=torch.float32)[:, None] * torch.rand(rot // 2, generator=g)[None, :]
+    table = dev(torch.cat([ang.cos(), ang.sin()], dim=1).contiguous())
+    slots = torch.randperm(pages * ps, generator=g)[:N].to(torch.int32)
+    slots[3] = -1
+    slots = dev(slots)
+    shape = (pages, nkv, ps, d)
+    k1, v1 = dev(torch.zeros(shape, dtype=dtype)), dev(torch.zeros(shape, dtype=dtype))
+    k2, v2 = k1.clone(), v1.clone()
+    a, b = qkv.clone(), qkv.clone()
+    ops.rope_cache_write(a, nh, nkv, d, pos, table, rot, neox, slots, k1, v1)
+    ref.rope_cache_write(b, nh, nkv, d, pos, table, rot, neox, slots, k2, v2)
+    assert torch.allclose(a.float(), b.float(), **tol(dtype))
+    assert torch.allclose(k1.float(), k2.float(), **tol(dtype)) and torch.equal(v1, v2)
+    # cache write alone and rotation alone
+    a, b = qkv.clone(), qkv.clone()
+    k1.zero_(); v1.zero_(); k2.zero_(); v2.zero_()
+    ops.rope_cache_write(a, nh, nkv, d, None, None, 0, True, slots, k1, v1)
+    ref.rope_cache_write(b, nh, nkv, d, None, None, 0, True, slots, k2, v2)
+    assert torch.equal(a, qkv) and torch.equal(k1, k2) and torch.equal(v1, v2)
+    ops.rope_cache_write(a, nh, nkv, d, pos, table, rot, neox, None, None, None)
+    ref.rope_cache_write(b, nh, nkv, d, pos, table, rot, neox, None, None, None)
+    assert torch.allclose(a.float(), b.float(), **tol(dtype))
+
+
+def _paged_case(dtype, nh, nkv, d, ps, seg_lens, ctx_lens, seed, spike=False):
+    """Segments with ``seg_lens`` query tokens each at the end of contexts of ``ctx_lens`` tokens; pages in
+    a scrambled order. Returns the kernel's arguments."""
+    g = torch.Generator().manual_seed(seed)
+    S = len(seg_lens)
+    blocks = [-(-c // ps) for c in ctx_lens]
+    total = sum(blocks) + 3
+    perm = torch.randperm(total, generator=g).tolist()
+    W = max(blocks)
+    bt = torch.zeros(S, W, dtype=torch.int32)
+    at = 0
+    for s in range(S):
+        for b in range(blocks[s]):
+            bt[s, b] = perm[at]
+            at += 1
+    k_pages = torch.randn(total, nkv, ps, d, generator=g)
+    v_pages = torch.randn(total, nkv, ps, d, generator=g)
+    N = sum(seg_lens)
+    q = torch.randn(N, nh * d + 8, generator=g)       # wider than nh*d: a strided view, like the fused QKV
+    seg, pos = [], []
+    for s in range(S):
+        for i in range(seg_lens[s]):
+            seg.append(s)
+            pos.append(ctx_lens[s] - seg_lens[s] + i)
+    if spike:
+        # one far key per kv head stands out: scale it and the matching query direction
+        for s in range(S):
+            j = 1 if ctx_lens[s] > 1 else 0
+            page, off = int(bt[s, j // ps]), j % ps
+            k_pages[page, :, off, :] *= 6.0
+    return (dev(q.to(dtype)), dev(k_pages.to(dtype)), dev(v_pages.to(dtype)), dev(bt),
+            dev(torch.tensor(seg, dtype=torch.int32)), dev(torch.tensor(pos, dtype=torch.int32)))
+
+
+ATT_SHAPES = [
+    # nh, nkv, d, page size, query tokens per segment, context per segment
+    (4, 2, 16, 8, [1, 7, 33], [1, 7, 33]),
+    (5, 5, 48, 16, [2, 1, 1], [300, 17, 256]),
+    (8, 1, 32, 16, [64, 1], [64, 513]),
+    (6, 3, 80, 4, [3, 5], [40, 5]),
+    (32, 8, 128, 16, [1, 1, 1, 16], [700, 1, 257, 16]),
+    (2, 1, 256, 32, [9], [70]),
+]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", ATT_SHAPES)
+@pytest.mark.parametrize("window", [0, 24])
+def test_paged_attention(ops, ref, dtype, shape, window):
+    nh, nkv, d, ps, seg_lens, ctx_lens = shape
+    q, kp, vp, bt, seg, pos = _paged_case(dtype, nh, nkv, d, ps, seg_lens, ctx_lens, seed=nh * d + ps, spike=True)
+    scale = 1.0 / math.sqrt(d)
+    a = ops.paged_attention(q, kp, vp, bt, seg, pos, nh, nkv, d, scale, window)
+    b = ref.paged_attention(q, kp, vp, bt, seg, pos, nh, nkv, d, scale, window)
+    assert a.shape == (q.shape[0], nh * d)
+    assert torch.allclose(a.float(), b.float(), **tol(dtype)), (a.float() - b.float()).abs().max()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_paged_attention_reduces_to_library_softmax(ops, dtype):
+    """One request, one head, no rotation: the kernel must equal softmax(q k^T / sqrt d) v of torch."""
+    d, ps, T = 64, 16, 50
+    g = torch.Generator().manual_seed(1)
+    q = torch.randn(T, d, generator=g).to(dtype)
+    k = torch.randn(T, d, generator=g).to(dtype)
+    v = torch.randn(T, d, generator=g).to(dtype)
+    pages = -(-T // ps)
+    kp = torch.zeros(pages, 1, ps, d, dtype=dtype)
+    vp = torch.zeros(pages, 1, ps, d, dtype=dtype)
+    kp.view(pages * ps, d)[:T] = k
+    vp.view(pages * ps, d)[:T] = v
+    bt = torch.arange(pages, dtype=torch.int32)[None, :]
+    out = ops.paged_attention(dev(q), dev(kp), dev(vp), dev(bt), dev(torch.zeros(T, dtype=torch.int32)),
+                              dev(torch.arange(T, dtype=torch.int32)), 1, 1, d, 1.0 / math.sqrt(d))
+    want = torch.nn.functional.scaled_dot_product_attention(q.float()[None], k.float()[None], v.float()[None],
+                                                            is_causal=True)[0]
+    assert torch.allclose(out.float().cpu(), want, **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("kind", ["silu", "gelu"])
+@pytest.mark.parametrize("N,I", [(3, 176), (17, 14336), (1, 5)])
+def test_gated_act(ops, ref, dtype, kind, N, I):
+    g = torch.Generator().manual_seed(I)
+    gu = dev((torch.randn(N, 2 * I, generator=g) * 4).to(dtype))
+    a, b = ops.gated_act(gu, kind), ref.gated_act(gu, kind)
+    assert torch.allclose(a.float(), b.float(), **tol(dtype))
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 1000, 128), (7, 331, 80), (65, 64, 176), (130, 257, 1030), (33, 4096, 4096)])
+@pytest.mark.parametrize("bias", [False, True])
+def test_linear_float32_is_exact_float32(ops, M, N, K, bias):
+    """The float32 product must agree with a float64 product to float32 rounding of a K-term sum: no
+    reduced-precision matrix mode."""
+    g = torch.Generator().manual_seed(M * N + K)
+    x, w = torch.randn(M, K, generator=g), torch.randn(N, K, generator=g)
+    b = torch.randn(N, generator=g) if bias else None
+    y = ops.linear(dev(x), dev(w), dev(b) if bias else None)
+    want = x.double() @ w.double().t() + (b.double() if bias else 0)
+    err = (y.cpu().double() - want).abs().max().item()
+    assert err < 2e-6 * math.sqrt(K) * 4, err
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 1000, 128), (7, 331, 80), (64, 640, 352), (65, 512, 176), (300, 1024, 512)])
+@pytest.mark.parametrize("bias", [False, True])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+def test_linear_bfloat16(ops, ref, M, N, K, bias, out_dtype):
+    g = torch.Generator().manual_seed(M + N + K)
+    x = dev(torch.randn(M, K, generator=g).to(torch.bfloat16))
+    w = dev((torch.randn(N, K, generator=g) * 0.1).to(torch.bfloat16))
+    b = dev(torch.randn(N, generator=g).to(torch.bfloat16)) if bias else None
+    y = ops.linear(x, w, b, out_dtype=out_dtype)
+    want = ref.linear(x, w, b, out_dtype=torch.float32)
+    assert y.dtype == out_dtype
+    t = dict(atol=1e-4, rtol=1e-4) if out_dtype == torch.float32 else dict(atol=3e-2, rtol=1.6e-2)
+    assert torch.allclose(y.float(), want, **t), (y.float() - want).abs().max()
+
+
+def test_linear_mixed_storage(ops, ref):
+    """A weight stored in 32 bits stays so and still multiplies bfloat16 activations."""
+    g = torch.Generator().manual_seed(5)
+    x = dev(torch.randn(5, 96, generator=g).to(torch.bfloat16))
+    w = dev(torch.randn(40, 96, generator=g))
+    y = ops.linear(x, w)
+    assert y.dtype == torch.bfloat16
+    assert torch.allclose(y.float(), ref.linear(x, w, None, torch.float32), atol=5e-2, rtol=1e-2)
+
+
+@pytest.mark.parametrize("V", [256, 1000, 128256])
+def test_sample_greedy_and_seeded(ops, ref, V):
+    g = torch.Generator().manual_seed(V)
+    R = 6
+    logits = torch.randn(R, V, generator=g) * 3
+    logits[0, 5] = logits[0, 77] = 50.0                 # a tie: the lowest index wins
+    lg = dev(logits)
+    assert ops.sample(lg).tolist() == torch.argmax(logits, dim=-1).tolist() and ops.sample(lg)[0].item() == 5
+    temp = dev(torch.tensor([0.0, 0.7, 1.0, 1.3, 0.7, 0.7]))
+    top_k = dev(torch.tensor([-1, -1, 5, 50, -1, 3], dtype=torch.int32))
+    top_p = dev(torch.tensor([1.0, 1.0, 1.0, 0.9, 0.5, 0.8]))
+    min_p = dev(torch.tensor([0.0, 0.0, 0.0, 0.0, 0.0, 0.05]))
+    seeds = dev(torch.tensor([1, 2, 3, 4, 5, 2 ** 40 + 17], dtype=torch.int64))
+    for draw in range(3):
+        draws = dev(torch.full((R,), draw, dtype=torch.int32))
+        a = ops.sample(lg, temp, top_k, top_p, min_p, seeds, draws)
+        b = ref.sample(lg, temp, top_k, top_p, min_p, seeds, draws)
+        assert a.tolist() == b.tolist(), (draw, a.tolist(), b.tolist())
+
+
+def test_sample_does_not_depend_on_batch(ops):
+    g = torch.Generator().manual_seed(9)
+    logits = dev(torch.randn(4, 777, generator=g))
+    temp = dev(torch.full((4,), 0.9))
+    seeds = dev(torch.tensor([11, 12, 13, 14], dtype=torch.int64))
+    draws = dev(torch.tensor([0, 5, 2, 9], dtype=torch.int32))
+    whole = ops.sample(logits, temp, None, None, None, seeds, draws).tolist()
+    for r in range(4):
+        one = ops.sample(logits[r:r + 1], temp[r:r + 1], None, None, None, seeds[r:r + 1], draws[r:r + 1]).tolist()
+        assert one == [whole[r]]
+
+
+def test_sample_frequencies_follow_softmax(ops):
+    """Over many draws the tokens come with the probabilities softmax(logits / T) gives (chi-square)."""
+    V, n = 12, 4000
+    g = torch.Generator().manual_seed(3)
+    row = torch.randn(V, generator=g)
+    T = 0.8
+    p = torch.softmax(row / T, dim=-1)
+    lg = dev(row[None, :].repeat(n, 1).contiguous())
+    out = ops.sample(lg, dev(torch.full((n,), T)), None, None, None,
+                     dev(torch.full((n,), 123, dtype=torch.int64)), dev(torch.arange(n, dtype=torch.int32)))
+    counts = torch.bincount(out.cpu().long(), minlength=V).float()
+    chi2 = (((counts - n * p) ** 2) / (n * p)).sum().item()
+    assert chi2 < 40.0, chi2           # 11 degrees of freedom: P(chi2 > 40) < 4e-5
+
+
+def test_apply_penalties(ops, ref):
+    g = torch.Generator().manual_seed(4)
+    R, V = 3, 500
+    logits = torch.randn(R, V, generator=g)
+    rows = [([1, 2, 3, 3], [3, 4, 4, 4]), ([7], []), ([], [9, 9, 499])]
+    tokens, offsets, plens = [], [0], []
+    for pr, out in rows:
+        tokens += pr + out
+        offsets.append(len(tokens))
+        plens.append(len(pr))
+    args = [dev(torch.tensor(tokens, dtype=torch.int32)), dev(torch.tensor(offsets, dtype=torch.int32)),
+            dev(torch.tensor(plens, dtype=torch.int32)), dev(torch.tensor([0.2, 0.0, 1.0])),
+            dev(torch.tensor([0.1, 0.0, 0.5])), dev(torch.tensor([1.3, 1.0, 0.8]))]
+    a, b = dev(logits.clone()), dev(logits.clone())
+    ops.apply_penalties(a, *args)
+    ref.apply_penalties(b, *args)
+    assert torch.allclose(a, b, atol=1e-6)
+    assert not torch.equal(a, dev(logits))

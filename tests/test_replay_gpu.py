@@ -1,0 +1,183 @@
+"""The engine against the plain implementation under every way of cutting the work, in float32
+and in bfloat16: each request alone and whole; most of it in one step and the last 32 tokens one
+by one; portions of changing size; up to four live requests mixed with so few pages that they are
+used again; long decoding; the first tokens of a sequence; and the same through bin/trace_run."""
+import os
+
+import pytest
+import torch
+
+from helpers import (TINY, make_model_folder, random_tokens, replay_in_process, replay_with_program, trace_bulk_then_single,
+                     trace_mixed, trace_portions, trace_whole)
+from plain_llama import plain_llama_forward, read_model_folder
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+TRACE_RUN = os.path.join(ROOT, "bin", "trace_run")
+
+
+def tolerance(dtype, ref):
+    """float32: rounding of sums of a few hundred terms. bfloat16: activations are rounded to 8 bits of
+    mantissa between kernels, a few times per layer; the bound is relative to the largest logit."""
+    scale = ref.abs().max().item()
+    return 3e-5 * max(1.0, scale) if dtype == "float32" else 4e-2 * max(0.25, scale)
+
+
+def check(got, refs, dtype, what):
+    for rid, ref in refs.items():
+        assert rid in got, (what, rid)
+        assert got[rid].shape == ref.shape, (what, rid, got[rid].shape, ref.shape)
+        err = (got[rid] - ref).abs()
+        t = tolerance(dtype, ref)
+        if err.max().item() > t:
+            pos = int(torch.nonzero(err.max(dim=1).values > t)[0])
+            raise AssertionError("%s: request %r first differs at position %d (page offset %d): max err %.3g > %.3g"
+                                 % (what, rid, pos, pos % 16, err.max().item(), t))
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    """{(config, storage dtype): (folder, plain config, plain weights)}; bfloat16 models are stored in
+    bfloat16, so the plain implementation sees exactly the engine's weights."""
+    root = tmp_path_factory.mktemp("models")
+    out = {}
+    for which in TINY:
+        for dtype in ("float32", "bfloat16"):
+            folder, _ = make_model_folder(root, which, dtype=dtype)
+            cfg, w = read_model_folder(folder)
+            out[(which, dtype)] = (folder, cfg, w)
+    return out
+
+
+def requests_for(cfg, which):
+    V = cfg["vocab_size"]
+    top = cfg["max_position_embeddings"]
+    lens = {"A": [1, 7, 33, 64, 128], "B": [3, 45, 130, 300, 77, 260], "C": [2, 100, 255, 31]}[which]
+    return {"r%d" % i: random_tokens(min(n, top), V, 100 + i) for i, n in enumerate(lens)}
+
+
+def engine(folder, which, dtype, num_pages):
+    from lmsf_amd.engine import load_engine_core
+    return load_engine_core(folder, dtype=dtype, block_size=TINY[which][2], num_pages=num_pages, max_num_seqs=8)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("which", ["A", "B", "C"])
+def test_every_way_of_cutting(models, which, dtype):
+    folder, cfg, w = models[(which, dtype)]
+    reqs = requests_for(cfg, which)
+    refs = {rid: plain_llama_forward(cfg, w, toks) for rid, toks in reqs.items()}
+    bs = TINY[which][2]
+    core = engine(folder, which, dtype, num_pages=-(-max(len(t) for t in reqs.values()) // bs) + 1)
+    ex = core.executor
+    check(replay_in_process(ex, trace_whole(reqs)), refs, dtype, "whole")
+    check(replay_in_process(ex, trace_bulk_then_single(reqs)), refs, dtype, "bulk then single")
+    check(replay_in_process(ex, trace_portions(reqs, seed=1)), refs, dtype, "portions")
+    core.storage.manager.check_invariants()
+    assert core.storage.manager.num_free_pages(0) == core.storage.groups[0].num_pages
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("which", ["A", "B", "C"])
+def test_mixed_requests_with_page_reuse(models, which, dtype):
+    folder, cfg, w = models[(which, dtype)]
+    reqs = requests_for(cfg, which)
+    reqs.update({"s%d" % i: random_tokens(20 + 9 * i, cfg["vocab_size"], 200 + i) for i in range(4)})
+    refs = {rid: plain_llama_forward(cfg, w, toks) for rid, toks in reqs.items()}
+    longest = -(-max(len(t) for t in reqs.values()) // 64) * 64
+    max_tokens = longest + 128            # the longest request and little else: pages must be reused
+    steps = trace_mixed(reqs, max_tokens, seed=5)
+    assert max(len(s["entries"]) for s in steps) >= 2
+    bs = TINY[which][2]
+    core = engine(folder, which, dtype, num_pages=max_tokens // bs)
+    check(replay_in_process(core.executor, steps), refs, dtype, "mixed")
+    core.storage.manager.check_invariants()
+    assert core.storage.manager.num_free_pages(0) == max_tokens // bs
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_and_first_tokens(models, dtype):
+    """One token at a time from the very first token to the end of the context."""
+    folder, cfg, w = models[("B", dtype)]
+    toks = random_tokens(cfg["max_position_embeddings"], cfg["vocab_size"], 77)
+    ref = plain_llama_forward(cfg, w, toks)
+    core = engine(folder, "B", dtype, num_pages=len(toks) // 16)
+    steps = [{"step": i, "entries": [{"id": "d", "tokens": [t], "want": [0]}], "end": []} for i, t in enumerate(toks)]
+    got = replay_in_process(core.executor, steps)
+    check(got, {"d": ref}, dtype, "token by token")
+    # the first tokens of a sequence alone
+    core.executor.release("d")
+    got = replay_in_process(core.executor, [{"step": 0, "entries": [{"id": "f", "tokens": toks[:1], "want": [0]}],
+                                             "end": ["f"]}])
+    check(got, {"f": ref[:1]}, dtype, "first token")
+
+
+def spike_far_key(folder, cfg, token=5, strength=8.0):
+    """A copy of the model folder whose first layer makes every query attend to the key of ``token``:
+    the slowest rotary pair of k carries ``strength`` for that token only (k_proj's row there is the
+    token's normalised embedding), and every q head carries ``strength`` there through its bias. The
+    slowest pair turns by less than a milliradian over the whole context, so the score stays high at
+    any distance."""
+    import shutil
+    from safetensors.torch import load_file, save_file
+    from plain_llama import plain_rms_norm
+    spiked = folder + "_spiked"
+    if os.path.isdir(spiked):
+        return spiked
+    shutil.copytree(folder, spiked)
+    t = load_file(os.path.join(folder, "model.safetensors"))
+    H, d, nh = cfg["hidden_size"], cfg["head_dim"], cfg["num_attention_heads"]
+    store = t["model.embed_tokens.weight"].dtype
+    slow = d // 2 - 1
+    h = plain_rms_norm(t["model.embed_tokens.weight"][token].float(), t["model.layers.0.input_layernorm.weight"].float(),
+                       cfg["rms_norm_eps"])
+    p = "model.layers.0.self_attn."
+    wk, bk = t[p + "k_proj.weight"].float(), t[p + "k_proj.bias"].float()
+    wq, bq = t[p + "q_proj.weight"].float(), t[p + "q_proj.bias"].float()
+    wk[slow] = strength * h / H
+    bk[slow] = 0.0
+    for head in range(nh):
+        wq[head * d + slow] = 0.0
+        bq[head * d + slow] = strength
+    for name, val in (("k_proj.weight", wk), ("k_proj.bias", bk), ("q_proj.weight", wq), ("q_proj.bias", bq)):
+        t[p + name] = val.to(store)
+    save_file(t, os.path.join(spiked, "model.safetensors"))
+    return spiked
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_far_key_among_hundreds(models, dtype):
+    """Random weights give nearly flat attention, which hides a lost key. Here the weights are made so
+    that one token's key stands out, and that token is placed once, early, in a long request: every
+    later position's logits depend on reading exactly that far key from its page."""
+    folder, cfg, _ = models[("B", dtype)]
+    spiked = spike_far_key(folder, cfg)
+    cfg, w = read_model_folder(spiked)
+    toks = [t if t != 5 else 6 for t in random_tokens(400, cfg["vocab_size"], 31)]
+    toks[18] = 5                          # in the second page, far from the end
+    ref = plain_llama_forward(cfg, w, toks)
+    flat = plain_llama_forward(cfg, w, toks[:18] + [6] + toks[19:])
+    assert (ref[300:] - flat[300:]).abs().max() > 10 * tolerance(dtype, ref), "the far key does not matter enough"
+    core = engine(spiked, "B", dtype, num_pages=26)
+    reqs = {"x": toks}
+    check(replay_in_process(core.executor, trace_whole(reqs)), {"x": ref}, dtype, "far key, whole")
+    check(replay_in_process(core.executor, trace_bulk_then_single(reqs)), {"x": ref}, dtype, "far key, decode")
+    check(replay_in_process(core.executor, trace_portions(reqs, seed=3)), {"x": ref}, dtype, "far key, portions")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(models, dtype, tmp_path):
+    """The same comparison through the replay program, as a user runs it."""
+    folder, cfg, w = models[("B", dtype)]
+    reqs = requests_for(cfg, "B")
+    refs = {rid: plain_llama_forward(cfg, w, toks) for rid, toks in reqs.items()}
+    max_tokens = 320 + 128
+    steps = trace_mixed(reqs, max_tokens, seed=11)
+    # some steps want nothing, and one request wants only a few places
+    steps[0]["entries"][0]["want"] = []
+    got = replay_with_program(TRACE_RUN, folder, dtype, steps, str(tmp_path / "out"), max_tokens, cfg["vocab_size"])
+    first = steps[0]["entries"][0]
+    refs_cut = dict(refs)
+    refs_cut[first["id"]] = refs[first["id"]][len(first["tokens"]):]
+    check(got, refs_cut, dtype, "trace_run mixed")

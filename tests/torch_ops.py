@@ -175,13 +175,9 @@ class TorchOps:
                 csum = torch.cumsum(e[order], dim=0)
                 # largest key whose mass of keys >= it reaches the target (ties counted together)
                 sk = keys[order]
-                best = cut
-                for i in range(V):
-                    if i + 1 < V and sk[i + 1] == sk[i]:
-                        continue
-                    if csum[i] >= target:
-                        best = max(best, int(sk[i]))
-                        break
+                group_end = torch.cat([sk[1:] != sk[:-1], torch.ones(1, dtype=torch.bool)])
+                hit = torch.nonzero(group_end & (csum >= target))
+                best = max(cut, int(sk[int(hit[0])])) if hit.numel() else cut
                 cut = best
             mp = float(min_p[r]) if min_p is not None else 0.0
             if mp > 0.0:
