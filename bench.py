@@ -1,0 +1,193 @@
+"""Decode and prefill throughput of the engine at Llama-3-8B shape on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one decode step of the whole engine (schedule, batch building, model, sampling) at
+batch 8: requests with 512-token random prompts are prefilled (untimed), W decode steps warm up,
+then exactly K decode steps are timed between device synchronisations. The same line carries the
+prefill of 2,048 tokens, the decode step's share of the HBM roofline, and decode at batch 1 and 64.
+Weights are random (N(0, 0.02), bfloat16, made on the device), token ids are seeded uniform-random.
+The reference publishes no numbers, so vs_baseline is null.
+"""
+import argparse
+import json
+import os
+import random
+import sys
+import tempfile
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+# MI355X published peaks
+HBM_BYTES_PER_S = 8.0e12
+PEAK_FLOPS = {"bf16": 2.5e15, "fp16": 2.5e15, "fp8": 5.0e15, "fp32": 157.3e12}
+
+LLAMA3_8B = dict(
+    architectures=["LlamaForCausalLM"], model_type="llama", vocab_size=128256, hidden_size=4096,
+    intermediate_size=14336, num_hidden_layers=32, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
+    rms_norm_eps=1e-5, rope_theta=500000.0, rope_scaling=None, max_position_embeddings=8192,
+    tie_word_embeddings=False, attention_bias=False, hidden_act="silu", torch_dtype="bfloat16",
+    bos_token_id=128000, eos_token_id=128001)
+
+
+def make_engine(cfg, args, max_num_seqs, dtype):
+    from lmsf_amd.engine import EngineArgs, LLMEngine
+    folder = tempfile.mkdtemp(prefix="lmsf_bench_")
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    return LLMEngine(EngineArgs(model=folder, dtype=dtype, block_size=16, load_format="random", seed=0,
+                                max_num_seqs=max_num_seqs, max_num_batched_tokens=args.max_num_batched_tokens,
+                                gpu_memory_utilization=args.gpu_memory_utilization))
+
+
+def weight_bytes(engine):
+    """Bytes of every weight a decode step reads once: all matrices and norm weights, the LM head, not
+    the embedding table (one row per token)."""
+    seen, total = set(), 0
+    emb = engine.core.model.embedding.weight
+    head = engine.core.model.head.weight
+    for p in engine.core.model.parts():
+        for name in ("weight", "bias"):
+            t = getattr(p, name, None)
+            if t is None or t.data_ptr() in seen:
+                continue
+            if t.data_ptr() == emb.data_ptr() and emb.data_ptr() != head.data_ptr():
+                continue
+            seen.add(t.data_ptr())
+            total += t.numel() * t.element_size()
+    return total
+
+
+def decode_run(engine, batch, prompt_len, steps, warmup, seed):
+    """Prefill ``batch`` prompts, warm up, time ``steps`` decode steps. Returns (seconds, mean context)."""
+    import torch
+    from lmsf_amd.sampling import SamplingParams
+    rng = random.Random(seed)
+    V = engine.core.config.vocab_size
+    ids = []
+    for i in range(batch):
+        rid = "b%d_%d" % (batch, i)
+        engine.add_request(rid, [rng.randrange(V) for _ in range(prompt_len)],
+                           SamplingParams(temperature=0.0, max_tokens=steps + warmup + 8, ignore_eos=True))
+        ids.append(rid)
+    while any(s.remaining > 1 for s in list(engine.scheduler.running) + list(engine.scheduler.waiting)) \
+            or engine.scheduler.waiting:
+        engine.step()
+    for _ in range(warmup):
+        engine.step()
+    ctx0 = sum(s.length for s in engine.scheduler.running) / batch
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        outs = engine.step()
+        assert len(outs) == batch
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    for rid in ids:
+        engine.abort_request(rid)
+    return dt, ctx0 + steps / 2.0
+
+
+def prefill_run(engine, n_tokens, reps, seed):
+    """Median seconds of a prefill of ``n_tokens`` tokens of one request (one step, logits of the last token)."""
+    import torch
+    from lmsf_amd.engine import StepEntry
+    rng = random.Random(seed)
+    V = engine.core.config.vocab_size
+    times = []
+    for r in range(reps + 1):
+        toks = [rng.randrange(V) for _ in range(n_tokens)]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        engine.core.executor.step([StepEntry("prefill", toks, [n_tokens - 1])])
+        torch.cuda.synchronize()
+        if r > 0:
+            times.append(time.perf_counter() - t0)
+        engine.core.executor.release("prefill")
+    times.sort()
+    return times[len(times) // 2]
+
+
+def prefill_flops(cfg, T):
+    """Multiply-adds times two of a causal prefill of T tokens: the linear layers on every token, the
+    attention scores and values over the causal half, the LM head on one row."""
+    H, I, L = cfg["hidden_size"], cfg["intermediate_size"], cfg["num_hidden_layers"]
+    nh, nkv, d = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    per_token = L * ((nh + 2 * nkv) * d * H + nh * d * H + 3 * I * H)
+    attn = L * nh * d * 2 * (T * (T + 1) // 2)
+    return 2.0 * (per_token * T + attn + cfg["vocab_size"] * H)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--prompt-len", type=int, default=512)
+    ap.add_argument("--prefill-tokens", type=int, default=2048)
+    ap.add_argument("--layers", type=int, default=None, help="run fewer layers than the configuration has")
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--max-num-batched-tokens", type=int, default=8192)
+    ap.add_argument("--gpu-memory-utilization", type=float, default=0.85)
+    ap.add_argument("--skip-points", action="store_true", help="leave out the batch 1 and batch 64 runs")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this engine runs on one GPU; --gpus %d is not supported" % args.gpus)
+        sys.exit(2)
+
+    import torch
+    cfg = dict(LLAMA3_8B)
+    full_layers = cfg["num_hidden_layers"]
+    if args.layers:
+        cfg["num_hidden_layers"] = args.layers
+    engine = make_engine(cfg, args, max_num_seqs=64, dtype=args.dtype)
+    wbytes = weight_bytes(engine)
+    kv_per_token = 2 * cfg["num_key_value_heads"] * cfg["head_dim"] * cfg["num_hidden_layers"] * \
+        (2 if args.dtype == "bfloat16" else 4)
+
+    dt, mean_ctx = decode_run(engine, args.batch, args.prompt_len, args.steps, args.warmup, seed=1)
+    ms_per_step = dt / args.steps * 1e3
+    value = args.batch * args.steps / dt
+    step_bytes = wbytes + args.batch * mean_ctx * kv_per_token
+    achieved = step_bytes / (dt / args.steps) / 1e9
+
+    points = {}
+    if not args.skip_points:
+        for b in (1, 64):
+            k = max(16, args.steps // 2)
+            d, _ = decode_run(engine, b, args.prompt_len, k, args.warmup, seed=2 + b)
+            points["decode_b%d" % b] = round(b * k / d, 1)
+
+    pt = prefill_run(engine, args.prefill_tokens, reps=5, seed=3)
+    pflops = prefill_flops(cfg, args.prefill_tokens)
+    peak = PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
+
+    line = {
+        "metric": "decode tok/s at batch 8 (Llama-3-8B bf16)",
+        "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
+        "config": {
+            "model": "Llama-3-8B shape, random weights", "global_batch": args.batch, "seq_len": args.prompt_len,
+            "parallelism": "single GPU", "layers": cfg["num_hidden_layers"], "layers_of_model": full_layers,
+            "hidden_size": cfg["hidden_size"], "heads": cfg["num_attention_heads"],
+            "kv_heads": cfg["num_key_value_heads"], "head_dim": cfg["head_dim"],
+            "intermediate_size": cfg["intermediate_size"], "vocab_size": cfg["vocab_size"],
+            "max_context": cfg["max_position_embeddings"], "block_size": 16, "prompt_len": args.prompt_len,
+            "mean_decode_context": round(mean_ctx, 1), "prefill_tokens": args.prefill_tokens,
+        },
+        "prefill": {"value": round(args.prefill_tokens / pt, 1), "tokens": args.prefill_tokens,
+                    "ms": round(pt * 1e3, 3), "frac": round(pflops / pt / peak, 4)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_BYTES_PER_S / 1e9, "unit": "GB/s",
+                     "frac": round(achieved / (HBM_BYTES_PER_S / 1e9), 4)},
+        "points": points,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,84 @@
+"""Engine arguments with the reference's option names and meanings
+(core/src/common/config.rs:9-87), as a dataclass and as command-line flags.
+
+Options of the reference that have no meaning here are still accepted, so that its command lines
+run: --swap-space, --max-paddings, --threads, --chat-template, --log-dir, --alsologtostderr are
+parsed and unused (as --threads and --chat-template are in the reference); --tp, --pp must be 1
+and --quantization must be absent, or the engine refuses to start.
+"""
+import argparse
+import dataclasses
+from dataclasses import dataclass
+from typing import Optional
+
+
+@dataclass
+class EngineArgs:
+    model: str = ""
+    dtype: Optional[str] = None                    # default: config.json's torch_dtype
+    max_model_len: Optional[int] = None            # default: config.json's max_position_embeddings
+    block_size: int = 16
+    seed: int = 0
+    gpu_memory_utilization: float = 0.9
+    max_num_batched_tokens: Optional[int] = None   # default: max(max_model_len, 2048)
+    max_num_seqs: int = 256
+    max_paddings: int = 256                        # unused: batches have no padding
+    swap_space: int = 4                            # unused: preemption recomputes
+    quantization: Optional[str] = None
+    chat_template: Optional[str] = ""
+    pipeline_parallel_size: int = 1
+    tensor_parallel_size: int = 1
+    threads: int = 4
+    log_dir: Optional[str] = None
+    alsologtostderr: bool = False
+    # beyond the reference
+    load_format: str = "auto"                      # "auto": safetensors of the folder; "random": random weights
+    prefill_chunk_size: Optional[int] = None
+    num_gpu_blocks_override: Optional[int] = None
+    device: str = "cuda:0"
+
+    def verify(self) -> None:
+        if self.quantization:
+            raise ValueError("--quantization %s: quantized weights are not supported" % self.quantization)
+        if self.pipeline_parallel_size != 1 or self.tensor_parallel_size != 1:
+            raise ValueError("--pp and --tp must be 1: this engine runs on one GPU")
+        if self.gpu_memory_utilization > 1.0 or self.gpu_memory_utilization <= 0.0:
+            # core/src/common/config.rs:245-250
+            raise ValueError("GPU memory utilization must be in (0, 1]. Got %r." % self.gpu_memory_utilization)
+        if self.load_format not in ("auto", "random"):
+            raise ValueError("--load-format must be auto or random")
+
+    @staticmethod
+    def add_cli_args(parser: argparse.ArgumentParser) -> argparse.ArgumentParser:
+        a = parser.add_argument
+        a("--model", required=True, help="path of the huggingface model folder to use")
+        a("--dtype", default=None, choices=["float32", "bfloat16", "float16", "half", "auto"],
+          help="the datatype to use for model (float16 runs as bfloat16)")
+        a("--max-model-len", type=int, default=None,
+          help="model context length. If unspecified, will be automatically derived from the model")
+        a("--block-size", type=int, default=16, help="token block size")
+        a("--seed", type=int, default=0, help="random seed")
+        a("--gpu-memory-utilization", type=float, default=0.9,
+          help="the percentage of GPU memory to be used for the model executor")
+        a("--max-num-batched-tokens", type=int, default=None, help="maximum number of batched tokens per iteration")
+        a("--max-num-seqs", type=int, default=256, help="maximum number of sequences per iteration")
+        a("--max-paddings", type=int, default=256, help="maximum number of paddings in a batch (unused)")
+        a("--swap-space", type=int, default=4, help="CPU swap space size (GiB) per GPU (unused)")
+        a("--quantization", default=None, help="specify quantize method (not supported)")
+        a("--chat-template", default="", help="chat template config file (unused)")
+        a("--pp", dest="pipeline_parallel_size", type=int, default=1, help="number of pipeline stages (1)")
+        a("--tp", dest="tensor_parallel_size", type=int, default=1, help="number of tensor parallel replicas (1)")
+        a("--threads", type=int, default=4, help="(unused)")
+        a("--log-dir", default=None, help="log dir (unused)")
+        a("--alsologtostderr", action="store_true", help="print log into stderr (unused)")
+        a("--load-format", default="auto", choices=["auto", "random"],
+          help="auto: the folder's safetensors; random: random weights for the folder's config.json")
+        a("--prefill-chunk-size", type=int, default=None, help="longest portion of a prompt in one step")
+        a("--num-gpu-blocks-override", type=int, default=None, help="pages of the cache instead of sizing from memory")
+        a("--device", default="cuda:0")
+        return parser
+
+    @classmethod
+    def from_cli_args(cls, ns: argparse.Namespace) -> "EngineArgs":
+        names = {f.name for f in dataclasses.fields(cls)}
+        return cls(**{k: v for k, v in vars(ns).items() if k in names})

@@ -1,0 +1,172 @@
+"""The engine: requests in, tokens out, one step at a time.
+
+LLMEngine mirrors the reference's (core/src/engine/llm_engine.rs:74-582): ``add_request``,
+``abort_request``, ``has_unfinished_requests`` and ``step``, which schedules, runs the model once,
+samples and applies the stop rules. ``LLM.generate`` is the convenience loop around it.
+"""
+import hashlib
+import time
+from typing import Any, Dict, Hashable, List, Optional, Sequence as Seq
+
+import torch
+
+from ..sampling.params import SamplingParams
+from ..sampling.sampler import Sampler, SamplingRow
+from .args import EngineArgs
+from .batch import StepEntry
+from .core import EngineCore, load_engine_core
+from .outputs import RequestOutput
+from .scheduler import Scheduler, SchedulerConfig, StepPlan
+from .sequence import Sequence, SequenceState
+
+
+class LLMEngine:
+    def __init__(self, args: EngineArgs, ops: Any = None):
+        args.verify()
+        self.args = args
+        self.core: EngineCore = load_engine_core(
+            args.model or None, dtype=args.dtype, block_size=args.block_size, max_model_len=args.max_model_len,
+            num_pages=args.num_gpu_blocks_override, gpu_memory_utilization=args.gpu_memory_utilization,
+            max_num_seqs=args.max_num_seqs, max_num_batched_tokens=args.max_num_batched_tokens, device=args.device,
+            ops=ops, load_format=args.load_format, seed=args.seed)
+        max_len = self.core.max_model_len
+        budget = args.max_num_batched_tokens or max(max_len, 2048)      # core/src/common/config.rs:301-307
+        self.scheduler = Scheduler(SchedulerConfig(budget, args.max_num_seqs, max_len, args.prefill_chunk_size),
+                                   self.core.storage.manager)
+        self.sampler = Sampler(self.core.rt.ops, self.core.rt.device)
+        self.eos_token_ids = set(self.core.config.eos_token_ids)
+        self._arrivals = 0
+        self._requests: Dict[Hashable, Sequence] = {}
+        self.stats = {"steps": 0, "tokens": 0, "generated_tokens": 0, "preemptions": 0}
+
+    @classmethod
+    def from_engine_args(cls, args: EngineArgs) -> "LLMEngine":
+        return cls(args)
+
+    # ------------------------------------------------------------------ requests
+
+    def add_request(self, request_id: Hashable, prompt_token_ids: Seq[int],
+                    sampling_params: Optional[SamplingParams] = None) -> None:
+        """core/src/engine/llm_engine.rs:136-169, on token ids."""
+        if request_id in self._requests:
+            raise ValueError("request id %r is already in use" % (request_id,))
+        params = sampling_params or SamplingParams()
+        params.verify()
+        ids = [int(t) for t in prompt_token_ids]
+        V = self.core.config.vocab_size
+        if not ids:
+            raise ValueError("request %r has an empty prompt" % (request_id,))
+        bad = [t for t in ids if not (0 <= t < V)]
+        if bad:
+            raise ValueError("request %r: token id %d outside the vocabulary of %d" % (request_id, bad[0], V))
+        seed = params.seed
+        if seed is None:
+            h = hashlib.sha256(("%d:%d" % (self.args.seed, self._arrivals)).encode()).digest()
+            seed = int.from_bytes(h[:8], "little")
+        seq = Sequence(request_id, ids, params, self._arrivals, seed)
+        self._arrivals += 1
+        self._requests[request_id] = seq
+        self.scheduler.add(seq)
+
+    def abort_request(self, request_id: Hashable) -> None:
+        """core/src/engine/llm_engine.rs:171-178."""
+        seq = self.scheduler.abort(request_id)
+        if seq is not None:
+            seq.metrics.finished_time = time.monotonic()
+        self._requests.pop(request_id, None)
+
+    def has_unfinished_requests(self) -> bool:
+        return self.scheduler.has_unfinished()
+
+    def get_num_unfinished_requests(self) -> int:
+        return self.scheduler.num_unfinished()
+
+    # ------------------------------------------------------------------ the step
+
+    def step(self) -> List[RequestOutput]:
+        """Schedule, run the model once, sample, apply the stop rules
+        (core/src/engine/llm_engine.rs:536-582)."""
+        plan: StepPlan = self.scheduler.schedule()
+        outputs: List[RequestOutput] = []
+        now = time.monotonic()
+        for seq in plan.ignored + plan.capped:
+            seq.metrics.finished_time = now
+            self._requests.pop(seq.request_id, None)
+            outputs.append(RequestOutput.from_sequence(seq, None))
+        self.stats["preemptions"] += len(plan.preempted)
+        if plan.empty:
+            return outputs
+        entries = [StepEntry(s.seq.request_id, s.seq.tokens(s.start, s.n_tokens),
+                             [s.n_tokens - 1] if s.samples else []) for s in plan.scheduled]
+        logits = self.core.executor.step(entries)
+        self.stats["steps"] += 1
+        sampled = []
+        for s in plan.scheduled:
+            s.seq.num_computed += s.n_tokens
+            if s.samples:
+                sampled.append(s.seq)
+        rows = [SamplingRow(seq.params, seq.seed, len(seq.output_token_ids), seq.prompt_token_ids,
+                            seq.output_token_ids) for seq in sampled]
+        tokens = self.sampler.sample(logits, rows)
+        now = time.monotonic()
+        for seq, tok in zip(sampled, tokens):
+            seq.output_token_ids.append(tok)
+            if seq.metrics.first_token_time is None:
+                seq.metrics.first_token_time = now
+            self._check_stop(seq)
+            if seq.state.finished:
+                seq.metrics.finished_time = now
+                self.scheduler.finish(seq)
+                self._requests.pop(seq.request_id, None)
+            outputs.append(RequestOutput.from_sequence(seq, tok))
+        self.stats["generated_tokens"] += len(sampled)
+        self.stats["tokens"] += plan.num_tokens
+        return outputs
+
+    def _check_stop(self, seq: Sequence) -> None:
+        """The reference's order without stop strings (core/src/engine/llm_engine.rs:221-258):
+        stop_token_ids, longer than max_model_len, max_tokens reached, EOS unless ignore_eos."""
+        p = seq.params
+        last = seq.last_token_id
+        if p.stop_token_ids and last in p.stop_token_ids:
+            seq.state = SequenceState.FINISHED_STOPPED
+        elif seq.length > self.core.max_model_len:
+            seq.state = SequenceState.FINISHED_LENGTH_CAPPED
+        elif len(seq.output_token_ids) >= p.max_tokens:
+            seq.state = SequenceState.FINISHED_LENGTH_CAPPED
+        elif not p.ignore_eos and last in self.eos_token_ids:
+            seq.state = SequenceState.FINISHED_STOPPED
+        elif seq.length >= self.core.max_model_len:
+            # the next token would have no position left
+            seq.state = SequenceState.FINISHED_LENGTH_CAPPED
+
+
+class LLM:
+    """``LLM(model=..., **engine options).generate(prompts, sampling_params)``: every prompt a list of
+    token ids; returns one finished RequestOutput per prompt, in the order given."""
+
+    def __init__(self, model: str, **kwargs):
+        self.engine = LLMEngine(EngineArgs(model=model, **kwargs))
+        self._next_id = 0
+
+    def generate(self, prompt_token_ids: Seq[Seq[int]], sampling_params=None) -> List[RequestOutput]:
+        if sampling_params is None or isinstance(sampling_params, SamplingParams):
+            params_list = [sampling_params] * len(prompt_token_ids)
+        else:
+            params_list = list(sampling_params)
+            if len(params_list) != len(prompt_token_ids):
+                raise ValueError("one SamplingParams per prompt, or one for all")
+        ids = []
+        for prompt, params in zip(prompt_token_ids, params_list):
+            rid = self._next_id
+            self._next_id += 1
+            # every request gets its own copy: verify() may normalise fields
+            p = None if params is None else SamplingParams(**vars(params))
+            self.engine.add_request(rid, prompt, p)
+            ids.append(rid)
+        done: Dict[Hashable, RequestOutput] = {}
+        while self.engine.has_unfinished_requests():
+            for out in self.engine.step():
+                if out.finished:
+                    done[out.request_id] = out
+        return [done[r] for r in ids]

@@ -1,0 +1,33 @@
+"""What the engine hands back per request and step
+(core/src/common/output.rs:5-132: RequestOutput with its CompletionOutputs). Text fields are
+absent: the engine works on token ids."""
+from dataclasses import dataclass, field
+from typing import Hashable, List, Optional
+
+from .sequence import RequestMetrics, Sequence
+
+
+@dataclass
+class CompletionOutput:
+    index: int
+    token_ids: List[int]
+    latest_token: Optional[int]          # the token this step produced (None if the step produced none)
+    finish_reason: Optional[str] = None  # "stop", "length", "abort"
+
+    def finished(self) -> bool:
+        return self.finish_reason is not None
+
+
+@dataclass
+class RequestOutput:
+    request_id: Hashable
+    prompt_token_ids: List[int]
+    outputs: List[CompletionOutput]
+    finished: bool
+    metrics: Optional[RequestMetrics] = None
+
+    @classmethod
+    def from_sequence(cls, seq: Sequence, latest: Optional[int]) -> "RequestOutput":
+        return cls(seq.request_id, list(seq.prompt_token_ids),
+                   [CompletionOutput(0, list(seq.output_token_ids), latest, seq.state.finish_reason)],
+                   seq.state.finished, seq.metrics)

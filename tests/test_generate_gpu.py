@@ -1,0 +1,76 @@
+"""Greedy generation through the entry points on the GPU: the Python one (LLM.generate) and the
+command line, in float32 and bfloat16, against the plain implementation."""
+import os
+import subprocess
+import sys
+
+import pytest
+import torch
+
+from helpers import TINY, make_model_folder, random_tokens
+from plain_llama import plain_greedy_generate, plain_llama_forward, read_model_folder
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.mark.parametrize("which", ["A", "B"])
+def test_llm_generate_greedy_float32(tmp_path, which):
+    from lmsf_amd import LLM, SamplingParams
+    folder, cfg = make_model_folder(tmp_path, which)
+    cfg_dict, w = read_model_folder(folder)
+    lens = (1, 7, 33, 64) if which == "A" else (3, 40, 150, 300, 17, 90)
+    prompts = [random_tokens(n, cfg.vocab_size, 20 + n) for n in lens]
+    llm = LLM(model=folder, dtype="float32", block_size=TINY[which][2], num_gpu_blocks_override=96,
+              max_num_seqs=8, prefill_chunk_size=64, max_num_batched_tokens=128)
+    outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_tokens=16, ignore_eos=True))
+    for p, o in zip(prompts, outs):
+        assert o.outputs[0].token_ids == plain_greedy_generate(cfg_dict, w, p, 16), len(p)
+    llm.engine.core.storage.manager.check_invariants()
+
+
+def test_llm_generate_bfloat16_follows_plain_argmax(tmp_path):
+    """In bfloat16 a near-tie may flip a token, after which the sequences differ for good; so every
+    generated token is checked against the plain logits of the engine's own prefix: it must be the
+    argmax or within the bfloat16 error of it."""
+    from lmsf_amd import LLM, SamplingParams
+    folder, cfg = make_model_folder(tmp_path, "B", dtype="bfloat16")
+    cfg_dict, w = read_model_folder(folder)
+    prompts = [random_tokens(n, cfg.vocab_size, 40 + n) for n in (5, 70, 200)]
+    llm = LLM(model=folder, dtype="bfloat16", block_size=16, num_gpu_blocks_override=64, max_num_seqs=4)
+    outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True))
+    for p, o in zip(prompts, outs):
+        gen = o.outputs[0].token_ids
+        assert len(gen) == 12
+        logits = plain_llama_forward(cfg_dict, w, p + gen[:-1])[len(p) - 1:]
+        for i, tok in enumerate(gen):
+            assert logits[i, tok] >= logits[i].max() - 0.05 * logits[i].abs().max(), (len(p), i)
+
+
+def test_temperature_sampling_seeded(tmp_path):
+    from lmsf_amd import LLM, SamplingParams
+    folder, cfg = make_model_folder(tmp_path, "B")
+    prompts = [random_tokens(n, cfg.vocab_size, 60 + n) for n in (9, 33)]
+    llm = LLM(model=folder, dtype="float32", block_size=16, num_gpu_blocks_override=64, max_num_seqs=4,
+              prefill_chunk_size=64)
+    sp = SamplingParams(temperature=0.7, max_tokens=24, ignore_eos=True, seed=5)
+    a = [o.outputs[0].token_ids for o in llm.generate(prompts, sp)]
+    b = [o.outputs[0].token_ids for o in llm.generate(prompts[::-1], sp)][::-1]
+    assert a == b and a[0] != a[1]
+    c = [o.outputs[0].token_ids for o in llm.generate(prompts, SamplingParams(temperature=0.7, max_tokens=24,
+                                                                              ignore_eos=True, seed=6))]
+    assert c != a
+
+
+def test_command_line(tmp_path):
+    folder, cfg = make_model_folder(tmp_path, "A")
+    cfg_dict, w = read_model_folder(folder)
+    prompt = random_tokens(11, cfg.vocab_size, 9)
+    proc = subprocess.run([os.path.join(ROOT, "bin", "lmsf_generate"), "--model", folder, "--dtype", "float32",
+                           "--gpu-memory-utilization", "0.5", "--block-size", "8", "--max-model-len", "64",
+                           "--prompt-ids", ",".join(map(str, prompt)), "--temperature", "0", "--max-tokens", "8",
+                           "--ignore-eos"], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    lines = proc.stdout.strip().splitlines()
+    assert [int(t) for t in lines[0].split()] == plain_greedy_generate(cfg_dict, w, prompt, 8)
+    assert lines[-1].startswith("cost ")
