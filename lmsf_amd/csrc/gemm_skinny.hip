@@ -1,0 +1,204 @@
+// Linear layer for few rows (decoding): y[M, N] = x[M, K] W[N, K]^T (+ bias), M <= 64, bfloat16
+// inputs, float32 accumulation on the matrix cores, bfloat16 or float32 output.
+//
+// With so few rows the product is a stream of the weight matrix: every weight is read once from
+// HBM and used M times, so the kernel is built around the memory system, not the arithmetic.
+// The reference leaves these products to cuBLASLt with an offline-tuned algorithm per shape
+// (tops/src/cublas.rs:29-114, tops/csrc/tops/tensorrt_llm/c_api/gemm.cc:43-150).
+//
+// Decomposition. One workgroup owns 16 rows of W (16 outputs per token) over the whole K. Its NW
+// waves split K in chunks of KC elements, wave w taking chunks w, w + NW, ...: at any moment the
+// workgroup reads NW * KC contiguous elements of each of its rows. Partial sums of the waves are
+// added in a fixed order through LDS, so the result does not depend on timing.
+//
+// Data path of one chunk in one wave. W tile (16 rows x KC) and x tile (16 tokens x KC, per token
+// tile) are fetched with 16-byte loads in which consecutive lanes read consecutive addresses of one
+// row (KC/8 lanes per row), so every load instruction covers whole cache lines. The matrix-core
+// operand layout wants lane (r, g) to hold row r, elements g*8..g*8+7 of a 32-wide step; the tiles go
+// through a wave-private LDS area (row stride padded by 16 bytes: conflict-free for both the write
+// and the read pattern) to change layout. The loads of the next chunk are issued before the current
+// chunk's LDS traffic and MFMAs, so a chunk per wave is always in flight.
+//
+// MFMA: v_mfma_f32_16x16x32_bf16, A = W tile (16 rows x 32 k), B = x tile (32 k x 16 tokens), D[n][m]:
+// lane l holds token m = l % 16 and the four outputs n = (l / 16) * 4 .. + 3.
+#include "common.h"
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));   // a 16-byte piece in flight
+
+template <int KC>
+struct SkinnyTile {
+  static constexpr int LANES_PER_ROW = KC / 8;              // 16-byte pieces per row of a tile
+  static constexpr int ROWS_PER_LOAD = 64 / LANES_PER_ROW;  // rows one load instruction covers
+  static constexpr int LOADS = 16 / ROWS_PER_LOAD;          // load instructions per tile
+  static constexpr int ROW_BYTES = KC * 2 + 16;             // padded LDS row
+  static constexpr int TILE_BYTES = 16 * ROW_BYTES;
+  static constexpr int STEPS = KC / 32;                     // MFMA steps per chunk
+};
+
+template <int MT, int KC, int NW, typename TOut>
+__global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ x, long ldx,
+                                                              const bf16_t* __restrict__ W, long ldw,
+                                                              const bf16_t* __restrict__ bias, TOut* __restrict__ y,
+                                                              long ldy, int M, int N, int K) {
+  using T = SkinnyTile<KC>;
+  extern __shared__ __align__(16) unsigned char lds[];
+  const int tid = threadIdx.x;
+  const int wave = tid / 64, lane = tid % 64;
+  const int n0 = blockIdx.x * 16;
+  unsigned char* my = lds + (size_t)wave * (1 + MT) * T::TILE_BYTES;
+
+  // global load coordinates of this lane inside a tile
+  const int lrow = lane / T::LANES_PER_ROW;      // + i * ROWS_PER_LOAD
+  const int lcol = (lane % T::LANES_PER_ROW) * 8;  // element offset inside the chunk
+  // LDS read coordinates (MFMA operand layout)
+  const int fr = lane % 16, fg = lane / 16;
+
+  // row offsets (in elements) of this lane's 16-byte pieces; rows beyond the matrix repeat the last row
+  long woff[T::LOADS], xoff[MT][T::LOADS];
+#pragma unroll
+  for (int i = 0; i < T::LOADS; ++i) {
+    int r = n0 + lrow + i * T::ROWS_PER_LOAD;
+    if (r > N - 1) r = N - 1;
+    woff[i] = (long)r * ldw + lcol;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      int m = mt * 16 + lrow + i * T::ROWS_PER_LOAD;
+      if (m > M - 1) m = M - 1;
+      xoff[mt][i] = (long)m * ldx + lcol;
+    }
+  }
+
+  f32x4_t acc[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) acc[mt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+
+  const int nchunks = (K + KC - 1) / KC;
+  u32x4_t wreg[T::LOADS], xreg[MT][T::LOADS];
+
+  // K is a multiple of 8, so a 16-byte piece is inside or outside the row as a whole; a piece outside
+  // is read from the start of the row instead and multiplied by nothing (its x piece is zeroed)
+#define SKINNY_FETCH(chunk)                                                                     \
+  {                                                                                             \
+    const int k_ = (chunk) * KC;                                                                \
+    const bool ok_ = (k_ + lcol) < K;                                                           \
+    const int kk_ = ok_ ? k_ : -lcol;                                                           \
+    const unsigned keep_ = ok_ ? 0xffffffffu : 0u;                                              \
+    _Pragma("unroll") for (int i = 0; i < T::LOADS; ++i) {                                      \
+      wreg[i] = *reinterpret_cast<const u32x4_t*>(W + woff[i] + kk_);                           \
+      _Pragma("unroll") for (int mt = 0; mt < MT; ++mt) {                                       \
+        xreg[mt][i] = *reinterpret_cast<const u32x4_t*>(x + xoff[mt][i] + kk_) & keep_;         \
+      }                                                                                         \
+    }                                                                                           \
+  }
+
+  // Every fetch is unconditional (a wave without a next chunk fetches its current one again, from
+  // cache), which keeps the staged pieces in registers across the loop.
+  int c = wave;
+  SKINNY_FETCH(c < nchunks ? c : 0);
+  while (c < nchunks) {
+    // registers -> LDS (load layout)
+#pragma unroll
+    for (int i = 0; i < T::LOADS; ++i) {
+      const int off = (lrow + i * T::ROWS_PER_LOAD) * T::ROW_BYTES + lcol * 2;
+      *reinterpret_cast<u32x4_t*>(my + off) = wreg[i];
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) *reinterpret_cast<u32x4_t*>(my + (1 + mt) * T::TILE_BYTES + off) = xreg[mt][i];
+    }
+    const int next = c + NW;
+    SKINNY_FETCH(next < nchunks ? next : c);
+    // LDS -> operands (MFMA layout), multiply
+#pragma unroll
+    for (int s = 0; s < T::STEPS; ++s) {
+      const int off = fr * T::ROW_BYTES + s * 64 + fg * 16;
+      const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(my + off);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const bf16x8_t b = *reinterpret_cast<const bf16x8_t*>(my + (1 + mt) * T::TILE_BYTES + off);
+        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[mt], 0, 0, 0);
+      }
+    }
+    c = next;
+  }
+#undef SKINNY_FETCH
+
+  // add the waves' partial sums in wave order
+  __syncthreads();
+  float* red = reinterpret_cast<float*>(lds);   // [NW][MT][64 lanes][4]
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+    *reinterpret_cast<f32x4_t*>(red + (((size_t)wave * MT + mt) * 64 + lane) * 4) = acc[mt];
+  __syncthreads();
+  for (int e = tid; e < MT * 256; e += NW * 64) {
+    const int mt = e / 256, l = (e % 256) / 4, j = e % 4;
+    float sum = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) sum += red[(((size_t)w * MT + mt) * 64 + l) * 4 + j];
+    const int n = n0 + (l / 16) * 4 + j, m = mt * 16 + l % 16;
+    if (n < N && m < M) {
+      if (bias) sum += bf16_to_f32(bias[n]);
+      y[(long)m * ldy + n] = from_f32<TOut>(sum);
+    }
+  }
+}
+
+template <int MT, int KC, int NW, typename TOut>
+static int launch_skinny(const void* x, long ldx, const void* W, long ldw, const void* bias, void* y, long ldy, int M,
+                         int N, int K, hipStream_t stream) {
+  using T = SkinnyTile<KC>;
+  const size_t stage = (size_t)NW * (1 + MT) * T::TILE_BYTES;
+  const size_t red = (size_t)NW * MT * 64 * 4 * sizeof(float);
+  const size_t smem = stage > red ? stage : red;
+  auto kernel = gemm_skinny_kernel<MT, KC, NW, TOut>;
+  static bool configured = false;   // per instantiation
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) {
+      lmsf_set_error("gemm_skinny: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
+      return 2;
+    }
+    configured = true;
+  }
+  hipLaunchKernelGGL(kernel, dim3((N + 15) / 16), dim3(NW * 64), smem, stream, (const bf16_t*)x, ldx,
+                     (const bf16_t*)W, ldw, (const bf16_t*)bias, (TOut*)y, ldy, M, N, K);
+  return 0;
+}
+
+// x [M, K] bfloat16 (row stride ldx), W [N, K] bfloat16 (row stride ldw), bias [N] bfloat16 or null,
+// y [M, N] of out_dtype. Needs M <= 64, K a multiple of 8, 16-byte aligned x and W and row strides
+// that are multiples of 8 elements; anything else is refused. ``variant`` picks the tiling (0: default).
+extern "C" int lmsf_gemm_skinny(const void* x, long ldx, const void* W, long ldw, const void* bias, void* y,
+                                int out_dtype, long ldy, int M, int N, int K, int variant, hipStream_t stream) {
+  LMSF_CHECK(x && W && y, "gemm_skinny: null pointer");
+  LMSF_CHECK(M >= 0 && M <= 64, "gemm_skinny: M=%d outside [0, 64]", M);
+  LMSF_CHECK(N > 0 && K > 0 && K % 8 == 0, "gemm_skinny: K=%d must be a positive multiple of 8 (N=%d)", K, N);
+  LMSF_CHECK(ldx >= K && ldw >= K && ldy >= N && ldx % 8 == 0 && ldw % 8 == 0,
+             "gemm_skinny: row strides must cover K and be multiples of 8");
+  LMSF_CHECK(lmsf_aligned16(x) && lmsf_aligned16(W), "gemm_skinny: x and W must be 16-byte aligned");
+  LMSF_CHECK(out_dtype == LMSF_F32 || out_dtype == LMSF_BF16, "gemm_skinny: unknown output dtype %d", out_dtype);
+  if (M == 0) return 0;
+  const int mt = (M + 15) / 16;
+  int rc = 0;
+#define SK(MT_, KC_, NW_)                                                                                       \
+  rc = out_dtype == LMSF_F32 ? launch_skinny<MT_, KC_, NW_, float>(x, ldx, W, ldw, bias, y, ldy, M, N, K, stream) \
+                             : launch_skinny<MT_, KC_, NW_, bf16_t>(x, ldx, W, ldw, bias, y, ldy, M, N, K, stream)
+  if (mt == 1) {
+    if (variant == 1) SK(1, 128, 8);
+    else if (variant == 2) SK(1, 64, 8);
+    else if (variant == 3) SK(1, 128, 16);
+    else SK(1, 64, 16);
+  } else if (mt == 2) {
+    if (variant == 1) SK(2, 128, 8);
+    else SK(2, 64, 16);
+  } else if (mt == 3) {
+    SK(3, 64, 8);
+  } else {
+    SK(4, 64, 8);
+  }
+#undef SK
+  if (rc) return rc;
+  LMSF_LAUNCH_CHECK("gemm_skinny");
+  return 0;
+}

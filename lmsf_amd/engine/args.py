@@ -35,6 +35,7 @@ class EngineArgs:
     load_format: str = "auto"                      # "auto": safetensors of the folder; "random": random weights
     prefill_chunk_size: Optional[int] = None
     num_gpu_blocks_override: Optional[int] = None
+    enforce_eager: bool = False                    # True: never capture decode steps as HIP graphs
     device: str = "cuda:0"
 
     def verify(self) -> None:
@@ -75,6 +76,7 @@ class EngineArgs:
           help="auto: the folder's safetensors; random: random weights for the folder's config.json")
         a("--prefill-chunk-size", type=int, default=None, help="longest portion of a prompt in one step")
         a("--num-gpu-blocks-override", type=int, default=None, help="pages of the cache instead of sizing from memory")
+        a("--enforce-eager", action="store_true", help="run decode steps kernel by kernel instead of as HIP graphs")
         a("--device", default="cuda:0")
         return parser
 

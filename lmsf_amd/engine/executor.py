@@ -26,7 +26,8 @@ def _align4(n: int) -> int:
 
 
 class ModelExecutor:
-    def __init__(self, model, storage: CacheStorage, rt: Runtime, max_model_len: int):
+    def __init__(self, model, storage: CacheStorage, rt: Runtime, max_model_len: int, use_graphs: bool = True,
+                 max_graph_batch: int = 256):
         self.model = model
         self.storage = storage
         self.manager: CacheManager = storage.manager
@@ -37,6 +38,11 @@ class ModelExecutor:
                              % (self.max_model_len, rt.max_positions))
         self.vocab_size = model.spec.vocab_size
         self._pinned: Optional[torch.Tensor] = None
+        # steps of single tokens are captured as HIP graphs, one per batch size
+        self.use_graphs = bool(use_graphs) and rt.device.type == "cuda"
+        self.max_graph_batch = int(max_graph_batch)
+        self._static: Dict[int, "_StaticBatch"] = {}
+        self._graph_pool = None
 
     # ------------------------------------------------------------------ the step
 
@@ -65,8 +71,17 @@ class ModelExecutor:
             for rid in added:
                 mgr.free_request(rid)
             raise
-        ctx = self._build_context(entries, starts)
-        logits = self.model.forward(ctx)
+        try:
+            if self.use_graphs and all(len(e.tokens) == 1 for e in entries) and len(entries) <= self.max_graph_batch:
+                logits = self._graph_step(entries, starts)
+            else:
+                logits = self.model.forward(self._build_context(entries, starts))
+        except Exception:
+            for rid in appended:
+                mgr.rollback(rid)
+            for rid in added:
+                mgr.free_request(rid)
+            raise
         for e in entries:
             mgr.commit(e.request_id)
         return logits
@@ -97,7 +112,12 @@ class ModelExecutor:
                 raise StepError("request %r would hold %d tokens, more than max_model_len %d"
                                 % (e.request_id, held + n, self.max_model_len))
 
-    def _build_context(self, entries: Sequence[StepEntry], starts: Sequence[int]) -> StepContext:
+    def _build_context(self, entries: Sequence[StepEntry], starts: Sequence[int],
+                       static: Optional["_StaticBatch"] = None) -> StepContext:
+        """Flatten the entries into the step's device tensors. Everything goes through one pinned staging
+        buffer and one copy. With ``static`` (a decode step that replays a captured graph) the copy goes
+        into that batch's fixed device buffer, block tables padded to their full width, and every
+        token's logits are asked for."""
         mgr = self.manager
         S = len(entries)
         lens = [len(e.tokens) for e in entries]
@@ -116,6 +136,8 @@ class ModelExecutor:
             seg_of.extend([s] * lens[s])
             logit_rows.extend(seg_starts[s] + int(w) for w in e.want)
             state_slots.append(mgr.request(e.request_id).state_slot)
+        if static is not None:
+            logit_rows = list(range(N))
         G = len(mgr.groups)
         group_slots: List[List[int]] = []
         group_tables: List[List[List[int]]] = []
@@ -128,20 +150,9 @@ class ModelExecutor:
                 tables.append([p if p >= 0 else 0 for p in mgr.block_table(e.request_id, gi)])
             group_slots.append(sl)
             group_tables.append(tables)
-            widths.append(max(1, max(len(t) for t in tables)))
-        # one pinned staging buffer, one copy to the device, views into it
+            widths.append(static.widths[gi] if static is not None else max(1, max(len(t) for t in tables)))
         R = len(logit_rows)
-        sections = [("token_ids", N), ("positions", N), ("seg_of", N), ("seg_starts", S + 1), ("seg_first", S),
-                    ("state_slots", S), ("logit_rows", R)]
-        for gi in range(G):
-            sections.append(("slots%d" % gi, N))
-            sections.append(("tables%d" % gi, S * widths[gi]))
-        offsets: Dict[str, Tuple[int, int]] = {}
-        total = 0
-        for name, n in sections:
-            offsets[name] = (total, n)
-            total += _align4(n)
-        total = max(total, 4)
+        offsets, total = self._layout(N, S, R, widths)
         if self._pinned is None or self._pinned.numel() < total:
             self._pinned = torch.empty(max(total, 4096), dtype=torch.int32,
                                        pin_memory=self.rt.device.type == "cuda")
@@ -165,8 +176,13 @@ class ModelExecutor:
             for t in group_tables[gi]:
                 flat.extend(t + [0] * (widths[gi] - len(t)))
             put("tables%d" % gi, flat)
-        if self.rt.device.type == "cuda":
-            # the staging buffer is reused by the next step: wait for earlier copies out of it
+        # the copy is synchronous: the staging buffer is free again when the next step fills it
+        if static is not None:
+            static.device_buffer.copy_(host, non_blocking=False)
+            if static.context is not None:
+                return static.context
+            dev = static.device_buffer
+        elif self.rt.device.type == "cuda":
             dev = torch.empty(total, dtype=torch.int32, device=self.rt.device)
             dev.copy_(host, non_blocking=False)
         else:
@@ -185,5 +201,68 @@ class ModelExecutor:
             state_slots=view("state_slots"), logit_rows=view("logit_rows"), n_logit_rows=R, groups=groups,
             host_seg_starts=seg_starts, host_seg_lens=lens, host_seg_first_pos=list(starts),
             host_state_slots=state_slots, request_ids=[e.request_id for e in entries],
-            max_seg_len=max(lens), max_context=max(st + n for st, n in zip(starts, lens)),
-            all_single=all(n == 1 for n in lens))
+            max_seg_len=max(lens),
+            max_context=self.max_model_len if static is not None else max(st + n for st, n in zip(starts, lens)),
+            all_single=all(n == 1 for n in lens), replayed=static is not None)
+
+    @staticmethod
+    def _layout(N: int, S: int, R: int, widths: Sequence[int]):
+        """Offsets (in int32 elements, 16-byte aligned) of the sections of a step's metadata buffer."""
+        sections = [("token_ids", N), ("positions", N), ("seg_of", N), ("seg_starts", S + 1), ("seg_first", S),
+                    ("state_slots", S), ("logit_rows", R)]
+        for gi, w in enumerate(widths):
+            sections.append(("slots%d" % gi, N))
+            sections.append(("tables%d" % gi, S * w))
+        offsets: Dict[str, Tuple[int, int]] = {}
+        total = 0
+        for name, n in sections:
+            offsets[name] = (total, n)
+            total += _align4(n)
+        return offsets, max(total, 4)
+
+    # ------------------------------------------------------------------ decode steps as HIP graphs
+
+    def _graph_step(self, entries: Sequence[StepEntry], starts: Sequence[int]) -> torch.Tensor:
+        """A step of single tokens. The first step of a batch size runs eagerly and is then captured as a
+        HIP graph over a fixed metadata buffer; later steps of that size copy their metadata into the
+        buffer and replay the graph: one launch instead of hundreds. The graph computes the logits of
+        every token; the wanted rows are picked afterwards."""
+        B = len(entries)
+        sb = self._static.get(B)
+        if sb is None:
+            widths = [-(-self.max_model_len // g.page_size) for g in self.manager.groups]
+            _, total = self._layout(B, B, B, widths)
+            sb = _StaticBatch(widths, torch.zeros(total, dtype=torch.int32, device=self.rt.device))
+            self._static[B] = sb
+        ctx = self._build_context(entries, starts, static=sb)
+        if sb.graph is None:
+            sb.context = ctx
+            logits = self.model.forward(ctx)                 # eager: this step's result, and the warm-up
+            torch.cuda.current_stream().synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, pool=self._graph_pool):
+                sb.logits = self.model.forward(ctx)
+            sb.graph = graph
+            if self._graph_pool is None:
+                self._graph_pool = graph.pool()
+        else:
+            sb.graph.replay()
+            logits = sb.logits
+        wanted = [i for i, e in enumerate(entries) if len(e.want)]
+        if len(wanted) == B:
+            return logits.clone()
+        if not wanted:
+            return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.rt.device)
+        return logits[torch.tensor(wanted, device=self.rt.device)]
+
+
+class _StaticBatch:
+    """What a captured decode step of one batch size keeps: the fixed metadata buffer, the context whose
+    tensors are views into it, the graph and its output."""
+
+    def __init__(self, widths: Sequence[int], device_buffer: torch.Tensor):
+        self.widths = list(widths)
+        self.device_buffer = device_buffer
+        self.context: Optional[StepContext] = None
+        self.graph = None
+        self.logits: Optional[torch.Tensor] = None

@@ -47,6 +47,8 @@ class HipOps:
                 "the kernels are built for gfx950 only; this device reports %r" % self.device_arch)
         self._bad_flag = None
         self.use_library_gemm = True   # bfloat16 matrix products of many rows go to the BLAS library
+        self.skinny_variant = 0        # tiling of the few-rows kernel (0: default; others for tuning)
+        self.skinny_max_rows = 16      # rows up to which the few-rows kernel beats the library (measured)
 
     # ------------------------------------------------------------------ helpers
 
@@ -238,14 +240,35 @@ class HipOps:
         if bias is not None and (bias.shape != (N,) or bias.dtype != weight.dtype or not bias.is_contiguous()):
             raise ValueError("linear: bias must be [%d] of the weight's dtype" % N)
         out_dtype = out_dtype or x.dtype
-        if (self.use_library_gemm and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
-                and out_dtype == torch.bfloat16 and M > 64):
-            return torch.nn.functional.linear(x, weight, bias)
+        both_bf16 = x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
+        if both_bf16 and self._skinny_ok(x, weight):
+            # few rows: the weight-streaming kernel. It also serves float32 output (logits), which the
+            # library does not offer, for any number of rows, 64 at a time.
+            limit = self.skinny_max_rows if out_dtype == torch.bfloat16 else 64
+            if M <= limit or out_dtype == torch.float32:
+                y = torch.empty((M, N), dtype=out_dtype, device=x.device)
+                for r0 in range(0, M, 64):
+                    rows = min(64, M - r0)
+                    xs, ys = x[r0:r0 + rows], y[r0:r0 + rows]
+                    self._check(self.lib.lmsf_gemm_skinny(
+                        _ptr(xs), xs.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(ys),
+                        _code(out_dtype), ys.stride(0), rows, N, K, self.skinny_variant, self._stream()))
+                return y
+        if self.use_library_gemm and both_bf16 and M > self.skinny_max_rows:
+            y = torch.nn.functional.linear(x, weight, bias)
+            return y if out_dtype == torch.bfloat16 else y.to(out_dtype)
         y = torch.empty((M, N), dtype=out_dtype, device=x.device)
         self._check(self.lib.lmsf_gemm_plain(_ptr(x), _code(x.dtype), x.stride(0), _ptr(weight), _code(weight.dtype),
                                              weight.stride(0), _ptr(bias), _ptr(y), _code(out_dtype), y.stride(0),
                                              M, N, K, self._stream()))
         return y
+
+    @staticmethod
+    def _skinny_ok(x: torch.Tensor, weight: torch.Tensor) -> bool:
+        """What the few-rows kernel asks of its operands: K and the row strides multiples of 8, 16-byte bases."""
+        K = x.shape[1]
+        return (K % 8 == 0 and x.stride(0) % 8 == 0 and weight.stride(0) % 8 == 0
+                and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
 
     # ------------------------------------------------------------------ sampling
 

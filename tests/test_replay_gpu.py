@@ -181,3 +181,26 @@ def test_trace_run_program(models, dtype, tmp_path):
     refs_cut = dict(refs)
     refs_cut[first["id"]] = refs[first["id"]][len(first["tokens"]):]
     check(got, refs_cut, dtype, "trace_run mixed")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_graph_replay_equals_eager(models, dtype):
+    """Decode steps are captured as HIP graphs and replayed. Every replay must give what the same step
+    gives kernel by kernel: the comparison is bitwise, over many replays, with eager steps of other
+    shapes (prompt portions) and synchronisations between the replays."""
+    folder, cfg, w = models[("B", dtype)]
+    from lmsf_amd.engine import load_engine_core
+    reqs = {"p": random_tokens(70, cfg["vocab_size"], 301), "q": random_tokens(45, cfg["vocab_size"], 302),
+            "r": random_tokens(33, cfg["vocab_size"], 303)}
+    steps = trace_mixed(reqs, 512, seed=21, prompt_fraction=0.3)
+    assert sum(1 for s in steps if all(len(e["tokens"]) == 1 for e in s["entries"])) > 40
+    outs = []
+    for eager in (True, False):
+        core = load_engine_core(folder, dtype=dtype, block_size=16, num_pages=32, max_num_seqs=8,
+                                enforce_eager=eager)
+        assert core.executor.use_graphs == (not eager)
+        outs.append(replay_in_process(core.executor, steps))
+        if not eager:
+            assert core.executor._static and all(sb.graph is not None for sb in core.executor._static.values())
+    for rid in reqs:
+        assert torch.equal(outs[0][rid], outs[1][rid]), rid
