@@ -2,8 +2,8 @@
 
 The reference allocates per layer K [blocks, kv_heads, d/x, block, x] and V [blocks, kv_heads, d, block]
 (core/src/worker/cache_engine.rs:107-160) and sizes the pool from free device memory
-(core/src/worker/model_worker.rs:128-162, block bytes :cache_engine.rs:88-105). Here both K and V
-are [pages, kv_heads, page_size, head_dim]; runs of layers whose mixers declare equal needs form
+(core/src/worker/model_worker.rs:128-162, block bytes :cache_engine.rs:88-105). Here K is
+[pages, kv_heads, page_size, head_dim] and V [pages, kv_heads, head_dim, page_size]; runs of layers whose mixers declare equal needs form
 a group that shares page ids, so one block table serves all of them.
 """
 from dataclasses import dataclass
@@ -72,9 +72,11 @@ class CacheStorage:
                 b.group = self.entry_group[i]
                 if src is None:
                     g = self.groups[b.group]
-                    shape = (max(1, g.num_pages), cspec.num_kv_heads, g.page_size, cspec.head_dim)
-                    b.k_pages = torch.zeros(shape, dtype=rt.dtype, device=rt.device)
-                    b.v_pages = torch.zeros(shape, dtype=rt.dtype, device=rt.device)
+                    n = max(1, g.num_pages)
+                    b.k_pages = torch.zeros((n, cspec.num_kv_heads, g.page_size, cspec.head_dim), dtype=rt.dtype,
+                                            device=rt.device)
+                    b.v_pages = torch.zeros((n, cspec.num_kv_heads, cspec.head_dim, g.page_size), dtype=rt.dtype,
+                                            device=rt.device)
                 else:
                     b.k_pages, b.v_pages = bindings[src].k_pages, bindings[src].v_pages
                     b.writes_cache = False

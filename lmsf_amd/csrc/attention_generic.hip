@@ -3,7 +3,8 @@
 //
 // Query token t belongs to request segment seg[t] and stands at position pos[t]. It attends to
 // the keys at positions j in [max(0, pos - window + 1), pos] of that request, read from the pages
-// (key j lives in page block_table[seg][j / page_size] at offset j % page_size). All keys of a step
+// (key j lives in page block_table[seg][j / page_size] at offset j % page_size; K pages are
+// [page, kv_head, offset, d], V pages [page, kv_head, d, offset]). All keys of a step
 // are written to the pages before this kernel runs, so prompts, portions of prompts and single
 // decoded tokens are one case.
 //
@@ -30,7 +31,7 @@ __global__ __launch_bounds__(GEN_THREADS) void paged_attention_generic_kernel(
   extern __shared__ float smem[];
   float* sq = smem;                       // [d] query, pre-scaled
   float* sp = sq + d;                     // [256] scores, then probabilities
-  int* srow = (int*)(sp + GEN_THREADS);   // [256] row index of each key in the pages
+  int* srow = (int*)(sp + GEN_THREADS);   // [256] (page * nkv + g) * ps + offset of each key
   float* sacc = (float*)(srow + GEN_THREADS);  // [256] partial outputs of the key groups
   __shared__ float red[16];
 
@@ -76,7 +77,10 @@ __global__ __launch_bounds__(GEN_THREADS) void paged_attention_generic_kernel(
     __syncthreads();
     if (pv_active) {
       const int n = min(GEN_THREADS, p - j0 + 1);
-      for (int jj = og; jj < n; jj += ngroups) acc += sp[jj] * to_f32<T>(v_pages[(long)srow[jj] * d + oi]);
+      for (int jj = og; jj < n; jj += ngroups) {
+        const int row = srow[jj], head_base = row / ps, off = row - head_base * ps;
+        acc += sp[jj] * to_f32<T>(v_pages[((long)head_base * d + oi) * ps + off]);
+      }
     }
     __syncthreads();
   }

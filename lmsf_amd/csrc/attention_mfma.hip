@@ -1,0 +1,554 @@
+// Paged attention on the matrix cores, bfloat16 storage, float32 softmax and accumulation.
+//
+// Two kernels over the same cache (K pages [page, kv_head, offset, d], V pages transposed
+// [page, kv_head, d, offset]):
+//   - "prefill": tiles of consecutive query tokens of one request, any number of tokens per tile;
+//   - "decode": one query token per workgroup and split of its keys, followed by a reduction over
+//     the splits.
+// Both compute, per query head h with kv head h / (nh / nkv),
+//   s_j = scale * <q, k_j>,  p = softmax_j(s) over lo <= j <= pos,  out = sum_j p_j v_j
+// (core/src/model_executor/layers/attention.rs:91-103, :139-155;
+// vllm/kernels/attention/attention_kernels.cu:82-414). The reference's decode kernel rounds p to
+// the model's dtype before the product with v (:337-351); so does the matrix-core product here.
+//
+// Layout of the products (v_mfma_f32_16x16x32_bf16: A is 16 rows x 32 k, lane l holds row l % 16 and
+// k = (l / 16) * 8 .. + 7; B is 32 k x 16 columns with the same lane pattern; D[row][col]: lane l holds
+// column l % 16 and rows (l / 16) * 4 .. + 3).
+//   S^T[key][row] = K[key][:] . Q[row][:]       A = 16 keys of K, B = 16 query rows, k runs over d.
+//   O^T[dv][row]  = V^T[dv][key] . P^T[key][row] A = 16 output dims of V^T, B = P^T, k runs over 32 keys.
+// A lane that holds column ``row`` of S^T for the keys 4g .. 4g+3 of two 16-key blocks holds exactly
+// the eight k-values of P^T that the second product wants from it, if the product's k index is read as
+// (block, 4g + i); V^T is fetched with the same reading. So the probabilities never leave the lane
+// that computed them, and both K and V^T come straight from global memory in operand layout: K rows
+// are contiguous in d, V^T rows are contiguous in the key offset.
+//
+// The query rows of a workgroup are (token, head of the kv group) pairs, so that the heads that
+// share a kv head share its keys in registers.
+#include "common.h"
+
+#include <limits.h>
+#include <math.h>
+
+union Frag8 {
+  bf16x8_t v;
+  uint4 q;
+  uint2 h[2];
+  uint32_t w[4];
+};
+
+__device__ __forceinline__ uint32_t pack2_bf16(float a, float b) {
+  return (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16);
+}
+
+__device__ __forceinline__ int wave_max_i(int v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = max(v, __shfl_xor(v, o, 64));
+  return v;
+}
+__device__ __forceinline__ int wave_min_i(int v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = min(v, __shfl_xor(v, o, 64));
+  return v;
+}
+
+struct KvView {
+  const bf16_t* k;
+  const bf16_t* v;
+  const int* bt;   // block table row of the request
+  int btw;         // its width
+  int nkv, d, ps, kvh;
+};
+
+// Element offset of key ``key``'s row in the K pages.
+__device__ __forceinline__ long k_row_offset(const KvView& G, int key) {
+  int blk = key / G.ps;
+  if (blk > G.btw - 1) blk = G.btw - 1;   // keys beyond the table are masked by the caller; stay inside it
+  const int page = G.bt[blk];
+  return ((long)(page * G.nkv + G.kvh) * G.ps + (key - (key / G.ps) * G.ps)) * G.d;
+}
+// Element offset of (dv = 0, key) in the transposed V pages; add dv * ps.
+__device__ __forceinline__ long v_col_offset(const KvView& G, int key) {
+  int blk = key / G.ps;
+  if (blk > G.btw - 1) blk = G.btw - 1;
+  const int page = G.bt[blk];
+  return (long)(page * G.nkv + G.kvh) * G.d * G.ps + (key - (key / G.ps) * G.ps);
+}
+
+// ---------------------------------------------------------------- prefill
+
+// One workgroup of 4 waves per (tile, kv head, block of HB heads of its group). Wave w owns the rows
+// (w * NQB + j) * 16 + c, j < NQB, c = lane % 16; row r is token r / HB of the tile and head r % HB of
+// the block. tiles[2 i], tiles[2 i + 1]: first flat token and number of tokens of tile i.
+template <int DPAD, int NQB>
+__global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
+    const bf16_t* __restrict__ q, long q_stride, bf16_t* __restrict__ out, long out_stride,
+    const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages, const int* __restrict__ block_tables,
+    int btw, const int* __restrict__ tiles, const int* __restrict__ seg, const int* __restrict__ pos, int nh, int nkv,
+    int d, int ps, float scale_log2, int window, int HB, int n_hb) {
+  constexpr int DS = DPAD / 32, DV = DPAD / 16;
+  const int tile = blockIdx.x;
+  const int kvh = blockIdx.y / n_hb, hb = blockIdx.y - kvh * n_hb;
+  const int n_rep = nh / nkv;
+  const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, c = l & 15, g = l >> 4;
+  const int t0 = tiles[2 * tile], ntok = tiles[2 * tile + 1];
+  KvView G;
+  G.k = k_pages; G.v = v_pages; G.btw = btw; G.nkv = nkv; G.d = d; G.ps = ps; G.kvh = kvh;
+  G.bt = block_tables + (long)seg[t0] * btw;
+
+  int rpos[NQB], rlo[NQB];
+  long qoff[NQB], ooff[NQB];
+  int wmax = -1, wlo = INT_MAX;
+#pragma unroll
+  for (int j = 0; j < NQB; ++j) {
+    const int row = (w * NQB + j) * 16 + c;
+    const int t = row / HB, hin = hb * HB + (row - t * HB);
+    const bool valid = t < ntok && hin < n_rep;
+    const int tok = t0 + (valid ? t : 0);
+    const int p = valid ? pos[tok] : -1;
+    rpos[j] = p;
+    rlo[j] = (window > 0 && p >= 0) ? max(0, p - window + 1) : 0;
+    const int head = kvh * n_rep + (valid ? hin : 0);
+    qoff[j] = (long)tok * q_stride + (long)head * d;
+    ooff[j] = (long)tok * out_stride + (long)head * d;
+    wmax = max(wmax, p);
+    if (valid) wlo = min(wlo, rlo[j]);
+  }
+  wmax = wave_max_i(wmax);
+  wlo = wave_min_i(wlo);
+  if (wmax < 0) return;   // no row of this wave is in use (waves share nothing, so it may leave)
+
+  Frag8 qf[NQB][DS];
+#pragma unroll
+  for (int j = 0; j < NQB; ++j)
+#pragma unroll
+    for (int s = 0; s < DS; ++s) {
+      const int d0 = s * 32 + g * 8;
+      if (rpos[j] >= 0 && d0 < d)
+        qf[j][s].q = *reinterpret_cast<const uint4*>(q + qoff[j] + d0);
+      else
+        qf[j][s].q = make_uint4(0, 0, 0, 0);
+    }
+
+  f32x4_t acc[DV][NQB];
+  float m[NQB], lsum[NQB];
+#pragma unroll
+  for (int j = 0; j < NQB; ++j) {
+    m[j] = -INFINITY;
+    lsum[j] = 0.f;
+#pragma unroll
+    for (int v = 0; v < DV; ++v) acc[v][j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+  }
+
+  for (int kbase = (wlo / 32) * 32; kbase <= wmax; kbase += 32) {
+    // S^T for two blocks of 16 keys
+    f32x4_t st[2][NQB];
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      const long kr = k_row_offset(G, kbase + b * 16 + c);
+      Frag8 kf[DS];
+#pragma unroll
+      for (int s = 0; s < DS; ++s) {
+        const int d0 = s * 32 + g * 8;
+        if (d0 < d)
+          kf[s].q = *reinterpret_cast<const uint4*>(k_pages + kr + d0);
+        else
+          kf[s].q = make_uint4(0, 0, 0, 0);
+      }
+#pragma unroll
+      for (int j = 0; j < NQB; ++j) {
+        f32x4_t a = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < DS; ++s) a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[s].v, qf[j][s].v, a, 0, 0, 0);
+        st[b][j] = a;
+      }
+    }
+    // V^T addresses of this lane's two groups of four keys (issued early, used after the softmax)
+    const long vo0 = v_col_offset(G, kbase + 4 * g), vo1 = v_col_offset(G, kbase + 16 + 4 * g);
+    // mask, online softmax, probabilities as the B operand of the second product
+    Frag8 pf[NQB];
+#pragma unroll
+    for (int j = 0; j < NQB; ++j) {
+      float sv[8];
+      float mx = -INFINITY;
+#pragma unroll
+      for (int b = 0; b < 2; ++b)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = kbase + b * 16 + g * 4 + i;
+          const bool ok = key <= rpos[j] && key >= rlo[j];
+          const float x = ok ? st[b][j][i] * scale_log2 : -INFINITY;
+          sv[b * 4 + i] = x;
+          mx = fmaxf(mx, x);
+        }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = fmaxf(m[j], mx);
+      const bool dead = m_new == -INFINITY;           // nothing seen yet by this row
+      const float corr = (m[j] == -INFINITY) ? (dead ? 1.f : 0.f) : exp2f(m[j] - m_new);
+      float ps_ = 0.f;
+      float pv[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        pv[e] = dead ? 0.f : exp2f(sv[e] - m_new);
+        ps_ += pv[e];
+      }
+      lsum[j] = lsum[j] * corr + ps_;
+      m[j] = m_new;
+#pragma unroll
+      for (int v = 0; v < DV; ++v) acc[v][j] *= corr;
+      pf[j].w[0] = pack2_bf16(pv[0], pv[1]);
+      pf[j].w[1] = pack2_bf16(pv[2], pv[3]);
+      pf[j].w[2] = pack2_bf16(pv[4], pv[5]);
+      pf[j].w[3] = pack2_bf16(pv[6], pv[7]);
+    }
+    // O^T += V^T P^T
+#pragma unroll
+    for (int v = 0; v < DV; ++v) {
+      if (v * 16 < d) {
+        const long dvo = (long)(v * 16 + c) * ps;
+        Frag8 vf;
+        vf.h[0] = *reinterpret_cast<const uint2*>(v_pages + vo0 + dvo);
+        vf.h[1] = *reinterpret_cast<const uint2*>(v_pages + vo1 + dvo);
+#pragma unroll
+        for (int j = 0; j < NQB; ++j) acc[v][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[j].v, acc[v][j], 0, 0, 0);
+      }
+    }
+  }
+
+#pragma unroll
+  for (int j = 0; j < NQB; ++j) {
+    float ls = lsum[j];
+    ls += __shfl_xor(ls, 16, 64);
+    ls += __shfl_xor(ls, 32, 64);
+    if (rpos[j] < 0) continue;
+    const float inv = 1.0f / ls;
+#pragma unroll
+    for (int v = 0; v < DV; ++v) {
+      const int dv = v * 16 + g * 4;
+      if (dv < d) {
+        uint2 o;
+        o.x = pack2_bf16(acc[v][j][0] * inv, acc[v][j][1] * inv);
+        o.y = pack2_bf16(acc[v][j][2] * inv, acc[v][j][3] * inv);
+        *reinterpret_cast<uint2*>(out + ooff[j] + dv) = o;
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------- decode
+
+// One workgroup of 4 waves per (query token, kv head and block of up to 16 heads of its group, split).
+// Split s covers the keys [s * chunk, (s + 1) * chunk); wave w takes the 32-key steps w, w + 4, ... of it.
+// The waves' results are merged through LDS and written as a partial result
+//   part_o[((i * nh + head) * n_splits + s) * d + dv]  (not normalised),
+//   part_ml[((i * nh + head) * n_splits + s) * 2 + {0, 1}] = (running maximum in log2 units, sum),
+// i being the index of the token in this launch. A split without keys writes nothing; the reduction
+// knows from the position which splits have keys.
+template <int DPAD>
+__global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
+    const bf16_t* __restrict__ q, long q_stride, const bf16_t* __restrict__ k_pages,
+    const bf16_t* __restrict__ v_pages, const int* __restrict__ block_tables, int btw,
+    const int* __restrict__ tok_idx, const int* __restrict__ seg, const int* __restrict__ pos, int nh, int nkv, int d,
+    int ps, float scale_log2, int window, int HB, int n_hb, int chunk, int n_splits, float* __restrict__ part_o,
+    float* __restrict__ part_ml) {
+  constexpr int DS = DPAD / 32, DV = DPAD / 16;
+  extern __shared__ float lds_f[];
+  const int i_tok = blockIdx.x;
+  const int tok = tok_idx ? tok_idx[i_tok] : i_tok;
+  const int kvh = blockIdx.y / n_hb, hb = blockIdx.y - kvh * n_hb;
+  const int split = blockIdx.z;
+  const int n_rep = nh / nkv;
+  const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, c = l & 15, g = l >> 4;
+  const int p = pos[tok];
+  const int lo = window > 0 ? max(0, p - window + 1) : 0;
+  const int c0 = max(split * chunk, (lo / 32) * 32), c1 = min((split + 1) * chunk, p + 1);   // keys [c0, c1)
+  if (c0 >= c1) return;
+  KvView G;
+  G.k = k_pages; G.v = v_pages; G.btw = btw; G.nkv = nkv; G.d = d; G.ps = ps; G.kvh = kvh;
+  G.bt = block_tables + (long)seg[tok] * btw;
+
+  const int hin = hb * HB + c;
+  const bool valid = c < HB && hin < n_rep;
+  const int head = kvh * n_rep + (valid ? hin : 0);
+  Frag8 qf[DS];
+#pragma unroll
+  for (int s = 0; s < DS; ++s) {
+    const int d0 = s * 32 + g * 8;
+    if (valid && d0 < d)
+      qf[s].q = *reinterpret_cast<const uint4*>(q + (long)tok * q_stride + (long)head * d + d0);
+    else
+      qf[s].q = make_uint4(0, 0, 0, 0);
+  }
+  f32x4_t acc[DV];
+#pragma unroll
+  for (int v = 0; v < DV; ++v) acc[v] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, lsum = 0.f;
+
+  for (int kbase = c0 + w * 32; kbase < c1; kbase += 128) {
+    Frag8 kf[2][DS];
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      const long kr = k_row_offset(G, kbase + b * 16 + c);
+#pragma unroll
+      for (int s = 0; s < DS; ++s) {
+        const int d0 = s * 32 + g * 8;
+        if (d0 < d)
+          kf[b][s].q = *reinterpret_cast<const uint4*>(k_pages + kr + d0);
+        else
+          kf[b][s].q = make_uint4(0, 0, 0, 0);
+      }
+    }
+    const long vo0 = v_col_offset(G, kbase + 4 * g), vo1 = v_col_offset(G, kbase + 16 + 4 * g);
+    Frag8 vf[DV];
+#pragma unroll
+    for (int v = 0; v < DV; ++v) {
+      if (v * 16 < d) {
+        const long dvo = (long)(v * 16 + c) * ps;
+        vf[v].h[0] = *reinterpret_cast<const uint2*>(v_pages + vo0 + dvo);
+        vf[v].h[1] = *reinterpret_cast<const uint2*>(v_pages + vo1 + dvo);
+      }
+    }
+    float sv[8];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      f32x4_t a = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < DS; ++s) a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[b][s].v, qf[s].v, a, 0, 0, 0);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = kbase + b * 16 + g * 4 + i;
+        const bool ok = valid && key <= p && key >= lo && key < c1;
+        const float x = ok ? a[i] * scale_log2 : -INFINITY;
+        sv[b * 4 + i] = x;
+        mx = fmaxf(mx, x);
+      }
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m, mx);
+    const bool dead = m_new == -INFINITY;
+    const float corr = (m == -INFINITY) ? (dead ? 1.f : 0.f) : exp2f(m - m_new);
+    float pv[8], ps_ = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      pv[e] = dead ? 0.f : exp2f(sv[e] - m_new);
+      ps_ += pv[e];
+    }
+    lsum = lsum * corr + ps_;
+    m = m_new;
+    Frag8 pf;
+    pf.w[0] = pack2_bf16(pv[0], pv[1]);
+    pf.w[1] = pack2_bf16(pv[2], pv[3]);
+    pf.w[2] = pack2_bf16(pv[4], pv[5]);
+    pf.w[3] = pack2_bf16(pv[6], pv[7]);
+#pragma unroll
+    for (int v = 0; v < DV; ++v) {
+      if (v * 16 < d) {
+        acc[v] *= corr;
+        acc[v] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[v].v, pf.v, acc[v], 0, 0, 0);
+      }
+    }
+  }
+  lsum += __shfl_xor(lsum, 16, 64);
+  lsum += __shfl_xor(lsum, 32, 64);
+
+  // merge the four waves: lds_o[w][row c][dv], lds_m[w][c], lds_l[w][c]
+  float* lds_o = lds_f;                       // 4 * 16 * (DPAD + 4)
+  float* lds_m = lds_o + 4 * 16 * (DPAD + 4);
+  float* lds_l = lds_m + 64;
+#pragma unroll
+  for (int v = 0; v < DV; ++v)
+    *reinterpret_cast<f32x4_t*>(lds_o + (w * 16 + c) * (DPAD + 4) + v * 16 + g * 4) = acc[v];
+  if (g == 0) {
+    lds_m[w * 16 + c] = m;
+    lds_l[w * 16 + c] = lsum;
+  }
+  __syncthreads();
+  const int rows = min(HB, n_rep - hb * HB);
+  for (int e = tid; e < rows * d; e += 256) {
+    const int r = e / d, dv = e - r * d;
+    float M = lds_m[r];
+#pragma unroll
+    for (int ww = 1; ww < 4; ++ww) M = fmaxf(M, lds_m[ww * 16 + r]);
+    float o = 0.f, ls = 0.f;
+#pragma unroll
+    for (int ww = 0; ww < 4; ++ww) {
+      const float mw = lds_m[ww * 16 + r];
+      const float f = (mw == -INFINITY) ? 0.f : exp2f(mw - M);
+      o += f * lds_o[(ww * 16 + r) * (DPAD + 4) + dv];
+      ls += f * lds_l[ww * 16 + r];
+    }
+    const long slot = ((long)i_tok * nh + (kvh * n_rep + hb * HB + r)) * n_splits + split;
+    part_o[slot * d + dv] = o;
+    if (dv == 0) {
+      part_ml[slot * 2] = M;
+      part_ml[slot * 2 + 1] = ls;
+    }
+  }
+}
+
+// out[tok, head, :] = sum_s 2^(m_s - M) o_s / sum_s 2^(m_s - M) l_s over the splits that have keys.
+__global__ __launch_bounds__(256) void attn_decode_reduce_kernel(
+    const float* __restrict__ part_o, const float* __restrict__ part_ml, bf16_t* __restrict__ out, long out_stride,
+    const int* __restrict__ tok_idx, const int* __restrict__ pos, int nh, int d, int window, int chunk, int n_splits) {
+  const int i_tok = blockIdx.x, head = blockIdx.y;
+  const int tok = tok_idx ? tok_idx[i_tok] : i_tok;
+  const int p = pos[tok];
+  const int lo = window > 0 ? max(0, p - window + 1) : 0;
+  const int s0 = ((lo / 32) * 32) / chunk, s1 = min(n_splits - 1, p / chunk);   // splits s0 .. s1 have keys
+  const long base = ((long)i_tok * nh + head) * n_splits;
+  float M = -INFINITY;
+  for (int s = s0; s <= s1; ++s) M = fmaxf(M, part_ml[(base + s) * 2]);
+  float ls = 0.f;
+  for (int s = s0; s <= s1; ++s) ls += exp2f(part_ml[(base + s) * 2] - M) * part_ml[(base + s) * 2 + 1];
+  const float inv = 1.0f / ls;
+  for (int dv = threadIdx.x; dv < d; dv += blockDim.x) {
+    float o = 0.f;
+    for (int s = s0; s <= s1; ++s) o += exp2f(part_ml[(base + s) * 2] - M) * part_o[(base + s) * d + dv];
+    out[(long)tok * out_stride + (long)head * d + dv] = f32_to_bf16(o * inv);
+  }
+}
+
+// ---------------------------------------------------------------- entry points
+
+static int check_common(const char* who, const void* q, const void* out, const void* k_pages, const void* v_pages,
+                        const int* block_tables, const int* seg, const int* pos, long q_stride, long out_stride,
+                        long num_pages, int btw, int nh, int nkv, int d, int ps, int window) {
+  LMSF_CHECK(q && out && k_pages && v_pages && block_tables && seg && pos, "%s: null pointer", who);
+  LMSF_CHECK(nh > 0 && nkv > 0 && nh % nkv == 0, "%s: heads %d not a multiple of kv heads %d", who, nh, nkv);
+  LMSF_CHECK(d >= 16 && d % 16 == 0 && d <= 256, "%s: head size %d not supported (multiples of 16 up to 256)", who, d);
+  LMSF_CHECK(ps > 0 && ps % 4 == 0, "%s: page size %d not supported (multiples of 4)", who, ps);
+  LMSF_CHECK(btw > 0 && num_pages > 0, "%s: bad page geometry", who);
+  LMSF_CHECK(num_pages * nkv * (long)ps * d < 2147483647L * 64, "%s: cache too large", who);
+  LMSF_CHECK(num_pages * nkv < 2147483647L / 2, "%s: too many pages for 32-bit page arithmetic", who);
+  LMSF_CHECK(q_stride >= (long)nh * d && out_stride >= (long)nh * d && q_stride % 8 == 0 && out_stride % 4 == 0,
+             "%s: row strides must cover nh*d and keep 16-byte (q) and 8-byte (out) alignment", who);
+  LMSF_CHECK(lmsf_aligned16(q) && lmsf_aligned16(k_pages) && lmsf_aligned16(v_pages) && lmsf_aligned16(out),
+             "%s: operands must be 16-byte aligned", who);
+  LMSF_CHECK(window >= 0, "%s: negative window", who);
+  return 0;
+}
+
+static inline int heads_per_block(int n_rep) { return n_rep < 16 ? n_rep : 16; }
+
+// Rows of query (token, head) pairs a prefill workgroup holds; a tile may have at most
+// lmsf_attention_tile_tokens(nh, nkv) tokens.
+#define PREFILL_NQB 2
+#define PREFILL_ROWS (4 * PREFILL_NQB * 16)
+
+extern "C" int lmsf_attention_tile_tokens(int nh, int nkv) {
+  if (nh <= 0 || nkv <= 0 || nh % nkv) return 0;
+  return PREFILL_ROWS / heads_per_block(nh / nkv);
+}
+
+// tiles: int32 [n_tiles, 2] = (first flat token, number of tokens <= lmsf_attention_tile_tokens); all tokens
+// of a tile belong to one request and stand at consecutive positions.
+extern "C" int lmsf_paged_attention_prefill_mfma(const void* q, long q_stride, void* out, long out_stride,
+                                                 const void* k_pages, const void* v_pages, long num_pages,
+                                                 const int* block_tables, int btw, const int* tiles, int n_tiles,
+                                                 const int* seg, const int* pos, int nh, int nkv, int d, int ps,
+                                                 float scale, int window, hipStream_t stream) {
+  if (int rc = check_common("paged_attention_prefill", q, out, k_pages, v_pages, block_tables, seg, pos, q_stride,
+                            out_stride, num_pages, btw, nh, nkv, d, ps, window))
+    return rc;
+  LMSF_CHECK(tiles != nullptr && n_tiles >= 0, "paged_attention_prefill: bad tile list");
+  if (n_tiles == 0) return 0;
+  const int n_rep = nh / nkv, HB = heads_per_block(n_rep), n_hb = (n_rep + HB - 1) / HB;
+  LMSF_CHECK((long)nkv * n_hb <= 65535, "paged_attention_prefill: too many kv heads");
+  const float scale_log2 = scale * 1.44269504088896340736f;
+  dim3 grid(n_tiles, nkv * n_hb), block(256);
+  const int dpad = (d + 31) / 32 * 32;
+#define LAUNCH(DP)                                                                                                  \
+  hipLaunchKernelGGL((attn_prefill_mfma_kernel<DP, PREFILL_NQB>), grid, block, 0, stream, (const bf16_t*)q, q_stride, \
+                     (bf16_t*)out, out_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_tables, btw,   \
+                     tiles, seg, pos, nh, nkv, d, ps, scale_log2, window, HB, n_hb)
+  switch (dpad) {
+    case 32: LAUNCH(32); break;
+    case 64: LAUNCH(64); break;
+    case 96: LAUNCH(96); break;
+    case 128: LAUNCH(128); break;
+    case 160: LAUNCH(160); break;
+    case 192: LAUNCH(192); break;
+    case 224: LAUNCH(224); break;
+    default: LAUNCH(256); break;
+  }
+#undef LAUNCH
+  LMSF_LAUNCH_CHECK("paged_attention_prefill");
+  return 0;
+}
+
+template <int DPAD>
+static int launch_decode(dim3 grid, hipStream_t stream, const bf16_t* q, long q_stride, const bf16_t* k_pages,
+                         const bf16_t* v_pages, const int* block_tables, int btw, const int* tok_idx, const int* seg,
+                         const int* pos, int nh, int nkv, int d, int ps, float scale_log2, int window, int HB, int n_hb,
+                         int chunk, int n_splits, float* part_o, float* part_ml) {
+  const size_t smem = (size_t)(4 * 16 * (DPAD + 4) + 128) * sizeof(float);
+  auto kernel = attn_decode_mfma_kernel<DPAD>;
+  static bool configured = false;   // per instantiation
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) {
+      lmsf_set_error("paged_attention_decode: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
+      return 2;
+    }
+    configured = true;
+  }
+  hipLaunchKernelGGL(kernel, grid, dim3(256), smem, stream, q, q_stride, k_pages, v_pages, block_tables, btw, tok_idx,
+                     seg, pos, nh, nkv, d, ps, scale_log2, window, HB, n_hb, chunk, n_splits, part_o, part_ml);
+  return 0;
+}
+
+// Floats that part_o and part_ml must hold for a decode launch of n tokens.
+extern "C" long lmsf_attention_decode_scratch_floats(int n, int nh, int d, int n_splits) {
+  return (long)n * nh * n_splits * (d + 2);
+}
+
+// One query token per entry of tok_idx (null: tokens 0 .. n - 1). chunk: keys per split, a multiple of 128;
+// n_splits * chunk must cover the longest context. scratch: lmsf_attention_decode_scratch_floats floats.
+extern "C" int lmsf_paged_attention_decode_mfma(const void* q, long q_stride, void* out, long out_stride,
+                                                const void* k_pages, const void* v_pages, long num_pages,
+                                                const int* block_tables, int btw, const int* tok_idx, int n,
+                                                const int* seg, const int* pos, int nh, int nkv, int d, int ps,
+                                                float scale, int window, int chunk, int n_splits, float* scratch,
+                                                hipStream_t stream) {
+  if (int rc = check_common("paged_attention_decode", q, out, k_pages, v_pages, block_tables, seg, pos, q_stride,
+                            out_stride, num_pages, btw, nh, nkv, d, ps, window))
+    return rc;
+  LMSF_CHECK(n >= 0 && scratch != nullptr, "paged_attention_decode: bad arguments");
+  LMSF_CHECK(chunk > 0 && chunk % 128 == 0 && n_splits > 0 && n_splits <= 65535,
+             "paged_attention_decode: chunk %d must be a positive multiple of 128 and splits %d in [1, 65535]", chunk,
+             n_splits);
+  if (n == 0) return 0;
+  const int n_rep = nh / nkv, HB = heads_per_block(n_rep), n_hb = (n_rep + HB - 1) / HB;
+  LMSF_CHECK((long)nkv * n_hb <= 65535 && nh <= 65535, "paged_attention_decode: too many heads");
+  const float scale_log2 = scale * 1.44269504088896340736f;
+  const int dpad = (d + 31) / 32 * 32;
+  float* part_o = scratch;
+  float* part_ml = scratch + (long)n * nh * n_splits * d;
+  dim3 grid(n, nkv * n_hb, n_splits);
+  int rc = 0;
+#define LAUNCH(DP)                                                                                              \
+  rc = launch_decode<DP>(grid, stream, (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, \
+                         block_tables, btw, tok_idx, seg, pos, nh, nkv, d, ps, scale_log2, window, HB, n_hb, chunk, \
+                         n_splits, part_o, part_ml)
+  switch (dpad) {
+    case 32: LAUNCH(32); break;
+    case 64: LAUNCH(64); break;
+    case 96: LAUNCH(96); break;
+    case 128: LAUNCH(128); break;
+    case 160: LAUNCH(160); break;
+    case 192: LAUNCH(192); break;
+    case 224: LAUNCH(224); break;
+    default: LAUNCH(256); break;
+  }
+#undef LAUNCH
+  if (rc) return rc;
+  LMSF_LAUNCH_CHECK("paged_attention_decode");
+  int threads = (d + 63) / 64 * 64;
+  hipLaunchKernelGGL(attn_decode_reduce_kernel, dim3(n, nh), dim3(threads), 0, stream, part_o, part_ml, (bf16_t*)out,
+                     out_stride, tok_idx, pos, nh, d, window, chunk, n_splits);
+  LMSF_LAUNCH_CHECK("paged_attention_decode_reduce");
+  return 0;
+}

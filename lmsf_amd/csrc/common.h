@@ -16,6 +16,10 @@ enum { LMSF_F32 = 0, LMSF_BF16 = 1 };
 
 typedef uint16_t bf16_t;  // raw bfloat16 bits
 
+// operand and accumulator registers of the bfloat16 matrix-core instructions
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
+
 void lmsf_set_error(const char* fmt, ...);
 
 #define LMSF_CHECK(cond, ...)            \

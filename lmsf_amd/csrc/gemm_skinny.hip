@@ -23,8 +23,6 @@
 // lane l holds token m = l % 16 and the four outputs n = (l / 16) * 4 .. + 3.
 #include "common.h"
 
-typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
-typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));   // a 16-byte piece in flight
 
 template <int KC>

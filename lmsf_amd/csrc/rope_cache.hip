@@ -9,8 +9,9 @@
 //
 // Cache write (vllm/kernels/cache_kernels.cu:190-232): the token's rotated k and its v go to slot
 // s = page * page_size + offset; a negative slot is skipped. Page layout here is
-// [page, kv_head, offset, d] for both K and V (the reference uses [page, head, d/x, offset, x] and
-// [page, head, d, offset]; only the slot arithmetic is shared).
+// [page, kv_head, offset, d] for K and [page, kv_head, d, offset] for V, which the attention kernels read
+// as matrix-core operands without a transposition (the reference uses [page, head, d/x, offset, x] and,
+// like here, [page, head, d, offset]).
 //
 // q, k, v point at the first column of their parts inside one row-strided buffer (the fused QKV
 // output); row_stride is in elements. Either half may be switched off: table == null leaves q and
@@ -25,11 +26,15 @@ __global__ __launch_bounds__(256) void rope_cache_write_kernel(
   const long t = blockIdx.x;
   const int half = rot / 2;
   const float* cs = table ? table + (long)positions[t] * rot : nullptr;
-  long kdst = -1;  // element offset of (page, head 0, offset, 0)
+  long kdst = -1;  // element offset of (page, head 0, offset, 0) in the K pages
+  long vdst = -1;  // element offset of (page, head 0, 0, offset) in the V pages
   long head_step = (long)ps * d;
   if (slots) {
     const int s = slots[t];
-    if (s >= 0) kdst = ((long)(s / ps) * nkv * ps + (s % ps)) * d;
+    if (s >= 0) {
+      kdst = ((long)(s / ps) * nkv * ps + (s % ps)) * d;
+      vdst = (long)(s / ps) * nkv * ps * d + (s % ps);
+    }
   }
   if (cs && q) {
     T* qt = q + t * row_stride;
@@ -68,11 +73,11 @@ __global__ __launch_bounds__(256) void rope_cache_write_kernel(
       }
     }
   }
-  if (v && kdst >= 0) {
+  if (v && vdst >= 0) {
     const T* vt = v + t * row_stride;
     for (int idx = threadIdx.x; idx < nkv * d; idx += blockDim.x) {
       const int h = idx / d, i = idx % d;
-      v_pages[kdst + h * head_step + i] = vt[h * d + i];
+      v_pages[vdst + h * head_step + (long)i * ps] = vt[h * d + i];
     }
   }
 }

@@ -51,5 +51,6 @@ class StepContext:
     max_seg_len: int = 0
     max_context: int = 0           # longest context (tokens in cache after this step) among the segments
     all_single: bool = False       # every segment has exactly one token (a pure decode step)
+    aux: dict = field(default_factory=dict)   # what a part derived from this batch and keeps for the next layers
     replayed: bool = False         # the step is captured as a graph: parts must decide nothing from host facts
                                    # that change from step to step (max_context is the model's limit then)

@@ -38,10 +38,10 @@ class ModelExecutor:
                              % (self.max_model_len, rt.max_positions))
         self.vocab_size = model.spec.vocab_size
         self._pinned: Optional[torch.Tensor] = None
-        # steps of single tokens are captured as HIP graphs, one per batch size
+        # steps of single tokens are captured as HIP graphs, one per batch size and context bucket
         self.use_graphs = bool(use_graphs) and rt.device.type == "cuda"
         self.max_graph_batch = int(max_graph_batch)
-        self._static: Dict[int, "_StaticBatch"] = {}
+        self._static: Dict[Tuple[int, int], "_StaticBatch"] = {}
         self._graph_pool = None
 
     # ------------------------------------------------------------------ the step
@@ -202,7 +202,7 @@ class ModelExecutor:
             host_seg_starts=seg_starts, host_seg_lens=lens, host_seg_first_pos=list(starts),
             host_state_slots=state_slots, request_ids=[e.request_id for e in entries],
             max_seg_len=max(lens),
-            max_context=self.max_model_len if static is not None else max(st + n for st, n in zip(starts, lens)),
+            max_context=static.max_context if static is not None else max(st + n for st, n in zip(starts, lens)),
             all_single=all(n == 1 for n in lens), replayed=static is not None)
 
     @staticmethod
@@ -223,17 +223,24 @@ class ModelExecutor:
     # ------------------------------------------------------------------ decode steps as HIP graphs
 
     def _graph_step(self, entries: Sequence[StepEntry], starts: Sequence[int]) -> torch.Tensor:
-        """A step of single tokens. The first step of a batch size runs eagerly and is then captured as a
-        HIP graph over a fixed metadata buffer; later steps of that size copy their metadata into the
-        buffer and replay the graph: one launch instead of hundreds. The graph computes the logits of
-        every token; the wanted rows are picked afterwards."""
+        """A step of single tokens. The first step of a batch size and context bucket (the longest context
+        rounded up to a power of two) runs eagerly and is then captured as a HIP graph over a fixed
+        metadata buffer; later steps of that kind copy their metadata into the buffer and replay the
+        graph: one launch instead of hundreds. Inside a graph nothing may depend on the step's actual
+        context lengths but through the device tensors, so the parts are told the bucket as the longest
+        context. The graph computes the logits of every token; the wanted rows are picked afterwards."""
         B = len(entries)
-        sb = self._static.get(B)
+        longest = max(starts) + 1
+        bucket = 256
+        while bucket < longest:
+            bucket *= 2
+        bucket = min(bucket, self.max_model_len)
+        sb = self._static.get((B, bucket))
         if sb is None:
-            widths = [-(-self.max_model_len // g.page_size) for g in self.manager.groups]
+            widths = [-(-bucket // g.page_size) for g in self.manager.groups]
             _, total = self._layout(B, B, B, widths)
-            sb = _StaticBatch(widths, torch.zeros(total, dtype=torch.int32, device=self.rt.device))
-            self._static[B] = sb
+            sb = _StaticBatch(widths, torch.zeros(total, dtype=torch.int32, device=self.rt.device), bucket)
+            self._static[(B, bucket)] = sb
         ctx = self._build_context(entries, starts, static=sb)
         if sb.graph is None:
             sb.context = ctx
@@ -260,8 +267,9 @@ class _StaticBatch:
     """What a captured decode step of one batch size keeps: the fixed metadata buffer, the context whose
     tensors are views into it, the graph and its output."""
 
-    def __init__(self, widths: Sequence[int], device_buffer: torch.Tensor):
+    def __init__(self, widths: Sequence[int], device_buffer: torch.Tensor, max_context: int):
         self.widths = list(widths)
+        self.max_context = int(max_context)
         self.device_buffer = device_buffer
         self.context: Optional[StepContext] = None
         self.graph = None

@@ -155,13 +155,13 @@ class HipOps:
         num_pages, ps = 0, 1
         if slots is not None:
             self._i32(slots, "slots", N)
-            for name, pg in (("k_pages", k_pages), ("v_pages", v_pages)):
-                if pg is None or pg.dim() != 4 or pg.shape[1] != nkv or pg.shape[3] != d or not pg.is_contiguous() \
-                        or pg.dtype != qkv.dtype:
-                    raise ValueError("%s must be contiguous [pages, %d, page_size, %d] of %s" % (name, nkv, d, qkv.dtype))
-            if k_pages.shape != v_pages.shape:
-                raise ValueError("k_pages and v_pages differ in shape")
+            if k_pages is None or k_pages.dim() != 4 or k_pages.shape[1] != nkv or k_pages.shape[3] != d \
+                    or not k_pages.is_contiguous() or k_pages.dtype != qkv.dtype:
+                raise ValueError("k_pages must be contiguous [pages, %d, page_size, %d] of %s" % (nkv, d, qkv.dtype))
             num_pages, ps = k_pages.shape[0], k_pages.shape[2]
+            if v_pages is None or tuple(v_pages.shape) != (num_pages, nkv, d, ps) or not v_pages.is_contiguous() \
+                    or v_pages.dtype != qkv.dtype:
+                raise ValueError("v_pages must be contiguous [%d, %d, %d, %d] of %s" % (num_pages, nkv, d, ps, qkv.dtype))
         base = qkv.data_ptr()
         q = ctypes.c_void_p(base)
         k = ctypes.c_void_p(base + nh * d * es)
@@ -174,35 +174,107 @@ class HipOps:
 
     def paged_attention(self, q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                         block_tables: torch.Tensor, seg: torch.Tensor, pos: torch.Tensor, nh: int, nkv: int, d: int,
-                        scale: float, window: int = 0, batch=None) -> torch.Tensor:
+                        scale: float, window: int = 0, batch=None, kernel: Optional[str] = None) -> torch.Tensor:
         """Attention of every query token over the cached keys of its request.
 
         ``q`` is [N, >= nh*d] with unit column stride (it may be the fused QKV buffer, of which the
-        first nh*d columns are read). ``block_tables`` int32 [S, W]; ``seg``, ``pos`` int32 [N].
-        ``batch`` carries host-side facts about the step for the choice of kernel.
-        Returns [N, nh*d] in q's dtype.
+        first nh*d columns are read). ``k_pages`` [pages, nkv, page_size, d], ``v_pages``
+        [pages, nkv, d, page_size]. ``block_tables`` int32 [S, W]; ``seg``, ``pos`` int32 [N].
+        ``batch`` (engine.batch.StepContext) carries host-side facts about the step for the choice of
+        kernel; without it they are read back from ``seg`` and ``pos``. ``kernel`` forces "generic" or
+        "mfma" (tests). Returns [N, nh*d] in q's dtype.
         """
         self._dev(q, k_pages, v_pages, block_tables, seg, pos)
         if q.dim() != 2 or q.stride(1) != 1 or q.shape[1] < nh * d:
             raise ValueError("q must be [N, >= %d] with unit column stride" % (nh * d))
         N = q.shape[0]
-        for name, pg in (("k_pages", k_pages), ("v_pages", v_pages)):
-            if pg.dim() != 4 or pg.shape[1] != nkv or pg.shape[3] != d or not pg.is_contiguous() or pg.dtype != q.dtype:
-                raise ValueError("%s must be contiguous [pages, %d, page_size, %d] of %s" % (name, nkv, d, q.dtype))
-        if k_pages.shape != v_pages.shape:
-            raise ValueError("k_pages and v_pages differ in shape")
+        if k_pages.dim() != 4 or k_pages.shape[1] != nkv or k_pages.shape[3] != d or not k_pages.is_contiguous() \
+                or k_pages.dtype != q.dtype:
+            raise ValueError("k_pages must be contiguous [pages, %d, page_size, %d] of %s" % (nkv, d, q.dtype))
+        num_pages, ps = k_pages.shape[0], k_pages.shape[2]
+        if tuple(v_pages.shape) != (num_pages, nkv, d, ps) or not v_pages.is_contiguous() or v_pages.dtype != q.dtype:
+            raise ValueError("v_pages must be contiguous [%d, %d, %d, %d] of %s" % (num_pages, nkv, d, ps, q.dtype))
         if block_tables.dim() != 2:
             raise ValueError("block_tables must be [segments, width]")
         self._i32(block_tables, "block_tables")
         self._i32(seg, "seg", N)
         self._i32(pos, "pos", N)
         out = torch.empty((N, nh * d), dtype=q.dtype, device=q.device)
-        num_pages, ps = k_pages.shape[0], k_pages.shape[2]
-        self._check(self.lib.lmsf_paged_attention_generic(
-            _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pages), _ptr(v_pages), num_pages,
-            _ptr(block_tables), block_tables.shape[1], _ptr(seg), _ptr(pos), N, nh, nkv, d, ps, float(scale),
-            int(window or 0), _code(q.dtype), self._stream()))
+        if N == 0:
+            return out
+        fast_ok = (q.dtype == torch.bfloat16 and d % 16 == 0 and 16 <= d <= 256 and ps % 4 == 0
+                   and q.stride(0) % 8 == 0 and q.data_ptr() % 16 == 0)
+        if kernel == "mfma" and not fast_ok:
+            raise ValueError("the matrix-core attention kernels need bfloat16, a head size that is a multiple of 16 "
+                             "up to 256, a page size that is a multiple of 4 and 16-byte aligned query rows")
+        if kernel == "generic" or not fast_ok:
+            self._check(self.lib.lmsf_paged_attention_generic(
+                _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pages), _ptr(v_pages), num_pages,
+                _ptr(block_tables), block_tables.shape[1], _ptr(seg), _ptr(pos), N, nh, nkv, d, ps, float(scale),
+                int(window or 0), _code(q.dtype), self._stream()))
+            return out
+        plan = self._attention_plan(batch, seg, pos, nh, nkv)
+        common = (_ptr(k_pages), _ptr(v_pages), num_pages, _ptr(block_tables), block_tables.shape[1])
+        if plan.tiles is not None:
+            self._check(self.lib.lmsf_paged_attention_prefill_mfma(
+                _ptr(q), q.stride(0), _ptr(out), out.stride(0), *common, _ptr(plan.tiles), plan.n_tiles,
+                _ptr(seg), _ptr(pos), nh, nkv, d, ps, float(scale), int(window or 0), self._stream()))
+        if plan.n_single:
+            n_hb = -(-(nh // nkv) // 16)
+            most = -(-plan.max_context // 128)
+            want = max(1, min(most, -(-1024 // (plan.n_single * nkv * n_hb))))
+            chunk = -(-(-(-plan.max_context // want)) // 128) * 128
+            n_splits = -(-plan.max_context // chunk)
+            floats = self.lib.lmsf_attention_decode_scratch_floats(plan.n_single, nh, d, n_splits)
+            scratch = torch.empty(floats, dtype=torch.float32, device=q.device)
+            self._check(self.lib.lmsf_paged_attention_decode_mfma(
+                _ptr(q), q.stride(0), _ptr(out), out.stride(0), *common, _ptr(plan.single_tokens), plan.n_single,
+                _ptr(seg), _ptr(pos), nh, nkv, d, ps, float(scale), int(window or 0), chunk, n_splits,
+                _ptr(scratch), self._stream()))
         return out
+
+    def _attention_plan(self, batch, seg: torch.Tensor, pos: torch.Tensor, nh: int, nkv: int) -> "_AttentionPlan":
+        """How a step's tokens are split between the two matrix-core kernels: requests with one token go
+        to the decode kernel, the others are cut into tiles for the prefill kernel. Computed once per step
+        and tile size, and kept on the batch for the other layers."""
+        tq = self.lib.lmsf_attention_tile_tokens(nh, nkv)
+        if batch is not None:
+            aux = batch.aux
+            key = ("attention_plan", tq)
+            if key in aux:
+                return aux[key]
+            lens, starts, max_context = batch.host_seg_lens, batch.host_seg_starts, batch.max_context
+            if batch.replayed or batch.all_single:
+                plan = _AttentionPlan(None, 0, None, batch.n_tokens, max_context)
+                aux[key] = plan
+                return plan
+        else:
+            seg_h = seg.tolist()
+            lens, starts = [], []
+            for i, sg in enumerate(seg_h):
+                if i == 0 or sg != seg_h[i - 1]:
+                    starts.append(i)
+                    lens.append(0)
+                lens[-1] += 1
+            max_context = int(pos.max().item()) + 1
+            aux, key = None, None
+        tiles, single = [], []
+        for st, n in zip(starts, lens):
+            if n == 1:
+                single.append(st)
+            else:
+                for t in range(0, n, tq):
+                    tiles.extend((st + t, min(tq, n - t)))
+        dev = seg.device
+        if len(single) == len(lens):
+            plan = _AttentionPlan(None, 0, None, len(single), max_context)
+        else:
+            both = torch.tensor(tiles + single, dtype=torch.int32).to(dev)
+            plan = _AttentionPlan(both[:len(tiles)], len(tiles) // 2,
+                                  both[len(tiles):] if single else None, len(single), max_context)
+        if aux is not None:
+            aux[key] = plan
+        return plan
 
     # ------------------------------------------------------------------ feed-forward
 
@@ -313,6 +385,17 @@ class HipOps:
         self._check(self.lib.lmsf_apply_penalties(_ptr(logits), logits.stride(0), R, V, _ptr(tokens), _ptr(offsets),
                                                   _ptr(prompt_lens), _ptr(counts), _ptr(presence), _ptr(frequency),
                                                   _ptr(repetition), self._stream()))
+
+
+class _AttentionPlan:
+    __slots__ = ("tiles", "n_tiles", "single_tokens", "n_single", "max_context")
+
+    def __init__(self, tiles, n_tiles, single_tokens, n_single, max_context):
+        self.tiles = tiles                    # int32 [n_tiles, 2] on the device, or None
+        self.n_tiles = n_tiles
+        self.single_tokens = single_tokens    # int32 flat indices of the one-token requests; None: every token
+        self.n_single = n_single
+        self.max_context = max_context
 
 
 _default_ops: Optional[HipOps] = None

@@ -116,7 +116,7 @@ class CacheBinding:
 
     group: Optional[int] = None            # index of the cache group (page pool + block tables)
     k_pages: Optional[torch.Tensor] = None  # [pages, kv_heads, page_size, head_dim]
-    v_pages: Optional[torch.Tensor] = None
+    v_pages: Optional[torch.Tensor] = None  # [pages, kv_heads, head_dim, page_size]
     writes_cache: bool = True              # False: reads another run's pages
     state: Optional[torch.Tensor] = None   # [slots, *StateSpec.shape]
 

@@ -101,8 +101,7 @@ def test_rope_cache_write(ops, ref, dtype, nh, nkv, d, rot, neox, ps):
     slots = torch.randperm(pages * ps, generator=g)[:N].to(torch.int32)
     slots[3] = -1
     slots = dev(slots)
-    shape = (pages, nkv, ps, d)
-    k1, v1 = dev(torch.zeros(shape, dtype=dtype)), dev(torch.zeros(shape, dtype=dtype))
+    k1, v1 = dev(torch.zeros((pages, nkv, ps, d), dtype=dtype)), dev(torch.zeros((pages, nkv, d, ps), dtype=dtype))
     k2, v2 = k1.clone(), v1.clone()
     a, b = qkv.clone(), qkv.clone()
     ops.rope_cache_write(a, nh, nkv, d, pos, table, rot, neox, slots, k1, v1)
@@ -136,7 +135,7 @@ def _paged_case(dtype, nh, nkv, d, ps, seg_lens, ctx_lens, seed, spike=False):
             bt[s, b] = perm[at]
             at += 1
     k_pages = torch.randn(total, nkv, ps, d, generator=g)
-    v_pages = torch.randn(total, nkv, ps, d, generator=g)
+    v_pages = torch.randn(total, nkv, d, ps, generator=g)
     N = sum(seg_lens)
     q = torch.randn(N, nh * d + 8, generator=g)       # wider than nh*d: a strided view, like the fused QKV
     seg, pos = [], []
@@ -178,6 +177,65 @@ def test_paged_attention(ops, ref, dtype, shape, window):
     assert torch.allclose(a.float(), b.float(), **tol(dtype)), (a.float() - b.float()).abs().max()
 
 
+MFMA_SHAPES = [
+    # nh, nkv, d, page size, query tokens per segment, context per segment
+    (4, 2, 16, 8, [1, 7, 33], [1, 7, 33]),                     # head size 16: half a step of the product is padding
+    (5, 5, 48, 16, [2, 1, 1], [300, 17, 256]),                 # portions beside single tokens: both kernels, one call
+    (8, 1, 32, 16, [64, 1], [64, 513]),                        # 8 heads on one kv head
+    (6, 3, 80, 4, [3, 5], [40, 5]),                            # pages of 4
+    (32, 8, 128, 16, [1, 1, 1, 1], [700, 1, 257, 16]),         # decoding only: splits and their reduction
+    (32, 8, 128, 16, [130, 40], [130, 1000]),                  # several tiles per request, a long context before one
+    (40, 2, 64, 16, [1, 9], [300, 64]),                        # 20 heads per kv head: more than one block of heads
+    (2, 1, 256, 32, [9, 1], [70, 2000]),
+    (3, 1, 112, 16, [17], [129]),
+]
+
+
+@pytest.mark.parametrize("shape", MFMA_SHAPES)
+@pytest.mark.parametrize("window", [0, 24, 200])
+def test_paged_attention_matrix_core_kernels(ops, ref, shape, window):
+    nh, nkv, d, ps, seg_lens, ctx_lens = shape
+    q, kp, vp, bt, seg, pos = _paged_case(torch.bfloat16, nh, nkv, d, ps, seg_lens, ctx_lens, seed=nh + d + ps, spike=True)
+    scale = 1.0 / math.sqrt(d)
+    a = ops.paged_attention(q, kp, vp, bt, seg, pos, nh, nkv, d, scale, window, kernel="mfma")
+    b = ref.paged_attention(q, kp, vp, bt, seg, pos, nh, nkv, d, scale, window)
+    c = ops.paged_attention(q, kp, vp, bt, seg, pos, nh, nkv, d, scale, window, kernel="generic")
+    assert torch.allclose(a.float(), b.float(), **tol(torch.bfloat16)), (a.float() - b.float()).abs().max()
+    assert torch.allclose(c.float(), b.float(), **tol(torch.bfloat16)), (c.float() - b.float()).abs().max()
+
+
+def test_matrix_core_attention_refuses_what_it_cannot_do(ops):
+    q, kp, vp, bt, seg, pos = _paged_case(torch.bfloat16, 2, 1, 24, 16, [3], [3], seed=1)
+    with pytest.raises(ValueError, match="multiple of 16"):
+        ops.paged_attention(q, kp, vp, bt, seg, pos, 2, 1, 24, 0.2, kernel="mfma")
+    out = ops.paged_attention(q, kp, vp, bt, seg, pos, 2, 1, 24, 0.2)      # the general kernel takes it
+    assert torch.isfinite(out.float()).all()
+
+
+def test_decode_attention_finds_a_far_key(ops):
+    """One key among thousands, in an early page, carries the answer; every split but one sees noise."""
+    nh, nkv, d, ps, ctx = 8, 2, 128, 16, 5000
+    g = torch.Generator().manual_seed(3)
+    pages = -(-ctx // ps)
+    perm = torch.randperm(pages, generator=g)
+    bt = perm.to(torch.int32)[None, :]
+    kp = torch.randn(pages, nkv, ps, d, generator=g) * 0.1
+    vp = torch.randn(pages, nkv, d, ps, generator=g) * 0.1
+    q = torch.randn(1, nh * d, generator=g)
+    far = 37
+    page, off = int(perm[far // ps]), far % ps
+    for h in range(nkv):
+        kp[page, h, off] = q[0, h * (nh // nkv) * d:h * (nh // nkv) * d + d] * 4.0     # matches the group's first head
+        vp[page, h, :, off] = 5.0
+    args = (dev(q.bfloat16()), dev(kp.bfloat16()), dev(vp.bfloat16()), dev(bt), dev(torch.zeros(1, dtype=torch.int32)),
+            dev(torch.tensor([ctx - 1], dtype=torch.int32)), nh, nkv, d, 1.0 / math.sqrt(d))
+    out = ops.paged_attention(*args, kernel="mfma").float().cpu().view(nh, d)
+    for h in range(nkv):
+        assert (out[h * (nh // nkv)] - 5.0).abs().max() < 0.1      # softmax is all on the far key
+    with_window = ops.paged_attention(*args, 64, kernel="mfma").float().cpu().view(nh, d)
+    assert with_window.abs().max() < 1.0                           # out of the window: gone
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_paged_attention_reduces_to_library_softmax(ops, dtype):
     """One request, one head, no rotation: the kernel must equal softmax(q k^T / sqrt d) v of torch."""
@@ -188,9 +246,10 @@ def test_paged_attention_reduces_to_library_softmax(ops, dtype):
     v = torch.randn(T, d, generator=g).to(dtype)
     pages = -(-T // ps)
     kp = torch.zeros(pages, 1, ps, d, dtype=dtype)
-    vp = torch.zeros(pages, 1, ps, d, dtype=dtype)
     kp.view(pages * ps, d)[:T] = k
-    vp.view(pages * ps, d)[:T] = v
+    vt = torch.zeros(pages * ps, d, dtype=dtype)
+    vt[:T] = v
+    vp = vt.view(pages, 1, ps, d).transpose(2, 3).contiguous()
     bt = torch.arange(pages, dtype=torch.int32)[None, :]
     out = ops.paged_attention(dev(q), dev(kp), dev(vp), dev(bt), dev(torch.zeros(T, dtype=torch.int32)),
                               dev(torch.arange(T, dtype=torch.int32)), 1, 1, d, 1.0 / math.sqrt(d))

@@ -109,7 +109,7 @@ class TorchOps:
             ok = sl >= 0
             page, off = sl[ok] // ps, sl[ok] % ps
             k_pages[page, :, off, :] = k[ok]
-            v_pages[page, :, off, :] = v[ok]
+            v_pages[page, :, :, off] = v[ok]
 
     # ------------------------------------------------------------ attention
     def paged_attention(self, q, k_pages, v_pages, block_tables, seg, pos, nh, nkv, d, scale, window=0, batch=None):
@@ -123,7 +123,7 @@ class TorchOps:
             js = torch.arange(lo, p + 1, device=q.device)
             pages = block_tables[s].long()[js // ps]
             keys = k_pages[pages, :, js % ps, :].to(torch.float32)      # [n, nkv, d]
-            vals = v_pages[pages, :, js % ps, :].to(torch.float32)
+            vals = v_pages[pages, :, :, js % ps].to(torch.float32)      # [n, nkv, d]
             qt = q[t, :nh * d].to(torch.float32).reshape(nh, d)
             keys = keys.repeat_interleave(rep, dim=1)                    # [n, nh, d]
             vals = vals.repeat_interleave(rep, dim=1)
