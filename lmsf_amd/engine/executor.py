@@ -39,7 +39,8 @@ class ModelExecutor:
         self.vocab_size = model.spec.vocab_size
         self._pinned: Optional[torch.Tensor] = None
         # steps of single tokens are captured as HIP graphs, one per batch size and context bucket
-        self.use_graphs = bool(use_graphs) and rt.device.type == "cuda"
+        self.use_graphs = bool(use_graphs) and rt.device.type == "cuda" and \
+            all(getattr(p, "graph_safe", False) for p in model.parts())
         self.max_graph_batch = int(max_graph_batch)
         self._static: Dict[Tuple[int, int], "_StaticBatch"] = {}
         self._graph_pool = None
@@ -202,8 +203,19 @@ class ModelExecutor:
             host_seg_starts=seg_starts, host_seg_lens=lens, host_seg_first_pos=list(starts),
             host_state_slots=state_slots, request_ids=[e.request_id for e in entries],
             max_seg_len=max(lens),
-            max_context=static.max_context if static is not None else max(st + n for st, n in zip(starts, lens)),
+            max_context=(static.max_context if static is not None else
+                         self._context_bucket(max(starts) + 1) if all(n == 1 for n in lens) else
+                         max(st + n for st, n in zip(starts, lens))),
             all_single=all(n == 1 for n in lens), replayed=static is not None)
+
+    def _context_bucket(self, longest: int) -> int:
+        """The longest context of a step of single tokens, rounded up to a power of two (at least 256, at
+        most the model's limit). Eager and replayed decode steps tell the parts this number instead of
+        the true one, so that both split the work alike and give the same bits."""
+        bucket = 256
+        while bucket < longest:
+            bucket *= 2
+        return min(bucket, self.max_model_len)
 
     @staticmethod
     def _layout(N: int, S: int, R: int, widths: Sequence[int]):
@@ -230,11 +242,7 @@ class ModelExecutor:
         context lengths but through the device tensors, so the parts are told the bucket as the longest
         context. The graph computes the logits of every token; the wanted rows are picked afterwards."""
         B = len(entries)
-        longest = max(starts) + 1
-        bucket = 256
-        while bucket < longest:
-            bucket *= 2
-        bucket = min(bucket, self.max_model_len)
+        bucket = self._context_bucket(max(starts) + 1)
         sb = self._static.get((B, bucket))
         if sb is None:
             widths = [-(-bucket // g.page_size) for g in self.manager.groups]

@@ -22,6 +22,8 @@ from .linear import FusedLinear, Linear
 
 @register_part("mixer", "paged_attention")
 class PagedAttention(Mixer):
+    graph_safe = True
+
     def __init__(self, prefix: str, rt: Runtime, hidden_size: int, num_heads: int, num_kv_heads: int,
                  head_dim: int, position: Optional[PartSpec] = None, qkv_bias: bool = False,
                  out_bias: bool = False, scale: Optional[float] = None, window: Optional[int] = None,

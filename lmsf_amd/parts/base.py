@@ -122,7 +122,15 @@ class CacheBinding:
 
 
 class Part:
-    """Base of every part. ``prefix`` is where its tensors live in the checkpoint."""
+    """Base of every part. ``prefix`` is where its tensors live in the checkpoint.
+
+    ``graph_safe`` says that the part's forward only launches work whose shapes and addresses follow
+    from the step's shapes (token count, table widths, ``max_context``), never from the values that
+    change from step to step on the host, so that a step can be captured as a HIP graph and replayed
+    with new contents in the same buffers. The engine captures decode steps only if every part of the
+    model says so; a part that loops over the step's requests in Python leaves it False."""
+
+    graph_safe = False
 
     def __init__(self, prefix: str, rt: Runtime):
         self.prefix = prefix

@@ -15,6 +15,8 @@ class PreNormResidualBlock(Block):
     previous block's output not yet added, and returns its feed-forward output not yet added.
     """
 
+    graph_safe = True
+
     ROLES = ("input", "post_mixer")
 
     def forward(self, branch: Optional[torch.Tensor], residual: torch.Tensor, ctx,

@@ -15,6 +15,8 @@ from .base import Part, Runtime, TensorDecl, register_part
 
 @register_part("embedding", "token_embedding")
 class TokenEmbedding(Part):
+    graph_safe = True
+
     def __init__(self, prefix: str, rt: Runtime, vocab_size: int, hidden_size: int, scale: float = 1.0,
                  weight_name: str = "weight"):
         super().__init__(prefix, rt)
@@ -37,6 +39,8 @@ class TokenEmbedding(Part):
 class LMHead(Part):
     """``weight_name`` is the full checkpoint name of the [V, H] matrix: the head's own, or the
     embedding table's when the two are tied (the loader then shares one device tensor)."""
+
+    graph_safe = True
 
     def __init__(self, prefix: str, rt: Runtime, vocab_size: int, hidden_size: int, weight_name: Optional[str] = None,
                  bias: bool = False):

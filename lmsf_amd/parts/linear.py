@@ -18,6 +18,8 @@ class FusedLinear(Part):
     ``sources`` is a list of (checkpoint sub-name, rows): the tensor ``prefix.sub-name.weight`` has
     shape [rows, in_features] and, with ``bias``, ``prefix.sub-name.bias`` has [rows]."""
 
+    graph_safe = True
+
     def __init__(self, prefix: str, rt: Runtime, in_features: int, sources: Sequence[Tuple[str, int]],
                  bias: bool = False):
         super().__init__(prefix, rt)

@@ -13,6 +13,8 @@ from .linear import FusedLinear, Linear
 
 @register_part("feed_forward", "gated_mlp")
 class GatedMLP(FeedForward):
+    graph_safe = True
+
     def __init__(self, prefix: str, rt: Runtime, hidden_size: int, intermediate_size: int, activation: str = "silu",
                  bias: bool = False, gate_name: str = "gate_proj", up_name: str = "up_proj",
                  down_name: str = "down_proj"):

@@ -43,6 +43,8 @@ class RotaryEncoding(PositionEncoding):
     """style "neox" pairs (i, i + rot/2), "gptj" pairs (2i, 2i+1)
     (vllm/kernels/pos_encoding_kernels.cu:12-36)."""
 
+    graph_safe = True
+
     def __init__(self, prefix: str, rt: Runtime, head_dim: int, theta: float, rotary_dim: Optional[int] = None,
                  scaling: Optional[Mapping[str, Any]] = None, style: str = "neox"):
         super().__init__(prefix, rt)

@@ -1,0 +1,188 @@
+"""Weights: reading by name, element types, the one error that lists everything, random-weights mode."""
+import json
+import os
+import struct
+
+import pytest
+import torch
+from safetensors.torch import load_file, save_file
+
+from helpers import TINY, TINY_A, TINY_B, make_model_folder
+
+from lmsf_amd.config import LlamaConfig, get_architecture
+from lmsf_amd.models import DecoderModel
+from lmsf_amd.parts import Runtime
+from lmsf_amd.weights import (SafetensorsError, SafetensorsFile, WeightsError, declared_tensors, list_weight_files,
+                              load_weights, write_random_model, write_safetensors)
+
+
+def cpu_model(cfg, dtype=torch.float32):
+    rt = Runtime(ops=None, device=torch.device("cpu"), dtype=dtype, max_positions=cfg.max_position_embeddings)
+    return DecoderModel(get_architecture(cfg.architecture).build_spec(cfg), rt)
+
+
+def rewrite(folder, change):
+    """Load model.safetensors, let ``change`` edit the dict of tensors, write it back."""
+    path = os.path.join(folder, "model.safetensors")
+    tensors = load_file(path)
+    change(tensors)
+    save_file(tensors, path)
+
+
+def test_declared_names_and_shapes_follow_the_configuration():
+    cfg = LlamaConfig.from_dict(TINY_B)
+    decls = declared_tensors(get_architecture(cfg.architecture), cfg)
+    assert decls["model.embed_tokens.weight"].shape == (1000, 128)
+    assert decls["model.layers.2.self_attn.q_proj.weight"].shape == (8 * 32, 128)
+    assert decls["model.layers.0.self_attn.k_proj.weight"].shape == (1 * 32, 128)
+    assert decls["model.layers.0.self_attn.k_proj.bias"].shape == (32,)
+    assert decls["model.layers.1.self_attn.o_proj.weight"].shape == (128, 256)
+    assert decls["model.layers.1.self_attn.o_proj.bias"].shape == (128,)
+    assert decls["model.layers.1.mlp.gate_proj.weight"].shape == (352, 128)
+    assert decls["model.layers.1.mlp.down_proj.weight"].shape == (128, 352)
+    assert decls["model.layers.1.input_layernorm.weight"].shape == (128,) and decls["model.norm.weight"].init == "ones"
+    assert decls["lm_head.weight"].shape == (1000, 128)
+    assert "model.layers.3.mlp.up_proj.weight" not in decls and "model.layers.0.mlp.up_proj.bias" not in decls
+    tied = declared_tensors(get_architecture("LlamaForCausalLM"), LlamaConfig.from_dict(TINY_A))
+    assert "lm_head.weight" not in tied and "model.layers.0.self_attn.q_proj.bias" not in tied
+
+
+def test_written_folder_is_read_by_the_safetensors_package_and_back(tmp_path):
+    folder, cfg = make_model_folder(tmp_path, "B")
+    theirs = load_file(os.path.join(folder, "model.safetensors"))
+    ours = SafetensorsFile(os.path.join(folder, "model.safetensors"))
+    assert set(theirs) == set(ours.entries)
+    for name in ("model.embed_tokens.weight", "model.layers.1.self_attn.v_proj.bias"):
+        assert torch.equal(theirs[name], ours.read(name))
+    ours.close()
+    with open(os.path.join(folder, "config.json")) as f:
+        assert LlamaConfig.from_dict(json.load(f)) == cfg
+    # same seed, same values; another seed, other values; norm weights are ones
+    again, _ = make_model_folder(tmp_path / "again", "B")
+    other, _ = make_model_folder(tmp_path / "other", "B", seed=5)
+    t2, t3 = load_file(os.path.join(again, "model.safetensors")), load_file(os.path.join(other, "model.safetensors"))
+    assert all(torch.equal(theirs[k], t2[k]) for k in theirs)
+    assert not torch.equal(theirs["lm_head.weight"], t3["lm_head.weight"])
+    assert torch.equal(theirs["model.norm.weight"], torch.ones(128))
+    w = theirs["model.layers.0.mlp.up_proj.weight"]
+    assert abs(w.std().item() - 0.02) < 0.002 and abs(w.mean().item()) < 0.002
+
+
+def test_fused_rows_and_tied_head(tmp_path):
+    folder, cfg = make_model_folder(tmp_path, "B")
+    model = cpu_model(cfg)
+    load_weights(model.parts(), folder, torch.device("cpu"), torch.float32)
+    raw = load_file(os.path.join(folder, "model.safetensors"))
+    att = model.blocks[1].mixer
+    p = "model.layers.1.self_attn."
+    assert torch.equal(att.qkv.weight, torch.cat([raw[p + "q_proj.weight"], raw[p + "k_proj.weight"],
+                                                  raw[p + "v_proj.weight"]]))
+    assert torch.equal(att.qkv.bias, torch.cat([raw[p + "q_proj.bias"], raw[p + "k_proj.bias"], raw[p + "v_proj.bias"]]))
+    ffn = model.blocks[1].feed_forward
+    assert torch.equal(ffn.gate_up.weight, torch.cat([raw["model.layers.1.mlp.gate_proj.weight"],
+                                                      raw["model.layers.1.mlp.up_proj.weight"]]))
+    folder_a, cfg_a = make_model_folder(tmp_path, "A")
+    tied = cpu_model(cfg_a)
+    load_weights(tied.parts(), folder_a, torch.device("cpu"), torch.float32)
+    assert tied.head.weight.data_ptr() == tied.embedding.weight.data_ptr()
+
+
+def test_element_types(tmp_path):
+    folder, cfg = make_model_folder(tmp_path, "A", dtype="bfloat16")
+    rewrite(folder, lambda t: t.update({"model.norm.weight": t["model.norm.weight"].float(),
+                                        "model.layers.0.mlp.down_proj.weight":
+                                            t["model.layers.0.mlp.down_proj.weight"].half()}))
+    m16 = cpu_model(cfg, torch.bfloat16)
+    load_weights(m16.parts(), folder, torch.device("cpu"), torch.bfloat16)
+    assert m16.embedding.weight.dtype == torch.bfloat16
+    assert m16.final_norm.weight.dtype == torch.float32                       # stored in 32 bits: stays so
+    assert m16.blocks[0].feed_forward.down.weight.dtype == torch.bfloat16     # float16 storage is converted
+    m32 = cpu_model(cfg, torch.float32)
+    load_weights(m32.parts(), folder, torch.device("cpu"), torch.float32)
+    assert all(p.weight.dtype == torch.float32 for p in m32.parts() if getattr(p, "weight", None) is not None)
+    rewrite(folder, lambda t: t.update({"model.norm.weight": torch.ones(64, dtype=torch.int32)}))
+    with pytest.raises(WeightsError, match="model.norm.weight.*stored as torch.int32"):
+        load_weights(cpu_model(cfg).parts(), folder, torch.device("cpu"), torch.float32)
+
+
+def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
+    folder, cfg = make_model_folder(tmp_path, "B")
+
+    def damage(t):
+        del t["model.layers.0.self_attn.q_proj.weight"]
+        del t["model.layers.2.mlp.down_proj.weight"]
+        t["model.layers.1.mlp.up_proj.weight"] = torch.zeros(352, 127)
+        t["model.norm.weight"] = torch.zeros(2, 64)
+        t["model.layers.7.input_layernorm.weight"] = torch.zeros(128)
+        t["model.layers.0.self_attn.rotary_emb.inv_freq"] = torch.zeros(16)   # tolerated: old exports carry it
+
+    rewrite(folder, damage)
+    with pytest.raises(WeightsError) as e:
+        load_weights(cpu_model(cfg).parts(), folder, torch.device("cpu"), torch.float32,
+                     tolerated=get_architecture(cfg.architecture).tolerated_tensors)
+    err = e.value
+    assert err.missing == ["model.layers.0.self_attn.q_proj.weight", "model.layers.2.mlp.down_proj.weight"]
+    assert err.unexpected == ["model.layers.7.input_layernorm.weight"]
+    assert err.wrong_shape == [("model.layers.1.mlp.up_proj.weight", (352, 128), (352, 127)),
+                               ("model.norm.weight", (128,), (2, 64))]
+    text = str(err)
+    for word in ("missing tensors (2)", "unexpected tensors (1)", "wrong shapes (2)", "q_proj.weight",
+                 "expected [352, 128] found [352, 127]", folder):
+        assert word in text
+    assert "rotary_emb" not in text
+
+
+def test_tied_checkpoint_may_carry_a_head(tmp_path):
+    folder, cfg = make_model_folder(tmp_path, "A")
+    rewrite(folder, lambda t: t.update({"lm_head.weight": t["model.embed_tokens.weight"].clone()}))
+    load_weights(cpu_model(cfg).parts(), folder, torch.device("cpu"), torch.float32,
+                 tolerated=get_architecture(cfg.architecture).tolerated_tensors)
+    with pytest.raises(WeightsError, match="unexpected tensors"):
+        load_weights(cpu_model(cfg).parts(), folder, torch.device("cpu"), torch.float32)
+
+
+def test_shards_with_index_equal_one_file(tmp_path):
+    folder, cfg = make_model_folder(tmp_path, "A")
+    tensors = load_file(os.path.join(folder, "model.safetensors"))
+    names = sorted(tensors)
+    shard = str(tmp_path / "sharded")
+    os.makedirs(shard)
+    halves = {"model-00001-of-00002.safetensors": names[::2], "model-00002-of-00002.safetensors": names[1::2]}
+    for fname, ns in halves.items():
+        write_safetensors(os.path.join(shard, fname), [(n, tensors[n]) for n in ns])
+    with open(os.path.join(shard, "model.safetensors.index.json"), "w") as f:
+        json.dump({"weight_map": {n: fname for fname, ns in halves.items() for n in ns}}, f)
+    assert [os.path.basename(p) for p in list_weight_files(shard)] == sorted(halves)
+    a, b = cpu_model(cfg), cpu_model(cfg)
+    load_weights(a.parts(), folder, torch.device("cpu"), torch.float32)
+    load_weights(b.parts(), shard, torch.device("cpu"), torch.float32)
+    assert torch.equal(a.blocks[1].mixer.qkv.weight, b.blocks[1].mixer.qkv.weight)
+    os.unlink(os.path.join(shard, "model-00002-of-00002.safetensors"))
+    with pytest.raises(WeightsError, match="not there"):
+        load_weights(cpu_model(cfg).parts(), shard, torch.device("cpu"), torch.float32)
+
+
+def test_broken_files_are_refused(tmp_path):
+    folder, cfg = make_model_folder(tmp_path, "A")
+    path = os.path.join(folder, "model.safetensors")
+    data = open(path, "rb").read()
+    with open(path, "wb") as f:
+        f.write(data[:len(data) - 100])
+    with pytest.raises(WeightsError, match="truncated"):
+        load_weights(cpu_model(cfg).parts(), folder, torch.device("cpu"), torch.float32)
+    with open(path, "wb") as f:
+        f.write(struct.pack("<Q", 1 << 40) + b"{}")
+    with pytest.raises(SafetensorsError, match="header length"):
+        SafetensorsFile(path)
+    os.unlink(path)
+    with pytest.raises(WeightsError, match="no safetensors file"):
+        load_weights(cpu_model(cfg).parts(), folder, torch.device("cpu"), torch.float32)
+
+
+def test_write_random_model_uses_the_requested_storage(tmp_path):
+    cfg = LlamaConfig.from_dict(TINY_A)
+    folder = write_random_model(str(tmp_path / "bf"), cfg, seed=3, dtype="bfloat16")
+    t = load_file(os.path.join(folder, "model.safetensors"))
+    assert all(v.dtype == torch.bfloat16 for v in t.values())
+    with open(os.path.join(folder, "config.json")) as f:
+        assert json.load(f)["torch_dtype"] == "bfloat16"
