@@ -19,6 +19,11 @@
 // and the read pattern) to change layout. The loads of the next chunk are issued before the current
 // chunk's LDS traffic and MFMAs, so a chunk per wave is always in flight.
 //
+// Gated form (GATED): W holds 2 N rows, the gate's N rows first and then the up projection's N rows (the
+// fused gate_up weight of a gated feed-forward). A workgroup then owns rows n0 .. n0 + 15 of both halves and
+// writes y[m][n] = act(g) * u with g and u the two products: the activation kernel and its traffic are gone
+// (the reference runs silu_and_mul as a kernel of its own, vllm/kernels/activation_kernels.cu:31-42).
+//
 // MFMA: v_mfma_f32_16x16x32_bf16, A = W tile (16 rows x 32 k), B = x tile (32 k x 16 tokens), D[n][m]:
 // lane l holds token m = l % 16 and the four outputs n = (l / 16) * 4 .. + 3.
 #include "common.h"
@@ -35,17 +40,19 @@ struct SkinnyTile {
   static constexpr int STEPS = KC / 32;                     // MFMA steps per chunk
 };
 
-template <int MT, int KC, int NW, typename TOut>
+// ACT: 0 none (plain linear layer), 1 silu-gated, 2 gelu-gated
+template <int MT, int KC, int NW, typename TOut, int ACT>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ x, long ldx,
                                                               const bf16_t* __restrict__ W, long ldw,
                                                               const bf16_t* __restrict__ bias, TOut* __restrict__ y,
                                                               long ldy, int M, int N, int K) {
   using T = SkinnyTile<KC>;
+  constexpr int WT = ACT ? 2 : 1;   // W tiles per chunk: gate and up, or one
   extern __shared__ __align__(16) unsigned char lds[];
   const int tid = threadIdx.x;
   const int wave = tid / 64, lane = tid % 64;
   const int n0 = blockIdx.x * 16;
-  unsigned char* my = lds + (size_t)wave * (1 + MT) * T::TILE_BYTES;
+  unsigned char* my = lds + (size_t)wave * (WT + MT) * T::TILE_BYTES;
 
   // global load coordinates of this lane inside a tile
   const int lrow = lane / T::LANES_PER_ROW;      // + i * ROWS_PER_LOAD
@@ -54,12 +61,13 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __re
   const int fr = lane % 16, fg = lane / 16;
 
   // row offsets (in elements) of this lane's 16-byte pieces; rows beyond the matrix repeat the last row
-  long woff[T::LOADS], xoff[MT][T::LOADS];
+  long woff[WT][T::LOADS], xoff[MT][T::LOADS];
 #pragma unroll
   for (int i = 0; i < T::LOADS; ++i) {
     int r = n0 + lrow + i * T::ROWS_PER_LOAD;
     if (r > N - 1) r = N - 1;
-    woff[i] = (long)r * ldw + lcol;
+#pragma unroll
+    for (int wt = 0; wt < WT; ++wt) woff[wt][i] = (long)(r + wt * N) * ldw + lcol;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       int m = mt * 16 + lrow + i * T::ROWS_PER_LOAD;
@@ -68,12 +76,14 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __re
     }
   }
 
-  f32x4_t acc[MT];
+  f32x4_t acc[WT][MT];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) acc[mt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+  for (int wt = 0; wt < WT; ++wt)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[wt][mt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 
   const int nchunks = (K + KC - 1) / KC;
-  u32x4_t wreg[T::LOADS], xreg[MT][T::LOADS];
+  u32x4_t wreg[WT][T::LOADS], xreg[MT][T::LOADS];
 
   // K is a multiple of 8, so a 16-byte piece is inside or outside the row as a whole; a piece outside
   // is read from the start of the row instead and multiplied by nothing (its x piece is zeroed)
@@ -84,7 +94,9 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __re
     const int kk_ = ok_ ? k_ : -lcol;                                                           \
     const unsigned keep_ = ok_ ? 0xffffffffu : 0u;                                              \
     _Pragma("unroll") for (int i = 0; i < T::LOADS; ++i) {                                      \
-      wreg[i] = *reinterpret_cast<const u32x4_t*>(W + woff[i] + kk_);                           \
+      _Pragma("unroll") for (int wt = 0; wt < WT; ++wt) {                                       \
+        wreg[wt][i] = *reinterpret_cast<const u32x4_t*>(W + woff[wt][i] + kk_);                 \
+      }                                                                                         \
       _Pragma("unroll") for (int mt = 0; mt < MT; ++mt) {                                       \
         xreg[mt][i] = *reinterpret_cast<const u32x4_t*>(x + xoff[mt][i] + kk_) & keep_;         \
       }                                                                                         \
@@ -100,9 +112,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __re
 #pragma unroll
     for (int i = 0; i < T::LOADS; ++i) {
       const int off = (lrow + i * T::ROWS_PER_LOAD) * T::ROW_BYTES + lcol * 2;
-      *reinterpret_cast<u32x4_t*>(my + off) = wreg[i];
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) *reinterpret_cast<u32x4_t*>(my + (1 + mt) * T::TILE_BYTES + off) = xreg[mt][i];
+      for (int wt = 0; wt < WT; ++wt) *reinterpret_cast<u32x4_t*>(my + wt * T::TILE_BYTES + off) = wreg[wt][i];
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) *reinterpret_cast<u32x4_t*>(my + (WT + mt) * T::TILE_BYTES + off) = xreg[mt][i];
     }
     const int next = c + NW;
     SKINNY_FETCH(next < nchunks ? next : c);
@@ -110,11 +123,14 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __re
 #pragma unroll
     for (int s = 0; s < T::STEPS; ++s) {
       const int off = fr * T::ROW_BYTES + s * 64 + fg * 16;
-      const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(my + off);
+      bf16x8_t a[WT];
+#pragma unroll
+      for (int wt = 0; wt < WT; ++wt) a[wt] = *reinterpret_cast<const bf16x8_t*>(my + wt * T::TILE_BYTES + off);
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
-        const bf16x8_t b = *reinterpret_cast<const bf16x8_t*>(my + (1 + mt) * T::TILE_BYTES + off);
-        acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, acc[mt], 0, 0, 0);
+        const bf16x8_t b = *reinterpret_cast<const bf16x8_t*>(my + (WT + mt) * T::TILE_BYTES + off);
+#pragma unroll
+        for (int wt = 0; wt < WT; ++wt) acc[wt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[wt], b, acc[wt][mt], 0, 0, 0);
       }
     }
     c = next;
@@ -123,32 +139,55 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __re
 
   // add the waves' partial sums in wave order
   __syncthreads();
-  float* red = reinterpret_cast<float*>(lds);   // [NW][MT][64 lanes][4]
+  float* red = reinterpret_cast<float*>(lds);   // [NW][WT][MT][64 lanes][4]
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt)
-    *reinterpret_cast<f32x4_t*>(red + (((size_t)wave * MT + mt) * 64 + lane) * 4) = acc[mt];
+  for (int wt = 0; wt < WT; ++wt)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+      *reinterpret_cast<f32x4_t*>(red + ((((size_t)wave * WT + wt) * MT + mt) * 64 + lane) * 4) = acc[wt][mt];
   __syncthreads();
   for (int e = tid; e < MT * 256; e += NW * 64) {
     const int mt = e / 256, l = (e % 256) / 4, j = e % 4;
-    float sum = 0.f;
+    float sum[WT];
 #pragma unroll
-    for (int w = 0; w < NW; ++w) sum += red[(((size_t)w * MT + mt) * 64 + l) * 4 + j];
+    for (int wt = 0; wt < WT; ++wt) {
+      sum[wt] = 0.f;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) sum[wt] += red[((((size_t)w * WT + wt) * MT + mt) * 64 + l) * 4 + j];
+    }
     const int n = n0 + (l / 16) * 4 + j, m = mt * 16 + l % 16;
     if (n < N && m < M) {
-      if (bias) sum += bf16_to_f32(bias[n]);
-      y[(long)m * ldy + n] = from_f32<TOut>(sum);
+      float r;
+      if (ACT == 0) {
+        r = sum[0];
+        if (bias) r += bf16_to_f32(bias[n]);
+      } else {
+        float g = sum[0], u = sum[WT - 1];
+        if (bias) {
+          g += bf16_to_f32(bias[n]);
+          u += bf16_to_f32(bias[N + n]);
+        }
+        // the two products are rounded to the storage type before the activation, as the unfused path
+        // stores them (so both paths give the same bits)
+        g = bf16_to_f32(f32_to_bf16(g));
+        u = bf16_to_f32(f32_to_bf16(u));
+        const float a = ACT == 1 ? g / (1.0f + expf(-g)) : 0.5f * g * (1.0f + erff(g * 0.70710678118654752f));
+        r = a * u;
+      }
+      y[(long)m * ldy + n] = from_f32<TOut>(r);
     }
   }
 }
 
-template <int MT, int KC, int NW, typename TOut>
+template <int MT, int KC, int NW, typename TOut, int ACT>
 static int launch_skinny(const void* x, long ldx, const void* W, long ldw, const void* bias, void* y, long ldy, int M,
                          int N, int K, hipStream_t stream) {
   using T = SkinnyTile<KC>;
-  const size_t stage = (size_t)NW * (1 + MT) * T::TILE_BYTES;
-  const size_t red = (size_t)NW * MT * 64 * 4 * sizeof(float);
+  constexpr int WT = ACT ? 2 : 1;
+  const size_t stage = (size_t)NW * (WT + MT) * T::TILE_BYTES;
+  const size_t red = (size_t)NW * WT * MT * 64 * 4 * sizeof(float);
   const size_t smem = stage > red ? stage : red;
-  auto kernel = gemm_skinny_kernel<MT, KC, NW, TOut>;
+  auto kernel = gemm_skinny_kernel<MT, KC, NW, TOut, ACT>;
   static bool configured = false;   // per instantiation
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -167,8 +206,11 @@ static int launch_skinny(const void* x, long ldx, const void* W, long ldw, const
 // x [M, K] bfloat16 (row stride ldx), W [N, K] bfloat16 (row stride ldw), bias [N] bfloat16 or null,
 // y [M, N] of out_dtype. Needs M <= 64, K a multiple of 8, 16-byte aligned x and W and row strides
 // that are multiples of 8 elements; anything else is refused. ``variant`` picks the tiling (0: default).
+// act 0: y = x W^T + bias. act 1 (silu) or 2 (gelu): W is [2 N, K] and bias [2 N], gate rows first;
+// y = act(x Wgate^T + bgate) * (x Wup^T + bup), bfloat16 output only.
 extern "C" int lmsf_gemm_skinny(const void* x, long ldx, const void* W, long ldw, const void* bias, void* y,
-                                int out_dtype, long ldy, int M, int N, int K, int variant, hipStream_t stream) {
+                                int out_dtype, long ldy, int M, int N, int K, int variant, int act,
+                                hipStream_t stream) {
   LMSF_CHECK(x && W && y, "gemm_skinny: null pointer");
   LMSF_CHECK(M >= 0 && M <= 64, "gemm_skinny: M=%d outside [0, 64]", M);
   LMSF_CHECK(N > 0 && K > 0 && K % 8 == 0, "gemm_skinny: K=%d must be a positive multiple of 8 (N=%d)", K, N);
@@ -176,12 +218,33 @@ extern "C" int lmsf_gemm_skinny(const void* x, long ldx, const void* W, long ldw
              "gemm_skinny: row strides must cover K and be multiples of 8");
   LMSF_CHECK(lmsf_aligned16(x) && lmsf_aligned16(W), "gemm_skinny: x and W must be 16-byte aligned");
   LMSF_CHECK(out_dtype == LMSF_F32 || out_dtype == LMSF_BF16, "gemm_skinny: unknown output dtype %d", out_dtype);
+  LMSF_CHECK(act >= 0 && act <= 2, "gemm_skinny: unknown activation %d", act);
+  LMSF_CHECK(act == 0 || out_dtype == LMSF_BF16, "gemm_skinny: the gated form writes bfloat16 only");
   if (M == 0) return 0;
   const int mt = (M + 15) / 16;
   int rc = 0;
-#define SK(MT_, KC_, NW_)                                                                                       \
-  rc = out_dtype == LMSF_F32 ? launch_skinny<MT_, KC_, NW_, float>(x, ldx, W, ldw, bias, y, ldy, M, N, K, stream) \
-                             : launch_skinny<MT_, KC_, NW_, bf16_t>(x, ldx, W, ldw, bias, y, ldy, M, N, K, stream)
+  if (act) {
+#define SKG(MT_, KC_, NW_)                                                                                     \
+  rc = act == 1 ? launch_skinny<MT_, KC_, NW_, bf16_t, 1>(x, ldx, W, ldw, bias, y, ldy, M, N, K, stream)       \
+                : launch_skinny<MT_, KC_, NW_, bf16_t, 2>(x, ldx, W, ldw, bias, y, ldy, M, N, K, stream)
+    if (mt == 1) {
+      if (variant == 1) SKG(1, 128, 8);
+      else SKG(1, 64, 16);
+    } else if (mt == 2) {
+      SKG(2, 64, 16);
+    } else if (mt == 3) {
+      SKG(3, 64, 8);
+    } else {
+      SKG(4, 64, 8);
+    }
+#undef SKG
+    if (rc) return rc;
+    LMSF_LAUNCH_CHECK("gemm_skinny (gated)");
+    return 0;
+  }
+#define SK(MT_, KC_, NW_)                                                                                          \
+  rc = out_dtype == LMSF_F32 ? launch_skinny<MT_, KC_, NW_, float, 0>(x, ldx, W, ldw, bias, y, ldy, M, N, K, stream) \
+                             : launch_skinny<MT_, KC_, NW_, bf16_t, 0>(x, ldx, W, ldw, bias, y, ldy, M, N, K, stream)
   if (mt == 1) {
     if (variant == 1) SK(1, 128, 8);
     else if (variant == 2) SK(1, 64, 8);

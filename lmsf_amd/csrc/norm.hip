@@ -49,9 +49,102 @@ __global__ __launch_bounds__(1024) void add_rms_norm_kernel(
   }
 }
 
+// The same for rows whose length is a multiple of 4 and at most 4 * 4 * 1024: every thread keeps its
+// elements in registers between the two passes (at most VPT vectors of 4), so the row is read once and
+// nothing is read back from memory that was just written. One workgroup per output row.
+template <typename T> struct Vec4;
+template <> struct Vec4<float> {
+  static __device__ __forceinline__ void load(const float* p, float* x) {
+    const float4 v = *reinterpret_cast<const float4*>(p);
+    x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
+  }
+  static __device__ __forceinline__ void store(float* p, const float* x) {
+    *reinterpret_cast<float4*>(p) = make_float4(x[0], x[1], x[2], x[3]);
+  }
+};
+template <> struct Vec4<bf16_t> {
+  static __device__ __forceinline__ void load(const bf16_t* p, float* x) {
+    const uint2 v = *reinterpret_cast<const uint2*>(p);
+    x[0] = __uint_as_float(v.x << 16); x[1] = __uint_as_float(v.x & 0xffff0000u);
+    x[2] = __uint_as_float(v.y << 16); x[3] = __uint_as_float(v.y & 0xffff0000u);
+  }
+  static __device__ __forceinline__ void store(bf16_t* p, const float* x) {
+    uint2 v;
+    v.x = (uint32_t)f32_to_bf16(x[0]) | ((uint32_t)f32_to_bf16(x[1]) << 16);
+    v.y = (uint32_t)f32_to_bf16(x[2]) | ((uint32_t)f32_to_bf16(x[3]) << 16);
+    *reinterpret_cast<uint2*>(p) = v;
+  }
+};
+
+template <typename TB, typename TO, typename TW, int VPT>
+__global__ __launch_bounds__(1024) void add_rms_norm_vec_kernel(
+    const TB* __restrict__ branch, float* __restrict__ residual, const TW* __restrict__ weight,
+    TO* __restrict__ out, const int* __restrict__ rows, int H, float eps, float weight_offset) {
+  __shared__ float red[16];
+  const int r = blockIdx.x;
+  const long src = rows ? (long)rows[r] : (long)r;
+  const TB* b = branch ? branch + src * H : nullptr;
+  float* res = residual ? residual + src * H : nullptr;
+  const bool write_res = (b != nullptr) && (res != nullptr) && (rows == nullptr);
+  const int nvec = H / 4;
+  float x[VPT][4];
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < VPT; ++k) {
+    const int v = threadIdx.x + k * blockDim.x;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) x[k][e] = 0.f;
+    if (v < nvec) {
+      if (b) Vec4<TB>::load(b + v * 4, x[k]);
+      if (res) {
+        float y[4];
+        Vec4<float>::load(res + v * 4, y);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) x[k][e] += y[e];
+      }
+      if (write_res) Vec4<float>::store(res + v * 4, x[k]);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) ss += x[k][e] * x[k][e];
+    }
+  }
+  ss = block_sum(ss, red);
+  const float inv = rsqrtf(ss / (float)H + eps);
+  TO* o = out + (long)r * H;
+#pragma unroll
+  for (int k = 0; k < VPT; ++k) {
+    const int v = threadIdx.x + k * blockDim.x;
+    if (v < nvec) {
+      float w[4], y[4];
+      Vec4<TW>::load(weight + v * 4, w);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) y[e] = x[k][e] * inv * (w[e] + weight_offset);
+      Vec4<TO>::store(o + v * 4, y);
+    }
+  }
+}
+
 template <typename TB, typename TO, typename TW>
 static void launch_norm(const void* branch, float* residual, const void* weight, void* out, const int* rows,
                         int n_out, int H, float eps, float woff, hipStream_t stream) {
+  const bool aligned = (branch == nullptr || (((uintptr_t)branch) & 15u) == 0) &&
+                       (residual == nullptr || (((uintptr_t)residual) & 15u) == 0) &&
+                       (((uintptr_t)weight) & 15u) == 0 && (((uintptr_t)out) & 15u) == 0;
+  if (H % 4 == 0 && H <= 16384 && aligned) {
+    const int nvec = H / 4;
+    int threads = (nvec + 63) / 64 * 64;
+    if (threads > 1024) threads = 1024;
+    // few vectors per thread also for short rows: at most 256 threads while one vector each suffices
+    const int vpt = (nvec + threads - 1) / threads;
+#define NORM_VEC(V)                                                                                          \
+  hipLaunchKernelGGL((add_rms_norm_vec_kernel<TB, TO, TW, V>), dim3(n_out), dim3(threads), 0, stream,         \
+                     (const TB*)branch, residual, (const TW*)weight, (TO*)out, rows, H, eps, woff)
+    if (vpt <= 1) NORM_VEC(1);
+    else if (vpt == 2) NORM_VEC(2);
+    else if (vpt == 3) NORM_VEC(3);
+    else NORM_VEC(4);
+#undef NORM_VEC
+    return;
+  }
   int threads = ((H + 3) / 4 + 63) / 64 * 64;
   if (threads > 1024) threads = 1024;
   if (threads < 64) threads = 64;

@@ -15,70 +15,63 @@
 //
 // q, k, v point at the first column of their parts inside one row-strided buffer (the fused QKV
 // output); row_stride is in elements. Either half may be switched off: table == null leaves q and
-// k unrotated, slots == null writes no cache. One workgroup per token.
+// k unrotated, slots == null writes no cache.
 #include "common.h"
 
+// One workgroup of 64 threads per (token, head): heads 0 .. nh-1 are q heads, then nkv k heads, then nkv
+// v heads. A decode step has few tokens, so the parallelism has to come from the heads.
 template <typename T>
-__global__ __launch_bounds__(256) void rope_cache_write_kernel(
+__global__ __launch_bounds__(64) void rope_cache_write_kernel(
     T* __restrict__ q, T* __restrict__ k, const T* __restrict__ v, long row_stride, const int* __restrict__ positions,
     const float* __restrict__ table, int rot, int neox, const int* __restrict__ slots, T* __restrict__ k_pages,
     T* __restrict__ v_pages, int nh, int nkv, int d, int ps) {
   const long t = blockIdx.x;
+  const int hy = blockIdx.y;
   const int half = rot / 2;
   const float* cs = table ? table + (long)positions[t] * rot : nullptr;
-  long kdst = -1;  // element offset of (page, head 0, offset, 0) in the K pages
-  long vdst = -1;  // element offset of (page, head 0, 0, offset) in the V pages
-  long head_step = (long)ps * d;
-  if (slots) {
-    const int s = slots[t];
-    if (s >= 0) {
-      kdst = ((long)(s / ps) * nkv * ps + (s % ps)) * d;
-      vdst = (long)(s / ps) * nkv * ps * d + (s % ps);
-    }
-  }
-  if (cs && q) {
-    T* qt = q + t * row_stride;
-    for (int idx = threadIdx.x; idx < nh * half; idx += blockDim.x) {
-      const int h = idx / half, i = idx % half;
+  int slot = -1;
+  if (slots) slot = slots[t];
+  if (hy < nh) {
+    if (!cs || !q) return;
+    T* x = q + t * row_stride + (long)hy * d;
+    for (int i = threadIdx.x; i < half; i += 64) {
       const int xi = neox ? i : 2 * i, yi = neox ? i + half : 2 * i + 1;
       const float c = cs[i], s = cs[half + i];
-      const float x = to_f32<T>(qt[h * d + xi]), y = to_f32<T>(qt[h * d + yi]);
-      qt[h * d + xi] = from_f32<T>(x * c - y * s);
-      qt[h * d + yi] = from_f32<T>(y * c + x * s);
+      const float a = to_f32<T>(x[xi]), b = to_f32<T>(x[yi]);
+      x[xi] = from_f32<T>(a * c - b * s);
+      x[yi] = from_f32<T>(b * c + a * s);
     }
-  }
-  if (k) {
-    T* kt = k + t * row_stride;
+  } else if (hy < nh + nkv) {
+    if (!k) return;
+    const int h = hy - nh;
+    T* x = k + t * row_stride + (long)h * d;
+    // element offset of (page, head h, offset, 0) in the K pages
+    T* dst = slot >= 0 ? k_pages + (((long)(slot / ps) * nkv + h) * ps + (slot % ps)) * d : nullptr;
     if (cs) {
-      for (int idx = threadIdx.x; idx < nkv * half; idx += blockDim.x) {
-        const int h = idx / half, i = idx % half;
+      for (int i = threadIdx.x; i < half; i += 64) {
         const int xi = neox ? i : 2 * i, yi = neox ? i + half : 2 * i + 1;
         const float c = cs[i], s = cs[half + i];
-        const float x = to_f32<T>(kt[h * d + xi]), y = to_f32<T>(kt[h * d + yi]);
-        const T xr = from_f32<T>(x * c - y * s), yr = from_f32<T>(y * c + x * s);
-        kt[h * d + xi] = xr;
-        kt[h * d + yi] = yr;
-        if (kdst >= 0) {
-          k_pages[kdst + h * head_step + xi] = xr;
-          k_pages[kdst + h * head_step + yi] = yr;
+        const float a = to_f32<T>(x[xi]), b = to_f32<T>(x[yi]);
+        const T xr = from_f32<T>(a * c - b * s), yr = from_f32<T>(b * c + a * s);
+        x[xi] = xr;
+        x[yi] = yr;
+        if (dst) {
+          dst[xi] = xr;
+          dst[yi] = yr;
         }
       }
     }
-    if (kdst >= 0) {
+    if (dst) {
       // the part of k that the rotation did not touch (all of it without a table)
-      const int lo = cs ? rot : 0, tail = d - lo;
-      for (int idx = threadIdx.x; idx < nkv * tail; idx += blockDim.x) {
-        const int h = idx / tail, i = lo + idx % tail;
-        k_pages[kdst + h * head_step + i] = kt[h * d + i];
-      }
+      for (int i = (cs ? rot : 0) + threadIdx.x; i < d; i += 64) dst[i] = x[i];
     }
-  }
-  if (v && vdst >= 0) {
-    const T* vt = v + t * row_stride;
-    for (int idx = threadIdx.x; idx < nkv * d; idx += blockDim.x) {
-      const int h = idx / d, i = idx % d;
-      v_pages[vdst + h * head_step + (long)i * ps] = vt[h * d + i];
-    }
+  } else {
+    if (!v || slot < 0) return;
+    const int h = hy - nh - nkv;
+    const T* x = v + t * row_stride + (long)h * d;
+    // element offset of (page, head h, 0, offset) in the transposed V pages
+    T* dst = v_pages + ((long)(slot / ps) * nkv + h) * ps * d + (slot % ps);
+    for (int i = threadIdx.x; i < d; i += 64) dst[(long)i * ps] = x[i];
   }
 }
 
@@ -100,12 +93,15 @@ extern "C" int lmsf_rope_cache_write(void* q, void* k, const void* v, int dtype,
     LMSF_CHECK(ps > 0 && num_pages > 0, "rope_cache_write: bad page geometry");
   }
   if (n_tokens == 0) return 0;
+  const int heads = nh + 2 * nkv;
+  LMSF_CHECK(heads > 0 && heads <= 65535, "rope_cache_write: %d heads do not fit the grid", heads);
+  dim3 grid(n_tokens, heads);
   if (dtype == LMSF_F32)
-    hipLaunchKernelGGL((rope_cache_write_kernel<float>), dim3(n_tokens), dim3(256), 0, stream, (float*)q, (float*)k,
+    hipLaunchKernelGGL((rope_cache_write_kernel<float>), grid, dim3(64), 0, stream, (float*)q, (float*)k,
                        (const float*)v, row_stride, positions, table, rot, neox, slots, (float*)k_pages,
                        (float*)v_pages, nh, nkv, d, ps);
   else
-    hipLaunchKernelGGL((rope_cache_write_kernel<bf16_t>), dim3(n_tokens), dim3(256), 0, stream, (bf16_t*)q,
+    hipLaunchKernelGGL((rope_cache_write_kernel<bf16_t>), grid, dim3(64), 0, stream, (bf16_t*)q,
                        (bf16_t*)k, (const bf16_t*)v, row_stride, positions, table, rot, neox, slots, (bf16_t*)k_pages,
                        (bf16_t*)v_pages, nh, nkv, d, ps);
   LMSF_LAUNCH_CHECK("rope_cache_write");

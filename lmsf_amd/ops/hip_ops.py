@@ -324,7 +324,7 @@ class HipOps:
                     xs, ys = x[r0:r0 + rows], y[r0:r0 + rows]
                     self._check(self.lib.lmsf_gemm_skinny(
                         _ptr(xs), xs.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(ys),
-                        _code(out_dtype), ys.stride(0), rows, N, K, self.skinny_variant, self._stream()))
+                        _code(out_dtype), ys.stride(0), rows, N, K, self.skinny_variant, 0, self._stream()))
                 return y
         if self.use_library_gemm and both_bf16 and M > self.skinny_max_rows:
             y = torch.nn.functional.linear(x, weight, bias)
@@ -334,6 +334,31 @@ class HipOps:
                                              weight.stride(0), _ptr(bias), _ptr(y), _code(out_dtype), y.stride(0),
                                              M, N, K, self._stream()))
         return y
+
+    def linear_gated(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                     kind: str = "silu") -> torch.Tensor:
+        """act(x Wg^T + bg) * (x Wu^T + bu) for the fused weight [2 I, K] = [Wg; Wu] (bias [2 I] likewise);
+        [M, I] in x's dtype. With few bfloat16 rows the activation is the epilogue of the weight-streaming
+        product; otherwise the product and the activation kernel run one after the other. Both ways round
+        the two products to the storage type before the activation, so they give the same bits."""
+        if weight.dim() != 2 or weight.shape[0] % 2 != 0:
+            raise ValueError("linear_gated: weight must be [2 I, K]")
+        kinds = {"silu": 1, "gelu": 2}
+        if kind not in kinds:
+            raise ValueError("unknown activation %r (known: %s)" % (kind, ", ".join(kinds)))
+        M, I = x.shape[0], weight.shape[0] // 2
+        if (x.dim() == 2 and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and 0 < M <= self.skinny_max_rows
+                and x.shape[1] == weight.shape[1] and x.stride(1) == 1 and weight.stride(1) == 1
+                and self._skinny_ok(x, weight)):
+            self._dev(x, weight, bias)
+            if bias is not None and (bias.shape != (2 * I,) or bias.dtype != weight.dtype or not bias.is_contiguous()):
+                raise ValueError("linear_gated: bias must be [%d] of the weight's dtype" % (2 * I))
+            y = torch.empty((M, I), dtype=x.dtype, device=x.device)
+            self._check(self.lib.lmsf_gemm_skinny(
+                _ptr(x), x.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(y), BF16, y.stride(0), M, I,
+                x.shape[1], self.skinny_variant, kinds[kind], self._stream()))
+            return y
+        return self.gated_act(self.linear(x, weight, bias), kind)
 
     @staticmethod
     def _skinny_ok(x: torch.Tensor, weight: torch.Tensor) -> bool:

@@ -30,6 +30,5 @@ class GatedMLP(FeedForward):
         return [self.gate_up, self.down]
 
     def forward(self, h: torch.Tensor) -> torch.Tensor:
-        gu = self.gate_up.forward(h)
-        a = self.rt.ops.gated_act(gu, self.activation)
+        a = self.rt.ops.linear_gated(h, self.gate_up.weight, self.gate_up.bias, self.activation)
         return self.down.forward(a)

@@ -300,6 +300,26 @@ def test_linear_bfloat16(ops, ref, M, N, K, bias, out_dtype):
     assert torch.allclose(y.float(), want, **t), (y.float() - want).abs().max()
 
 
+@pytest.mark.parametrize("M,I,K", [(1, 176, 64), (8, 14336, 4096), (16, 208, 80), (13, 1000, 328), (40, 352, 128)])
+@pytest.mark.parametrize("kind", ["silu", "gelu"])
+@pytest.mark.parametrize("bias", [False, True])
+def test_linear_gated(ops, ref, M, I, K, kind, bias):
+    """The gated feed-forward's first half: with few rows the activation is the product's epilogue. It must
+    give the bits of the product followed by the activation kernel, and both the plain formula."""
+    g = torch.Generator().manual_seed(M * I + K)
+    x = dev((torch.randn(M, K, generator=g)).bfloat16())
+    w = dev((torch.randn(2 * I, K, generator=g) * K ** -0.5).bfloat16())
+    b = dev(torch.randn(2 * I, generator=g).bfloat16()) if bias else None
+    fused = ops.linear_gated(x, w, b, kind)
+    two = ops.gated_act(ops.linear(x, w, b), kind)
+    assert fused.shape == (M, I) and fused.dtype == torch.bfloat16
+    assert torch.equal(fused, two)
+    want = ref.linear_gated(x.float(), w.float(), None if b is None else b.float(), kind)
+    assert (fused.float() - want).abs().max().item() <= 2e-2 * max(1.0, want.abs().max().item())
+    f32 = ops.linear_gated(x.float(), w.float(), None if b is None else b.float(), kind)      # float32: no fusion, no rounding
+    assert f32.dtype == torch.float32 and torch.allclose(f32, want, atol=1e-4, rtol=1e-4)
+
+
 def test_linear_mixed_storage(ops, ref):
     """A weight stored in 32 bits stays so and still multiplies bfloat16 activations."""
     g = torch.Generator().manual_seed(5)

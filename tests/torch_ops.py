@@ -144,6 +144,9 @@ class TorchOps:
             raise ValueError(kind)
         return (a * u).to(gu.dtype)
 
+    def linear_gated(self, x, weight, bias=None, kind="silu"):
+        return self.gated_act(self.linear(x, weight, bias), kind)
+
     def linear(self, x, weight, bias=None, out_dtype=None):
         y = x.to(torch.float32) @ weight.to(torch.float32).t()
         if bias is not None:
