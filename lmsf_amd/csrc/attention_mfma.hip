@@ -36,8 +36,18 @@ union Frag8 {
   uint32_t w[4];
 };
 
-__device__ __forceinline__ uint32_t pack2_bf16(float a, float b) {
-  return (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16);
+// Maximum over the four lanes l, l ^ 16, l ^ 32, l ^ 48 (the lanes that hold one query row's scores), with
+// gfx950's row and half-wave swaps: two VALU instructions each instead of two trips through LDS.
+// v_permlane16_swap exchanges the odd rows of 16 lanes of its first operand with the even rows of its
+// second, v_permlane32_swap the upper half of the first with the lower half of the second; with the same
+// value in both operands, the two results hold the two partners side by side.
+__device__ __forceinline__ float max_over_lane_groups(float x) {
+  unsigned u = __float_as_uint(x);
+  auto a = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  x = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  u = __float_as_uint(x);
+  auto b = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
 }
 
 __device__ __forceinline__ int wave_max_i(int v) {
@@ -180,8 +190,7 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
           sv[b * 4 + i] = x;
           mx = fmaxf(mx, x);
         }
-      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      mx = max_over_lane_groups(mx);
       const float m_new = fmaxf(m[j], mx);
       const bool dead = m_new == -INFINITY;           // nothing seen yet by this row
       const float corr = (m[j] == -INFINITY) ? (dead ? 1.f : 0.f) : exp2f(m[j] - m_new);
@@ -233,6 +242,322 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
       }
     }
   }
+}
+
+// The same with the keys and values staged in LDS by the workgroup and read from there by its four waves;
+// the kernel above has every wave fetch them from global memory for itself and spends its time waiting.
+// Here tiles of 32 keys travel from global memory straight into LDS (global_load_lds_dwordx4: lane i of a
+// wave writes its 16 bytes at the wave's LDS base + 16 i, whatever global address it reads), STAGES - 1
+// steps ahead of the one being multiplied, so that the memory latency is covered by several steps of work
+// and no registers are held by data in flight. One barrier per step.
+//
+// A stage holds the K tile [32 keys][DPAD] and the V^T tile [DPAD][32 keys], both without padding (the
+// transfer writes lane after lane). Bank conflicts of the operand reads are avoided by choosing which
+// piece each lane fetches: 16-byte piece ``col`` of K row ``row`` lies in slot (col - row) mod PR of its row,
+// piece ``p`` of V^T row ``dv`` in slot (p + dv / 4) mod 4. The request's block table is copied to LDS first,
+// so that no address waits for a lookup in global memory. Needs pages of 8, 16, 32, ... tokens.
+//
+// The transfer instruction is written as inline assembly: through the compiler's builtin every LDS read
+// that follows would first wait for all transfers in flight (the compiler cannot tell that they write other
+// stages), which undoes the pipelining. The waits are therefore explicit: s_waitcnt vmcnt(n) before the
+// barrier of each step.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"   // m0 is named as clobbered on purpose
+__device__ __forceinline__ void global_to_lds_16(const void* src, unsigned lds_base_uniform) {
+  // lane i's 16 bytes go to LDS address m0 + 16 i
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(lds_base_uniform)
+               : "memory", "m0");
+}
+#pragma clang diagnostic pop
+__device__ __forceinline__ unsigned lds_address(const void* p) {
+  return (unsigned)(size_t)(__attribute__((address_space(3))) const unsigned char*)p;
+}
+
+// A step of 32 keys costs a wave 32 matrix-core instructions (512 cycles); everything else has to stay below
+// that, so whatever does not change from step to step (which piece a lane moves, where it reads its
+// operands in a stage) is worked out before the loop, pages are powers of two (shifts, no divisions), the
+// mask is only applied in steps that touch the diagonal or the window's edge, and the accumulators are
+// only rescaled when a row's maximum has moved.
+template <int DPAD, int NQB, int STAGES>
+__global__ __launch_bounds__(256) void attn_prefill_dma_kernel(
+    const bf16_t* __restrict__ q, long q_stride, bf16_t* __restrict__ out, long out_stride,
+    const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages, const int* __restrict__ block_tables,
+    int btw, const int* __restrict__ tiles, const int* __restrict__ seg, const int* __restrict__ pos, int nh, int nkv,
+    int d, int ps_log2, float scale_log2, int window, int HB, int n_hb, int bt_cap) {
+  constexpr int DS = DPAD / 32, DV = DPAD / 16;
+  constexpr int PR = DPAD / 8;                   // 16-byte pieces per K row
+  constexpr int KTILE = 32 * DPAD * 2;           // bytes; the V^T tile has the same size
+  constexpr int STAGE = 2 * KTILE;
+  constexpr int LPW = DPAD / 32;                 // transfers per wave and stage (DPAD / 8 in all)
+  extern __shared__ __align__(16) unsigned char lds_raw[];   // [STAGES][STAGE], then the block table
+  int* lds_bt = reinterpret_cast<int*>(lds_raw + STAGES * STAGE);
+  const int tile = blockIdx.x;
+  const int kvh = blockIdx.y / n_hb, hb = blockIdx.y - kvh * n_hb;
+  const int n_rep = nh / nkv;
+  const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, c = l & 15, g = l >> 4;
+  const int t0 = tiles[2 * tile], ntok = tiles[2 * tile + 1];
+  const int* bt = block_tables + (long)seg[t0] * btw;
+  const int ps = 1 << ps_log2, pm = ps - 1;
+
+  // the workgroup's range of keys: positions of a tile are consecutive
+  const int p_first = pos[t0], p_last = p_first + ntok - 1;
+  const int k_begin = window > 0 ? (max(0, p_first - window + 1) / 32) * 32 : 0;
+  const int n_steps = (p_last - k_begin) / 32 + 1;
+  const int blk0 = k_begin >> ps_log2;                                   // first block of the table that is needed
+  const int n_blk = min(min(btw, (p_last >> ps_log2) + 1) - blk0, bt_cap);   // the host made sure bt_cap suffices
+  for (int i = tid; i < n_blk; i += 256) lds_bt[i] = bt[blk0 + i];
+
+  int rpos[NQB], rlo[NQB];
+  long qoff[NQB], ooff[NQB];
+  int wmax = -1, wlo = INT_MAX, wminpos = INT_MAX, wmaxlo = 0;
+#pragma unroll
+  for (int j = 0; j < NQB; ++j) {
+    const int row = (w * NQB + j) * 16 + c;
+    const int t = row / HB, hin = hb * HB + (row - t * HB);
+    const bool valid = t < ntok && hin < n_rep;
+    const int tok = t0 + (valid ? t : 0);
+    const int p = valid ? p_first + t : -1;
+    rpos[j] = p;
+    rlo[j] = (window > 0 && p >= 0) ? max(0, p - window + 1) : 0;
+    const int head = kvh * n_rep + (valid ? hin : 0);
+    qoff[j] = (long)tok * q_stride + (long)head * d;
+    ooff[j] = (long)tok * out_stride + (long)head * d;
+    wmax = max(wmax, p);
+    if (valid) {
+      wlo = min(wlo, rlo[j]);
+      wminpos = min(wminpos, p);
+      wmaxlo = max(wmaxlo, rlo[j]);
+    }
+  }
+  wmax = wave_max_i(wmax);
+  wlo = wave_min_i(wlo);
+  wminpos = wave_min_i(wminpos);   // a step whose keys all lie in [wmaxlo, wminpos] needs no mask
+  wmaxlo = wave_max_i(wmaxlo);
+
+  Frag8 qf[NQB][DS];
+#pragma unroll
+  for (int j = 0; j < NQB; ++j)
+#pragma unroll
+    for (int s = 0; s < DS; ++s) {
+      const int d0 = s * 32 + g * 8;
+      if (rpos[j] >= 0 && d0 < d)
+        qf[j][s].q = *reinterpret_cast<const uint4*>(q + qoff[j] + d0);
+      else
+        qf[j][s].q = make_uint4(0, 0, 0, 0);
+    }
+
+  f32x4_t acc[DV][NQB];
+  float m[NQB], lsum[NQB];
+#pragma unroll
+  for (int j = 0; j < NQB; ++j) {
+    m[j] = -INFINITY;
+    lsum[j] = 0.f;
+#pragma unroll
+    for (int v = 0; v < DV; ++v) acc[v][j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+  }
+
+  // what this lane moves in every step: transfer i of the wave covers pieces j * 64 .. j * 64 + 63 of a stage,
+  // j = w + 4 i; the first DPAD / 16 transfers are the K tile, the others the V^T tile
+  const long page_stride = (long)nkv * d << ps_log2;   // elements per page, K and V alike
+  int t_key[LPW], t_mul[LPW];
+  long t_fixed[LPW];
+  const bf16_t* t_base[LPW];
+#pragma unroll
+  for (int i = 0; i < LPW; ++i) {
+    const int j = w + 4 * i;
+    if (j < DPAD / 16) {
+      const int P = j * 64 + l;
+      const int row = P / PR, slot = P - row * PR;
+      int col = slot + row % PR;
+      if (col >= PR) col -= PR;
+      if (col * 8 >= d) col = 0;                   // beyond the head: any finite data, the query is zero there
+      t_key[i] = row;
+      t_mul[i] = d;
+      t_fixed[i] = ((long)kvh * d << ps_log2) + col * 8;
+      t_base[i] = k_pages;
+    } else {
+      const int P = (j - DPAD / 16) * 64 + l;
+      int dv = P >> 2;
+      const int slot = P & 3;
+      const int piece = (slot - (dv >> 2)) & 3;
+      if (dv >= d) dv = 0;                         // rows beyond the head are never read
+      t_key[i] = piece * 8;
+      t_mul[i] = 1;
+      t_fixed[i] = ((long)(kvh * d + dv) << ps_log2);
+      t_base[i] = v_pages;
+    }
+  }
+  // where this lane reads its operands in a stage (bytes)
+  int koff[2][DS];
+#pragma unroll
+  for (int b = 0; b < 2; ++b)
+#pragma unroll
+    for (int s = 0; s < DS; ++s) {
+      const int row = b * 16 + c;
+      int slot = s * 4 + g - row % PR;
+      if (slot < 0) slot += PR;
+      koff[b][s] = (row * PR + slot) * 16;
+    }
+  const int vrot = (g >> 1) + (c >> 2);            // (piece + dv / 4) mod 4 with dv = 16 v + c
+  const int voff0 = KTILE + c * 64 + (g & 1) * 8 + (vrot & 3) * 16;
+  const int voff1 = KTILE + c * 64 + (g & 1) * 8 + ((vrot + 2) & 3) * 16;
+
+  // The query fragments are pinned here, so that the compiler waits for their loads now and not, with a
+  // wait for everything in flight, inside the loop.
+#pragma unroll
+  for (int j = 0; j < NQB; ++j)
+#pragma unroll
+    for (int s = 0; s < DS; ++s) asm volatile("" : "+v"(qf[j][s].v));
+  __syncthreads();   // the block table is in LDS
+
+  // this wave's transfers of the step that starts at key kb, into the stage at byte ``stage_byte``
+  auto issue = [&](int kb, int stage_byte) {
+#pragma unroll
+    for (int i = 0; i < LPW; ++i) {
+      const int key = kb + t_key[i];
+      int blk = (key >> ps_log2) - blk0;
+      blk = min(blk, n_blk - 1);                   // keys beyond the last block are masked: any valid page
+      const long off = (long)lds_bt[blk] * page_stride + t_fixed[i] + (key & pm) * t_mul[i];
+      global_to_lds_16(t_base[i] + off, __builtin_amdgcn_readfirstlane(lds_address(lds_raw) + stage_byte +
+                                                                       (w + 4 * i) * 1024));
+    }
+  };
+
+#pragma unroll
+  for (int s = 0; s < STAGES - 1; ++s)
+    if (s < n_steps) issue(k_begin + s * 32, s * STAGE);
+
+  int consume = 0, produce = (STAGES - 1) * STAGE;   // byte offsets of the stage read now and of the one filled now
+  for (int it = 0; it < n_steps; ++it) {
+    const int kbase = k_begin + it * 32;
+    // step ``it`` has arrived when at most the transfers of the later steps are outstanding
+    if (it + STAGES - 2 < n_steps)
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"((STAGES - 2) * LPW) : "memory");
+    else
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();   // everybody's part of step ``it`` is there, and everybody is done with step ``it - 1``
+    if (it + STAGES - 1 < n_steps) issue(kbase + (STAGES - 1) * 32, produce);
+    produce = produce + STAGE == STAGES * STAGE ? 0 : produce + STAGE;
+    if (kbase <= wmax && kbase + 31 >= wlo) {
+      const unsigned char* st_base = lds_raw + consume;
+      f32x4_t st[2][NQB];
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        Frag8 kf[DS];
+#pragma unroll
+        for (int s = 0; s < DS; ++s) kf[s].q = *reinterpret_cast<const uint4*>(st_base + koff[b][s]);
+#pragma unroll
+        for (int j = 0; j < NQB; ++j) {
+          f32x4_t a = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int s = 0; s < DS; ++s) a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[s].v, qf[j][s].v, a, 0, 0, 0);
+          st[b][j] = a;
+        }
+      }
+      const bool need_mask = kbase + 31 > wminpos || kbase < wmaxlo;   // the same for the whole wave
+      Frag8 pf[NQB];
+#pragma unroll
+      for (int j = 0; j < NQB; ++j) {
+        float r[8];
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) r[b * 4 + i] = st[b][j][i];
+        if (need_mask) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const int key = kbase + (e >> 2) * 16 + g * 4 + (e & 3);
+            if (key > rpos[j] || key < rlo[j]) r[e] = -INFINITY;
+          }
+        }
+        float mx = fmaxf(fmaxf(fmaxf(r[0], r[1]), fmaxf(r[2], r[3])), fmaxf(fmaxf(r[4], r[5]), fmaxf(r[6], r[7])));
+        mx = max_over_lane_groups(mx);
+        const float m_new = fmaxf(m[j], mx * scale_log2);      // the scale is positive
+        if (__any(m_new > m[j])) {
+          // rows whose maximum moved rescale what they have; the others multiply by one
+          const float corr = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m[j] - m_new);
+          lsum[j] *= corr;
+#pragma unroll
+          for (int v = 0; v < DV; ++v) acc[v][j] *= corr;
+          m[j] = m_new;
+        }
+        // a row that has seen nothing yet has only masked keys here: exp2(-inf) = 0 whatever is subtracted
+        const float neg_m = (m[j] == -INFINITY) ? 0.f : -m[j];
+        float pv[8], ps_ = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          pv[e] = __builtin_amdgcn_exp2f(fmaf(r[e], scale_log2, neg_m));
+          ps_ += pv[e];
+        }
+        lsum[j] += ps_;
+        pf[j].w[0] = pack2_bf16(pv[0], pv[1]);
+        pf[j].w[1] = pack2_bf16(pv[2], pv[3]);
+        pf[j].w[2] = pack2_bf16(pv[4], pv[5]);
+        pf[j].w[3] = pack2_bf16(pv[6], pv[7]);
+      }
+#pragma unroll
+      for (int v = 0; v < DV; ++v) {
+        if (v * 16 < d) {
+          Frag8 vf;
+          vf.h[0] = *reinterpret_cast<const uint2*>(st_base + voff0 + v * 1024);
+          vf.h[1] = *reinterpret_cast<const uint2*>(st_base + voff1 + v * 1024);
+#pragma unroll
+          for (int j = 0; j < NQB; ++j) acc[v][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[j].v, acc[v][j], 0, 0, 0);
+        }
+      }
+    }
+    consume = consume + STAGE == STAGES * STAGE ? 0 : consume + STAGE;
+  }
+
+#pragma unroll
+  for (int j = 0; j < NQB; ++j) {
+    float ls = lsum[j];
+    ls += __shfl_xor(ls, 16, 64);
+    ls += __shfl_xor(ls, 32, 64);
+    if (rpos[j] < 0) continue;
+    const float inv = 1.0f / ls;
+#pragma unroll
+    for (int v = 0; v < DV; ++v) {
+      const int dv = v * 16 + g * 4;
+      if (dv < d) {
+        uint2 o;
+        o.x = pack2_bf16(acc[v][j][0] * inv, acc[v][j][1] * inv);
+        o.y = pack2_bf16(acc[v][j][2] * inv, acc[v][j][3] * inv);
+        *reinterpret_cast<uint2*>(out + ooff[j] + dv) = o;
+      }
+    }
+  }
+}
+
+// Entries of a block table that the LDS-staged kernel can keep beside its stages.
+#define PREFILL_BT_CAP 2048
+
+template <int DPAD>
+static int launch_prefill_dma(dim3 grid, hipStream_t stream, const bf16_t* q, long q_stride, bf16_t* out,
+                              long out_stride, const bf16_t* k_pages, const bf16_t* v_pages, const int* block_tables,
+                              int btw, const int* tiles, const int* seg, const int* pos, int nh, int nkv, int d, int ps,
+                              float scale_log2, int window, int HB, int n_hb) {
+  int ps_log2 = 0;
+  while ((1 << ps_log2) < ps) ++ps_log2;
+  // four stages of a head size of 128 and the table are 72 KB: two workgroups share a compute unit's LDS,
+  // and one's softmax runs beside the other's matrix products
+  constexpr int STAGES = DPAD <= 128 ? 4 : 3;
+  const size_t smem = (size_t)STAGES * 4 * 32 * DPAD + PREFILL_BT_CAP * sizeof(int);
+  auto kernel = attn_prefill_dma_kernel<DPAD, 2, STAGES>;
+  static bool configured = false;   // per instantiation
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) {
+      lmsf_set_error("paged_attention_prefill: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
+      return 2;
+    }
+    configured = true;
+  }
+  hipLaunchKernelGGL(kernel, grid, dim3(256), smem, stream, q, q_stride, out, out_stride, k_pages, v_pages,
+                     block_tables, btw, tiles, seg, pos, nh, nkv, d, ps_log2, scale_log2, window, HB, n_hb,
+                     PREFILL_BT_CAP);
+  return 0;
 }
 
 // ---------------------------------------------------------------- decode
@@ -324,8 +649,7 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
         mx = fmaxf(mx, x);
       }
     }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    mx = max_over_lane_groups(mx);
     const float m_new = fmaxf(m, mx);
     const bool dead = m_new == -INFINITY;
     const float corr = (m == -INFINITY) ? (dead ? 1.f : 0.f) : exp2f(m - m_new);
@@ -443,22 +767,46 @@ extern "C" int lmsf_attention_tile_tokens(int nh, int nkv) {
 }
 
 // tiles: int32 [n_tiles, 2] = (first flat token, number of tokens <= lmsf_attention_tile_tokens); all tokens
-// of a tile belong to one request and stand at consecutive positions.
+// of a tile belong to one request and stand at consecutive positions. variant 0: keys and values staged in
+// LDS where the page size and the table's width allow it (the default); 1: every wave fetches them itself.
 extern "C" int lmsf_paged_attention_prefill_mfma(const void* q, long q_stride, void* out, long out_stride,
                                                  const void* k_pages, const void* v_pages, long num_pages,
                                                  const int* block_tables, int btw, const int* tiles, int n_tiles,
                                                  const int* seg, const int* pos, int nh, int nkv, int d, int ps,
-                                                 float scale, int window, hipStream_t stream) {
+                                                 float scale, int window, int variant, hipStream_t stream) {
   if (int rc = check_common("paged_attention_prefill", q, out, k_pages, v_pages, block_tables, seg, pos, q_stride,
                             out_stride, num_pages, btw, nh, nkv, d, ps, window))
     return rc;
   LMSF_CHECK(tiles != nullptr && n_tiles >= 0, "paged_attention_prefill: bad tile list");
+  LMSF_CHECK(scale > 0.f, "paged_attention_prefill: the scale must be positive, got %g", (double)scale);
   if (n_tiles == 0) return 0;
   const int n_rep = nh / nkv, HB = heads_per_block(n_rep), n_hb = (n_rep + HB - 1) / HB;
   LMSF_CHECK((long)nkv * n_hb <= 65535, "paged_attention_prefill: too many kv heads");
   const float scale_log2 = scale * 1.44269504088896340736f;
   dim3 grid(n_tiles, nkv * n_hb), block(256);
   const int dpad = (d + 31) / 32 * 32;
+  if (variant == 0 && ps >= 8 && (ps & (ps - 1)) == 0 && btw <= PREFILL_BT_CAP) {
+    // tiles staged in LDS
+    int rc = 0;
+#define LAUNCH_LDS(DP)                                                                                           \
+  rc = launch_prefill_dma<DP>(grid, stream, (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride,                \
+                              (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_tables, btw, tiles, seg, pos, \
+                              nh, nkv, d, ps, scale_log2, window, HB, n_hb)
+    switch (dpad) {
+      case 32: LAUNCH_LDS(32); break;
+      case 64: LAUNCH_LDS(64); break;
+      case 96: LAUNCH_LDS(96); break;
+      case 128: LAUNCH_LDS(128); break;
+      case 160: LAUNCH_LDS(160); break;
+      case 192: LAUNCH_LDS(192); break;
+      case 224: LAUNCH_LDS(224); break;
+      default: LAUNCH_LDS(256); break;
+    }
+#undef LAUNCH_LDS
+    if (rc) return rc;
+    LMSF_LAUNCH_CHECK("paged_attention_prefill");
+    return 0;
+  }
 #define LAUNCH(DP)                                                                                                  \
   hipLaunchKernelGGL((attn_prefill_mfma_kernel<DP, PREFILL_NQB>), grid, block, 0, stream, (const bf16_t*)q, q_stride, \
                      (bf16_t*)out, out_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_tables, btw,   \

@@ -43,12 +43,18 @@ void lmsf_set_error(const char* fmt, ...);
 
 __device__ __forceinline__ float bf16_to_f32(bf16_t v) { return __uint_as_float(((uint32_t)v) << 16); }
 
-// round to nearest even; NaN stays NaN
+// round to nearest even (one v_cvt_pk_bf16_f32 on gfx950)
 __device__ __forceinline__ bf16_t f32_to_bf16(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (bf16_t)(u >> 16);
+  const __bf16 b = (__bf16)f;
+  return *reinterpret_cast<const bf16_t*>(&b);
+}
+// two values in one register, a in the low half
+typedef __bf16 lmsf_bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float lmsf_f32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack2_bf16(float a, float b) {
+  const lmsf_f32x2_t v = {a, b};
+  const lmsf_bf16x2_t r = __builtin_convertvector(v, lmsf_bf16x2_t);
+  return *reinterpret_cast<const uint32_t*>(&r);
 }
 
 template <typename T> __device__ __forceinline__ float to_f32(T v);

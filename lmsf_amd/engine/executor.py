@@ -9,9 +9,10 @@ trace replay can take the logits.
 """
 from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
+import numpy as np
 import torch
 
-from ..cache.manager import CacheManager, OutOfPages
+from ..cache.manager import CacheError, CacheManager, OutOfPages
 from ..cache.storage import CacheStorage
 from ..parts.base import Runtime
 from .batch import GroupView, StepContext, StepEntry
@@ -38,6 +39,7 @@ class ModelExecutor:
                              % (self.max_model_len, rt.max_positions))
         self.vocab_size = model.spec.vocab_size
         self._pinned: Optional[torch.Tensor] = None
+        self._pinned_np: Optional[np.ndarray] = None
         # steps of single tokens are captured as HIP graphs, one per batch size and context bucket
         self.use_graphs = bool(use_graphs) and rt.device.type == "cuda" and \
             all(getattr(p, "graph_safe", False) for p in model.parts())
@@ -123,60 +125,66 @@ class ModelExecutor:
         S = len(entries)
         lens = [len(e.tokens) for e in entries]
         N = sum(lens)
-        seg_starts = [0]
-        for n in lens:
-            seg_starts.append(seg_starts[-1] + n)
-        token_ids: List[int] = []
-        positions: List[int] = []
-        seg_of: List[int] = []
-        logit_rows: List[int] = []
-        state_slots: List[int] = []
-        for s, (e, st) in enumerate(zip(entries, starts)):
-            token_ids.extend(int(t) for t in e.tokens)
-            positions.extend(range(st, st + lens[s]))
-            seg_of.extend([s] * lens[s])
-            logit_rows.extend(seg_starts[s] + int(w) for w in e.want)
-            state_slots.append(mgr.request(e.request_id).state_slot)
+        lens_a = np.asarray(lens, dtype=np.int64)
+        starts_a = np.asarray(starts, dtype=np.int64)
+        seg_starts_a = np.zeros(S + 1, dtype=np.int64)
+        np.cumsum(lens_a, out=seg_starts_a[1:])
+        seg_starts = seg_starts_a.tolist()
+        caches = [mgr.request(e.request_id) for e in entries]
+        state_slots = [rc.state_slot for rc in caches]
         if static is not None:
-            logit_rows = list(range(N))
+            logit_rows = np.arange(N, dtype=np.int64)
+        else:
+            logit_rows = np.fromiter((seg_starts[s] + int(w) for s, e in enumerate(entries) for w in e.want),
+                                     dtype=np.int64)
+        R = int(logit_rows.shape[0])
         G = len(mgr.groups)
-        group_slots: List[List[int]] = []
-        group_tables: List[List[List[int]]] = []
         widths: List[int] = []
         for gi in range(G):
-            sl: List[int] = []
-            tables = []
-            for e, st, n in zip(entries, starts, lens):
-                sl.extend(mgr.slot_mapping(e.request_id, gi, st, n))
-                tables.append([p if p >= 0 else 0 for p in mgr.block_table(e.request_id, gi)])
-            group_slots.append(sl)
-            group_tables.append(tables)
-            widths.append(static.widths[gi] if static is not None else max(1, max(len(t) for t in tables)))
-        R = len(logit_rows)
+            widths.append(static.widths[gi] if static is not None else
+                          max(1, max(len(rc.tables[gi]) for rc in caches)))
         offsets, total = self._layout(N, S, R, widths)
         if self._pinned is None or self._pinned.numel() < total:
             self._pinned = torch.empty(max(total, 4096), dtype=torch.int32,
                                        pin_memory=self.rt.device.type == "cuda")
+            self._pinned_np = self._pinned.numpy()
         host = self._pinned[:total]
+        host_np = self._pinned_np
 
-        def put(name: str, values: Sequence[int]):
+        def section(name: str) -> np.ndarray:
             o, n = offsets[name]
-            if n:
-                host[o:o + n] = torch.tensor(values, dtype=torch.int32)
+            return host_np[o:o + n]
 
-        put("token_ids", token_ids)
-        put("positions", positions)
-        put("seg_of", seg_of)
-        put("seg_starts", seg_starts)
-        put("seg_first", list(starts))
-        put("state_slots", state_slots)
-        put("logit_rows", logit_rows)
+        seg_of = np.repeat(np.arange(S, dtype=np.int64), lens_a)
+        within = np.arange(N, dtype=np.int64) - seg_starts_a[:-1][seg_of]       # index of a token in its segment
+        positions = starts_a[seg_of] + within
+        if N == S:
+            section("token_ids")[:] = [e.tokens[0] for e in entries]
+        else:
+            section("token_ids")[:] = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in entries])
+        section("positions")[:] = positions
+        section("seg_of")[:] = seg_of
+        section("seg_starts")[:] = seg_starts_a
+        section("seg_first")[:] = starts_a
+        section("state_slots")[:] = state_slots
+        if R:
+            section("logit_rows")[:] = logit_rows
         for gi in range(G):
-            put("slots%d" % gi, group_slots[gi])
-            flat: List[int] = []
-            for t in group_tables[gi]:
-                flat.extend(t + [0] * (widths[gi] - len(t)))
-            put("tables%d" % gi, flat)
+            ps = mgr.groups[gi].page_size
+            w = widths[gi]
+            tables = section("tables%d" % gi).reshape(S, w)
+            tables[:] = 0
+            for s, rc in enumerate(caches):
+                t = rc.tables[gi]
+                tables[s, :len(t)] = t
+            # slot of every token: page of its block, times the page size, plus its offset in the page
+            pages = tables[seg_of, positions // ps].astype(np.int64)
+            if (pages < 0).any():
+                bad = int(np.nonzero(pages < 0)[0][0])
+                raise CacheError("position %d of request %r lies in a page that was given back"
+                                 % (int(positions[bad]), entries[int(seg_of[bad])].request_id))
+            section("slots%d" % gi)[:] = pages * ps + positions % ps
+            np.maximum(tables, 0, out=tables)            # pages that a window has passed: any valid page id
         # the copy is synchronous: the staging buffer is free again when the next step fills it
         if static is not None:
             static.device_buffer.copy_(host, non_blocking=False)
@@ -201,7 +209,7 @@ class ModelExecutor:
             seg_of_token=view("seg_of"), seg_starts=view("seg_starts"), seg_first_pos=view("seg_first"),
             state_slots=view("state_slots"), logit_rows=view("logit_rows"), n_logit_rows=R, groups=groups,
             host_seg_starts=seg_starts, host_seg_lens=lens, host_seg_first_pos=list(starts),
-            host_state_slots=state_slots, request_ids=[e.request_id for e in entries],
+            host_state_slots=list(state_slots), request_ids=[e.request_id for e in entries],
             max_seg_len=max(lens),
             max_context=(static.max_context if static is not None else
                          self._context_bucket(max(starts) + 1) if all(n == 1 for n in lens) else

@@ -28,6 +28,10 @@ class RequestOutput:
 
     @classmethod
     def from_sequence(cls, seq: Sequence, latest: Optional[int]) -> "RequestOutput":
-        return cls(seq.request_id, list(seq.prompt_token_ids),
-                   [CompletionOutput(0, list(seq.output_token_ids), latest, seq.state.finish_reason)],
-                   seq.state.finished, seq.metrics)
+        # a finished request gets lists of its own; while it runs, the output shows the request's live lists
+        # (copying a long prompt for every request at every step costs more than the step's host work)
+        done = seq.state.finished
+        return cls(seq.request_id, list(seq.prompt_token_ids) if done else seq.prompt_token_ids,
+                   [CompletionOutput(0, list(seq.output_token_ids) if done else seq.output_token_ids, latest,
+                                     seq.state.finish_reason)],
+                   done, seq.metrics)

@@ -119,15 +119,21 @@ class Scheduler:
         planned_slots = 0
         watermark = [int(round(cfg.watermark * g.num_pages)) for g in cache.groups]
 
+        last_need = [None, None, None]             # (request, tokens) of the last question and its answer
+
+        def needed(rid, n):
+            if last_need[0] != rid or last_need[1] != n or rid is None:
+                last_need[0], last_need[1], last_need[2] = rid, n, cache.pages_needed(rid, n)
+            return last_need[2]
+
         def fits(rid, n, reserve=False) -> bool:
-            need = cache.pages_needed(rid, n)
-            for gi, k in enumerate(need):
+            for gi, k in enumerate(needed(rid, n)):
                 if cache.num_free_pages(gi) - planned[gi] - k < (watermark[gi] if reserve else 0):
                     return False
             return True
 
         def take(rid, n) -> None:
-            for gi, k in enumerate(cache.pages_needed(rid, n)):
+            for gi, k in enumerate(needed(rid, n)):
                 planned[gi] += k
 
         self.running.sort(key=lambda s: s.arrival)

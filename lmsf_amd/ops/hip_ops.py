@@ -47,6 +47,7 @@ class HipOps:
                 "the kernels are built for gfx950 only; this device reports %r" % self.device_arch)
         self._bad_flag = None
         self.use_library_gemm = True   # bfloat16 matrix products of many rows go to the BLAS library
+        self.prefill_attention_variant = 0   # 0: keys and values staged in LDS; 1: fetched by every wave for itself
         self.skinny_variant = 0        # tiling of the few-rows kernel (0: default; others for tuning)
         self.skinny_max_rows = 16      # rows up to which the few-rows kernel beats the library (measured)
 
@@ -203,10 +204,10 @@ class HipOps:
         if N == 0:
             return out
         fast_ok = (q.dtype == torch.bfloat16 and d % 16 == 0 and 16 <= d <= 256 and ps % 4 == 0
-                   and q.stride(0) % 8 == 0 and q.data_ptr() % 16 == 0)
+                   and q.stride(0) % 8 == 0 and q.data_ptr() % 16 == 0 and scale > 0)
         if kernel == "mfma" and not fast_ok:
             raise ValueError("the matrix-core attention kernels need bfloat16, a head size that is a multiple of 16 "
-                             "up to 256, a page size that is a multiple of 4 and 16-byte aligned query rows")
+                             "up to 256, a page size that is a multiple of 4, 16-byte aligned query rows and a positive scale")
         if kernel == "generic" or not fast_ok:
             self._check(self.lib.lmsf_paged_attention_generic(
                 _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pages), _ptr(v_pages), num_pages,
@@ -218,7 +219,8 @@ class HipOps:
         if plan.tiles is not None:
             self._check(self.lib.lmsf_paged_attention_prefill_mfma(
                 _ptr(q), q.stride(0), _ptr(out), out.stride(0), *common, _ptr(plan.tiles), plan.n_tiles,
-                _ptr(seg), _ptr(pos), nh, nkv, d, ps, float(scale), int(window or 0), self._stream()))
+                _ptr(seg), _ptr(pos), nh, nkv, d, ps, float(scale), int(window or 0), self.prefill_attention_variant,
+                self._stream()))
         if plan.n_single:
             n_hb = -(-(nh // nkv) // 16)
             most = -(-plan.max_context // 128)
