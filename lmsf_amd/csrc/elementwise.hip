@@ -59,6 +59,30 @@ __global__ __launch_bounds__(256) void gated_act_kernel(const T* __restrict__ in
   out[t * (long)I + i] = from_f32<T>(a * u);
 }
 
+// The same with 16-byte accesses: 8 bfloat16 or 4 float32 per thread.
+template <typename T, int KIND>
+__global__ __launch_bounds__(256) void gated_act_vec_kernel(const T* __restrict__ in, T* __restrict__ out, int I,
+                                                            long in_stride) {
+  constexpr int N = Vec16<T>::N;
+  const long t = blockIdx.x;
+  const int i = (blockIdx.y * blockDim.x + threadIdx.x) * N;
+  if (i >= I) return;
+  Vec16<T> g, u, o;
+  g.load(in + t * in_stride + i);
+  u.load(in + t * in_stride + I + i);
+#pragma unroll
+  for (int e = 0; e < N; ++e) {
+    const float x = g.get(e);
+    float a;
+    if (KIND == 0)
+      a = x / (1.0f + expf(-x));
+    else
+      a = 0.5f * x * (1.0f + erff(x * 0.70710678118654752f));
+    o.set(e, a * u.get(e));
+  }
+  o.store(out + t * (long)I + i);
+}
+
 extern "C" int lmsf_gated_act(const void* in, void* out, int dtype, int n_tokens, int I, long in_stride, int kind,
                               hipStream_t stream) {
   LMSF_CHECK(in && out, "gated_act: null pointer");
@@ -68,6 +92,21 @@ extern "C" int lmsf_gated_act(const void* in, void* out, int dtype, int n_tokens
   LMSF_CHECK(kind == 0 || kind == 1, "gated_act: unknown activation %d", kind);
   LMSF_CHECK(dtype == LMSF_F32 || dtype == LMSF_BF16, "gated_act: unknown dtype code %d", dtype);
   if (n_tokens == 0) return 0;
+  const int per = dtype == LMSF_F32 ? 4 : 8;   // elements of a 16-byte access
+  if (I % per == 0 && in_stride % per == 0 && lmsf_aligned16(in) && lmsf_aligned16(out)) {
+    const int vecs = I / per;
+    dim3 vgrid(n_tokens, (vecs + 255) / 256), vblock(256);
+#define GAV(T, K) \
+  hipLaunchKernelGGL((gated_act_vec_kernel<T, K>), vgrid, vblock, 0, stream, (const T*)in, (T*)out, I, in_stride)
+    if (dtype == LMSF_F32) {
+      if (kind == 0) GAV(float, 0); else GAV(float, 1);
+    } else {
+      if (kind == 0) GAV(bf16_t, 0); else GAV(bf16_t, 1);
+    }
+#undef GAV
+    LMSF_LAUNCH_CHECK("gated_act");
+    return 0;
+  }
   dim3 grid(n_tokens, (I + 255) / 256), block(256);
 #define GA(T, K) hipLaunchKernelGGL((gated_act_kernel<T, K>), grid, block, 0, stream, (const T*)in, (T*)out, I, in_stride)
   if (dtype == LMSF_F32) {
