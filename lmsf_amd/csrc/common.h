@@ -93,6 +93,13 @@ template <> struct Vec16<bf16_t> {
   }
 };
 
+// One rotation pair of the rotary embedding, x' = x cos - y sin, y' = y cos + x sin, with the roundings
+// pinned (a product, then one fused multiply-add), so that every kernel that rotates gives the same bits.
+__device__ __forceinline__ void rope_rotate(float x, float y, float c, float s, float* xr, float* yr) {
+  *xr = __fmaf_rn(x, c, -__fmul_rn(y, s));
+  *yr = __fmaf_rn(y, c, __fmul_rn(x, s));
+}
+
 // ---------------------------------------------------------------- wave64 and block reductions
 
 __device__ __forceinline__ float wave_sum(float v) {

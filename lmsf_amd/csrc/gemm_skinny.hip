@@ -24,6 +24,13 @@
 // writes y[m][n] = act(g) * u with g and u the two products: the activation kernel and its traffic are gone
 // (the reference runs silu_and_mul as a kernel of its own, vllm/kernels/activation_kernels.cu:31-42).
 //
+// Rotary form (ACT == 3): the product is the fused QKV projection of an attention layer with NeoX rotary
+// embedding over the whole head. A workgroup owns rows i .. i + 15 and i + d/2 .. i + d/2 + 15 of one head,
+// that is, both members of 16 rotation pairs, and its epilogue rotates q and k by the token's position,
+// stores q (and k, v) in the output and k, v in the token's slot of the paged cache: the kernel that
+// would do this afterwards (vllm/kernels/pos_encoding_kernels.cu:38-77 and cache_kernels.cu:190-232 in the
+// reference) and its launch are gone from a decode step.
+//
 // MFMA: v_mfma_f32_16x16x32_bf16, A = W tile (16 rows x 32 k), B = x tile (32 k x 16 tokens), D[n][m]:
 // lane l holds token m = l % 16 and the four outputs n = (l / 16) * 4 .. + 3.
 #include "common.h"
@@ -40,18 +47,31 @@ struct SkinnyTile {
   static constexpr int STEPS = KC / 32;                     // MFMA steps per chunk
 };
 
-// ACT: 0 none (plain linear layer), 1 silu-gated, 2 gelu-gated
+// What the rotary epilogue needs beside the product's own arguments.
+struct RopeCacheArgs {
+  const int* positions;    // [M]
+  const float* table;      // [max_pos, d] = [cos(d/2) | sin(d/2)]
+  const int* slots;        // [M]: page * page_size + offset of the token in the cache, negative: not stored
+  bf16_t* k_pages;         // [pages, nkv, page_size, d]
+  bf16_t* v_pages;         // [pages, nkv, d, page_size]
+  int nh, nkv, d, ps;
+};
+
+// ACT: 0 none (plain linear layer), 1 silu-gated, 2 gelu-gated, 3 rotary embedding and cache write
 template <int MT, int KC, int NW, typename TOut, int ACT>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ x, long ldx,
                                                               const bf16_t* __restrict__ W, long ldw,
                                                               const bf16_t* __restrict__ bias, TOut* __restrict__ y,
-                                                              long ldy, int M, int N, int K) {
+                                                              long ldy, int M, int N, int K, RopeCacheArgs rc) {
   using T = SkinnyTile<KC>;
-  constexpr int WT = ACT ? 2 : 1;   // W tiles per chunk: gate and up, or one
+  constexpr int WT = ACT ? 2 : 1;   // W tiles per chunk: gate and up, the two halves of a head, or one
   extern __shared__ __align__(16) unsigned char lds[];
   const int tid = threadIdx.x;
   const int wave = tid / 64, lane = tid % 64;
-  const int n0 = blockIdx.x * 16;
+  const int half = rc.d / 2;
+  // first row of the first tile; the second tile starts tile_step rows further
+  const int n0 = ACT == 3 ? (blockIdx.x / (half / 16)) * rc.d + (blockIdx.x % (half / 16)) * 16 : blockIdx.x * 16;
+  const int tile_step = ACT == 3 ? half : N;
   unsigned char* my = lds + (size_t)wave * (WT + MT) * T::TILE_BYTES;
 
   // global load coordinates of this lane inside a tile
@@ -67,7 +87,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __re
     int r = n0 + lrow + i * T::ROWS_PER_LOAD;
     if (r > N - 1) r = N - 1;
 #pragma unroll
-    for (int wt = 0; wt < WT; ++wt) woff[wt][i] = (long)(r + wt * N) * ldw + lcol;
+    for (int wt = 0; wt < WT; ++wt) woff[wt][i] = (long)(r + wt * tile_step) * ldw + lcol;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       int m = mt * 16 + lrow + i * T::ROWS_PER_LOAD;
@@ -156,6 +176,47 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __re
       for (int w = 0; w < NW; ++w) sum[wt] += red[((((size_t)w * WT + wt) * MT + mt) * 64 + l) * 4 + j];
     }
     const int n = n0 + (l / 16) * 4 + j, m = mt * 16 + l % 16;
+    if (ACT == 3) {
+      if (m >= M) continue;
+      float a = sum[0], b = sum[WT - 1];
+      if (bias) {
+        a += bf16_to_f32(bias[n]);
+        b += bf16_to_f32(bias[n + half]);
+      }
+      // rounded to the storage type first, as the product stores them when the rotation is a kernel of its own
+      a = bf16_to_f32(f32_to_bf16(a));
+      b = bf16_to_f32(f32_to_bf16(b));
+      const int head = n / rc.d, i = n - head * rc.d;   // i < d / 2: index of the rotation pair
+      bf16_t lo, hi;
+      if (head < rc.nh + rc.nkv) {
+        const float* cs = rc.table + (long)rc.positions[m] * rc.d;
+        const float c = cs[i], sn = cs[half + i];
+        float xr, yr;
+        rope_rotate(a, b, c, sn, &xr, &yr);
+        lo = f32_to_bf16(xr);
+        hi = f32_to_bf16(yr);
+      } else {
+        lo = f32_to_bf16(a);
+        hi = f32_to_bf16(b);
+      }
+      bf16_t* yo = reinterpret_cast<bf16_t*>(y);   // this form writes bfloat16 only
+      yo[(long)m * ldy + n] = lo;
+      yo[(long)m * ldy + n + half] = hi;
+      const int slot = rc.slots[m];
+      if (head >= rc.nh && slot >= 0) {
+        const int page = slot / rc.ps, off = slot - page * rc.ps;
+        if (head < rc.nh + rc.nkv) {
+          bf16_t* dst = rc.k_pages + (((long)page * rc.nkv + (head - rc.nh)) * rc.ps + off) * rc.d;
+          dst[i] = lo;
+          dst[i + half] = hi;
+        } else {
+          bf16_t* dst = rc.v_pages + ((long)page * rc.nkv + (head - rc.nh - rc.nkv)) * rc.d * rc.ps + off;
+          dst[(long)i * rc.ps] = lo;
+          dst[(long)(i + half) * rc.ps] = hi;
+        }
+      }
+      continue;
+    }
     if (n < N && m < M) {
       float r;
       if (ACT == 0) {
@@ -181,7 +242,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __re
 
 template <int MT, int KC, int NW, typename TOut, int ACT>
 static int launch_skinny(const void* x, long ldx, const void* W, long ldw, const void* bias, void* y, long ldy, int M,
-                         int N, int K, hipStream_t stream) {
+                         int N, int K, hipStream_t stream, RopeCacheArgs rc = RopeCacheArgs()) {
   using T = SkinnyTile<KC>;
   constexpr int WT = ACT ? 2 : 1;
   const size_t stage = (size_t)NW * (WT + MT) * T::TILE_BYTES;
@@ -198,8 +259,10 @@ static int launch_skinny(const void* x, long ldx, const void* W, long ldw, const
     }
     configured = true;
   }
-  hipLaunchKernelGGL(kernel, dim3((N + 15) / 16), dim3(NW * 64), smem, stream, (const bf16_t*)x, ldx,
-                     (const bf16_t*)W, ldw, (const bf16_t*)bias, (TOut*)y, ldy, M, N, K);
+  // the gated form has a workgroup per 16 outputs, the rotary form one per 32 rows of W, the plain one per 16
+  const int blocks = ACT == 3 ? N / 32 : (N + 15) / 16;
+  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(NW * 64), smem, stream, (const bf16_t*)x, ldx, (const bf16_t*)W, ldw,
+                     (const bf16_t*)bias, (TOut*)y, ldy, M, N, K, rc);
   return 0;
 }
 
@@ -261,5 +324,38 @@ extern "C" int lmsf_gemm_skinny(const void* x, long ldx, const void* W, long ldw
 #undef SK
   if (rc) return rc;
   LMSF_LAUNCH_CHECK("gemm_skinny");
+  return 0;
+}
+
+// The fused QKV projection with rotary embedding and cache write as its epilogue, for M <= 16 tokens:
+// y[M, (nh + 2 nkv) d] = x W^T (+ bias), then q and k heads rotated in NeoX style over the whole head by
+// table[positions[m]] ([max_pos, d] = cos | sin, float32), k and v stored in the pages at slots[m]
+// (negative: not stored). Needs what lmsf_gemm_skinny needs and d a multiple of 32.
+extern "C" int lmsf_gemm_qkv_rope_cache(const void* x, long ldx, const void* W, long ldw, const void* bias, void* y,
+                                        long ldy, int M, int K, const int* positions, const float* table, int max_pos,
+                                        const int* slots, void* k_pages, void* v_pages, long num_pages, int nh,
+                                        int nkv, int d, int ps, int variant, hipStream_t stream) {
+  LMSF_CHECK(x && W && y && positions && table && slots && k_pages && v_pages, "gemm_qkv_rope_cache: null pointer");
+  LMSF_CHECK(M >= 0 && M <= 16, "gemm_qkv_rope_cache: M=%d outside [0, 16]", M);
+  LMSF_CHECK(nh > 0 && nkv > 0 && d >= 32 && d % 32 == 0, "gemm_qkv_rope_cache: head size %d must be a multiple of 32", d);
+  const long N = (long)(nh + 2 * nkv) * d;
+  LMSF_CHECK(N / 32 <= 2147483647L, "gemm_qkv_rope_cache: too many rows");
+  LMSF_CHECK(K > 0 && K % 8 == 0, "gemm_qkv_rope_cache: K=%d must be a positive multiple of 8", K);
+  LMSF_CHECK(ldx >= K && ldw >= K && ldy >= N && ldx % 8 == 0 && ldw % 8 == 0,
+             "gemm_qkv_rope_cache: row strides must cover K and be multiples of 8");
+  LMSF_CHECK(lmsf_aligned16(x) && lmsf_aligned16(W), "gemm_qkv_rope_cache: x and W must be 16-byte aligned");
+  LMSF_CHECK(ps > 0 && num_pages > 0 && max_pos > 0, "gemm_qkv_rope_cache: bad page geometry or empty table");
+  if (M == 0) return 0;
+  RopeCacheArgs rc;
+  rc.positions = positions; rc.table = table; rc.slots = slots;
+  rc.k_pages = (bf16_t*)k_pages; rc.v_pages = (bf16_t*)v_pages;
+  rc.nh = nh; rc.nkv = nkv; rc.d = d; rc.ps = ps;
+  int r;
+  if (variant == 1)
+    r = launch_skinny<1, 64, 8, bf16_t, 3>(x, ldx, W, ldw, bias, y, ldy, M, (int)N, K, stream, rc);
+  else
+    r = launch_skinny<1, 64, 16, bf16_t, 3>(x, ldx, W, ldw, bias, y, ldy, M, (int)N, K, stream, rc);
+  if (r) return r;
+  LMSF_LAUNCH_CHECK("gemm_qkv_rope_cache");
   return 0;
 }

@@ -37,9 +37,10 @@ __global__ __launch_bounds__(64) void rope_cache_write_kernel(
     for (int i = threadIdx.x; i < half; i += 64) {
       const int xi = neox ? i : 2 * i, yi = neox ? i + half : 2 * i + 1;
       const float c = cs[i], s = cs[half + i];
-      const float a = to_f32<T>(x[xi]), b = to_f32<T>(x[yi]);
-      x[xi] = from_f32<T>(a * c - b * s);
-      x[yi] = from_f32<T>(b * c + a * s);
+      float xr, yr;
+      rope_rotate(to_f32<T>(x[xi]), to_f32<T>(x[yi]), c, s, &xr, &yr);
+      x[xi] = from_f32<T>(xr);
+      x[yi] = from_f32<T>(yr);
     }
   } else if (hy < nh + nkv) {
     if (!k) return;
@@ -51,8 +52,9 @@ __global__ __launch_bounds__(64) void rope_cache_write_kernel(
       for (int i = threadIdx.x; i < half; i += 64) {
         const int xi = neox ? i : 2 * i, yi = neox ? i + half : 2 * i + 1;
         const float c = cs[i], s = cs[half + i];
-        const float a = to_f32<T>(x[xi]), b = to_f32<T>(x[yi]);
-        const T xr = from_f32<T>(a * c - b * s), yr = from_f32<T>(b * c + a * s);
+        float xf, yf;
+        rope_rotate(to_f32<T>(x[xi]), to_f32<T>(x[yi]), c, s, &xf, &yf);
+        const T xr = from_f32<T>(xf), yr = from_f32<T>(yf);
         x[xi] = xr;
         x[yi] = yr;
         if (dst) {

@@ -171,6 +171,43 @@ class HipOps:
             q, k, v, _code(qkv.dtype), N, qkv.stride(0), _ptr(positions), _ptr(table), rot_dim, 1 if neox else 0,
             max_pos, _ptr(slots), _ptr(k_pages), _ptr(v_pages), num_pages, nh, nkv, d, ps, self._stream()))
 
+    def qkv_rope_cache(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], nh: int, nkv: int,
+                       d: int, positions: torch.Tensor, table: Optional[torch.Tensor], rot_dim: int, neox: bool,
+                       slots: Optional[torch.Tensor], k_pages: Optional[torch.Tensor],
+                       v_pages: Optional[torch.Tensor]) -> torch.Tensor:
+        """The fused QKV projection, the rotation of its q and k heads and the write of k and v into the
+        pages: ``linear`` followed by ``rope_cache_write``, with the same results. With few bfloat16 rows and
+        a NeoX rotation over the whole head, the rotation and the write are the product's epilogue."""
+        M, K = x.shape
+        N = (nh + 2 * nkv) * d
+        if (table is not None and slots is not None and neox and rot_dim == d and d % 32 == 0
+                and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and 0 < M <= self.skinny_max_rows
+                and tuple(weight.shape) == (N, K) and x.stride(1) == 1 and weight.stride(1) == 1
+                and self._skinny_ok(x, weight) and k_pages is not None and k_pages.dtype == torch.bfloat16):
+            self._dev(x, weight, bias, positions, table, slots, k_pages, v_pages)
+            if bias is not None and (bias.shape != (N,) or bias.dtype != weight.dtype or not bias.is_contiguous()):
+                raise ValueError("qkv_rope_cache: bias must be [%d] of the weight's dtype" % N)
+            if table.dtype != torch.float32 or table.dim() != 2 or table.shape[1] != d or not table.is_contiguous():
+                raise ValueError("rotary table must be contiguous float32 [max_pos, %d]" % d)
+            self._i32(positions, "positions", M)
+            self._i32(slots, "slots", M)
+            if k_pages.dim() != 4 or k_pages.shape[1] != nkv or k_pages.shape[3] != d or not k_pages.is_contiguous():
+                raise ValueError("k_pages must be contiguous [pages, %d, page_size, %d]" % (nkv, d))
+            num_pages, ps = k_pages.shape[0], k_pages.shape[2]
+            if v_pages is None or tuple(v_pages.shape) != (num_pages, nkv, d, ps) or not v_pages.is_contiguous() \
+                    or v_pages.dtype != torch.bfloat16:
+                raise ValueError("v_pages must be contiguous bfloat16 [%d, %d, %d, %d]" % (num_pages, nkv, d, ps))
+            y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+            self._check(self.lib.lmsf_gemm_qkv_rope_cache(
+                _ptr(x), x.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(y), y.stride(0), M, K,
+                _ptr(positions), _ptr(table), table.shape[0], _ptr(slots), _ptr(k_pages), _ptr(v_pages), num_pages,
+                nh, nkv, d, ps, self.skinny_variant, self._stream()))
+            return y
+        y = self.linear(x, weight, bias)
+        if table is not None or slots is not None:
+            self.rope_cache_write(y, nh, nkv, d, positions, table, rot_dim, neox, slots, k_pages, v_pages)
+        return y
+
     # ------------------------------------------------------------------ attention
 
     def paged_attention(self, q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,

@@ -9,7 +9,7 @@ from typing import Optional
 
 from ..csrc import build as _build
 
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 _lib: Optional[ctypes.CDLL] = None
 _lib_path: Optional[str] = None
@@ -39,6 +39,8 @@ _SIGNATURES = {
     "lmsf_gated_act": (c_int, [_P, _P, c_int, c_int, c_int, c_long, c_int, _P]),
     "lmsf_gemm_plain": (c_int, [_P, c_int, c_long, _P, c_int, c_long, _P, _P, c_int, c_long, c_int, c_int, c_int, _P]),
     "lmsf_gemm_skinny": (c_int, [_P, c_long, _P, c_long, _P, _P, c_int, c_long, c_int, c_int, c_int, c_int, c_int, _P]),
+    "lmsf_gemm_qkv_rope_cache": (c_int, [_P, c_long, _P, c_long, _P, _P, c_long, c_int, c_int, _P, _P, c_int, _P, _P, _P,
+                                         c_long, c_int, c_int, c_int, c_int, c_int, _P]),
     "lmsf_sample": (c_int, [_P, c_long, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, _P]),
     "lmsf_apply_penalties": (c_int, [_P, c_long, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, _P]),
 }

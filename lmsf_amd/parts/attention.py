@@ -51,17 +51,18 @@ class PagedAttention(Mixer):
     def forward(self, h: torch.Tensor, ctx, binding: CacheBinding) -> torch.Tensor:
         ops = self.rt.ops
         group = ctx.groups[binding.group]
-        qkv = self.qkv.forward(h)
-        table, rot, neox = (None, 0, True)
-        if self.position is not None:
-            if hasattr(self.position, "rotary_table"):
-                table, rot, neox = self.position.rotary_table()
-            else:
-                self.position.apply(qkv, self.nh, self.nkv, self.d, ctx.positions)
         slots = group.slots if binding.writes_cache else None
-        if table is not None or slots is not None:
-            ops.rope_cache_write(qkv, self.nh, self.nkv, self.d, ctx.positions, table, rot, neox, slots,
-                                 binding.k_pages, binding.v_pages)
+        if self.position is not None and not hasattr(self.position, "rotary_table"):
+            # an encoding that acts on the projections itself
+            qkv = self.qkv.forward(h)
+            self.position.apply(qkv, self.nh, self.nkv, self.d, ctx.positions)
+            if slots is not None:
+                ops.rope_cache_write(qkv, self.nh, self.nkv, self.d, ctx.positions, None, 0, True, slots,
+                                     binding.k_pages, binding.v_pages)
+        else:
+            table, rot, neox = self.position.rotary_table() if self.position is not None else (None, 0, True)
+            qkv = ops.qkv_rope_cache(h, self.qkv.weight, self.qkv.bias, self.nh, self.nkv, self.d, ctx.positions,
+                                     table, rot, neox, slots, binding.k_pages, binding.v_pages)
         a = ops.paged_attention(qkv, binding.k_pages, binding.v_pages, group.block_tables, ctx.seg_of_token,
                                 ctx.positions, self.nh, self.nkv, self.d, self.scale, self.window or 0, batch=ctx)
         return self.o.forward(a)

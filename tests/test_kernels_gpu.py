@@ -320,6 +320,42 @@ def test_linear_gated(ops, ref, M, I, K, kind, bias):
     assert f32.dtype == torch.float32 and torch.allclose(f32, want, atol=1e-4, rtol=1e-4)
 
 
+@pytest.mark.parametrize("M,H,nh,nkv,d,ps", [(1, 128, 8, 1, 32, 16), (8, 4096, 32, 8, 128, 16), (16, 80, 3, 3, 64, 8),
+                                             (5, 256, 4, 2, 96, 4)])
+@pytest.mark.parametrize("bias", [False, True])
+def test_qkv_rope_cache_fused_equals_the_three_steps(ops, ref, M, H, nh, nkv, d, ps, bias):
+    """With few rows the rotation and the cache write are the epilogue of the QKV product; the result must be
+    the bits of product, rotation kernel and cache write one after the other, and the plain formulas."""
+    g = torch.Generator().manual_seed(M * H + d)
+    N = (nh + 2 * nkv) * d
+    x = dev(torch.randn(M, H, generator=g).bfloat16())
+    w = dev((torch.randn(N, H, generator=g) * H ** -0.5).bfloat16())
+    b = dev(torch.randn(N, generator=g).bfloat16()) if bias else None
+    max_pos, pages = 50, 7
+    pos = dev(torch.randint(0, max_pos, (M,), generator=g, dtype=torch.int32))
+    ang = torch.arange(max_pos, dtype=torch.float32)[:, None] * torch.rand(d // 2, generator=g)[None, :]
+    table = dev(torch.cat([ang.cos(), ang.sin()], dim=1).contiguous())
+    slots = torch.randperm(pages * ps, generator=g)[:M].to(torch.int32)
+    if M > 2:
+        slots[2] = -1
+    slots = dev(slots)
+    k1, v1 = dev(torch.zeros(pages, nkv, ps, d).bfloat16()), dev(torch.zeros(pages, nkv, d, ps).bfloat16())
+    k2, v2, k3, v3 = k1.clone(), v1.clone(), k1.clone(), v1.clone()
+    fused = ops.qkv_rope_cache(x, w, b, nh, nkv, d, pos, table, d, True, slots, k1, v1)
+    steps = ops.linear(x, w, b)
+    ops.rope_cache_write(steps, nh, nkv, d, pos, table, d, True, slots, k2, v2)
+    assert torch.equal(fused, steps) and torch.equal(k1, k2) and torch.equal(v1, v2)
+    plain = ref.qkv_rope_cache(x, w, b, nh, nkv, d, pos, table, d, True, slots, k3, v3)
+    scale = max(1.0, plain.float().abs().max().item())
+    assert (fused.float() - plain.float()).abs().max().item() <= 2e-2 * scale
+    assert (k1.float() - k3.float()).abs().max().item() <= 2e-2 * scale and (v1.float() - v3.float()).abs().max().item() <= 2e-2 * scale
+    # what the fused kernel does not take falls back to the three steps: GPT-J pairing, partial rotation
+    k4, v4, k5, v5 = k3.clone().zero_(), v3.clone().zero_(), k3.clone().zero_(), v3.clone().zero_()
+    a = ops.qkv_rope_cache(x, w, b, nh, nkv, d, pos, table[:, :d // 2].contiguous(), d // 2, False, slots, k4, v4)
+    c = ref.qkv_rope_cache(x, w, b, nh, nkv, d, pos, table[:, :d // 2].contiguous(), d // 2, False, slots, k5, v5)
+    assert (a.float() - c.float()).abs().max().item() <= 2e-2 * scale and (k4.float() - k5.float()).abs().max().item() <= 2e-2 * scale
+
+
 def test_linear_mixed_storage(ops, ref):
     """A weight stored in 32 bits stays so and still multiplies bfloat16 activations."""
     g = torch.Generator().manual_seed(5)

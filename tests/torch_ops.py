@@ -111,6 +111,12 @@ class TorchOps:
             k_pages[page, :, off, :] = k[ok]
             v_pages[page, :, :, off] = v[ok]
 
+    def qkv_rope_cache(self, x, weight, bias, nh, nkv, d, positions, table, rot_dim, neox, slots, k_pages, v_pages):
+        y = self.linear(x, weight, bias)
+        if table is not None or slots is not None:
+            self.rope_cache_write(y, nh, nkv, d, positions, table, rot_dim, neox, slots, k_pages, v_pages)
+        return y
+
     # ------------------------------------------------------------ attention
     def paged_attention(self, q, k_pages, v_pages, block_tables, seg, pos, nh, nkv, d, scale, window=0, batch=None):
         N = q.shape[0]
