@@ -1,0 +1,284 @@
+// Linear layer for 17 to 64 rows (decoding at larger batches): y[M, N] = x[M, K] W[N, K]^T (+ bias),
+// bfloat16 inputs, float32 accumulation on the matrix cores, bfloat16 output; optionally the gated
+// activation of a feed-forward as epilogue.
+//
+// The product is still a stream of the weight matrix, but with this many rows the activations are no
+// longer negligible: a workgroup that owns 16 rows of W reads four times as many bytes of x as of W. Here
+// a workgroup owns 64 rows of W (16 per wave) and all rows of x, so x is read once per 64 rows of W; where
+// that leaves too few workgroups to fill the chip (N = 4096: 64 of them), K is split over several
+// workgroups, which write float32 partial sums that a second small kernel adds in a fixed order (and
+// applies bias and activation to). The reference leaves these products to cuBLASLt
+// (tops/src/cublas.rs:29-114).
+//
+// Tiles of 64 k travel from global memory straight into LDS (global_load_lds_dwordx4: lane i of a wave
+// writes its 16 bytes at the wave's LDS base + 16 i), three steps ahead of the one being multiplied; each
+// wave moves its own rows of W and a quarter of x. A tile is 16 rows of 128 bytes; the 16-byte piece c of
+// row r lies in slot (c + r / 2) mod 8 of its row, which keeps the operand reads of a wave on distinct
+// banks without padding (the transfer cannot pad). One barrier per step.
+//
+// v_mfma_f32_16x16x32_bf16: A = 16 rows of W, B = 16 rows of x, both with lane (r, g) = (l % 16, l / 16)
+// holding row r, elements 8 g .. 8 g + 7 of a 32-wide step; D[n][m]: lane l holds token m = l % 16 and the
+// four outputs n = (l / 16) * 4 .. + 3.
+#include "common.h"
+
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"   // m0 is named as clobbered on purpose
+// The transfer is inline assembly: through the compiler's builtin every LDS read that follows would first
+// wait for all transfers in flight. The waits are explicit (s_waitcnt vmcnt before each step's barrier).
+__device__ __forceinline__ void mid_global_to_lds_16(const void* src, unsigned lds_base_uniform) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(lds_base_uniform)
+               : "memory", "m0");
+}
+#pragma clang diagnostic pop
+__device__ __forceinline__ unsigned mid_lds_address(const void* p) {
+  return (unsigned)(size_t)(__attribute__((address_space(3))) const unsigned char*)p;
+}
+
+__device__ __forceinline__ float mid_activation(float g, float u, int act) {
+  // the two products are rounded to the storage type before the activation, as the unfused path stores them
+  g = bf16_to_f32(f32_to_bf16(g));
+  u = bf16_to_f32(f32_to_bf16(u));
+  const float a = act == 1 ? g / (1.0f + expf(-g)) : 0.5f * g * (1.0f + erff(g * 0.70710678118654752f));
+  return a * u;
+}
+
+#define MID_STAGES 5
+#define MID_TILE 2048
+
+// MT: tiles of 16 rows of x (2 or 4). ACT: 0 none, 1 silu-gated, 2 gelu-gated (W = [gate rows; up rows], N
+// outputs). PARTIAL: write float32 partial sums of this workgroup's part of K instead of the result.
+template <int MT, int ACT, bool PARTIAL>
+__global__ __launch_bounds__(256) void gemm_mid_kernel(const bf16_t* __restrict__ x, long ldx,
+                                                       const bf16_t* __restrict__ W, long ldw,
+                                                       const bf16_t* __restrict__ bias, bf16_t* __restrict__ y,
+                                                       long ldy, float* __restrict__ part, int M, int N, int K,
+                                                       int n_split) {
+  constexpr int WT = ACT ? 2 : 1;
+  constexpr int STAGE = (4 * WT + MT) * MID_TILE;
+  constexpr int XL = MT / 2;           // halves of x tiles this wave moves per step (2 MT halves over 4 waves)
+  constexpr int LPW = 2 * WT + XL;     // transfers per wave and step
+  extern __shared__ __align__(16) unsigned char lds[];
+  const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
+  const int n0 = blockIdx.x * 64, split = blockIdx.y;
+  const int chunks = K / 64;
+  const int c_begin = (int)((long)split * chunks / n_split), c_end = (int)((long)(split + 1) * chunks / n_split);
+  const int n_steps = c_end - c_begin;
+
+  // what this lane moves in every step: lane i of a transfer fills slot i % 8 of row i / 8 of half a tile
+  const int trow = l >> 3, tslot = l & 7;
+  const bf16_t* src[LPW];
+  unsigned dst[LPW];                   // byte offset inside a stage; the same for all lanes of the wave
+#pragma unroll
+  for (int t = 0; t < WT; ++t)
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int row = 8 * h + trow, piece = (tslot - (row >> 1)) & 7;
+      int n = n0 + 16 * w + row;
+      if (n > N - 1) n = N - 1;        // rows beyond the matrix repeat the last row and are not stored
+      src[t * 2 + h] = W + (long)(n + t * N) * ldw + piece * 8 + (long)c_begin * 64;
+      dst[t * 2 + h] = (w * WT + t) * MID_TILE + h * 1024;
+    }
+#pragma unroll
+  for (int j = 0; j < XL; ++j) {
+    const int qh = w * XL + j, tile = qh >> 1, h = qh & 1;
+    const int row = 8 * h + trow, piece = (tslot - (row >> 1)) & 7;
+    int m = tile * 16 + row;
+    if (m > M - 1) m = M - 1;
+    src[2 * WT + j] = x + (long)m * ldx + piece * 8 + (long)c_begin * 64;
+    dst[2 * WT + j] = (4 * WT + tile) * MID_TILE + h * 1024;
+  }
+  // where this lane reads its operands in a tile: row r, pieces 4 s + g of the two 32-wide steps
+  int foff[2];
+#pragma unroll
+  for (int s = 0; s < 2; ++s) foff[s] = r * 128 + (((s * 4 + g) + (r >> 1)) & 7) * 16;
+
+  f32x4_t acc[WT][MT];
+#pragma unroll
+  for (int t = 0; t < WT; ++t)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[t][mt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+
+  const unsigned lds0 = mid_lds_address(lds);
+  auto issue = [&](int step, int stage_byte) {
+#pragma unroll
+    for (int i = 0; i < LPW; ++i)
+      mid_global_to_lds_16(src[i] + (long)step * 64, __builtin_amdgcn_readfirstlane(lds0 + stage_byte + dst[i]));
+  };
+#pragma unroll
+  for (int s = 0; s < MID_STAGES - 1; ++s)
+    if (s < n_steps) issue(s, s * STAGE);
+
+  int consume = 0, produce = (MID_STAGES - 1) * STAGE;
+  for (int it = 0; it < n_steps; ++it) {
+    // step ``it`` has arrived when at most the transfers of the later steps are outstanding
+    if (it + MID_STAGES - 2 < n_steps)
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"((MID_STAGES - 2) * LPW) : "memory");
+    else
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();   // everybody's part of step ``it`` is there, and everybody is done with step ``it - 1``
+    if (it + MID_STAGES - 1 < n_steps) issue(it + MID_STAGES - 1, produce);
+    produce = produce + STAGE == MID_STAGES * STAGE ? 0 : produce + STAGE;
+    const unsigned char* st = lds + consume;
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      bf16x8_t a[WT], b[MT];
+#pragma unroll
+      for (int t = 0; t < WT; ++t) a[t] = *reinterpret_cast<const bf16x8_t*>(st + (w * WT + t) * MID_TILE + foff[s]);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) b[mt] = *reinterpret_cast<const bf16x8_t*>(st + (4 * WT + mt) * MID_TILE + foff[s]);
+#pragma unroll
+      for (int t = 0; t < WT; ++t)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t], b[mt], acc[t][mt], 0, 0, 0);
+    }
+    consume = consume + STAGE == MID_STAGES * STAGE ? 0 : consume + STAGE;
+  }
+
+  // this lane holds, for token m = mt * 16 + r, the outputs n = n0 + 16 w + 4 g .. + 3
+  const int n = n0 + 16 * w + 4 * g;
+  if (n >= N) return;                  // N is a multiple of 4 where it is not a multiple of 64 (checked by the host)
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int m = mt * 16 + r;
+    if (m >= M) continue;
+    if (PARTIAL) {
+      // partial sums: [split][tile of W rows (gate, up)][M][N]
+#pragma unroll
+      for (int t = 0; t < WT; ++t)
+        *reinterpret_cast<f32x4_t*>(part + (((long)split * WT + t) * M + m) * N + n) = acc[t][mt];
+    } else {
+      float o[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (ACT == 0) {
+          o[i] = acc[0][mt][i] + (bias ? bf16_to_f32(bias[n + i]) : 0.f);
+        } else {
+          const float gg = acc[0][mt][i] + (bias ? bf16_to_f32(bias[n + i]) : 0.f);
+          const float uu = acc[WT - 1][mt][i] + (bias ? bf16_to_f32(bias[N + n + i]) : 0.f);
+          o[i] = mid_activation(gg, uu, ACT);
+        }
+      }
+      uint2 v;
+      v.x = pack2_bf16(o[0], o[1]);
+      v.y = pack2_bf16(o[2], o[3]);
+      *reinterpret_cast<uint2*>(y + (long)m * ldy + n) = v;
+    }
+  }
+}
+
+// y[m][n] = (act of) the sum over the splits of the partial sums, in the order of the splits, plus bias.
+__global__ __launch_bounds__(256) void gemm_mid_reduce_kernel(const float* __restrict__ part,
+                                                              const bf16_t* __restrict__ bias, bf16_t* __restrict__ y,
+                                                              long ldy, int M, int N, int n_split, int act) {
+  const long idx = ((long)blockIdx.x * 256 + threadIdx.x) * 4;   // over M * N, four outputs of a row at a time
+  if (idx >= (long)M * N) return;
+  const int m = (int)(idx / N), n = (int)(idx - (long)m * N);
+  const int wt = act ? 2 : 1;
+  f32x4_t sg = (f32x4_t){0.f, 0.f, 0.f, 0.f}, su = sg;
+  for (int s = 0; s < n_split; ++s) {
+    sg += *reinterpret_cast<const f32x4_t*>(part + (((long)s * wt) * M + m) * N + n);
+    if (act) su += *reinterpret_cast<const f32x4_t*>(part + (((long)s * wt + 1) * M + m) * N + n);
+  }
+  float o[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float gg = sg[i] + (bias ? bf16_to_f32(bias[n + i]) : 0.f);
+    if (act) {
+      const float uu = su[i] + (bias ? bf16_to_f32(bias[N + n + i]) : 0.f);
+      o[i] = mid_activation(gg, uu, act);
+    } else {
+      o[i] = gg;
+    }
+  }
+  uint2 v;
+  v.x = pack2_bf16(o[0], o[1]);
+  v.y = pack2_bf16(o[2], o[3]);
+  *reinterpret_cast<uint2*>(y + (long)m * ldy + n) = v;
+}
+
+template <int MT, int ACT, bool PARTIAL>
+static int launch_mid(dim3 grid, hipStream_t stream, const bf16_t* x, long ldx, const bf16_t* W, long ldw,
+                      const bf16_t* bias, bf16_t* y, long ldy, float* part, int M, int N, int K, int n_split) {
+  constexpr int WT = ACT ? 2 : 1;
+  const size_t smem = (size_t)MID_STAGES * (4 * WT + MT) * MID_TILE;
+  auto kernel = gemm_mid_kernel<MT, ACT, PARTIAL>;
+  static bool configured = false;   // per instantiation
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) {
+      lmsf_set_error("gemm_mid: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
+      return 2;
+    }
+    configured = true;
+  }
+  hipLaunchKernelGGL(kernel, grid, dim3(256), smem, stream, x, ldx, W, ldw, bias, y, ldy, part, M, N, K, n_split);
+  return 0;
+}
+
+// Splits of K proposed for these sizes (1: no partial sums, no second kernel). The time of the product is
+// that of the compute unit with the most workgroups, so the number of workgroups should fill the last round
+// over the 256 compute units; against that stand the partial sums, which are written and read once. The
+// proposal minimises bytes / (share of the last round that is filled) + bytes of the partial sums.
+extern "C" int lmsf_gemm_mid_splits(int M, int N, int K, int act) {
+  const int wt = act ? 2 : 1;
+  const long blocks = (N + 63) / 64, chunks = K / 64;
+  const double w_bytes = 2.0 * wt * (double)N * K;
+  int best = 1;
+  double best_cost = 0;
+  for (int s = 1; s <= 8; ++s) {
+    if (s > 1 && chunks / s < 8) break;       // at least 8 steps per workgroup
+    const long wg = blocks * s, rounds = (wg + 255) / 256;
+    const double fill = (double)wg / (256.0 * rounds);
+    const double cost = w_bytes / fill + (s > 1 ? 2.0 * s * wt * (double)M * N * 4 : 0.0);
+    if (s == 1 || cost < best_cost) {
+      best = s;
+      best_cost = cost;
+    }
+  }
+  return best;
+}
+extern "C" long lmsf_gemm_mid_scratch_floats(int M, int N, int n_split, int act) {
+  return n_split > 1 ? (long)n_split * (act ? 2 : 1) * M * N : 0;
+}
+
+// x [M, K] bfloat16 (row stride ldx), W [N, K] (act 0) or [2 N, K] (act 1 silu, 2 gelu: gate rows first),
+// bias [N] or [2 N] or null, y [M, N] bfloat16. Needs 1 <= M <= 64, K a multiple of 64, N a multiple of 4,
+// 16-byte aligned x and W, row strides of x and W that are multiples of 8 and of y of 4; anything else is
+// refused. n_split: parts of K that go to different workgroups (lmsf_gemm_mid_splits proposes a number);
+// scratch: lmsf_gemm_mid_scratch_floats floats (may be null when that is 0).
+extern "C" int lmsf_gemm_mid(const void* x, long ldx, const void* W, long ldw, const void* bias, void* y, long ldy,
+                             int M, int N, int K, int act, int n_split, float* scratch, hipStream_t stream) {
+  LMSF_CHECK(x && W && y, "gemm_mid: null pointer");
+  LMSF_CHECK(M >= 0 && M <= 64, "gemm_mid: M=%d outside [0, 64]", M);
+  LMSF_CHECK(N > 0 && N % 4 == 0 && K > 0 && K % 64 == 0, "gemm_mid: N=%d must be a multiple of 4 and K=%d of 64", N, K);
+  LMSF_CHECK(ldx >= K && ldw >= K && ldy >= N && ldx % 8 == 0 && ldw % 8 == 0 && ldy % 4 == 0,
+             "gemm_mid: row strides must cover the rows, be multiples of 8 (x, W) and of 4 (y)");
+  LMSF_CHECK(lmsf_aligned16(x) && lmsf_aligned16(W) && (((uintptr_t)y) & 7u) == 0, "gemm_mid: operands must be aligned");
+  LMSF_CHECK(act >= 0 && act <= 2, "gemm_mid: unknown activation %d", act);
+  if (M == 0) return 0;
+  LMSF_CHECK(n_split >= 1 && n_split <= 64 && n_split <= K / 64, "gemm_mid: %d splits of K=%d", n_split, K);
+  LMSF_CHECK(n_split == 1 || scratch != nullptr, "gemm_mid: %d splits need scratch", n_split);
+  dim3 grid((N + 63) / 64, n_split);
+  const bf16_t *xb = (const bf16_t*)x, *Wb = (const bf16_t*)W, *bb = (const bf16_t*)bias;
+  bf16_t* yb = (bf16_t*)y;
+  int rc = 0;
+#define MID(MT_, ACT_)                                                                                           \
+  rc = n_split > 1 ? launch_mid<MT_, ACT_, true>(grid, stream, xb, ldx, Wb, ldw, bb, yb, ldy, scratch, M, N, K, n_split) \
+                   : launch_mid<MT_, ACT_, false>(grid, stream, xb, ldx, Wb, ldw, bb, yb, ldy, scratch, M, N, K, n_split)
+  if (M <= 32) {
+    if (act == 0) MID(2, 0); else if (act == 1) MID(2, 1); else MID(2, 2);
+  } else {
+    if (act == 0) MID(4, 0); else if (act == 1) MID(4, 1); else MID(4, 2);
+  }
+#undef MID
+  if (rc) return rc;
+  LMSF_LAUNCH_CHECK("gemm_mid");
+  if (n_split > 1) {
+    const long quads = ((long)M * N + 3) / 4;
+    hipLaunchKernelGGL(gemm_mid_reduce_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream, scratch, bb,
+                       yb, ldy, M, N, n_split, act);
+    LMSF_LAUNCH_CHECK("gemm_mid_reduce");
+  }
+  return 0;
+}

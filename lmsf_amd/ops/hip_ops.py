@@ -365,6 +365,8 @@ class HipOps:
                         _ptr(xs), xs.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(ys),
                         _code(out_dtype), ys.stride(0), rows, N, K, self.skinny_variant, 0, self._stream()))
                 return y
+        if both_bf16 and out_dtype == torch.bfloat16 and self.skinny_max_rows < M <= 64 and self._mid_ok(x, weight):
+            return self._linear_mid(x, weight, bias, 0)
         if self.use_library_gemm and both_bf16 and M > self.skinny_max_rows:
             y = torch.nn.functional.linear(x, weight, bias)
             return y if out_dtype == torch.bfloat16 else y.to(out_dtype)
@@ -377,9 +379,10 @@ class HipOps:
     def linear_gated(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
                      kind: str = "silu") -> torch.Tensor:
         """act(x Wg^T + bg) * (x Wu^T + bu) for the fused weight [2 I, K] = [Wg; Wu] (bias [2 I] likewise);
-        [M, I] in x's dtype. With few bfloat16 rows the activation is the epilogue of the weight-streaming
+        [M, I] in x's dtype. With up to 64 bfloat16 rows the activation is the epilogue of the weight-streaming
         product; otherwise the product and the activation kernel run one after the other. Both ways round
-        the two products to the storage type before the activation, so they give the same bits."""
+        the two products to the storage type before the activation, so they give the same bits wherever
+        they add up K in the same order."""
         if weight.dim() != 2 or weight.shape[0] % 2 != 0:
             raise ValueError("linear_gated: weight must be [2 I, K]")
         kinds = {"silu": 1, "gelu": 2}
@@ -397,7 +400,34 @@ class HipOps:
                 _ptr(x), x.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(y), BF16, y.stride(0), M, I,
                 x.shape[1], self.skinny_variant, kinds[kind], self._stream()))
             return y
+        if (x.dim() == 2 and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
+                and self.skinny_max_rows < M <= 64 and x.shape[1] == weight.shape[1] and self._mid_ok(x, weight)):
+            return self._linear_mid(x, weight, bias, kinds[kind])
         return self.gated_act(self.linear(x, weight, bias), kind)
+
+    @staticmethod
+    def _mid_ok(x: torch.Tensor, weight: torch.Tensor) -> bool:
+        """What the kernel for 17 to 64 rows asks: K a multiple of 64, N of 4, unit column strides, row strides
+        that are multiples of 8, 16-byte bases."""
+        K = x.shape[1]
+        return (K % 64 == 0 and weight.shape[0] % 8 == 0 and x.stride(1) == 1 and weight.stride(1) == 1
+                and x.stride(0) % 8 == 0 and weight.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
+                and weight.data_ptr() % 16 == 0)
+
+    def _linear_mid(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], act: int) -> torch.Tensor:
+        self._dev(x, weight, bias)
+        M, K = x.shape
+        N = weight.shape[0] // 2 if act else weight.shape[0]
+        if bias is not None and (bias.shape != (weight.shape[0],) or bias.dtype != weight.dtype
+                                 or not bias.is_contiguous()):
+            raise ValueError("linear: bias must be [%d] of the weight's dtype" % weight.shape[0])
+        splits = self.lib.lmsf_gemm_mid_splits(M, N, K, act)
+        floats = self.lib.lmsf_gemm_mid_scratch_floats(M, N, splits, act)
+        scratch = torch.empty(floats, dtype=torch.float32, device=x.device) if floats else None
+        y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+        self._check(self.lib.lmsf_gemm_mid(_ptr(x), x.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(y),
+                                           y.stride(0), M, N, K, act, splits, _ptr(scratch), self._stream()))
+        return y
 
     @staticmethod
     def _skinny_ok(x: torch.Tensor, weight: torch.Tensor) -> bool:
