@@ -33,14 +33,15 @@ LLAMA3_8B = dict(
     bos_token_id=128000, eos_token_id=128001)
 
 
-def make_engine(cfg, args, max_num_seqs, dtype):
+def make_engine(cfg, args, max_num_seqs, dtype, prefill_chunk_size=None):
     from lmsf_amd.engine import EngineArgs, LLMEngine
     folder = tempfile.mkdtemp(prefix="lmsf_bench_")
     with open(os.path.join(folder, "config.json"), "w") as f:
         json.dump(cfg, f)
     return LLMEngine(EngineArgs(model=folder, dtype=dtype, block_size=16, load_format="random", seed=0,
                                 max_num_seqs=max_num_seqs, max_num_batched_tokens=args.max_num_batched_tokens,
-                                gpu_memory_utilization=args.gpu_memory_utilization))
+                                gpu_memory_utilization=args.gpu_memory_utilization,
+                                prefill_chunk_size=prefill_chunk_size))
 
 
 def weight_bytes(engine):
@@ -111,6 +112,57 @@ def prefill_run(engine, n_tokens, reps, seed):
     return times[len(times) // 2]
 
 
+LLAMA2_7B = dict(
+    architectures=["LlamaForCausalLM"], model_type="llama", vocab_size=32000, hidden_size=4096,
+    intermediate_size=11008, num_hidden_layers=32, num_attention_heads=32, num_key_value_heads=32, head_dim=128,
+    rms_norm_eps=1e-5, rope_theta=10000.0, rope_scaling=None, max_position_embeddings=4096,
+    tie_word_embeddings=False, attention_bias=False, hidden_act="silu", torch_dtype="bfloat16",
+    bos_token_id=1, eos_token_id=2)
+
+
+def serve_run(args):
+    """Continuous batching at Llama-2-7B shape: 64 requests arrive at once, prompts of 128 to 2,048 random
+    tokens, 128 generated tokens each, prompts cut into portions that run beside the decoding requests."""
+    import torch
+    from lmsf_amd.sampling import SamplingParams
+    cfg = dict(LLAMA2_7B)
+    if args.layers:
+        cfg["num_hidden_layers"] = args.layers
+    engine = make_engine(cfg, args, max_num_seqs=64, dtype=args.dtype, prefill_chunk_size=args.prefill_chunk_size)
+    rng = random.Random(7)
+    V = cfg["vocab_size"]
+
+    def load(n_req, n_out):
+        prompts = [[rng.randrange(V) for _ in range(rng.randint(128, 2048))] for _ in range(n_req)]
+        for i, p in enumerate(prompts):
+            engine.add_request("s%d_%d" % (n_req, i), p, SamplingParams(temperature=0.0, max_tokens=n_out, ignore_eos=True))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        steps = 0
+        while engine.has_unfinished_requests():
+            engine.step()
+            steps += 1
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0, steps, sum(len(p) for p in prompts)
+
+    load(8, 8)                                   # warm-up: kernels, graphs of the small batch sizes
+    dt, steps, prompt_tokens = load(64, 128)
+    out_tokens = 64 * 128
+    line = {
+        "metric": "continuous batching, generated tok/s (Llama-2-7B bf16, 64 requests)", "value": round(out_tokens / dt, 1),
+        "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": 0, "ms_per_step": round(dt / steps * 1e3, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
+        "config": {"model": "Llama-2-7B shape, random weights", "global_batch": 64, "seq_len": 2048,
+                   "parallelism": "single GPU", "layers": cfg["num_hidden_layers"], "layers_of_model": 32,
+                   "requests": 64, "prompt_tokens": prompt_tokens, "generated_tokens": out_tokens,
+                   "prefill_chunk_size": args.prefill_chunk_size, "max_num_batched_tokens": args.max_num_batched_tokens,
+                   "total_tok_per_s": round((prompt_tokens + out_tokens) / dt, 1), "seconds": round(dt, 3),
+                   "preemptions": engine.stats["preemptions"]},
+    }
+    print(json.dumps(line))
+
+
 def prefill_flops(cfg, T):
     """Multiply-adds times two of a causal prefill of T tokens: the linear layers on every token, the
     attention scores and values over the causal half, the LM head on one row."""
@@ -134,11 +186,18 @@ def main():
     ap.add_argument("--max-num-batched-tokens", type=int, default=8192)
     ap.add_argument("--gpu-memory-utilization", type=float, default=0.85)
     ap.add_argument("--skip-points", action="store_true", help="leave out the batch 1 and batch 64 runs")
+    ap.add_argument("--workload", default="decode", choices=["decode", "serve"],
+                    help="decode: the default line (Llama-3-8B shape); serve: continuous batching of 64 requests at "
+                         "Llama-2-7B shape, a line of its own")
+    ap.add_argument("--prefill-chunk-size", type=int, default=1024, help="serve: longest portion of a prompt in a step")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this engine runs on one GPU; --gpus %d is not supported" % args.gpus)
         sys.exit(2)
 
+    if args.workload == "serve":
+        serve_run(args)
+        return
     import torch
     cfg = dict(LLAMA3_8B)
     full_layers = cfg["num_hidden_layers"]

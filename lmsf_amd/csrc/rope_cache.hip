@@ -18,14 +18,16 @@
 // k unrotated, slots == null writes no cache.
 #include "common.h"
 
-// One workgroup of 64 threads per (token, head): heads 0 .. nh-1 are q heads, then nkv k heads, then nkv
-// v heads. A decode step has few tokens, so the parallelism has to come from the heads.
+// One wave per (token, head): heads 0 .. nh-1 are q heads, then nkv k heads, then nkv v heads (a decode step
+// has few tokens, so the parallelism has to come from the heads); a workgroup holds the waves of
+// blockDim.y consecutive tokens of one head.
 template <typename T>
-__global__ __launch_bounds__(64) void rope_cache_write_kernel(
+__global__ __launch_bounds__(256) void rope_cache_write_kernel(
     T* __restrict__ q, T* __restrict__ k, const T* __restrict__ v, long row_stride, const int* __restrict__ positions,
     const float* __restrict__ table, int rot, int neox, const int* __restrict__ slots, T* __restrict__ k_pages,
-    T* __restrict__ v_pages, int nh, int nkv, int d, int ps) {
-  const long t = blockIdx.x;
+    T* __restrict__ v_pages, int nh, int nkv, int d, int ps, int n_tokens) {
+  const long t = (long)blockIdx.x * blockDim.y + threadIdx.y;
+  if (t >= n_tokens) return;
   const int hy = blockIdx.y;
   const int half = rot / 2;
   const float* cs = table ? table + (long)positions[t] * rot : nullptr;
@@ -97,15 +99,16 @@ extern "C" int lmsf_rope_cache_write(void* q, void* k, const void* v, int dtype,
   if (n_tokens == 0) return 0;
   const int heads = nh + 2 * nkv;
   LMSF_CHECK(heads > 0 && heads <= 65535, "rope_cache_write: %d heads do not fit the grid", heads);
-  dim3 grid(n_tokens, heads);
+  const int per_block = n_tokens >= 64 ? 4 : 1;   // tokens per workgroup: many small workgroups cost a long prompt time
+  dim3 grid((n_tokens + per_block - 1) / per_block, heads), block(64, per_block);
   if (dtype == LMSF_F32)
-    hipLaunchKernelGGL((rope_cache_write_kernel<float>), grid, dim3(64), 0, stream, (float*)q, (float*)k,
+    hipLaunchKernelGGL((rope_cache_write_kernel<float>), grid, block, 0, stream, (float*)q, (float*)k,
                        (const float*)v, row_stride, positions, table, rot, neox, slots, (float*)k_pages,
-                       (float*)v_pages, nh, nkv, d, ps);
+                       (float*)v_pages, nh, nkv, d, ps, n_tokens);
   else
-    hipLaunchKernelGGL((rope_cache_write_kernel<bf16_t>), grid, dim3(64), 0, stream, (bf16_t*)q,
+    hipLaunchKernelGGL((rope_cache_write_kernel<bf16_t>), grid, block, 0, stream, (bf16_t*)q,
                        (bf16_t*)k, (const bf16_t*)v, row_stride, positions, table, rot, neox, slots, (bf16_t*)k_pages,
-                       (bf16_t*)v_pages, nh, nkv, d, ps);
+                       (bf16_t*)v_pages, nh, nkv, d, ps, n_tokens);
   LMSF_LAUNCH_CHECK("rope_cache_write");
   return 0;
 }
