@@ -42,15 +42,26 @@ __device__ __forceinline__ float mid_activation(float g, float u, int act) {
   return a * u;
 }
 
+// four consecutive outputs of a row
+__device__ __forceinline__ void mid_store4(bf16_t* p, const float* o) {
+  uint2 v;
+  v.x = pack2_bf16(o[0], o[1]);
+  v.y = pack2_bf16(o[2], o[3]);
+  *reinterpret_cast<uint2*>(p) = v;
+}
+__device__ __forceinline__ void mid_store4(float* p, const float* o) {
+  *reinterpret_cast<float4*>(p) = make_float4(o[0], o[1], o[2], o[3]);
+}
+
 #define MID_STAGES 5
 #define MID_TILE 2048
 
 // MT: tiles of 16 rows of x (2 or 4). ACT: 0 none, 1 silu-gated, 2 gelu-gated (W = [gate rows; up rows], N
 // outputs). PARTIAL: write float32 partial sums of this workgroup's part of K instead of the result.
-template <int MT, int ACT, bool PARTIAL>
+template <int MT, int ACT, bool PARTIAL, typename TOut>
 __global__ __launch_bounds__(256) void gemm_mid_kernel(const bf16_t* __restrict__ x, long ldx,
                                                        const bf16_t* __restrict__ W, long ldw,
-                                                       const bf16_t* __restrict__ bias, bf16_t* __restrict__ y,
+                                                       const bf16_t* __restrict__ bias, TOut* __restrict__ y,
                                                        long ldy, float* __restrict__ part, int M, int N, int K,
                                                        int n_split) {
   constexpr int WT = ACT ? 2 : 1;
@@ -158,17 +169,15 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const bf16_t* __restrict_
           o[i] = mid_activation(gg, uu, ACT);
         }
       }
-      uint2 v;
-      v.x = pack2_bf16(o[0], o[1]);
-      v.y = pack2_bf16(o[2], o[3]);
-      *reinterpret_cast<uint2*>(y + (long)m * ldy + n) = v;
+      mid_store4(y + (long)m * ldy + n, o);
     }
   }
 }
 
 // y[m][n] = (act of) the sum over the splits of the partial sums, in the order of the splits, plus bias.
+template <typename TOut>
 __global__ __launch_bounds__(256) void gemm_mid_reduce_kernel(const float* __restrict__ part,
-                                                              const bf16_t* __restrict__ bias, bf16_t* __restrict__ y,
+                                                              const bf16_t* __restrict__ bias, TOut* __restrict__ y,
                                                               long ldy, int M, int N, int n_split, int act) {
   const long idx = ((long)blockIdx.x * 256 + threadIdx.x) * 4;   // over M * N, four outputs of a row at a time
   if (idx >= (long)M * N) return;
@@ -190,18 +199,15 @@ __global__ __launch_bounds__(256) void gemm_mid_reduce_kernel(const float* __res
       o[i] = gg;
     }
   }
-  uint2 v;
-  v.x = pack2_bf16(o[0], o[1]);
-  v.y = pack2_bf16(o[2], o[3]);
-  *reinterpret_cast<uint2*>(y + (long)m * ldy + n) = v;
+  mid_store4(y + (long)m * ldy + n, o);
 }
 
-template <int MT, int ACT, bool PARTIAL>
+template <int MT, int ACT, bool PARTIAL, typename TOut>
 static int launch_mid(dim3 grid, hipStream_t stream, const bf16_t* x, long ldx, const bf16_t* W, long ldw,
-                      const bf16_t* bias, bf16_t* y, long ldy, float* part, int M, int N, int K, int n_split) {
+                      const bf16_t* bias, TOut* y, long ldy, float* part, int M, int N, int K, int n_split) {
   constexpr int WT = ACT ? 2 : 1;
   const size_t smem = (size_t)MID_STAGES * (4 * WT + MT) * MID_TILE;
-  auto kernel = gemm_mid_kernel<MT, ACT, PARTIAL>;
+  auto kernel = gemm_mid_kernel<MT, ACT, PARTIAL, TOut>;
   static bool configured = false;   // per instantiation
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -243,41 +249,51 @@ extern "C" long lmsf_gemm_mid_scratch_floats(int M, int N, int n_split, int act)
 }
 
 // x [M, K] bfloat16 (row stride ldx), W [N, K] (act 0) or [2 N, K] (act 1 silu, 2 gelu: gate rows first),
-// bias [N] or [2 N] or null, y [M, N] bfloat16. Needs 1 <= M <= 64, K a multiple of 64, N a multiple of 4,
+// bias [N] or [2 N] or null, y [M, N] of out_dtype (float32 only without activation). Needs 1 <= M <= 64, K a multiple of 64, N a multiple of 4,
 // 16-byte aligned x and W, row strides of x and W that are multiples of 8 and of y of 4; anything else is
 // refused. n_split: parts of K that go to different workgroups (lmsf_gemm_mid_splits proposes a number);
 // scratch: lmsf_gemm_mid_scratch_floats floats (may be null when that is 0).
-extern "C" int lmsf_gemm_mid(const void* x, long ldx, const void* W, long ldw, const void* bias, void* y, long ldy,
-                             int M, int N, int K, int act, int n_split, float* scratch, hipStream_t stream) {
+extern "C" int lmsf_gemm_mid(const void* x, long ldx, const void* W, long ldw, const void* bias, void* y,
+                             int out_dtype, long ldy, int M, int N, int K, int act, int n_split, float* scratch,
+                             hipStream_t stream) {
   LMSF_CHECK(x && W && y, "gemm_mid: null pointer");
   LMSF_CHECK(M >= 0 && M <= 64, "gemm_mid: M=%d outside [0, 64]", M);
   LMSF_CHECK(N > 0 && N % 4 == 0 && K > 0 && K % 64 == 0, "gemm_mid: N=%d must be a multiple of 4 and K=%d of 64", N, K);
   LMSF_CHECK(ldx >= K && ldw >= K && ldy >= N && ldx % 8 == 0 && ldw % 8 == 0 && ldy % 4 == 0,
              "gemm_mid: row strides must cover the rows, be multiples of 8 (x, W) and of 4 (y)");
-  LMSF_CHECK(lmsf_aligned16(x) && lmsf_aligned16(W) && (((uintptr_t)y) & 7u) == 0, "gemm_mid: operands must be aligned");
+  LMSF_CHECK(lmsf_aligned16(x) && lmsf_aligned16(W) && lmsf_aligned16(y), "gemm_mid: operands must be 16-byte aligned");
   LMSF_CHECK(act >= 0 && act <= 2, "gemm_mid: unknown activation %d", act);
+  LMSF_CHECK(out_dtype == LMSF_BF16 || (out_dtype == LMSF_F32 && act == 0),
+             "gemm_mid: output is bfloat16, or float32 without activation");
   if (M == 0) return 0;
   LMSF_CHECK(n_split >= 1 && n_split <= 64 && n_split <= K / 64, "gemm_mid: %d splits of K=%d", n_split, K);
   LMSF_CHECK(n_split == 1 || scratch != nullptr, "gemm_mid: %d splits need scratch", n_split);
   dim3 grid((N + 63) / 64, n_split);
   const bf16_t *xb = (const bf16_t*)x, *Wb = (const bf16_t*)W, *bb = (const bf16_t*)bias;
-  bf16_t* yb = (bf16_t*)y;
   int rc = 0;
-#define MID(MT_, ACT_)                                                                                           \
-  rc = n_split > 1 ? launch_mid<MT_, ACT_, true>(grid, stream, xb, ldx, Wb, ldw, bb, yb, ldy, scratch, M, N, K, n_split) \
-                   : launch_mid<MT_, ACT_, false>(grid, stream, xb, ldx, Wb, ldw, bb, yb, ldy, scratch, M, N, K, n_split)
-  if (M <= 32) {
-    if (act == 0) MID(2, 0); else if (act == 1) MID(2, 1); else MID(2, 2);
+#define MID(MT_, ACT_, T_)                                                                                          \
+  rc = n_split > 1                                                                                                  \
+           ? launch_mid<MT_, ACT_, true, T_>(grid, stream, xb, ldx, Wb, ldw, bb, (T_*)y, ldy, scratch, M, N, K, n_split) \
+           : launch_mid<MT_, ACT_, false, T_>(grid, stream, xb, ldx, Wb, ldw, bb, (T_*)y, ldy, scratch, M, N, K, n_split)
+  if (out_dtype == LMSF_F32) {
+    if (M <= 32) MID(2, 0, float); else MID(4, 0, float);
+  } else if (M <= 32) {
+    if (act == 0) MID(2, 0, bf16_t); else if (act == 1) MID(2, 1, bf16_t); else MID(2, 2, bf16_t);
   } else {
-    if (act == 0) MID(4, 0); else if (act == 1) MID(4, 1); else MID(4, 2);
+    if (act == 0) MID(4, 0, bf16_t); else if (act == 1) MID(4, 1, bf16_t); else MID(4, 2, bf16_t);
   }
 #undef MID
   if (rc) return rc;
   LMSF_LAUNCH_CHECK("gemm_mid");
   if (n_split > 1) {
     const long quads = ((long)M * N + 3) / 4;
-    hipLaunchKernelGGL(gemm_mid_reduce_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream, scratch, bb,
-                       yb, ldy, M, N, n_split, act);
+    const dim3 rgrid((unsigned)((quads + 255) / 256));
+    if (out_dtype == LMSF_F32)
+      hipLaunchKernelGGL(gemm_mid_reduce_kernel<float>, rgrid, dim3(256), 0, stream, scratch, bb, (float*)y, ldy, M, N,
+                         n_split, act);
+    else
+      hipLaunchKernelGGL(gemm_mid_reduce_kernel<bf16_t>, rgrid, dim3(256), 0, stream, scratch, bb, (bf16_t*)y, ldy, M,
+                         N, n_split, act);
     LMSF_LAUNCH_CHECK("gemm_mid_reduce");
   }
   return 0;

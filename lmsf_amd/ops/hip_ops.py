@@ -352,6 +352,8 @@ class HipOps:
             raise ValueError("linear: bias must be [%d] of the weight's dtype" % N)
         out_dtype = out_dtype or x.dtype
         both_bf16 = x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
+        if both_bf16 and self.skinny_max_rows < M <= 64 and self._mid_ok(x, weight):
+            return self._linear_mid(x, weight, bias, 0, out_dtype)
         if both_bf16 and self._skinny_ok(x, weight):
             # few rows: the weight-streaming kernel. It also serves float32 output (logits), which the
             # library does not offer, for any number of rows, 64 at a time.
@@ -365,8 +367,6 @@ class HipOps:
                         _ptr(xs), xs.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(ys),
                         _code(out_dtype), ys.stride(0), rows, N, K, self.skinny_variant, 0, self._stream()))
                 return y
-        if both_bf16 and out_dtype == torch.bfloat16 and self.skinny_max_rows < M <= 64 and self._mid_ok(x, weight):
-            return self._linear_mid(x, weight, bias, 0)
         if self.use_library_gemm and both_bf16 and M > self.skinny_max_rows:
             y = torch.nn.functional.linear(x, weight, bias)
             return y if out_dtype == torch.bfloat16 else y.to(out_dtype)
@@ -414,7 +414,8 @@ class HipOps:
                 and x.stride(0) % 8 == 0 and weight.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
                 and weight.data_ptr() % 16 == 0)
 
-    def _linear_mid(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], act: int) -> torch.Tensor:
+    def _linear_mid(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], act: int,
+                    out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
         self._dev(x, weight, bias)
         M, K = x.shape
         N = weight.shape[0] // 2 if act else weight.shape[0]
@@ -424,9 +425,10 @@ class HipOps:
         splits = self.lib.lmsf_gemm_mid_splits(M, N, K, act)
         floats = self.lib.lmsf_gemm_mid_scratch_floats(M, N, splits, act)
         scratch = torch.empty(floats, dtype=torch.float32, device=x.device) if floats else None
-        y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+        y = torch.empty((M, N), dtype=out_dtype, device=x.device)
         self._check(self.lib.lmsf_gemm_mid(_ptr(x), x.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(y),
-                                           y.stride(0), M, N, K, act, splits, _ptr(scratch), self._stream()))
+                                           _code(out_dtype), y.stride(0), M, N, K, act, splits, _ptr(scratch),
+                                           self._stream()))
         return y
 
     @staticmethod
