@@ -168,14 +168,66 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(
   if (tid == 0) out[r] = best < V ? best : 0;
 }
 
+// Greedy rows of a large vocabulary, in two small kernels: each of SPLIT workgroups finds the first maximum
+// of its share of the row, then one wave per row picks among the shares (the lowest index wins ties, as in
+// the kernel above). One workgroup per row leaves most of the chip idle when there are few rows.
+#define ARGMAX_SPLIT 32
+__global__ __launch_bounds__(256) void argmax_partial_kernel(const float* __restrict__ logits, long ld, int V,
+                                                             float* __restrict__ pval, int* __restrict__ pidx) {
+  __shared__ float redf[16];
+  __shared__ int redi[16];
+  const int r = blockIdx.x, part = blockIdx.y, tid = threadIdx.x;
+  const int per = (V + ARGMAX_SPLIT - 1) / ARGMAX_SPLIT;
+  const int lo = part * per, hi = min(V, lo + per);
+  const float* row = logits + (long)r * ld;
+  float bv = -INFINITY;
+  int bi = 0x7fffffff;
+  for (int i = lo + tid; i < hi; i += 256) {
+    const float x = row[i];
+    if (x > bv) { bv = x; bi = i; }
+  }
+  const int best = block_argmax(bv, bi, redf, redi);
+  if (tid == 0) {
+    pidx[r * ARGMAX_SPLIT + part] = best;
+    pval[r * ARGMAX_SPLIT + part] = best < V ? row[best] : -INFINITY;
+  }
+}
+__global__ __launch_bounds__(64) void argmax_final_kernel(const float* __restrict__ pval, const int* __restrict__ pidx,
+                                                          int V, int* __restrict__ out) {
+  const int r = blockIdx.x, l = threadIdx.x;
+  float v = l < ARGMAX_SPLIT ? pval[r * ARGMAX_SPLIT + l] : -INFINITY;
+  int idx = l < ARGMAX_SPLIT ? pidx[r * ARGMAX_SPLIT + l] : 0x7fffffff;
+#pragma unroll
+  for (int o = LMSF_WAVE / 2; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(v, o, LMSF_WAVE);
+    const int oi = __shfl_xor(idx, o, LMSF_WAVE);
+    if (ov > v || (ov == v && oi < idx)) { v = ov; idx = oi; }
+  }
+  if (l == 0) out[r] = idx < V ? idx : 0;
+}
+
+// Floats (and as many ints) of scratch that lmsf_sample wants for R greedy rows; 0: none needed.
+extern "C" long lmsf_sample_scratch_elems(int R, int V) { return (V >= 16384 && R <= 256) ? (long)R * ARGMAX_SPLIT : 0; }
+
 // logits [R, V] float32 with row stride ld. temperature/top_k/top_p/min_p/seeds/draws are per-row
 // device arrays; any of them may be null (greedy, no cut, seed 0, draw 0).
+// scratch (optional): lmsf_sample_scratch_elems(R, V) floats followed by as many ints; with it, and with
+// no temperature (all rows greedy), a large vocabulary is searched by several workgroups per row.
 extern "C" int lmsf_sample(const float* logits, long ld, int R, int V, const float* temperature, const int* top_k,
                            const float* top_p, const float* min_p, const unsigned long long* seeds,
-                           const unsigned int* draws, int* out, hipStream_t stream) {
+                           const unsigned int* draws, int* out, void* scratch, hipStream_t stream) {
   LMSF_CHECK(logits && out, "sample: null pointer");
   LMSF_CHECK(R >= 0 && V > 0 && ld >= V, "sample: bad sizes R=%d V=%d ld=%ld", R, V, ld);
   if (R == 0) return 0;
+  const long elems = lmsf_sample_scratch_elems(R, V);
+  if (temperature == nullptr && scratch != nullptr && elems > 0) {
+    float* pval = (float*)scratch;
+    int* pidx = (int*)(pval + elems);
+    hipLaunchKernelGGL(argmax_partial_kernel, dim3(R, ARGMAX_SPLIT), dim3(256), 0, stream, logits, ld, V, pval, pidx);
+    hipLaunchKernelGGL(argmax_final_kernel, dim3(R), dim3(64), 0, stream, pval, pidx, V, out);
+    LMSF_LAUNCH_CHECK("sample (greedy)");
+    return 0;
+  }
   hipLaunchKernelGGL(sample_kernel, dim3(R), dim3(SAMP_THREADS), 0, stream, logits, ld, V, temperature, top_k, top_p,
                      min_p, seeds, draws, out);
   LMSF_LAUNCH_CHECK("sample");

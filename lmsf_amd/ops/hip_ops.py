@@ -456,9 +456,14 @@ class HipOps:
             if t is not None and (t.dtype != dt or t.numel() != R or not t.is_contiguous()):
                 raise ValueError("sample: %s must be a contiguous %s tensor of %d elements" % (name, dt, R))
         out = torch.empty((R,), dtype=torch.int32, device=logits.device)
+        scratch = None
+        if temperature is None:
+            elems = self.lib.lmsf_sample_scratch_elems(R, V)
+            if elems:
+                scratch = torch.empty(2 * elems, dtype=torch.float32, device=logits.device)
         self._check(self.lib.lmsf_sample(_ptr(logits), logits.stride(0), R, V, _ptr(temperature), _ptr(top_k),
                                          _ptr(top_p), _ptr(min_p), _ptr(seeds), _ptr(draws), _ptr(out),
-                                         self._stream()))
+                                         _ptr(scratch), self._stream()))
         return out
 
     def apply_penalties(self, logits: torch.Tensor, tokens: torch.Tensor, offsets: torch.Tensor,

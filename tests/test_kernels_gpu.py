@@ -392,6 +392,19 @@ def test_sample_greedy_and_seeded(ops, ref, V):
         assert a.tolist() == b.tolist(), (draw, a.tolist(), b.tolist())
 
 
+@pytest.mark.parametrize("V", [1000, 16384, 128256])
+def test_greedy_takes_the_first_of_equal_maxima(ops, V):
+    g = torch.Generator().manual_seed(V)
+    logits = torch.randn(5, V, generator=g)
+    logits[0, [V - 1, V // 2, 7]] = 9.0          # equal maxima far apart (different workgroups of a large vocabulary)
+    logits[1, V - 1] = 9.0                        # the last entry
+    logits[2, 0] = 9.0
+    logits[3] = -1.0                              # all equal
+    logits[4, V // 2 + 1] = float("inf")
+    out = ops.sample(dev(logits)).cpu().tolist()
+    assert out == [7, V - 1, 0, 0, V // 2 + 1]
+
+
 def test_sample_does_not_depend_on_batch(ops):
     g = torch.Generator().manual_seed(9)
     logits = dev(torch.randn(4, 777, generator=g))
