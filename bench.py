@@ -120,6 +120,19 @@ LLAMA2_7B = dict(
     bos_token_id=1, eos_token_id=2)
 
 
+LLAMA31_70B = dict(
+    architectures=["LlamaForCausalLM"], model_type="llama", vocab_size=128256, hidden_size=8192,
+    intermediate_size=28672, num_hidden_layers=80, num_attention_heads=64, num_key_value_heads=8, head_dim=128,
+    rms_norm_eps=1e-5, rope_theta=500000.0,
+    rope_scaling=dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                      original_max_position_embeddings=8192),
+    max_position_embeddings=16384, tie_word_embeddings=False, attention_bias=False, hidden_act="silu",
+    torch_dtype="bfloat16", bos_token_id=128000, eos_token_id=128001)
+
+SHAPES = {"llama3-8b": ("Llama-3-8B", LLAMA3_8B), "llama2-7b": ("Llama-2-7B", LLAMA2_7B),
+          "llama3.1-70b": ("Llama-3.1-70B", LLAMA31_70B)}
+
+
 def serve_run(args):
     """Continuous batching at Llama-2-7B shape: 64 requests arrive at once, prompts of 128 to 2,048 random
     tokens, 128 generated tokens each, prompts cut into portions that run beside the decoding requests."""
@@ -190,6 +203,9 @@ def main():
                     help="decode: the default line (Llama-3-8B shape); serve: continuous batching of 64 requests at "
                          "Llama-2-7B shape, a line of its own")
     ap.add_argument("--prefill-chunk-size", type=int, default=1024, help="serve: longest portion of a prompt in a step")
+    ap.add_argument("--shape", default="llama3-8b", choices=sorted(SHAPES),
+                    help="decode: the model whose layer sizes are measured (default: the headline configuration)")
+    ap.add_argument("--points", default="1,64", help="decode: further batch sizes, comma separated")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this engine runs on one GPU; --gpus %d is not supported" % args.gpus)
@@ -199,7 +215,8 @@ def main():
         serve_run(args)
         return
     import torch
-    cfg = dict(LLAMA3_8B)
+    shape_name, shape_cfg = SHAPES[args.shape]
+    cfg = dict(shape_cfg)
     full_layers = cfg["num_hidden_layers"]
     if args.layers:
         cfg["num_hidden_layers"] = args.layers
@@ -216,7 +233,7 @@ def main():
 
     points = {}
     if not args.skip_points:
-        for b in (1, 64):
+        for b in [int(x) for x in args.points.split(",") if x]:
             k = max(16, args.steps // 2)
             d, _ = decode_run(engine, b, args.prompt_len, k, args.warmup, seed=2 + b)
             points["decode_b%d" % b] = round(b * k / d, 1)
@@ -226,12 +243,12 @@ def main():
     peak = PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
 
     line = {
-        "metric": "decode tok/s at batch 8 (Llama-3-8B bf16)",
+        "metric": "decode tok/s at batch %d (%s %s)" % (args.batch, shape_name, "bf16" if args.dtype == "bfloat16" else "fp32"),
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic",
         "config": {
-            "model": "Llama-3-8B shape, random weights", "global_batch": args.batch, "seq_len": args.prompt_len,
+            "model": "%s shape, random weights" % shape_name, "global_batch": args.batch, "seq_len": args.prompt_len,
             "parallelism": "single GPU", "layers": cfg["num_hidden_layers"], "layers_of_model": full_layers,
             "hidden_size": cfg["hidden_size"], "heads": cfg["num_attention_heads"],
             "kv_heads": cfg["num_key_value_heads"], "head_dim": cfg["head_dim"],
