@@ -69,10 +69,12 @@ def decode_run(engine, batch, prompt_len, steps, warmup, seed):
     rng = random.Random(seed)
     V = engine.core.config.vocab_size
     ids = []
+    # requests whose prompts are done first decode while the others are still being prefilled: room for that
+    slack = batch * prompt_len // 1024 + 16
     for i in range(batch):
         rid = "b%d_%d" % (batch, i)
         engine.add_request(rid, [rng.randrange(V) for _ in range(prompt_len)],
-                           SamplingParams(temperature=0.0, max_tokens=steps + warmup + 8, ignore_eos=True))
+                           SamplingParams(temperature=0.0, max_tokens=steps + warmup + slack, ignore_eos=True))
         ids.append(rid)
     while any(s.remaining > 1 for s in list(engine.scheduler.running) + list(engine.scheduler.waiting)) \
             or engine.scheduler.waiting:
