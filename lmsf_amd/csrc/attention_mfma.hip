@@ -568,14 +568,15 @@ static int launch_prefill_dma(dim3 grid, hipStream_t stream, const bf16_t* q, lo
 //   part_o[((i * nh + head) * n_splits + s) * d + dv]  (not normalised),
 //   part_ml[((i * nh + head) * n_splits + s) * 2 + {0, 1}] = (running maximum in log2 units, sum),
 // i being the index of the token in this launch. A split without keys writes nothing; the reduction
-// knows from the position which splits have keys.
+// knows from the position which splits have keys. With n_splits == 1 there is nothing to reduce and the
+// workgroup writes out[tok, head, :] itself.
 template <int DPAD>
 __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
     const bf16_t* __restrict__ q, long q_stride, const bf16_t* __restrict__ k_pages,
     const bf16_t* __restrict__ v_pages, const int* __restrict__ block_tables, int btw,
     const int* __restrict__ tok_idx, const int* __restrict__ seg, const int* __restrict__ pos, int nh, int nkv, int d,
     int ps, float scale_log2, int window, int HB, int n_hb, int chunk, int n_splits, float* __restrict__ part_o,
-    float* __restrict__ part_ml) {
+    float* __restrict__ part_ml, bf16_t* __restrict__ out, long out_stride) {
   constexpr int DS = DPAD / 32, DV = DPAD / 16;
   extern __shared__ float lds_f[];
   const int i_tok = blockIdx.x;
@@ -703,7 +704,12 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
       o += f * lds_o[(ww * 16 + r) * (DPAD + 4) + dv];
       ls += f * lds_l[ww * 16 + r];
     }
-    const long slot = ((long)i_tok * nh + (kvh * n_rep + hb * HB + r)) * n_splits + split;
+    const int hd = kvh * n_rep + hb * HB + r;
+    if (n_splits == 1) {
+      out[(long)tok * out_stride + (long)hd * d + dv] = f32_to_bf16(o / ls);
+      continue;
+    }
+    const long slot = ((long)i_tok * nh + hd) * n_splits + split;
     part_o[slot * d + dv] = o;
     if (dv == 0) {
       part_ml[slot * 2] = M;
@@ -830,7 +836,7 @@ template <int DPAD>
 static int launch_decode(dim3 grid, hipStream_t stream, const bf16_t* q, long q_stride, const bf16_t* k_pages,
                          const bf16_t* v_pages, const int* block_tables, int btw, const int* tok_idx, const int* seg,
                          const int* pos, int nh, int nkv, int d, int ps, float scale_log2, int window, int HB, int n_hb,
-                         int chunk, int n_splits, float* part_o, float* part_ml) {
+                         int chunk, int n_splits, float* part_o, float* part_ml, bf16_t* out, long out_stride) {
   const size_t smem = (size_t)(4 * 16 * (DPAD + 4) + 128) * sizeof(float);
   auto kernel = attn_decode_mfma_kernel<DPAD>;
   static bool configured = false;   // per instantiation
@@ -844,7 +850,8 @@ static int launch_decode(dim3 grid, hipStream_t stream, const bf16_t* q, long q_
     configured = true;
   }
   hipLaunchKernelGGL(kernel, grid, dim3(256), smem, stream, q, q_stride, k_pages, v_pages, block_tables, btw, tok_idx,
-                     seg, pos, nh, nkv, d, ps, scale_log2, window, HB, n_hb, chunk, n_splits, part_o, part_ml);
+                     seg, pos, nh, nkv, d, ps, scale_log2, window, HB, n_hb, chunk, n_splits, part_o, part_ml, out,
+                     out_stride);
   return 0;
 }
 
@@ -854,7 +861,8 @@ extern "C" long lmsf_attention_decode_scratch_floats(int n, int nh, int d, int n
 }
 
 // One query token per entry of tok_idx (null: tokens 0 .. n - 1). chunk: keys per split, a multiple of 128;
-// n_splits * chunk must cover the longest context. scratch: lmsf_attention_decode_scratch_floats floats.
+// n_splits * chunk must cover the longest context. scratch: lmsf_attention_decode_scratch_floats floats
+// (not touched with n_splits == 1).
 extern "C" int lmsf_paged_attention_decode_mfma(const void* q, long q_stride, void* out, long out_stride,
                                                 const void* k_pages, const void* v_pages, long num_pages,
                                                 const int* block_tables, int btw, const int* tok_idx, int n,
@@ -880,7 +888,7 @@ extern "C" int lmsf_paged_attention_decode_mfma(const void* q, long q_stride, vo
 #define LAUNCH(DP)                                                                                              \
   rc = launch_decode<DP>(grid, stream, (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, \
                          block_tables, btw, tok_idx, seg, pos, nh, nkv, d, ps, scale_log2, window, HB, n_hb, chunk, \
-                         n_splits, part_o, part_ml)
+                         n_splits, part_o, part_ml, (bf16_t*)out, out_stride)
   switch (dpad) {
     case 32: LAUNCH(32); break;
     case 64: LAUNCH(64); break;
@@ -894,6 +902,7 @@ extern "C" int lmsf_paged_attention_decode_mfma(const void* q, long q_stride, vo
 #undef LAUNCH
   if (rc) return rc;
   LMSF_LAUNCH_CHECK("paged_attention_decode");
+  if (n_splits == 1) return 0;
   int threads = (d + 63) / 64 * 64;
   hipLaunchKernelGGL(attn_decode_reduce_kernel, dim3(n, nh), dim3(threads), 0, stream, part_o, part_ml, (bf16_t*)out,
                      out_stride, tok_idx, pos, nh, d, window, chunk, n_splits);

@@ -48,6 +48,7 @@ class HipOps:
         self._bad_flag = None
         self.use_library_gemm = True   # bfloat16 matrix products of many rows go to the BLAS library
         self.prefill_attention_variant = 0   # 0: keys and values staged in LDS; 1: fetched by every wave for itself
+        self.decode_attention_splits = 0     # 0: chosen from the batch and the context; n: at most n splits of the keys
         self.skinny_variant = 0        # tiling of the few-rows kernel (0: default; others for tuning)
         self.skinny_max_rows = 16      # rows up to which the few-rows kernel beats the library (measured)
 
@@ -261,11 +262,17 @@ class HipOps:
         if plan.n_single:
             n_hb = -(-(nh // nkv) // 16)
             most = -(-plan.max_context // 128)
-            want = max(1, min(most, -(-1024 // (plan.n_single * nkv * n_hb))))
+            # Measured: about 512 workgroups fill the chip; beyond that a split only adds partial results,
+            # and with two short halves the reduction kernel costs more than the second half saves.
+            want = max(1, min(most, 512 // (plan.n_single * nkv * n_hb)))
+            if want == 2 and plan.max_context <= 512:
+                want = 1
+            if self.decode_attention_splits:
+                want = min(most, self.decode_attention_splits)
             chunk = -(-(-(-plan.max_context // want)) // 128) * 128
             n_splits = -(-plan.max_context // chunk)
             floats = self.lib.lmsf_attention_decode_scratch_floats(plan.n_single, nh, d, n_splits)
-            scratch = torch.empty(floats, dtype=torch.float32, device=q.device)
+            scratch = torch.empty(floats if n_splits > 1 else 1, dtype=torch.float32, device=q.device)
             self._check(self.lib.lmsf_paged_attention_decode_mfma(
                 _ptr(q), q.stride(0), _ptr(out), out.stride(0), *common, _ptr(plan.single_tokens), plan.n_single,
                 _ptr(seg), _ptr(pos), nh, nkv, d, ps, float(scale), int(window or 0), chunk, n_splits,
