@@ -65,6 +65,36 @@ template <typename T> __device__ __forceinline__ T from_f32(float v);
 template <> __device__ __forceinline__ float from_f32<float>(float v) { return v; }
 template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float v) { return f32_to_bf16(v); }
 
+// A bfloat16 product [M, N] left as float32 partial sums over parts of K: element (m, n) is the sum over
+// s = 0 .. n_split-1, in that order, of part[(s * M + m) * N + n], plus bias[n] (bias may be null), rounded
+// to bfloat16: the value that the reduction kernel of the product would have stored. Kernels that take one
+// do that reduction while they load their operand. N is a multiple of 4 and part is 16-byte aligned.
+struct LmsfPartialSum {
+  const float* part;
+  const bf16_t* bias;
+  int n_split, M, N;
+};
+__device__ __forceinline__ float partial_sum_value(const LmsfPartialSum& p, int m, int n) {
+  float s = 0.f;
+  for (int i = 0; i < p.n_split; ++i) s += p.part[((long)i * p.M + m) * p.N + n];
+  if (p.bias) s += bf16_to_f32(p.bias[n]);
+  return bf16_to_f32(f32_to_bf16(s));
+}
+// four neighbours (n a multiple of 4)
+__device__ __forceinline__ void partial_sum_value4(const LmsfPartialSum& p, int m, int n, float* x) {
+  float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int i = 0; i < p.n_split; ++i) {
+    const float4 v = *reinterpret_cast<const float4*>(p.part + ((long)i * p.M + m) * p.N + n);
+    s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+  }
+  x[0] = s.x; x[1] = s.y; x[2] = s.z; x[3] = s.w;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    if (p.bias) x[e] += bf16_to_f32(p.bias[n + e]);
+    x[e] = bf16_to_f32(f32_to_bf16(x[e]));
+  }
+}
+
 // 16-byte vectors: 4 floats or 8 bfloat16
 template <typename T> struct Vec16;
 template <> struct Vec16<float> {

@@ -253,23 +253,24 @@ extern "C" long lmsf_gemm_mid_scratch_floats(int M, int N, int n_split, int act)
 // 16-byte aligned x and W, row strides of x and W that are multiples of 8 and of y of 4; anything else is
 // refused. n_split: parts of K that go to different workgroups (lmsf_gemm_mid_splits proposes a number);
 // scratch: lmsf_gemm_mid_scratch_floats floats (may be null when that is 0).
-extern "C" int lmsf_gemm_mid(const void* x, long ldx, const void* W, long ldw, const void* bias, void* y,
-                             int out_dtype, long ldy, int M, int N, int K, int act, int n_split, float* scratch,
-                             hipStream_t stream) {
-  LMSF_CHECK(x && W && y, "gemm_mid: null pointer");
+static int mid_check(const void* x, long ldx, const void* W, long ldw, int M, int N, int K, int n_split,
+                     const float* scratch) {
+  LMSF_CHECK(x && W, "gemm_mid: null pointer");
   LMSF_CHECK(M >= 0 && M <= 64, "gemm_mid: M=%d outside [0, 64]", M);
   LMSF_CHECK(N > 0 && N % 4 == 0 && K > 0 && K % 64 == 0, "gemm_mid: N=%d must be a multiple of 4 and K=%d of 64", N, K);
-  LMSF_CHECK(ldx >= K && ldw >= K && ldy >= N && ldx % 8 == 0 && ldw % 8 == 0 && ldy % 4 == 0,
-             "gemm_mid: row strides must cover the rows, be multiples of 8 (x, W) and of 4 (y)");
-  LMSF_CHECK(lmsf_aligned16(x) && lmsf_aligned16(W) && lmsf_aligned16(y), "gemm_mid: operands must be 16-byte aligned");
-  LMSF_CHECK(act >= 0 && act <= 2, "gemm_mid: unknown activation %d", act);
-  LMSF_CHECK(out_dtype == LMSF_BF16 || (out_dtype == LMSF_F32 && act == 0),
-             "gemm_mid: output is bfloat16, or float32 without activation");
-  if (M == 0) return 0;
+  LMSF_CHECK(ldx >= K && ldw >= K && ldx % 8 == 0 && ldw % 8 == 0,
+             "gemm_mid: row strides of x and W must cover the rows and be multiples of 8");
+  LMSF_CHECK(lmsf_aligned16(x) && lmsf_aligned16(W), "gemm_mid: operands must be 16-byte aligned");
   LMSF_CHECK(n_split >= 1 && n_split <= 64 && n_split <= K / 64, "gemm_mid: %d splits of K=%d", n_split, K);
-  LMSF_CHECK(n_split == 1 || scratch != nullptr, "gemm_mid: %d splits need scratch", n_split);
+  LMSF_CHECK(n_split == 1 || (scratch != nullptr && lmsf_aligned16(scratch)),
+             "gemm_mid: %d splits need 16-byte aligned scratch", n_split);
+  return 0;
+}
+
+// The product's kernel: the result into y (n_split == 1) or partial sums into scratch.
+static int mid_product(const bf16_t* xb, long ldx, const bf16_t* Wb, long ldw, const bf16_t* bb, void* y, int out_dtype,
+                       long ldy, int M, int N, int K, int act, int n_split, float* scratch, hipStream_t stream) {
   dim3 grid((N + 63) / 64, n_split);
-  const bf16_t *xb = (const bf16_t*)x, *Wb = (const bf16_t*)W, *bb = (const bf16_t*)bias;
   int rc = 0;
 #define MID(MT_, ACT_, T_)                                                                                          \
   rc = n_split > 1                                                                                                  \
@@ -285,16 +286,56 @@ extern "C" int lmsf_gemm_mid(const void* x, long ldx, const void* W, long ldw, c
 #undef MID
   if (rc) return rc;
   LMSF_LAUNCH_CHECK("gemm_mid");
-  if (n_split > 1) {
-    const long quads = ((long)M * N + 3) / 4;
-    const dim3 rgrid((unsigned)((quads + 255) / 256));
-    if (out_dtype == LMSF_F32)
-      hipLaunchKernelGGL(gemm_mid_reduce_kernel<float>, rgrid, dim3(256), 0, stream, scratch, bb, (float*)y, ldy, M, N,
-                         n_split, act);
-    else
-      hipLaunchKernelGGL(gemm_mid_reduce_kernel<bf16_t>, rgrid, dim3(256), 0, stream, scratch, bb, (bf16_t*)y, ldy, M,
-                         N, n_split, act);
-    LMSF_LAUNCH_CHECK("gemm_mid_reduce");
-  }
   return 0;
+}
+
+static int mid_reduce(const float* scratch, const bf16_t* bb, void* y, int out_dtype, long ldy, int M, int N,
+                      int act, int n_split, hipStream_t stream) {
+  const long quads = ((long)M * N + 3) / 4;
+  const dim3 rgrid((unsigned)((quads + 255) / 256));
+  if (out_dtype == LMSF_F32)
+    hipLaunchKernelGGL(gemm_mid_reduce_kernel<float>, rgrid, dim3(256), 0, stream, scratch, bb, (float*)y, ldy, M, N,
+                       n_split, act);
+  else
+    hipLaunchKernelGGL(gemm_mid_reduce_kernel<bf16_t>, rgrid, dim3(256), 0, stream, scratch, bb, (bf16_t*)y, ldy, M,
+                       N, n_split, act);
+  LMSF_LAUNCH_CHECK("gemm_mid_reduce");
+  return 0;
+}
+
+extern "C" int lmsf_gemm_mid(const void* x, long ldx, const void* W, long ldw, const void* bias, void* y,
+                             int out_dtype, long ldy, int M, int N, int K, int act, int n_split, float* scratch,
+                             hipStream_t stream) {
+  if (int rc = mid_check(x, ldx, W, ldw, M, N, K, M == 0 ? 1 : n_split, scratch)) return rc;
+  LMSF_CHECK(y != nullptr && lmsf_aligned16(y) && ldy >= N && ldy % 4 == 0,
+             "gemm_mid: y must be 16-byte aligned with a row stride that covers N and is a multiple of 4");
+  LMSF_CHECK(act >= 0 && act <= 2, "gemm_mid: unknown activation %d", act);
+  LMSF_CHECK(out_dtype == LMSF_BF16 || (out_dtype == LMSF_F32 && act == 0),
+             "gemm_mid: output is bfloat16, or float32 without activation");
+  if (M == 0) return 0;
+  const bf16_t *xb = (const bf16_t*)x, *Wb = (const bf16_t*)W, *bb = (const bf16_t*)bias;
+  if (int rc = mid_product(xb, ldx, Wb, ldw, bb, y, out_dtype, ldy, M, N, K, act, n_split, scratch, stream)) return rc;
+  if (n_split > 1) return mid_reduce(scratch, bb, y, out_dtype, ldy, M, N, act, n_split, stream);
+  return 0;
+}
+
+// The two halves of a product without activation whose K is split (n_split >= 2): the partial sums alone,
+// scratch[(s * M + m) * N + n], for a kernel that reduces them while it loads its operand (LmsfPartialSum);
+// and the reduction alone, y = sum over s + bias, for a caller that turns out to need the plain result.
+extern "C" int lmsf_gemm_mid_partial(const void* x, long ldx, const void* W, long ldw, int M, int N, int K,
+                                     int n_split, float* scratch, hipStream_t stream) {
+  if (int rc = mid_check(x, ldx, W, ldw, M, N, K, n_split, scratch)) return rc;
+  LMSF_CHECK(n_split >= 2, "gemm_mid_partial: needs at least two splits, got %d", n_split);
+  if (M == 0) return 0;
+  return mid_product((const bf16_t*)x, ldx, (const bf16_t*)W, ldw, nullptr, nullptr, LMSF_BF16, N, M, N, K, 0, n_split,
+                     scratch, stream);
+}
+extern "C" int lmsf_gemm_mid_reduce(const float* scratch, const void* bias, void* y, int out_dtype, long ldy, int M,
+                                    int N, int n_split, hipStream_t stream) {
+  LMSF_CHECK(scratch && y && lmsf_aligned16(scratch) && lmsf_aligned16(y), "gemm_mid_reduce: null or unaligned pointer");
+  LMSF_CHECK(M >= 0 && N > 0 && N % 4 == 0 && ldy >= N && ldy % 4 == 0 && n_split >= 1,
+             "gemm_mid_reduce: bad sizes M=%d N=%d ldy=%ld splits=%d", M, N, ldy, n_split);
+  LMSF_CHECK(out_dtype == LMSF_BF16 || out_dtype == LMSF_F32, "gemm_mid_reduce: unknown dtype code %d", out_dtype);
+  if (M == 0) return 0;
+  return mid_reduce(scratch, (const bf16_t*)bias, y, out_dtype, ldy, M, N, 0, n_split, stream);
 }

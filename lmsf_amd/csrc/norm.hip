@@ -76,16 +76,18 @@ template <> struct Vec4<bf16_t> {
   }
 };
 
-template <typename TB, typename TO, typename TW, int VPT>
+// PART: the branch is a product left as partial sums (``partial``; ``branch`` is not read).
+template <typename TB, typename TO, typename TW, int VPT, bool PART>
 __global__ __launch_bounds__(1024) void add_rms_norm_vec_kernel(
     const TB* __restrict__ branch, float* __restrict__ residual, const TW* __restrict__ weight,
-    TO* __restrict__ out, const int* __restrict__ rows, int H, float eps, float weight_offset) {
+    TO* __restrict__ out, const int* __restrict__ rows, int H, float eps, float weight_offset,
+    LmsfPartialSum partial) {
   __shared__ float red[16];
   const int r = blockIdx.x;
   const long src = rows ? (long)rows[r] : (long)r;
-  const TB* b = branch ? branch + src * H : nullptr;
+  const TB* b = (!PART && branch) ? branch + src * H : nullptr;
   float* res = residual ? residual + src * H : nullptr;
-  const bool write_res = (b != nullptr) && (res != nullptr) && (rows == nullptr);
+  const bool write_res = (PART || b != nullptr) && (res != nullptr) && (rows == nullptr);
   const int nvec = H / 4;
   float x[VPT][4];
   float ss = 0.f;
@@ -95,7 +97,8 @@ __global__ __launch_bounds__(1024) void add_rms_norm_vec_kernel(
 #pragma unroll
     for (int e = 0; e < 4; ++e) x[k][e] = 0.f;
     if (v < nvec) {
-      if (b) Vec4<TB>::load(b + v * 4, x[k]);
+      if (PART) partial_sum_value4(partial, (int)src, v * 4, x[k]);
+      else if (b) Vec4<TB>::load(b + v * 4, x[k]);
       if (res) {
         float y[4];
         Vec4<float>::load(res + v * 4, y);
@@ -126,6 +129,7 @@ __global__ __launch_bounds__(1024) void add_rms_norm_vec_kernel(
 template <typename TB, typename TO, typename TW>
 static void launch_norm(const void* branch, float* residual, const void* weight, void* out, const int* rows,
                         int n_out, int H, float eps, float woff, hipStream_t stream) {
+  const LmsfPartialSum none = {nullptr, nullptr, 0, 0, 0};
   const bool aligned = (branch == nullptr || (((uintptr_t)branch) & 15u) == 0) &&
                        (residual == nullptr || (((uintptr_t)residual) & 15u) == 0) &&
                        (((uintptr_t)weight) & 15u) == 0 && (((uintptr_t)out) & 15u) == 0;
@@ -136,8 +140,8 @@ static void launch_norm(const void* branch, float* residual, const void* weight,
     // few vectors per thread also for short rows: at most 256 threads while one vector each suffices
     const int vpt = (nvec + threads - 1) / threads;
 #define NORM_VEC(V)                                                                                          \
-  hipLaunchKernelGGL((add_rms_norm_vec_kernel<TB, TO, TW, V>), dim3(n_out), dim3(threads), 0, stream,         \
-                     (const TB*)branch, residual, (const TW*)weight, (TO*)out, rows, H, eps, woff)
+  hipLaunchKernelGGL((add_rms_norm_vec_kernel<TB, TO, TW, V, false>), dim3(n_out), dim3(threads), 0, stream,  \
+                     (const TB*)branch, residual, (const TW*)weight, (TO*)out, rows, H, eps, woff, none)
     if (vpt <= 1) NORM_VEC(1);
     else if (vpt == 2) NORM_VEC(2);
     else if (vpt == 3) NORM_VEC(3);
@@ -178,5 +182,53 @@ extern "C" int lmsf_add_rms_norm(const void* branch, int branch_dtype, float* re
     default: launch_norm<bf16_t, bf16_t, bf16_t>(branch, residual, weight, out, rows, n_out, H, eps, weight_offset, stream); break;
   }
   LMSF_LAUNCH_CHECK("add_rms_norm");
+  return 0;
+}
+
+template <typename TO, typename TW>
+static void launch_norm_partial(const LmsfPartialSum& ps, float* residual, const void* weight, void* out,
+                                const int* rows, int n_out, int H, float eps, float woff, hipStream_t stream) {
+  const int nvec = H / 4;
+  int threads = (nvec + 63) / 64 * 64;
+  if (threads > 1024) threads = 1024;
+  const int vpt = (nvec + threads - 1) / threads;
+#define NORM_PART(V)                                                                                              \
+  hipLaunchKernelGGL((add_rms_norm_vec_kernel<bf16_t, TO, TW, V, true>), dim3(n_out), dim3(threads), 0, stream,   \
+                     (const bf16_t*)nullptr, residual, (const TW*)weight, (TO*)out, rows, H, eps, woff, ps)
+  if (vpt <= 1) NORM_PART(1);
+  else if (vpt == 2) NORM_PART(2);
+  else if (vpt == 3) NORM_PART(3);
+  else NORM_PART(4);
+#undef NORM_PART
+}
+
+// The same with the branch given as the partial sums of a bfloat16 product [M, H] whose K was split
+// (lmsf_gemm_mid_partial): the reduction, the addition and the norm in one kernel. part: float32
+// [n_split, M, H]; bias bfloat16 [H] or null. residual [M, H] float32 or null; rows as above, entries < M.
+// Needs H a multiple of 4 and at most 16,384 and 16-byte aligned operands.
+extern "C" int lmsf_add_rms_norm_partial(const float* part, const void* bias, int n_split, int M, float* residual,
+                                         const void* weight, int weight_dtype, void* out, int out_dtype,
+                                         const int* rows, int n_out, int H, float eps, float weight_offset,
+                                         hipStream_t stream) {
+  LMSF_CHECK(part != nullptr && weight != nullptr && out != nullptr, "add_rms_norm_partial: null pointer");
+  LMSF_CHECK(n_split >= 1 && M >= 0 && n_out >= 0 && (rows != nullptr || n_out <= M),
+             "add_rms_norm_partial: bad sizes splits=%d M=%d n_out=%d", n_split, M, n_out);
+  LMSF_CHECK(H > 0 && H % 4 == 0 && H <= 16384, "add_rms_norm_partial: H=%d must be a multiple of 4 up to 16384", H);
+  LMSF_CHECK(eps > 0.f, "add_rms_norm_partial: eps must be > 0");
+  LMSF_CHECK((weight_dtype == LMSF_F32 || weight_dtype == LMSF_BF16) && (out_dtype == LMSF_F32 || out_dtype == LMSF_BF16),
+             "add_rms_norm_partial: unknown dtype code");
+  LMSF_CHECK(lmsf_aligned16(part) && lmsf_aligned16(weight) && lmsf_aligned16(out) &&
+                 (residual == nullptr || lmsf_aligned16(residual)) && (bias == nullptr || (((uintptr_t)bias) & 7u) == 0),
+             "add_rms_norm_partial: operands must be 16-byte aligned");
+  if (n_out == 0) return 0;
+  const LmsfPartialSum ps = {part, (const bf16_t*)bias, n_split, M, H};
+  const int key = out_dtype * 2 + weight_dtype;
+  switch (key) {
+    case 0: launch_norm_partial<float, float>(ps, residual, weight, out, rows, n_out, H, eps, weight_offset, stream); break;
+    case 1: launch_norm_partial<float, bf16_t>(ps, residual, weight, out, rows, n_out, H, eps, weight_offset, stream); break;
+    case 2: launch_norm_partial<bf16_t, float>(ps, residual, weight, out, rows, n_out, H, eps, weight_offset, stream); break;
+    default: launch_norm_partial<bf16_t, bf16_t>(ps, residual, weight, out, rows, n_out, H, eps, weight_offset, stream); break;
+  }
+  LMSF_LAUNCH_CHECK("add_rms_norm_partial");
   return 0;
 }

@@ -21,29 +21,39 @@
 // One wave per (token, head): heads 0 .. nh-1 are q heads, then nkv k heads, then nkv v heads (a decode step
 // has few tokens, so the parallelism has to come from the heads); a workgroup holds the waves of
 // blockDim.y consecutive tokens of one head.
-template <typename T>
+// PART: the values come from the partial sums of the fused QKV product (column (head index) * d + i of row
+// t) and q, k, v are only written: the reduction, the rotation and the cache write in one kernel.
+template <typename T, bool PART>
 __global__ __launch_bounds__(256) void rope_cache_write_kernel(
-    T* __restrict__ q, T* __restrict__ k, const T* __restrict__ v, long row_stride, const int* __restrict__ positions,
+    T* __restrict__ q, T* __restrict__ k, T* __restrict__ v, long row_stride, const int* __restrict__ positions,
     const float* __restrict__ table, int rot, int neox, const int* __restrict__ slots, T* __restrict__ k_pages,
-    T* __restrict__ v_pages, int nh, int nkv, int d, int ps, int n_tokens) {
+    T* __restrict__ v_pages, int nh, int nkv, int d, int ps, int n_tokens, LmsfPartialSum partial) {
   const long t = (long)blockIdx.x * blockDim.y + threadIdx.y;
   if (t >= n_tokens) return;
   const int hy = blockIdx.y;
   const int half = rot / 2;
+  const int col0 = hy * d;
+  auto rd = [&](const T* x, int i) -> float {
+    return PART ? partial_sum_value(partial, (int)t, col0 + i) : to_f32<T>(x[i]);
+  };
   const float* cs = table ? table + (long)positions[t] * rot : nullptr;
   int slot = -1;
   if (slots) slot = slots[t];
   if (hy < nh) {
-    if (!cs || !q) return;
+    if (!q || (!cs && !PART)) return;
     T* x = q + t * row_stride + (long)hy * d;
-    for (int i = threadIdx.x; i < half; i += 64) {
-      const int xi = neox ? i : 2 * i, yi = neox ? i + half : 2 * i + 1;
-      const float c = cs[i], s = cs[half + i];
-      float xr, yr;
-      rope_rotate(to_f32<T>(x[xi]), to_f32<T>(x[yi]), c, s, &xr, &yr);
-      x[xi] = from_f32<T>(xr);
-      x[yi] = from_f32<T>(yr);
+    if (cs) {
+      for (int i = threadIdx.x; i < half; i += 64) {
+        const int xi = neox ? i : 2 * i, yi = neox ? i + half : 2 * i + 1;
+        const float c = cs[i], s = cs[half + i];
+        float xr, yr;
+        rope_rotate(rd(x, xi), rd(x, yi), c, s, &xr, &yr);
+        x[xi] = from_f32<T>(xr);
+        x[yi] = from_f32<T>(yr);
+      }
     }
+    if (PART)
+      for (int i = (cs ? rot : 0) + threadIdx.x; i < d; i += 64) x[i] = from_f32<T>(rd(x, i));
   } else if (hy < nh + nkv) {
     if (!k) return;
     const int h = hy - nh;
@@ -55,7 +65,7 @@ __global__ __launch_bounds__(256) void rope_cache_write_kernel(
         const int xi = neox ? i : 2 * i, yi = neox ? i + half : 2 * i + 1;
         const float c = cs[i], s = cs[half + i];
         float xf, yf;
-        rope_rotate(to_f32<T>(x[xi]), to_f32<T>(x[yi]), c, s, &xf, &yf);
+        rope_rotate(rd(x, xi), rd(x, yi), c, s, &xf, &yf);
         const T xr = from_f32<T>(xf), yr = from_f32<T>(yf);
         x[xi] = xr;
         x[yi] = yr;
@@ -65,50 +75,93 @@ __global__ __launch_bounds__(256) void rope_cache_write_kernel(
         }
       }
     }
-    if (dst) {
+    if (dst || PART) {
       // the part of k that the rotation did not touch (all of it without a table)
-      for (int i = (cs ? rot : 0) + threadIdx.x; i < d; i += 64) dst[i] = x[i];
+      for (int i = (cs ? rot : 0) + threadIdx.x; i < d; i += 64) {
+        const T val = PART ? from_f32<T>(rd(x, i)) : x[i];
+        if (PART) x[i] = val;
+        if (dst) dst[i] = val;
+      }
     }
   } else {
-    if (!v || slot < 0) return;
+    if (!v || (slot < 0 && !PART)) return;
     const int h = hy - nh - nkv;
-    const T* x = v + t * row_stride + (long)h * d;
+    T* x = v + t * row_stride + (long)h * d;
     // element offset of (page, head h, 0, offset) in the transposed V pages
-    T* dst = v_pages + ((long)(slot / ps) * nkv + h) * ps * d + (slot % ps);
-    for (int i = threadIdx.x; i < d; i += 64) dst[(long)i * ps] = x[i];
+    T* dst = slot >= 0 ? v_pages + ((long)(slot / ps) * nkv + h) * ps * d + (slot % ps) : nullptr;
+    for (int i = threadIdx.x; i < d; i += 64) {
+      const T val = PART ? from_f32<T>(rd(x, i)) : x[i];
+      if (PART) x[i] = val;
+      if (dst) dst[(long)i * ps] = val;
+    }
   }
 }
 
-extern "C" int lmsf_rope_cache_write(void* q, void* k, const void* v, int dtype, int n_tokens, long row_stride,
+static int rope_cache_check(const char* who, const void* k, const void* v, int n_tokens, long row_stride,
+                            const int* positions, const float* table, int rot, int max_pos, const int* slots,
+                            const void* k_pages, const void* v_pages, long num_pages, int nh, int nkv, int d, int ps) {
+  LMSF_CHECK(n_tokens >= 0 && nh >= 0 && nkv >= 0 && d > 0, "%s: bad sizes", who);
+  LMSF_CHECK(row_stride >= 0, "%s: bad row stride", who);
+  if (table) {
+    LMSF_CHECK(positions != nullptr, "%s: rotation needs positions", who);
+    LMSF_CHECK(rot > 0 && rot % 2 == 0 && rot <= d, "%s: rotary_dim %d must be even and <= head_dim %d", who, rot, d);
+    LMSF_CHECK(max_pos > 0, "%s: empty table", who);
+  }
+  if (slots) {
+    LMSF_CHECK(k && v && k_pages && v_pages, "%s: cache write needs k, v and both page tensors", who);
+    LMSF_CHECK(ps > 0 && num_pages > 0, "%s: bad page geometry", who);
+  }
+  const int heads = nh + 2 * nkv;
+  LMSF_CHECK(heads > 0 && heads <= 65535, "%s: %d heads do not fit the grid", who, heads);
+  return 0;
+}
+
+extern "C" int lmsf_rope_cache_write(void* q, void* k, void* v, int dtype, int n_tokens, long row_stride,
                                      const int* positions, const float* table, int rot, int neox, int max_pos,
                                      const int* slots, void* k_pages, void* v_pages, long num_pages, int nh, int nkv,
                                      int d, int ps, hipStream_t stream) {
   LMSF_CHECK(dtype == LMSF_F32 || dtype == LMSF_BF16, "rope_cache_write: unknown dtype code %d", dtype);
-  LMSF_CHECK(n_tokens >= 0 && nh >= 0 && nkv >= 0 && d > 0, "rope_cache_write: bad sizes");
-  LMSF_CHECK(row_stride >= 0, "rope_cache_write: bad row stride");
-  if (table) {
-    LMSF_CHECK(positions != nullptr, "rope_cache_write: rotation needs positions");
-    LMSF_CHECK(rot > 0 && rot % 2 == 0 && rot <= d, "rope_cache_write: rotary_dim %d must be even and <= head_dim %d",
-               rot, d);
-    LMSF_CHECK(max_pos > 0, "rope_cache_write: empty table");
-  }
-  if (slots) {
-    LMSF_CHECK(k && v && k_pages && v_pages, "rope_cache_write: cache write needs k, v and both page tensors");
-    LMSF_CHECK(ps > 0 && num_pages > 0, "rope_cache_write: bad page geometry");
-  }
+  if (int rc = rope_cache_check("rope_cache_write", k, v, n_tokens, row_stride, positions, table, rot, max_pos, slots,
+                                k_pages, v_pages, num_pages, nh, nkv, d, ps))
+    return rc;
   if (n_tokens == 0) return 0;
   const int heads = nh + 2 * nkv;
-  LMSF_CHECK(heads > 0 && heads <= 65535, "rope_cache_write: %d heads do not fit the grid", heads);
+  const LmsfPartialSum none = {nullptr, nullptr, 0, 0, 0};
   const int per_block = n_tokens >= 64 ? 4 : 1;   // tokens per workgroup: many small workgroups cost a long prompt time
   dim3 grid((n_tokens + per_block - 1) / per_block, heads), block(64, per_block);
   if (dtype == LMSF_F32)
-    hipLaunchKernelGGL((rope_cache_write_kernel<float>), grid, block, 0, stream, (float*)q, (float*)k,
-                       (const float*)v, row_stride, positions, table, rot, neox, slots, (float*)k_pages,
-                       (float*)v_pages, nh, nkv, d, ps, n_tokens);
+    hipLaunchKernelGGL((rope_cache_write_kernel<float, false>), grid, block, 0, stream, (float*)q, (float*)k,
+                       (float*)v, row_stride, positions, table, rot, neox, slots, (float*)k_pages,
+                       (float*)v_pages, nh, nkv, d, ps, n_tokens, none);
   else
-    hipLaunchKernelGGL((rope_cache_write_kernel<bf16_t>), grid, block, 0, stream, (bf16_t*)q,
-                       (bf16_t*)k, (const bf16_t*)v, row_stride, positions, table, rot, neox, slots, (bf16_t*)k_pages,
-                       (bf16_t*)v_pages, nh, nkv, d, ps, n_tokens);
+    hipLaunchKernelGGL((rope_cache_write_kernel<bf16_t, false>), grid, block, 0, stream, (bf16_t*)q,
+                       (bf16_t*)k, (bf16_t*)v, row_stride, positions, table, rot, neox, slots, (bf16_t*)k_pages,
+                       (bf16_t*)v_pages, nh, nkv, d, ps, n_tokens, none);
   LMSF_LAUNCH_CHECK("rope_cache_write");
+  return 0;
+}
+
+// The same for a fused QKV product that was left as partial sums (lmsf_gemm_mid_partial with
+// N = (nh + 2 nkv) * d): part float32 [n_split, n_tokens, N], bias bfloat16 [N] or null. y [n_tokens, N]
+// bfloat16 (row stride ldy) receives the rotated q and k and v; the cache receives k and v.
+extern "C" int lmsf_rope_cache_write_partial(const float* part, const void* bias, int n_split, void* y, long ldy,
+                                             int n_tokens, const int* positions, const float* table, int rot,
+                                             int neox, int max_pos, const int* slots, void* k_pages, void* v_pages,
+                                             long num_pages, int nh, int nkv, int d, int ps, hipStream_t stream) {
+  LMSF_CHECK(part != nullptr && y != nullptr && n_split >= 1, "rope_cache_write_partial: bad arguments");
+  const long N = (long)(nh + 2 * nkv) * d;
+  LMSF_CHECK(ldy >= N && N <= 2147483647L, "rope_cache_write_partial: row stride %ld below %ld columns", ldy, N);
+  if (int rc = rope_cache_check("rope_cache_write_partial", y, y, n_tokens, ldy, positions, table, rot, max_pos, slots,
+                                k_pages, v_pages, num_pages, nh, nkv, d, ps))
+    return rc;
+  if (n_tokens == 0) return 0;
+  const LmsfPartialSum ps_ = {part, (const bf16_t*)bias, n_split, n_tokens, (int)N};
+  bf16_t* yb = (bf16_t*)y;
+  const int per_block = n_tokens >= 64 ? 4 : 1;
+  dim3 grid((n_tokens + per_block - 1) / per_block, nh + 2 * nkv), block(64, per_block);
+  hipLaunchKernelGGL((rope_cache_write_kernel<bf16_t, true>), grid, block, 0, stream, yb, yb + (long)nh * d,
+                     yb + (long)(nh + nkv) * d, ldy, positions, table, rot, neox, slots, (bf16_t*)k_pages,
+                     (bf16_t*)v_pages, nh, nkv, d, ps, n_tokens, ps_);
+  LMSF_LAUNCH_CHECK("rope_cache_write_partial");
   return 0;
 }

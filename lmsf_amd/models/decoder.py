@@ -43,6 +43,11 @@ class DecoderModel:
                     raise ValueError("schedule entry %d cannot read the cache of entry %d: cache shapes differ"
                                      % (i, e.cache_from))
         self.bindings: List[CacheBinding] = [CacheBinding() for _ in self.schedule]
+        # a block may return an unfinished product where everything that ever receives it can take one
+        takes = [self.blocks[e.layer].accepts_pending_branch for e in self.schedule[1:]] + [self.final_norm.accepts_pending]
+        for li, b in enumerate(self.blocks):
+            after = [t for e, t in zip(self.schedule, takes) if e.layer == li]
+            b.pending_output_ok = bool(after) and all(after)
 
     # ------------------------------------------------------------------ structure
 

@@ -11,6 +11,7 @@ from typing import Optional
 import torch
 
 from . import library
+from .handles import PendingProduct
 
 F32 = 0
 BF16 = 1
@@ -110,7 +111,10 @@ class HipOps:
 
         ``residual`` (float32 [N, H]) is updated to the sum in place when both operands are given
         and ``rows`` is None. ``rows`` (int32 [R]) selects input rows; the output then has R rows.
+        ``branch`` may be a ``PendingProduct``: its partial sums are added up on the way in.
         """
+        if isinstance(branch, PendingProduct):
+            return self._add_rms_norm_pending(branch, residual, weight, eps, out_dtype, rows, weight_offset)
         self._dev(branch, residual, weight, rows)
         ref = branch if branch is not None else residual
         if ref is None:
@@ -131,6 +135,36 @@ class HipOps:
             _ptr(branch), _code(branch.dtype) if branch is not None else F32, _ptr(residual), _ptr(weight),
             _code(weight.dtype), _ptr(out), _code(out_dtype), _ptr(rows), n_out, H, float(eps),
             float(weight_offset), self._stream()))
+        return out
+
+    def _add_rms_norm_pending(self, branch: PendingProduct, residual: Optional[torch.Tensor], weight: torch.Tensor,
+                              eps: float, out_dtype: torch.dtype, rows: Optional[torch.Tensor],
+                              weight_offset: float) -> torch.Tensor:
+        M, H = branch.shape
+        fits = (H % 4 == 0 and H <= 16384 and weight.shape == (H,) and weight.is_contiguous()
+                and weight.data_ptr() % 16 == 0
+                and (residual is None or (residual.dtype == torch.float32 and residual.is_contiguous()
+                                          and tuple(residual.shape) == (M, H) and residual.data_ptr() % 16 == 0)))
+        if not fits:
+            return self.add_rms_norm(self.materialize(branch), residual, weight, eps, out_dtype, rows, weight_offset)
+        self._dev(residual, weight, rows)
+        self._i32(rows, "rows")
+        n_out = M if rows is None else rows.numel()
+        out = torch.empty((n_out, H), dtype=out_dtype, device=branch.device)
+        self._check(self.lib.lmsf_add_rms_norm_partial(
+            _ptr(branch.partials), _ptr(branch.bias), branch.partials.shape[0], M, _ptr(residual), _ptr(weight),
+            _code(weight.dtype), _ptr(out), _code(out_dtype), _ptr(rows), n_out, H, float(eps), float(weight_offset),
+            self._stream()))
+        return out
+
+    def materialize(self, y):
+        """The tensor behind ``y``: ``y`` itself, or the finished sum of a ``PendingProduct``."""
+        if not isinstance(y, PendingProduct):
+            return y
+        M, N = y.shape
+        out = torch.empty((M, N), dtype=y.dtype, device=y.device)
+        self._check(self.lib.lmsf_gemm_mid_reduce(_ptr(y.partials), _ptr(y.bias), _ptr(out), _code(y.dtype),
+                                                  out.stride(0), M, N, y.partials.shape[0], self._stream()))
         return out
 
     # ------------------------------------------------------------------ rotary + cache write
@@ -204,9 +238,46 @@ class HipOps:
                 _ptr(positions), _ptr(table), table.shape[0], _ptr(slots), _ptr(k_pages), _ptr(v_pages), num_pages,
                 nh, nkv, d, ps, self.skinny_variant, self._stream()))
             return y
-        y = self.linear(x, weight, bias)
+        y = self.linear(x, weight, bias, pending_ok=True)
+        if isinstance(y, PendingProduct):
+            # 17 to 64 rows with K split: the rotation and the cache write add up the partial sums themselves
+            if (table is None and slots is None) or tuple(weight.shape) != (N, K):
+                return self.materialize(y)
+            return self._rope_cache_write_pending(y, nh, nkv, d, positions, table, rot_dim, neox, slots, k_pages,
+                                                  v_pages)
         if table is not None or slots is not None:
             self.rope_cache_write(y, nh, nkv, d, positions, table, rot_dim, neox, slots, k_pages, v_pages)
+        return y
+
+    def _rope_cache_write_pending(self, p: PendingProduct, nh: int, nkv: int, d: int,
+                                  positions: Optional[torch.Tensor], table: Optional[torch.Tensor], rot_dim: int,
+                                  neox: bool, slots: Optional[torch.Tensor], k_pages: Optional[torch.Tensor],
+                                  v_pages: Optional[torch.Tensor]) -> torch.Tensor:
+        M, N = p.shape
+        y = torch.empty((M, N), dtype=torch.bfloat16, device=p.device)
+        self._dev(positions, table, slots, k_pages, v_pages)
+        max_pos = 0
+        if table is not None:
+            if table.dtype != torch.float32 or table.dim() != 2 or table.shape[1] != rot_dim or not table.is_contiguous():
+                raise ValueError("rotary table must be contiguous float32 [max_pos, %d]" % rot_dim)
+            if positions is None:
+                raise ValueError("rotation needs positions")
+            self._i32(positions, "positions", M)
+            max_pos = table.shape[0]
+        num_pages, ps = 0, 1
+        if slots is not None:
+            self._i32(slots, "slots", M)
+            if k_pages is None or k_pages.dim() != 4 or k_pages.shape[1] != nkv or k_pages.shape[3] != d \
+                    or not k_pages.is_contiguous() or k_pages.dtype != torch.bfloat16:
+                raise ValueError("k_pages must be contiguous bfloat16 [pages, %d, page_size, %d]" % (nkv, d))
+            num_pages, ps = k_pages.shape[0], k_pages.shape[2]
+            if v_pages is None or tuple(v_pages.shape) != (num_pages, nkv, d, ps) or not v_pages.is_contiguous() \
+                    or v_pages.dtype != torch.bfloat16:
+                raise ValueError("v_pages must be contiguous bfloat16 [%d, %d, %d, %d]" % (num_pages, nkv, d, ps))
+        self._check(self.lib.lmsf_rope_cache_write_partial(
+            _ptr(p.partials), _ptr(p.bias), p.partials.shape[0], _ptr(y), y.stride(0), M, _ptr(positions), _ptr(table),
+            rot_dim, 1 if neox else 0, max_pos, _ptr(slots), _ptr(k_pages), _ptr(v_pages), num_pages, nh, nkv, d, ps,
+            self._stream()))
         return y
 
     # ------------------------------------------------------------------ attention
@@ -341,8 +412,10 @@ class HipOps:
     # ------------------------------------------------------------------ matrix products
 
     def linear(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
-               out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+               out_dtype: Optional[torch.dtype] = None, pending_ok: bool = False):
         """y = x weight^T (+ bias); x [M, K], weight [N, K]; y [M, N] in ``out_dtype`` (default x's).
+        With ``pending_ok`` the caller takes a ``PendingProduct`` as well, which comes back where the
+        product splits K over workgroups (17 to 64 rows, few columns).
 
         float32 operands always run the float32 multiply-add kernel. bfloat16 products with bfloat16
         output and many rows go to the BLAS library, as the reference's do
@@ -360,7 +433,7 @@ class HipOps:
         out_dtype = out_dtype or x.dtype
         both_bf16 = x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
         if both_bf16 and self.skinny_max_rows < M <= 64 and self._mid_ok(x, weight):
-            return self._linear_mid(x, weight, bias, 0, out_dtype)
+            return self._linear_mid(x, weight, bias, 0, out_dtype, pending_ok and out_dtype == torch.bfloat16)
         if both_bf16 and self._skinny_ok(x, weight):
             # few rows: the weight-streaming kernel. It also serves float32 output (logits), which the
             # library does not offer, for any number of rows, 64 at a time.
@@ -422,7 +495,7 @@ class HipOps:
                 and weight.data_ptr() % 16 == 0)
 
     def _linear_mid(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], act: int,
-                    out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+                    out_dtype: torch.dtype = torch.bfloat16, pending_ok: bool = False):
         self._dev(x, weight, bias)
         M, K = x.shape
         N = weight.shape[0] // 2 if act else weight.shape[0]
@@ -430,6 +503,11 @@ class HipOps:
                                  or not bias.is_contiguous()):
             raise ValueError("linear: bias must be [%d] of the weight's dtype" % weight.shape[0])
         splits = self.lib.lmsf_gemm_mid_splits(M, N, K, act)
+        if pending_ok and act == 0 and splits > 1:
+            partials = torch.empty((splits, M, N), dtype=torch.float32, device=x.device)
+            self._check(self.lib.lmsf_gemm_mid_partial(_ptr(x), x.stride(0), _ptr(weight), weight.stride(0), M, N, K,
+                                                       splits, _ptr(partials), self._stream()))
+            return PendingProduct(partials, bias, out_dtype)
         floats = self.lib.lmsf_gemm_mid_scratch_floats(M, N, splits, act)
         scratch = torch.empty(floats, dtype=torch.float32, device=x.device) if floats else None
         y = torch.empty((M, N), dtype=out_dtype, device=x.device)

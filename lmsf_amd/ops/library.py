@@ -9,7 +9,7 @@ from typing import Optional
 
 from ..csrc import build as _build
 
-ABI_VERSION = 11
+ABI_VERSION = 12
 
 _lib: Optional[ctypes.CDLL] = None
 _lib_path: Optional[str] = None
@@ -44,6 +44,12 @@ _SIGNATURES = {
     "lmsf_gemm_mid_splits": (c_int, [c_int, c_int, c_int, c_int]),
     "lmsf_gemm_mid_scratch_floats": (c_long, [c_int, c_int, c_int, c_int]),
     "lmsf_gemm_mid": (c_int, [_P, c_long, _P, c_long, _P, _P, c_int, c_long, c_int, c_int, c_int, c_int, c_int, _P, _P]),
+    "lmsf_gemm_mid_partial": (c_int, [_P, c_long, _P, c_long, c_int, c_int, c_int, c_int, _P, _P]),
+    "lmsf_gemm_mid_reduce": (c_int, [_P, _P, _P, c_int, c_long, c_int, c_int, c_int, _P]),
+    "lmsf_add_rms_norm_partial": (c_int, [_P, _P, c_int, c_int, _P, _P, c_int, _P, c_int, _P, c_int, c_int, c_float,
+                                          c_float, _P]),
+    "lmsf_rope_cache_write_partial": (c_int, [_P, _P, c_int, _P, c_long, c_int, _P, _P, c_int, c_int, c_int, _P, _P, _P,
+                                              c_long, c_int, c_int, c_int, c_int, _P]),
     "lmsf_sample": (c_int, [_P, c_long, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, _P, _P]),
     "lmsf_sample_scratch_elems": (c_long, [c_int, c_int]),
     "lmsf_apply_penalties": (c_int, [_P, c_long, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, _P]),

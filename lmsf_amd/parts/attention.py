@@ -48,7 +48,9 @@ class PagedAttention(Mixer):
     def cache_spec(self) -> Optional[CacheSpec]:
         return CacheSpec(num_kv_heads=self.nkv, head_dim=self.d, window=self.window)
 
-    def forward(self, h: torch.Tensor, ctx, binding: CacheBinding) -> torch.Tensor:
+    may_return_pending = True
+
+    def forward(self, h: torch.Tensor, ctx, binding: CacheBinding, pending_ok: bool = False):
         ops = self.rt.ops
         group = ctx.groups[binding.group]
         slots = group.slots if binding.writes_cache else None
@@ -65,4 +67,4 @@ class PagedAttention(Mixer):
                                      table, rot, neox, slots, binding.k_pages, binding.v_pages)
         a = ops.paged_attention(qkv, binding.k_pages, binding.v_pages, group.block_tables, ctx.seg_of_token,
                                 ctx.positions, self.nh, self.nkv, self.d, self.scale, self.window or 0, batch=ctx)
-        return self.o.forward(a)
+        return self.o.forward(a, pending_ok=pending_ok)

@@ -132,6 +132,13 @@ class Part:
 
     graph_safe = False
 
+    # A mixer or feed-forward whose ``forward`` takes ``pending_ok=True`` and may then return its last
+    # product unfinished (ops.handles.PendingProduct) sets this; a norm that takes such a branch in
+    # ``forward_add`` sets ``accepts_pending``. A block hands a pending product only to a norm that accepts
+    # it; ``rt.ops.materialize`` finishes one anywhere else. Parts that know nothing of this never see one.
+    may_return_pending = False
+    accepts_pending = False
+
     def __init__(self, prefix: str, rt: Runtime):
         self.prefix = prefix
         self.rt = rt
@@ -206,6 +213,15 @@ class Block(Part):
     so that the addition fuses with the next norm."""
 
     ROLES: Tuple[str, ...] = ()   # names of the norms this arrangement needs
+
+    # Set by the model where whatever receives this block's returned branch (the next block's first norm,
+    # the final norm) accepts a pending product; a block that does not look at it always returns a tensor.
+    pending_output_ok = False
+
+    @property
+    def accepts_pending_branch(self) -> bool:
+        """Whether the ``branch`` argument of ``forward`` may be a pending product."""
+        return False
 
     def __init__(self, prefix: str, rt: Runtime, mixer: Mixer, feed_forward: FeedForward, norms: Dict[str, Norm]):
         super().__init__(prefix, rt)

@@ -13,15 +13,27 @@ class PreNormResidualBlock(Block):
     core/src/model_executor/models/llama/llama.rs:286-340. As there, an addition is carried out by
     the norm that follows it (vllm/kernels/layernorm_kernels.cu:41-68): the block receives the
     previous block's output not yet added, and returns its feed-forward output not yet added.
+    Where the norm that follows accepts it, the o and down products may stay unfinished
+    (``PendingProduct``) and the norm's kernel adds up their partial sums.
     """
 
     graph_safe = True
 
     ROLES = ("input", "post_mixer")
 
+    @property
+    def accepts_pending_branch(self) -> bool:
+        return self.norms["input"].accepts_pending
+
     def forward(self, branch: Optional[torch.Tensor], residual: torch.Tensor, ctx,
                 binding: CacheBinding) -> torch.Tensor:
+        post = self.norms["post_mixer"]
         h = self.norms["input"].forward_add(branch, residual)
-        a = self.mixer.forward(h, ctx, binding)
-        h = self.norms["post_mixer"].forward_add(a, residual)
+        if self.mixer.may_return_pending and post.accepts_pending:
+            a = self.mixer.forward(h, ctx, binding, pending_ok=True)
+        else:
+            a = self.mixer.forward(h, ctx, binding)
+        h = post.forward_add(a, residual)
+        if self.feed_forward.may_return_pending and self.pending_output_ok:
+            return self.feed_forward.forward(h, pending_ok=True)
         return self.feed_forward.forward(h)

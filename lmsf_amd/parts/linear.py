@@ -57,7 +57,9 @@ class FusedLinear(Part):
             b = self._cat([fetch(self._name(sub, "bias")) for sub, _ in self.sources])
             self.bias = b.to(self.weight.dtype)
 
-    def forward(self, x: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, out_dtype: Optional[torch.dtype] = None, pending_ok: bool = False):
+        if pending_ok:
+            return self.rt.ops.linear(x, self.weight, self.bias, out_dtype=out_dtype, pending_ok=True)
         return self.rt.ops.linear(x, self.weight, self.bias, out_dtype=out_dtype)
 
 

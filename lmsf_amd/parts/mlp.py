@@ -29,6 +29,8 @@ class GatedMLP(FeedForward):
     def children(self):
         return [self.gate_up, self.down]
 
-    def forward(self, h: torch.Tensor) -> torch.Tensor:
+    may_return_pending = True
+
+    def forward(self, h: torch.Tensor, pending_ok: bool = False):
         a = self.rt.ops.linear_gated(h, self.gate_up.weight, self.gate_up.bias, self.activation)
-        return self.down.forward(a)
+        return self.down.forward(a, pending_ok=pending_ok)

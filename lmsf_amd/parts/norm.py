@@ -15,6 +15,7 @@ from .base import Norm, Runtime, TensorDecl, register_part
 @register_part("norm", "rms_norm")
 class RMSNorm(Norm):
     graph_safe = True
+    accepts_pending = True
 
     def __init__(self, prefix: str, rt: Runtime, size: int, eps: float, weight_offset: float = 0.0,
                  weight_name: str = "weight"):

@@ -29,7 +29,15 @@ TINY_C = dict(
     rope_theta=1000.0, rope_scaling=None, max_position_embeddings=256, tie_word_embeddings=False,
     attention_bias=False, mlp_bias=True, hidden_act="silu", torch_dtype="float32", bos_token_id=1, eos_token_id=2)
 
-TINY = {"A": (TINY_A, 0, 8), "B": (TINY_B, 1, 16), "C": (TINY_C, 2, 16)}   # config, seed, block size
+# A wide one: with 17 to 64 tokens in a step its products split K over workgroups and the engine leaves them
+# as partial sums for the next kernel, which the narrow configurations never reach.
+TINY_W = dict(
+    architectures=["LlamaForCausalLM"], model_type="llama", vocab_size=520, hidden_size=1024, intermediate_size=2048,
+    num_hidden_layers=2, num_attention_heads=8, num_key_value_heads=2, head_dim=128, rms_norm_eps=1e-5,
+    rope_theta=10000.0, rope_scaling=None, max_position_embeddings=256, tie_word_embeddings=False,
+    attention_bias=True, hidden_act="silu", torch_dtype="float32", bos_token_id=1, eos_token_id=2)
+
+TINY = {"A": (TINY_A, 0, 8), "B": (TINY_B, 1, 16), "C": (TINY_C, 2, 16), "W": (TINY_W, 3, 16)}   # config, seed, block size
 
 
 def make_model_folder(tmp_path, which, dtype="float32", seed=None):

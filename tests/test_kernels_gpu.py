@@ -362,6 +362,77 @@ def test_qkv_rope_cache_fused_equals_the_three_steps(ops, ref, M, H, nh, nkv, d,
     assert (a.float() - c.float()).abs().max().item() <= 2e-2 * scale and (k4.float() - k5.float()).abs().max().item() <= 2e-2 * scale
 
 
+@pytest.mark.parametrize("M,N,K", [(17, 256, 1024), (40, 4096, 4096), (64, 80, 1280), (33, 1000, 2048)])
+@pytest.mark.parametrize("bias", [False, True])
+def test_unfinished_product_is_finished_by_the_norm(ops, ref, M, N, K, bias):
+    """A product of 17 to 64 rows whose K is split may stay as partial sums; the norm that takes it as its
+    branch adds them up. The bits are those of product, then addition and norm, and the plain formulas hold."""
+    from lmsf_amd.ops.handles import PendingProduct
+    g = torch.Generator().manual_seed(M + N + K)
+    x = dev(torch.randn(M, K, generator=g).bfloat16())
+    w = dev((torch.randn(N, K, generator=g) * K ** -0.5).bfloat16())
+    b = dev(torch.randn(N, generator=g).bfloat16()) if bias else None
+    p = ops.linear(x, w, b, pending_ok=True)
+    assert isinstance(p, PendingProduct) and p.shape == (M, N) and p.partials.shape[0] >= 2
+    y = ops.linear(x, w, b)
+    assert torch.equal(ops.materialize(p), y) and ops.materialize(y) is y
+    nw = dev(torch.randn(N, generator=g).bfloat16())
+    res0 = dev(torch.randn(M, N, generator=g))
+    for out_dtype, weight in ((torch.bfloat16, nw), (torch.float32, nw.float())):
+        r1, r2 = res0.clone(), res0.clone()
+        a = ops.add_rms_norm(p, r1, weight, 1e-5, out_dtype, weight_offset=0.25)
+        c = ops.add_rms_norm(y, r2, weight, 1e-5, out_dtype, weight_offset=0.25)
+        assert torch.equal(a, c) and torch.equal(r1, r2) and not torch.equal(r1, res0)
+        want = ref.add_rms_norm(y, res0.clone(), weight, 1e-5, torch.float32, weight_offset=0.25)
+        assert (a.float() - want).abs().max().item() <= 2e-2 * max(1.0, want.abs().max().item())
+    rows = dev(torch.tensor([M - 1, 0, 5], dtype=torch.int32))
+    r1 = res0.clone()
+    a = ops.add_rms_norm(p, r1, nw, 1e-5, torch.bfloat16, rows=rows)
+    c = ops.add_rms_norm(y, res0.clone(), nw, 1e-5, torch.bfloat16, rows=rows)
+    assert torch.equal(a, c) and torch.equal(r1, res0)
+    # without a residual: the norm of the product alone
+    assert torch.equal(ops.add_rms_norm(p, None, nw, 1e-5, torch.bfloat16), ops.add_rms_norm(y, None, nw, 1e-5, torch.bfloat16))
+
+
+@pytest.mark.parametrize("M,H,nh,nkv,d,ps,rot,neox", [(17, 1024, 8, 2, 64, 16, 64, True), (64, 4096, 32, 8, 128, 16, 128, True),
+                                                      (40, 1024, 6, 3, 48, 8, 24, False), (33, 1280, 5, 5, 80, 4, 80, False)])
+@pytest.mark.parametrize("bias", [False, True])
+def test_qkv_rope_cache_from_partial_sums(ops, ref, M, H, nh, nkv, d, ps, rot, neox, bias):
+    """With 17 to 64 rows the QKV product splits K, and the rotation kernel adds up the partial sums before it
+    rotates and stores: the bits are those of product, rotation and cache write one after the other."""
+    g = torch.Generator().manual_seed(M * H + d)
+    N = (nh + 2 * nkv) * d
+    x = dev(torch.randn(M, H, generator=g).bfloat16())
+    w = dev((torch.randn(N, H, generator=g) * H ** -0.5).bfloat16())
+    b = dev(torch.randn(N, generator=g).bfloat16()) if bias else None
+    assert ops.lib.lmsf_gemm_mid_splits(M, N, H, 0) >= 2
+    max_pos, pages = 50, -(-M // ps) + 3
+    pos = dev(torch.randint(0, max_pos, (M,), generator=g, dtype=torch.int32))
+    ang = torch.arange(max_pos, dtype=torch.float32)[:, None] * torch.rand(rot // 2, generator=g)[None, :]
+    table = dev(torch.cat([ang.cos(), ang.sin()], dim=1).contiguous())
+    slots = torch.randperm(pages * ps, generator=g)[:M].to(torch.int32)
+    slots[2] = -1
+    slots = dev(slots)
+    k1, v1 = dev(torch.zeros(pages, nkv, ps, d).bfloat16()), dev(torch.zeros(pages, nkv, d, ps).bfloat16())
+    k2, v2, k3, v3 = k1.clone(), v1.clone(), k1.clone(), v1.clone()
+    fused = ops.qkv_rope_cache(x, w, b, nh, nkv, d, pos, table, rot, neox, slots, k1, v1)
+    steps = ops.linear(x, w, b)
+    ops.rope_cache_write(steps, nh, nkv, d, pos, table, rot, neox, slots, k2, v2)
+    assert torch.equal(fused, steps) and torch.equal(k1, k2) and torch.equal(v1, v2)
+    plain = ref.qkv_rope_cache(x, w, b, nh, nkv, d, pos, table, rot, neox, slots, k3, v3)
+    scale = max(1.0, plain.float().abs().max().item())
+    assert (fused.float() - plain.float()).abs().max().item() <= 2e-2 * scale
+    assert (k1.float() - k3.float()).abs().max().item() <= 2e-2 * scale and (v1.float() - v3.float()).abs().max().item() <= 2e-2 * scale
+    # no rotation and no cache: the product alone
+    assert torch.equal(ops.qkv_rope_cache(x, w, b, nh, nkv, d, pos, None, 0, True, None, None, None), ops.linear(x, w, b))
+    # no rotation, cache write only
+    k4, v4, k5, v5 = k1.clone().zero_(), v1.clone().zero_(), k1.clone().zero_(), v1.clone().zero_()
+    a = ops.qkv_rope_cache(x, w, b, nh, nkv, d, pos, None, 0, True, slots, k4, v4)
+    c = ops.linear(x, w, b)
+    ops.rope_cache_write(c, nh, nkv, d, pos, None, 0, True, slots, k5, v5)
+    assert torch.equal(a, c) and torch.equal(k4, k5) and torch.equal(v4, v5)
+
+
 def test_linear_mixed_storage(ops, ref):
     """A weight stored in 32 bits stays so and still multiplies bfloat16 activations."""
     g = torch.Generator().manual_seed(5)

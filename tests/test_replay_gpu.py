@@ -53,7 +53,8 @@ def models(tmp_path_factory):
 def requests_for(cfg, which):
     V = cfg["vocab_size"]
     top = cfg["max_position_embeddings"]
-    lens = {"A": [1, 7, 33, 64, 128], "B": [3, 45, 130, 300, 77, 260], "C": [2, 100, 255, 31]}[which]
+    lens = {"A": [1, 7, 33, 64, 128], "B": [3, 45, 130, 300, 77, 260], "C": [2, 100, 255, 31],
+            "W": [5, 40, 150, 64, 200]}[which]
     return {"r%d" % i: random_tokens(min(n, top), V, 100 + i) for i, n in enumerate(lens)}
 
 
@@ -63,7 +64,7 @@ def engine(folder, which, dtype, num_pages):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("which", ["A", "B", "C"])
+@pytest.mark.parametrize("which", ["A", "B", "C", "W"])
 def test_every_way_of_cutting(models, which, dtype):
     folder, cfg, w = models[(which, dtype)]
     reqs = requests_for(cfg, which)
@@ -79,7 +80,7 @@ def test_every_way_of_cutting(models, which, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("which", ["A", "B", "C"])
+@pytest.mark.parametrize("which", ["A", "B", "C", "W"])
 def test_mixed_requests_with_page_reuse(models, which, dtype):
     folder, cfg, w = models[(which, dtype)]
     reqs = requests_for(cfg, which)
@@ -94,6 +95,34 @@ def test_mixed_requests_with_page_reuse(models, which, dtype):
     check(replay_in_process(core.executor, steps), refs, dtype, "mixed")
     core.storage.manager.check_invariants()
     assert core.storage.manager.num_free_pages(0) == max_tokens // bs
+
+
+def test_wide_model_leaves_products_unfinished(models, monkeypatch):
+    """The wide configuration does reach the kernels that add up partial sums (a step of 40 tokens in
+    bfloat16): twice per layer the norm, once per layer the rotation; a step of 8 tokens reaches neither."""
+    folder, cfg, w = models[("W", "bfloat16")]
+    core = engine(folder, "W", "bfloat16", num_pages=8)
+    ops = core.executor.rt.ops
+    seen = {"norm": 0, "rope": 0}
+    norm, rope = ops._add_rms_norm_pending, ops._rope_cache_write_pending
+
+    def count(key, f):
+        def g(*a, **k):
+            seen[key] += 1
+            return f(*a, **k)
+        return g
+    monkeypatch.setattr(ops, "_add_rms_norm_pending", count("norm", norm))
+    monkeypatch.setattr(ops, "_rope_cache_write_pending", count("rope", rope))
+    toks = random_tokens(48, cfg["vocab_size"], 77)
+    ref = plain_llama_forward(cfg, w, toks)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": toks[:40], "want": list(range(40))}], "end": []}]
+    got = replay_in_process(core.executor, steps)
+    L = cfg["num_hidden_layers"]
+    assert seen == {"norm": 2 * L, "rope": L}
+    steps = [{"step": 1, "entries": [{"id": "a", "tokens": toks[40:], "want": list(range(8))}], "end": ["a"]}]
+    got2 = replay_in_process(core.executor, steps)
+    assert seen == {"norm": 2 * L, "rope": L}
+    check({"a": torch.cat([got["a"], got2["a"]])}, {"a": ref}, "bfloat16", "wide")
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

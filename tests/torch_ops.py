@@ -153,11 +153,14 @@ class TorchOps:
     def linear_gated(self, x, weight, bias=None, kind="silu"):
         return self.gated_act(self.linear(x, weight, bias), kind)
 
-    def linear(self, x, weight, bias=None, out_dtype=None):
+    def linear(self, x, weight, bias=None, out_dtype=None, pending_ok=False):
         y = x.to(torch.float32) @ weight.to(torch.float32).t()
         if bias is not None:
             y = y + bias.to(torch.float32)
         return y.to(out_dtype or x.dtype)
+
+    def materialize(self, y):
+        return y
 
     # ------------------------------------------------------------ sampling
     def sample(self, logits, temperature=None, top_k=None, top_p=None, min_p=None, seeds=None, draws=None):
