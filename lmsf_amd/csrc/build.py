@@ -1,10 +1,13 @@
-"""Compiles the HIP sources of this folder for gfx950 into one shared library.
+"""Compiles the HIP sources of this folder for gfx950 into one shared library, and the C++ host
+sources under ``host/`` (cache manager, scheduler, step metadata; no GPU code) into another.
 
 ``build()`` always compiles. ``ensure_built()`` compiles only if no library matching the
 sources is there (a fresh checkout, or a source changed since the last build); it is what the
 loader calls, and it prints a line now and then while hipcc runs, so that a first call does
 not look hung. The library is written beside the sources; if that folder cannot be written
 (another user's checkout), a per-user folder under the system's temporary directory is used.
+``build_host()`` / ``ensure_host_built()`` do the same for the host library, which needs a C++
+compiler only and is what the CPU side of the engine runs on.
 """
 import concurrent.futures
 import hashlib
@@ -71,11 +74,9 @@ def _candidate_dirs() -> List[str]:
     return [CSRC_DIR, fallback]
 
 
-def find_library() -> Optional[str]:
-    """Path of a built library whose stamp matches the current sources, or None."""
-    digest = source_digest()
+def _find(lib_name: str, digest: str) -> Optional[str]:
     for folder in _candidate_dirs():
-        lib = os.path.join(folder, LIB_NAME)
+        lib = os.path.join(folder, lib_name)
         stamp = lib + ".stamp"
         if os.path.isfile(lib) and os.path.isfile(stamp):
             try:
@@ -85,6 +86,11 @@ def find_library() -> Optional[str]:
             except OSError:
                 pass
     return None
+
+
+def find_library() -> Optional[str]:
+    """Path of a built library whose stamp matches the current sources, or None."""
+    return _find(LIB_NAME, source_digest())
 
 
 def _say(msg: str) -> None:
@@ -153,5 +159,65 @@ def ensure_built(verbose: bool = True) -> str:
     return build(verbose=verbose)
 
 
+# ---------------------------------------------------------------- the host library
+
+HOST_DIR = os.path.join(CSRC_DIR, "host")
+HOST_LIB_NAME = "liblmsf_host.so"
+HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-shared", "-Wall"]
+
+
+def host_sources() -> List[str]:
+    return sorted(f for f in os.listdir(HOST_DIR) if f.endswith(".cc"))
+
+
+def host_digest() -> str:
+    h = hashlib.sha256()
+    for name in sorted(os.listdir(HOST_DIR)):
+        if name.endswith((".cc", ".h")):
+            h.update(name.encode())
+            with open(os.path.join(HOST_DIR, name), "rb") as f:
+                h.update(f.read())
+    h.update(" ".join(HOST_FLAGS).encode())
+    return h.hexdigest()
+
+
+def _cxx() -> str:
+    for cand in (os.environ.get("CXX"), shutil.which("g++"), shutil.which("c++"), shutil.which("clang++"),
+                 "/opt/rocm/llvm/bin/clang++"):
+        if cand and (os.path.isfile(cand) or shutil.which(cand)):
+            return cand
+    raise RuntimeError("no C++ compiler found (looked at $CXX, g++, c++, clang++); the host library of lmsf_amd "
+                       "cannot be built")
+
+
+def build_host(verbose: bool = True) -> str:
+    """Compile the host library; returns its path."""
+    out_dir = next((d for d in _candidate_dirs() if _writable(d)), None)
+    if out_dir is None:
+        raise RuntimeError("no writable folder for the host library among %s" % _candidate_dirs())
+    digest = host_digest()
+    lib = os.path.join(out_dir, HOST_LIB_NAME)
+    tmp = lib + ".tmp%d" % os.getpid()
+    t0 = time.time()
+    cmd = [_cxx()] + HOST_FLAGS + ["-I", HOST_DIR, "-o", tmp] + [os.path.join(HOST_DIR, s) for s in host_sources()]
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("compiling %s failed:\n%s" % (HOST_LIB_NAME, proc.stdout))
+    os.replace(tmp, lib)
+    with open(lib + ".stamp", "w") as f:
+        f.write(digest + "\n")
+    if verbose:
+        _say("built %s in %.0f s" % (lib, time.time() - t0))
+    return lib
+
+
+def ensure_host_built(verbose: bool = True) -> str:
+    lib = _find(HOST_LIB_NAME, host_digest())
+    if lib is not None:
+        return lib
+    return build_host(verbose=verbose)
+
+
 if __name__ == "__main__":
+    print(build_host())
     print(build())

@@ -7,12 +7,12 @@ produces logits: it takes pages for the new tokens, builds the flat batch, runs 
 exactly the tokens it was given, and commits them to the cache. Sampling is a separate call, so that
 trace replay can take the logits.
 """
-from typing import Dict, Hashable, List, Optional, Sequence, Tuple
+from typing import Dict, Hashable, Optional, Sequence, Tuple
 
 import numpy as np
 import torch
 
-from ..cache.manager import CacheError, CacheManager, OutOfPages
+from ..cache.manager import CacheError, CacheManager
 from ..cache.storage import CacheStorage
 from ..parts.base import Runtime
 from .batch import GroupView, StepContext, StepEntry
@@ -20,10 +20,6 @@ from .batch import GroupView, StepContext, StepEntry
 
 class StepError(ValueError):
     """A step that cannot be run as given (unknown token id, too long a request, bad ``want``)."""
-
-
-def _align4(n: int) -> int:
-    return (n + 3) // 4 * 4
 
 
 class ModelExecutor:
@@ -58,35 +54,18 @@ class ModelExecutor:
         if not entries:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.rt.device)
         mgr = self.manager
-        added: List[Hashable] = []
-        appended: List[Hashable] = []
-        starts: List[int] = []
+        rids = [e.request_id for e in entries]
+        lens = [len(e.tokens) for e in entries]
+        handles, starts, added = mgr.begin_step(rids, lens)      # OutOfPages: nothing was taken
         try:
-            for e in entries:
-                if not mgr.has_request(e.request_id):
-                    mgr.add_request(e.request_id)
-                    added.append(e.request_id)
-                starts.append(mgr.append(e.request_id, len(e.tokens)))
-                appended.append(e.request_id)
-        except OutOfPages:
-            for rid in appended:
-                mgr.rollback(rid)
-            for rid in added:
-                mgr.free_request(rid)
-            raise
-        try:
-            if self.use_graphs and all(len(e.tokens) == 1 for e in entries) and len(entries) <= self.max_graph_batch:
-                logits = self._graph_step(entries, starts)
+            if self.use_graphs and all(n == 1 for n in lens) and len(entries) <= self.max_graph_batch:
+                logits = self._graph_step(entries, handles, starts)
             else:
-                logits = self.model.forward(self._build_context(entries, starts))
+                logits = self.model.forward(self._build_context(entries, handles, starts))
         except Exception:
-            for rid in appended:
-                mgr.rollback(rid)
-            for rid in added:
-                mgr.free_request(rid)
+            mgr.abort_step(rids, handles, added)
             raise
-        for e in entries:
-            mgr.commit(e.request_id)
+        mgr.commit_step(handles)
         return logits
 
     def release(self, request_id: Hashable) -> None:
@@ -115,35 +94,29 @@ class ModelExecutor:
                 raise StepError("request %r would hold %d tokens, more than max_model_len %d"
                                 % (e.request_id, held + n, self.max_model_len))
 
-    def _build_context(self, entries: Sequence[StepEntry], starts: Sequence[int],
+    def _build_context(self, entries: Sequence[StepEntry], handles: np.ndarray, starts_a: np.ndarray,
                        static: Optional["_StaticBatch"] = None) -> StepContext:
         """Flatten the entries into the step's device tensors. Everything goes through one pinned staging
-        buffer and one copy. With ``static`` (a decode step that replays a captured graph) the copy goes
-        into that batch's fixed device buffer, block tables padded to their full width, and every
-        token's logits are asked for."""
+        buffer, which the host library fills, and one copy. With ``static`` (a decode step that replays a
+        captured graph) the copy goes into that batch's fixed device buffer, block tables padded to their
+        full width, and every token's logits are asked for."""
         mgr = self.manager
         S = len(entries)
         lens = [len(e.tokens) for e in entries]
         N = sum(lens)
-        lens_a = np.asarray(lens, dtype=np.int64)
-        starts_a = np.asarray(starts, dtype=np.int64)
-        seg_starts_a = np.zeros(S + 1, dtype=np.int64)
-        np.cumsum(lens_a, out=seg_starts_a[1:])
-        seg_starts = seg_starts_a.tolist()
-        caches = [mgr.request(e.request_id) for e in entries]
-        state_slots = [rc.state_slot for rc in caches]
+        starts = starts_a.tolist()
         if static is not None:
-            logit_rows = np.arange(N, dtype=np.int64)
+            logit_rows = np.arange(N, dtype=np.int32)
         else:
-            logit_rows = np.fromiter((seg_starts[s] + int(w) for s, e in enumerate(entries) for w in e.want),
-                                     dtype=np.int64)
+            seg_start, rows = 0, []
+            for e, n in zip(entries, lens):
+                rows.extend(seg_start + int(w) for w in e.want)
+                seg_start += n
+            logit_rows = np.asarray(rows, dtype=np.int32)
         R = int(logit_rows.shape[0])
         G = len(mgr.groups)
-        widths: List[int] = []
-        for gi in range(G):
-            widths.append(static.widths[gi] if static is not None else
-                          max(1, max(len(rc.tables[gi]) for rc in caches)))
-        offsets, total = self._layout(N, S, R, widths)
+        widths = static.widths if static is not None else mgr.step_widths(handles)
+        offsets, raw_offsets, total = mgr.step_layout(N, S, R, widths)
         if self._pinned is None or self._pinned.numel() < total:
             self._pinned = torch.empty(max(total, 4096), dtype=torch.int32,
                                        pin_memory=self.rt.device.type == "cuda")
@@ -155,36 +128,18 @@ class ModelExecutor:
             o, n = offsets[name]
             return host_np[o:o + n]
 
-        seg_of = np.repeat(np.arange(S, dtype=np.int64), lens_a)
-        within = np.arange(N, dtype=np.int64) - seg_starts_a[:-1][seg_of]       # index of a token in its segment
-        positions = starts_a[seg_of] + within
         if N == S:
             section("token_ids")[:] = [e.tokens[0] for e in entries]
         else:
             section("token_ids")[:] = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in entries])
-        section("positions")[:] = positions
-        section("seg_of")[:] = seg_of
-        section("seg_starts")[:] = seg_starts_a
-        section("seg_first")[:] = starts_a
-        section("state_slots")[:] = state_slots
         if R:
             section("logit_rows")[:] = logit_rows
-        for gi in range(G):
-            ps = mgr.groups[gi].page_size
-            w = widths[gi]
-            tables = section("tables%d" % gi).reshape(S, w)
-            tables[:] = 0
-            for s, rc in enumerate(caches):
-                t = rc.tables[gi]
-                tables[s, :len(t)] = t
-            # slot of every token: page of its block, times the page size, plus its offset in the page
-            pages = tables[seg_of, positions // ps].astype(np.int64)
-            if (pages < 0).any():
-                bad = int(np.nonzero(pages < 0)[0][0])
-                raise CacheError("position %d of request %r lies in a page that was given back"
-                                 % (int(positions[bad]), entries[int(seg_of[bad])].request_id))
-            section("slots%d" % gi)[:] = pages * ps + positions % ps
-            np.maximum(tables, 0, out=tables)            # pages that a window has passed: any valid page id
+        try:
+            mgr.fill_step(handles, starts_a, lens, widths, raw_offsets, host_np)
+        except CacheError as e:
+            raise CacheError("%s (requests %s)" % (e, ", ".join(repr(x.request_id) for x in entries)))
+        seg_starts = section("seg_starts").tolist()
+        state_slots = section("state_slots").tolist()
         # the copy is synchronous: the staging buffer is free again when the next step fills it
         if static is not None:
             static.device_buffer.copy_(host, non_blocking=False)
@@ -225,24 +180,9 @@ class ModelExecutor:
             bucket *= 2
         return min(bucket, self.max_model_len)
 
-    @staticmethod
-    def _layout(N: int, S: int, R: int, widths: Sequence[int]):
-        """Offsets (in int32 elements, 16-byte aligned) of the sections of a step's metadata buffer."""
-        sections = [("token_ids", N), ("positions", N), ("seg_of", N), ("seg_starts", S + 1), ("seg_first", S),
-                    ("state_slots", S), ("logit_rows", R)]
-        for gi, w in enumerate(widths):
-            sections.append(("slots%d" % gi, N))
-            sections.append(("tables%d" % gi, S * w))
-        offsets: Dict[str, Tuple[int, int]] = {}
-        total = 0
-        for name, n in sections:
-            offsets[name] = (total, n)
-            total += _align4(n)
-        return offsets, max(total, 4)
-
     # ------------------------------------------------------------------ decode steps as HIP graphs
 
-    def _graph_step(self, entries: Sequence[StepEntry], starts: Sequence[int]) -> torch.Tensor:
+    def _graph_step(self, entries: Sequence[StepEntry], handles: np.ndarray, starts: np.ndarray) -> torch.Tensor:
         """A step of single tokens. The first step of a batch size and context bucket (the longest context
         rounded up to a power of two) runs eagerly and is then captured as a HIP graph over a fixed
         metadata buffer; later steps of that kind copy their metadata into the buffer and replay the
@@ -250,14 +190,14 @@ class ModelExecutor:
         context lengths but through the device tensors, so the parts are told the bucket as the longest
         context. The graph computes the logits of every token; the wanted rows are picked afterwards."""
         B = len(entries)
-        bucket = self._context_bucket(max(starts) + 1)
+        bucket = self._context_bucket(int(starts.max()) + 1)
         sb = self._static.get((B, bucket))
         if sb is None:
             widths = [-(-bucket // g.page_size) for g in self.manager.groups]
-            _, total = self._layout(B, B, B, widths)
+            _, _, total = self.manager.step_layout(B, B, B, widths)
             sb = _StaticBatch(widths, torch.zeros(total, dtype=torch.int32, device=self.rt.device), bucket)
             self._static[(B, bucket)] = sb
-        ctx = self._build_context(entries, starts, static=sb)
+        ctx = self._build_context(entries, handles, starts, static=sb)
         if sb.graph is None:
             sb.context = ctx
             logits = self.model.forward(ctx)                 # eager: this step's result, and the warm-up

@@ -1,15 +1,11 @@
 """Continuous batching above the step function: admits requests, cuts prompts into portions under
 a token budget, decodes, and decides what happens when pages run out.
 
-The reference's scheduler (core/src/sched/scheduler.rs:343-543) runs either a batch of whole
-prompts or a batch of decode tokens, admits a prompt only when all its blocks fit
-(core/src/sched/block_manager.rs:104-122), and on shortage preempts the latest arrival by
-recompute (:253-284, :459-490). Kept from it: first come first served by arrival, head-of-line
-admission with a watermark of free pages, preemption by recompute of the latest arrival with
-re-insertion at the front of the waiting queue, and prompts longer than the limit being ignored
-(:368-381). Different: a step holds real tokens under ``max_num_batched_tokens``: first one token
-for every decoding request, then portions of prompts in arrival order, each at most
-``prefill_chunk_size`` long.
+The decisions are made by the C++ scheduler of the host library (``lmsf_amd/csrc/host/scheduler.cc``;
+its header says what is kept from the reference's scheduler, core/src/sched/scheduler.rs:343-543, and
+what is different). This module is its Python face: it owns the ``Sequence`` objects (token ids,
+sampling parameters), tells the library each request's length and progress before a plan is made, and
+writes the plan's consequences (state, progress, counters) back to them.
 
 What happens when pages run out:
 - a new request is not admitted while its first portion does not fit above the watermark (it waits);
@@ -20,12 +16,15 @@ What happens when pages run out:
   reason "length";
 - a prompt that would not fit the whole pool even alone is ignored at admission (reason "length").
 """
+import ctypes
 import time
-from collections import deque
 from dataclasses import dataclass, field
-from typing import Deque, Dict, Hashable, List, Optional
+from typing import Dict, Hashable, List, Optional
 
-from ..cache.manager import CacheManager
+import numpy as np
+
+from ..cache.manager import CacheManager, _ptr, _raise
+from ..host import library as _host
 from .sequence import Sequence, SequenceState
 
 
@@ -73,172 +72,138 @@ class Scheduler:
     def __init__(self, config: SchedulerConfig, cache: CacheManager):
         self.config = config
         self.cache = cache
-        self.waiting: Deque[Sequence] = deque()
-        self.running: List[Sequence] = []
-        self.num_preemptions = 0
+        self._lib = _host.load_host_library()
+        h = ctypes.c_void_p()
+        rc = self._lib.lmsf_sched_create(cache.native, int(config.max_num_batched_tokens), int(config.max_num_seqs),
+                                         int(config.max_model_len), int(config.prefill_chunk_size or 0),
+                                         float(config.watermark), ctypes.byref(h))
+        if rc:
+            _raise(self._lib, rc)
+        self._h = h
+        self._seqs: Dict[int, Sequence] = {}        # the library's integer -> the request, while it is scheduled
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            self._lib.lmsf_sched_destroy(self._h)
+            self._h = None
 
     # ------------------------------------------------------------------ queue operations
 
     def add(self, seq: Sequence) -> None:
-        self.waiting.append(seq)
+        h = self.cache.pin(seq.request_id)
+        rc = self._lib.lmsf_sched_add(self._h, h, int(seq.arrival), int(seq.length))
+        if rc:
+            self.cache.unpin(seq.request_id)
+            _raise(self._lib, rc, "request %r" % (seq.request_id,))
+        self._seqs[h] = seq
+
+    def _drop(self, h: int) -> Optional[Sequence]:
+        seq = self._seqs.pop(h, None)
+        if seq is not None:
+            self.cache.unpin(seq.request_id)
+        return seq
+
+    def _handle(self, request_id: Hashable) -> Optional[int]:
+        h = self.cache.known_handle(request_id)
+        return h if h in self._seqs else None
 
     def abort(self, request_id: Hashable) -> Optional[Sequence]:
         """core/src/sched/scheduler.rs:160-196: by request id, in whichever queue."""
-        for q in (self.waiting, self.running):
-            for seq in list(q):
-                if seq.request_id == request_id:
-                    q.remove(seq)
-                    seq.state = SequenceState.FINISHED_ABORTED
-                    self._release(seq)
-                    return seq
-        return None
+        h = self._handle(request_id)
+        if h is None:
+            return None
+        found = ctypes.c_int()
+        rc = self._lib.lmsf_sched_abort(self._h, h, ctypes.byref(found))
+        if rc:
+            _raise(self._lib, rc)
+        seq = self._drop(h)
+        seq.state = SequenceState.FINISHED_ABORTED
+        return seq
 
     def has_unfinished(self) -> bool:
-        return bool(self.waiting or self.running)
+        return bool(self._seqs)
 
     def num_unfinished(self) -> int:
-        return len(self.waiting) + len(self.running)
+        return len(self._seqs)
 
     def finish(self, seq: Sequence) -> None:
         """The engine decided that ``seq`` is done: drop it and give back what it holds."""
-        if seq in self.running:
-            self.running.remove(seq)
-        self._release(seq)
+        h = self._handle(seq.request_id)
+        if h is None:
+            return
+        rc = self._lib.lmsf_sched_finish(self._h, h)
+        if rc:
+            _raise(self._lib, rc)
+        self._drop(h)
 
-    def _release(self, seq: Sequence) -> None:
-        if self.cache.has_request(seq.request_id):
-            self.cache.free_request(seq.request_id)
+    def _queue(self, which: int) -> List[Sequence]:
+        n = ctypes.c_int()
+        self._lib.lmsf_sched_queue(self._h, which, None, 0, ctypes.byref(n))
+        out = np.zeros(max(n.value, 1), dtype=np.int64)
+        self._lib.lmsf_sched_queue(self._h, which, _ptr(out), out.shape[0], ctypes.byref(n))
+        return [self._seqs[int(h)] for h in out[:n.value]]
+
+    @property
+    def waiting(self) -> List[Sequence]:
+        """The waiting requests, the head of the line first."""
+        return self._queue(0)
+
+    @property
+    def running(self) -> List[Sequence]:
+        return self._queue(1)
+
+    @property
+    def num_preemptions(self) -> int:
+        return int(self._lib.lmsf_sched_num_preemptions(self._h))
 
     # ------------------------------------------------------------------ planning
 
     def schedule(self) -> StepPlan:
-        cfg, cache = self.config, self.cache
+        n = len(self._seqs)
+        if n:
+            ids = np.fromiter(self._seqs.keys(), dtype=np.int64, count=n)
+            lengths = np.fromiter((s.length for s in self._seqs.values()), dtype=np.int64, count=n)
+            computed = np.fromiter((s.num_computed for s in self._seqs.values()), dtype=np.int64, count=n)
+            rc = self._lib.lmsf_sched_set_progress(self._h, n, _ptr(ids), _ptr(lengths), _ptr(computed))
+            if rc:
+                _raise(self._lib, rc)
+        counts = np.zeros(4, dtype=np.int32)
+        rc = self._lib.lmsf_sched_schedule(self._h, _ptr(counts))
+        if rc:
+            _raise(self._lib, rc)
+        ns, npre, nig, ncap = (int(c) for c in counts)
+        ids, starts, toks = (np.zeros(max(ns, 1), dtype=np.int64) for _ in range(3))
+        samples = np.zeros(max(ns, 1), dtype=np.int32)
+        pre, ign, cap = (np.zeros(max(k, 1), dtype=np.int64) for k in (npre, nig, ncap))
+        rc = self._lib.lmsf_sched_plan(self._h, _ptr(ids), _ptr(starts), _ptr(toks), _ptr(samples), _ptr(pre), _ptr(ign),
+                                       _ptr(cap))
+        if rc:
+            _raise(self._lib, rc)
         plan = StepPlan()
-        budget = cfg.max_num_batched_tokens
-        planned = [0] * len(cache.groups)          # pages promised to earlier entries of this plan
-        planned_slots = 0
-        watermark = [int(round(cfg.watermark * g.num_pages)) for g in cache.groups]
-
-        last_need = [None, None, None]             # (request, tokens) of the last question and its answer
-
-        def needed(rid, n):
-            if last_need[0] != rid or last_need[1] != n or rid is None:
-                last_need[0], last_need[1], last_need[2] = rid, n, cache.pages_needed(rid, n)
-            return last_need[2]
-
-        def fits(rid, n, reserve=False) -> bool:
-            for gi, k in enumerate(needed(rid, n)):
-                if cache.num_free_pages(gi) - planned[gi] - k < (watermark[gi] if reserve else 0):
-                    return False
-            return True
-
-        def take(rid, n) -> None:
-            for gi, k in enumerate(needed(rid, n)):
-                planned[gi] += k
-
-        self.running.sort(key=lambda s: s.arrival)
-        todo = list(self.running)                  # in arrival order; victims come from its end
-        while todo:
-            seq = todo.pop(0)
-            if budget <= 0:
-                break
-            n = seq.remaining
-            if n > 1:
-                n = min(n, budget, cfg.prefill_chunk_size or n)
-            while not fits(seq.request_id, n):
-                if n > 1:
-                    # a shorter portion may fit
-                    room = min(self._room_tokens(seq, planned), n - 1)
-                    if room >= 1:
-                        n = room
-                        continue
-                if todo:
-                    victim = todo.pop()            # the latest arrival
-                    self._preempt(victim, plan)
-                elif not plan.scheduled:
-                    # alone and still no room: it can never continue
-                    self.running.remove(seq)
-                    seq.state = SequenceState.FINISHED_LENGTH_CAPPED
-                    self._release(seq)
-                    plan.capped.append(seq)
-                    seq = None
-                    break
-                else:
-                    self._preempt(seq, plan)
-                    seq = None
-                    break
-            if seq is None:
-                continue
-            take(seq.request_id, n)
-            plan.scheduled.append(ScheduledSequence(seq, seq.num_computed, n, seq.num_computed + n == seq.length))
-            budget -= n
-
-        # admission, head of line only; nothing is admitted in a step that had to preempt
-        while self.waiting and not plan.preempted and budget > 0 and \
-                len(self.running) < cfg.max_num_seqs:
-            seq = self.waiting[0]
-            limit = min(cfg.max_model_len, cache_capacity_tokens(cache))
-            if seq.length > limit or seq.length == 0:
-                self.waiting.popleft()
-                seq.state = SequenceState.FINISHED_IGNORED
-                plan.ignored.append(seq)
-                continue
-            if cache.num_free_state_slots() - planned_slots <= 0:
-                break
-            n = min(seq.remaining, budget, cfg.prefill_chunk_size or seq.remaining)
-            if not fits(None, n, reserve=True):
-                room = min(self._room_tokens(None, planned, watermark), n)
-                idle = not self.running and not plan.scheduled
-                if room < 1:
-                    if not idle:
-                        break                      # wait for pages
-                    # every page is free and not one token fits above the watermark: it never will
-                    self.waiting.popleft()
-                    seq.state = SequenceState.FINISHED_IGNORED
-                    plan.ignored.append(seq)
-                    continue
-                if room < min(n, 16) and not idle:
-                    break                          # wait for pages rather than crawl
-                n = room
-            self.waiting.popleft()
-            take(None, n)
-            planned_slots += 1
-            seq.state = SequenceState.RUNNING
-            if seq.metrics.first_scheduled_time is None:
-                seq.metrics.first_scheduled_time = time.monotonic()
-            self.running.append(seq)
-            plan.scheduled.append(ScheduledSequence(seq, seq.num_computed, n, seq.num_computed + n == seq.length))
-            budget -= n
+        for h in pre[:npre]:
+            seq = self._seqs[int(h)]
+            seq.num_computed = 0
+            seq.num_preemptions += 1
+            seq.state = SequenceState.WAITING
+            plan.preempted.append(seq)
+        for h in ign[:nig]:
+            seq = self._drop(int(h))
+            seq.state = SequenceState.FINISHED_IGNORED
+            plan.ignored.append(seq)
+        for h in cap[:ncap]:
+            seq = self._drop(int(h))
+            seq.state = SequenceState.FINISHED_LENGTH_CAPPED
+            plan.capped.append(seq)
+        for i in range(ns):
+            seq = self._seqs[int(ids[i])]
+            if seq.state != SequenceState.RUNNING:
+                seq.state = SequenceState.RUNNING
+                if seq.metrics.first_scheduled_time is None:
+                    seq.metrics.first_scheduled_time = time.monotonic()
+            plan.scheduled.append(ScheduledSequence(seq, int(starts[i]), int(toks[i]), bool(samples[i])))
+        if npre or ncap:
+            self.cache.forget_released()
         return plan
-
-    def _room_tokens(self, seq: Optional[Sequence], planned: List[int], watermark: Optional[List[int]] = None) -> int:
-        """How many more tokens of ``seq`` (None: a new request) fit in the pages that are free now."""
-        cache = self.cache
-        room = None
-        for gi, g in enumerate(cache.groups):
-            free = cache.num_free_pages(gi) - planned[gi] - (watermark[gi] if watermark else 0)
-            held = 0
-            slack = 0
-            if seq is not None and cache.has_request(seq.request_id):
-                rc = cache.request(seq.request_id)
-                held = rc.num_tokens
-                slack = len(rc.tables[gi]) * g.page_size - held
-            r = max(0, free) * g.page_size + slack
-            room = r if room is None else min(room, r)
-        return room or 0
-
-    def _preempt(self, seq: Sequence, plan: StepPlan) -> None:
-        """Preemption by recompute (core/src/sched/scheduler.rs:274-284): everything the request holds
-        goes back, and it returns to the front of the waiting queue."""
-        if seq in self.running:
-            self.running.remove(seq)
-        self._release(seq)
-        seq.num_computed = 0
-        seq.num_preemptions += 1
-        seq.state = SequenceState.WAITING
-        self.waiting.appendleft(seq)
-        plan.preempted.append(seq)
-        self.num_preemptions += 1
 
 
 def cache_capacity_tokens(cache: CacheManager) -> int:
