@@ -253,8 +253,10 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
 //
 // A stage holds the K tile [32 keys][DPAD] and the V^T tile [DPAD][32 keys], both without padding (the
 // transfer writes lane after lane). Bank conflicts of the operand reads are avoided by choosing which
-// piece each lane fetches: 16-byte piece ``col`` of K row ``row`` lies in slot (col - row) mod PR of its row,
-// piece ``p`` of V^T row ``dv`` in slot (p + dv / 4) mod 4. The request's block table is copied to LDS first,
+// piece each lane fetches: 16-byte piece ``col`` of K row ``row`` lies in slot col xor (row mod PR) of its row
+// where a row has a power of two of pieces (measured: full rate; the rotation (col - row) mod PR, used for the
+// other head sizes, loses 40 % of the rate when two workgroups share a compute unit), piece ``p`` of V^T row
+// ``dv`` in slot (p + dv / 4) mod 4. The request's block table is copied to LDS first,
 // so that no address waits for a lookup in global memory. Needs pages of 8, 16, 32, ... tokens.
 //
 // The transfer instruction is written as inline assembly: through the compiler's builtin every LDS read
@@ -286,6 +288,7 @@ __global__ __launch_bounds__(256) void attn_prefill_dma_kernel(
     int d, int ps_log2, float scale_log2, int window, int HB, int n_hb, int bt_cap) {
   constexpr int DS = DPAD / 32, DV = DPAD / 16;
   constexpr int PR = DPAD / 8;                   // 16-byte pieces per K row
+  constexpr bool PR_POW2 = (PR & (PR - 1)) == 0;
   constexpr int KTILE = 32 * DPAD * 2;           // bytes; the V^T tile has the same size
   constexpr int STAGE = 2 * KTILE;
   constexpr int LPW = DPAD / 32;                 // transfers per wave and stage (DPAD / 8 in all)
@@ -368,8 +371,13 @@ __global__ __launch_bounds__(256) void attn_prefill_dma_kernel(
     if (j < DPAD / 16) {
       const int P = j * 64 + l;
       const int row = P / PR, slot = P - row * PR;
-      int col = slot + row % PR;
-      if (col >= PR) col -= PR;
+      int col;
+      if (PR_POW2) {
+        col = slot ^ (row & (PR - 1));
+      } else {
+        col = slot + row % PR;
+        if (col >= PR) col -= PR;
+      }
       if (col * 8 >= d) col = 0;                   // beyond the head: any finite data, the query is zero there
       t_key[i] = row;
       t_mul[i] = d;
@@ -394,8 +402,13 @@ __global__ __launch_bounds__(256) void attn_prefill_dma_kernel(
 #pragma unroll
     for (int s = 0; s < DS; ++s) {
       const int row = b * 16 + c;
-      int slot = s * 4 + g - row % PR;
-      if (slot < 0) slot += PR;
+      int slot;
+      if (PR_POW2) {
+        slot = (s * 4 + g) ^ (row & (PR - 1));
+      } else {
+        slot = s * 4 + g - row % PR;
+        if (slot < 0) slot += PR;
+      }
       koff[b][s] = (row * PR + slot) * 16;
     }
   const int vrot = (g >> 1) + (c >> 2);            // (piece + dv / 4) mod 4 with dv = 16 v + c

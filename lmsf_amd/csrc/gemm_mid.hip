@@ -13,7 +13,7 @@
 // Tiles of 64 k travel from global memory straight into LDS (global_load_lds_dwordx4: lane i of a wave
 // writes its 16 bytes at the wave's LDS base + 16 i), three steps ahead of the one being multiplied; each
 // wave moves its own rows of W and a quarter of x. A tile is 16 rows of 128 bytes; the 16-byte piece c of
-// row r lies in slot (c + r / 2) mod 8 of its row, which keeps the operand reads of a wave on distinct
+// row r lies in slot (c + r) mod 8 of its row, which keeps the operand reads of a wave on distinct
 // banks without padding (the transfer cannot pad). One barrier per step.
 //
 // v_mfma_f32_16x16x32_bf16: A = 16 rows of W, B = 16 rows of x, both with lane (r, g) = (l % 16, l / 16)
@@ -83,7 +83,7 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const bf16_t* __restrict_
   for (int t = 0; t < WT; ++t)
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
-      const int row = 8 * h + trow, piece = (tslot - (row >> 1)) & 7;
+      const int row = 8 * h + trow, piece = (tslot - row) & 7;
       int n = n0 + 16 * w + row;
       if (n > N - 1) n = N - 1;        // rows beyond the matrix repeat the last row and are not stored
       src[t * 2 + h] = W + (long)(n + t * N) * ldw + piece * 8 + (long)c_begin * 64;
@@ -92,7 +92,7 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const bf16_t* __restrict_
 #pragma unroll
   for (int j = 0; j < XL; ++j) {
     const int qh = w * XL + j, tile = qh >> 1, h = qh & 1;
-    const int row = 8 * h + trow, piece = (tslot - (row >> 1)) & 7;
+    const int row = 8 * h + trow, piece = (tslot - row) & 7;
     int m = tile * 16 + row;
     if (m > M - 1) m = M - 1;
     src[2 * WT + j] = x + (long)m * ldx + piece * 8 + (long)c_begin * 64;
@@ -101,7 +101,7 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const bf16_t* __restrict_
   // where this lane reads its operands in a tile: row r, pieces 4 s + g of the two 32-wide steps
   int foff[2];
 #pragma unroll
-  for (int s = 0; s < 2; ++s) foff[s] = r * 128 + (((s * 4 + g) + (r >> 1)) & 7) * 16;
+  for (int s = 0; s < 2; ++s) foff[s] = r * 128 + (((s * 4 + g) + r) & 7) * 16;
 
   f32x4_t acc[WT][MT];
 #pragma unroll
