@@ -103,6 +103,7 @@ template <> struct Vec16<float> {
   __device__ __forceinline__ void load(const float* p) { v = *reinterpret_cast<const float4*>(p); }
   __device__ __forceinline__ void store(float* p) const { *reinterpret_cast<float4*>(p) = v; }
   __device__ __forceinline__ float get(int i) const { return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w; }
+  __device__ __forceinline__ float raw(int i) const { return get(i); }   // element i as stored
   __device__ __forceinline__ void set(int i, float f) {
     if (i == 0) v.x = f; else if (i == 1) v.y = f; else if (i == 2) v.z = f; else v.w = f;
   }
@@ -115,6 +116,10 @@ template <> struct Vec16<bf16_t> {
   __device__ __forceinline__ float get(int i) const {
     uint32_t w = (i >> 1) == 0 ? v.x : (i >> 1) == 1 ? v.y : (i >> 1) == 2 ? v.z : v.w;
     return __uint_as_float((i & 1) ? (w & 0xffff0000u) : (w << 16));
+  }
+  __device__ __forceinline__ bf16_t raw(int i) const {                    // element i as stored
+    uint32_t w = (i >> 1) == 0 ? v.x : (i >> 1) == 1 ? v.y : (i >> 1) == 2 ? v.z : v.w;
+    return (bf16_t)((i & 1) ? (w >> 16) : (w & 0xffffu));
   }
   __device__ __forceinline__ void set(int i, float f) {
     uint32_t b = f32_to_bf16(f);

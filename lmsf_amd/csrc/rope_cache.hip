@@ -97,6 +97,111 @@ __global__ __launch_bounds__(256) void rope_cache_write_kernel(
   }
 }
 
+// The same work for steps of many tokens (prompts): a workgroup takes 16 consecutive tokens of one head and
+// moves 16-byte pieces, so q, k and the K cache are read and written in whole pieces, and the transposed V
+// cache, whose rows run along the tokens of a page, is written through an LDS tile with the 16 tokens of a
+// value next to each other: where their slots are consecutive, 16 lanes write 16 neighbouring elements. Needs
+// d, rot (GPT-J pairing) or rot / 2 (NeoX pairing) to be multiples of the piece (8 bfloat16, 4 float32) and
+// rows that start on 16-byte boundaries; the kernel above serves the rest and the steps of few tokens.
+template <typename T>
+__global__ __launch_bounds__(256) void rope_cache_tile_kernel(
+    T* __restrict__ q, T* __restrict__ k, T* __restrict__ v, long row_stride, const int* __restrict__ positions,
+    const float* __restrict__ table, int rot, int neox, const int* __restrict__ slots, T* __restrict__ k_pages,
+    T* __restrict__ v_pages, int nh, int nkv, int d, int ps, int n_tokens) {
+  constexpr int VEC = 16 / (int)sizeof(T);
+  constexpr int TOK = 16;
+  extern __shared__ __align__(16) unsigned char tile_raw[];
+  const int t0 = blockIdx.x * TOK, hy = blockIdx.y, tid = threadIdx.x;
+  const int ntok = min(TOK, n_tokens - t0);
+  const int half = rot / 2;
+  if (hy < nh + nkv) {
+    const bool is_k = hy >= nh;
+    const int h = hy - nh;
+    T* base = is_k ? k + (long)h * d : q + (long)hy * d;
+    const bool to_cache = is_k && slots != nullptr;
+    if (!base || (!table && !to_cache)) return;
+    auto cache_row = [&](int t) -> T* {
+      const int slot = to_cache ? slots[t] : -1;
+      return slot >= 0 ? k_pages + (((long)(slot / ps) * nkv + h) * ps + (slot % ps)) * d : nullptr;
+    };
+    if (table) {
+      if (neox) {
+        const int pieces = half / VEC;
+        for (int item = tid; item < ntok * pieces; item += 256) {
+          const int tt = item / pieces, pc = item - tt * pieces, t = t0 + tt;
+          T* x = base + (long)t * row_stride;
+          const float* cs = table + (long)positions[t] * rot + pc * VEC;
+          Vec16<T> lo, hi;
+          lo.load(x + pc * VEC);
+          hi.load(x + half + pc * VEC);
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) {
+            float xr, yr;
+            rope_rotate(lo.get(e), hi.get(e), cs[e], cs[half + e], &xr, &yr);
+            lo.set(e, xr);
+            hi.set(e, yr);
+          }
+          lo.store(x + pc * VEC);
+          hi.store(x + half + pc * VEC);
+          if (T* dst = cache_row(t)) {
+            lo.store(dst + pc * VEC);
+            hi.store(dst + half + pc * VEC);
+          }
+        }
+      } else {
+        const int pieces = rot / VEC;
+        for (int item = tid; item < ntok * pieces; item += 256) {
+          const int tt = item / pieces, pc = item - tt * pieces, t = t0 + tt;
+          T* x = base + (long)t * row_stride;
+          const float* cs = table + (long)positions[t] * rot + pc * (VEC / 2);
+          Vec16<T> a;
+          a.load(x + pc * VEC);
+#pragma unroll
+          for (int e = 0; e < VEC / 2; ++e) {
+            float xr, yr;
+            rope_rotate(a.get(2 * e), a.get(2 * e + 1), cs[e], cs[half + e], &xr, &yr);
+            a.set(2 * e, xr);
+            a.set(2 * e + 1, yr);
+          }
+          a.store(x + pc * VEC);
+          if (T* dst = cache_row(t)) a.store(dst + pc * VEC);
+        }
+      }
+    }
+    if (to_cache) {
+      // the part of k that the rotation did not touch (all of it without a table)
+      const int start = table ? rot : 0, pieces = (d - start) / VEC;
+      for (int item = tid; item < ntok * pieces; item += 256) {
+        const int tt = item / pieces, pc = item - tt * pieces, t = t0 + tt;
+        if (T* dst = cache_row(t)) {
+          Vec16<T> a;
+          a.load(base + (long)t * row_stride + start + pc * VEC);
+          a.store(dst + start + pc * VEC);
+        }
+      }
+    }
+  } else {
+    if (!v || !slots) return;
+    const int h = hy - nh - nkv;
+    T* tile = reinterpret_cast<T*>(tile_raw);
+    const int ld = d + (sizeof(T) == 2 ? 2 : 1);   // rows an odd number of 4-byte words apart: no bank conflicts
+    const int pieces = d / VEC;
+    for (int item = tid; item < ntok * pieces; item += 256) {
+      const int tt = item / pieces, pc = item - tt * pieces;
+      Vec16<T> a;
+      a.load(v + (long)(t0 + tt) * row_stride + (long)h * d + pc * VEC);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) tile[tt * ld + pc * VEC + e] = a.raw(e);
+    }
+    __syncthreads();
+    for (int e = tid; e < ntok * d; e += 256) {
+      const int dv = e / ntok, tt = e - dv * ntok;
+      const int slot = slots[t0 + tt];
+      if (slot >= 0) v_pages[(((long)(slot / ps) * nkv + h) * d + dv) * ps + (slot % ps)] = tile[tt * ld + dv];
+    }
+  }
+}
+
 static int rope_cache_check(const char* who, const void* k, const void* v, int n_tokens, long row_stride,
                             const int* positions, const float* table, int rot, int max_pos, const int* slots,
                             const void* k_pages, const void* v_pages, long num_pages, int nh, int nkv, int d, int ps) {
@@ -127,6 +232,25 @@ extern "C" int lmsf_rope_cache_write(void* q, void* k, void* v, int dtype, int n
   if (n_tokens == 0) return 0;
   const int heads = nh + 2 * nkv;
   const LmsfPartialSum none = {nullptr, nullptr, 0, 0, 0};
+  // steps of many tokens go in tiles of 16 tokens with 16-byte accesses where the sizes allow it
+  const int vec = dtype == LMSF_F32 ? 4 : 8;
+  const bool rot_ok = !table || (neox ? (rot / 2) % vec == 0 : rot % vec == 0);
+  const auto al16 = [](const void* p) { return p == nullptr || lmsf_aligned16(p); };
+  if (n_tokens >= 64 && d % vec == 0 && rot_ok && row_stride % vec == 0 && al16(q) && al16(k) && al16(v) &&
+      al16(k_pages) && al16(table)) {
+    dim3 tgrid((n_tokens + 15) / 16, heads);
+    const size_t smem = (size_t)16 * (d + 4) * (dtype == LMSF_F32 ? 4 : 2);
+    if (dtype == LMSF_F32)
+      hipLaunchKernelGGL((rope_cache_tile_kernel<float>), tgrid, dim3(256), smem, stream, (float*)q, (float*)k, (float*)v,
+                         row_stride, positions, table, rot, neox, slots, (float*)k_pages, (float*)v_pages, nh, nkv, d,
+                         ps, n_tokens);
+    else
+      hipLaunchKernelGGL((rope_cache_tile_kernel<bf16_t>), tgrid, dim3(256), smem, stream, (bf16_t*)q, (bf16_t*)k,
+                         (bf16_t*)v, row_stride, positions, table, rot, neox, slots, (bf16_t*)k_pages, (bf16_t*)v_pages,
+                         nh, nkv, d, ps, n_tokens);
+    LMSF_LAUNCH_CHECK("rope_cache_write (tiles)");
+    return 0;
+  }
   const int per_block = n_tokens >= 64 ? 4 : 1;   // tokens per workgroup: many small workgroups cost a long prompt time
   dim3 grid((n_tokens + per_block - 1) / per_block, heads), block(64, per_block);
   if (dtype == LMSF_F32)

@@ -91,14 +91,22 @@ def test_add_rms_norm(ops, ref, dtype, N, H):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("nh,nkv,d,rot,neox,ps", [(5, 5, 48, 48, True, 16), (6, 2, 64, 32, False, 8),
                                                  (8, 1, 128, 128, True, 16), (3, 3, 16, 16, True, 4)])
-def test_rope_cache_write(ops, ref, dtype, nh, nkv, d, rot, neox, ps):
+@pytest.mark.parametrize("N", [11, 150])
+def test_rope_cache_write(ops, ref, dtype, nh, nkv, d, rot, neox, ps, N):
+    """N = 150: the kernel for steps of many tokens (tiles of 16 tokens, 16-byte pieces) where the sizes
+    allow it; slots partly in runs (a prompt's portion), partly scattered."""
     g = torch.Generator().manual_seed(nh * d)
-    N, max_pos, pages = 11, 64, 9
+    max_pos, pages = 64, -(-N // ps) + 6
     qkv = dev(torch.randn(N, (nh + 2 * nkv) * d, generator=g).to(dtype))
     pos = dev(torch.randint(0, max_pos, (N,), generator=g, dtype=torch.int32))
     ang = torch.arange(max_pos, dtype=torch.float32)[:, None] * torch.rand(rot // 2, generator=g)[None, :]
     table = dev(torch.cat([ang.cos(), ang.sin()], dim=1).contiguous())
     slots = torch.randperm(pages * ps, generator=g)[:N].to(torch.int32)
+    if N > 64:
+        run = torch.arange(5, 5 + 100, dtype=torch.int32)          # 100 consecutive slots from an odd start
+        rest = torch.tensor([s for s in slots.tolist() if s < 5 or s >= 105][:N - 100], dtype=torch.int32)
+        slots = torch.cat([rest[:7], run, rest[7:]])
+        assert slots.numel() == N and len(set(slots.tolist())) == N
     slots[3] = -1
     slots = dev(slots)
     k1, v1 = dev(torch.zeros((pages, nkv, ps, d), dtype=dtype)), dev(torch.zeros((pages, nkv, d, ps), dtype=dtype))
