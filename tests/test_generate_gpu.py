@@ -47,6 +47,35 @@ def test_llm_generate_bfloat16_follows_plain_argmax(tmp_path):
             assert logits[i, tok] >= logits[i].max() - 0.05 * logits[i].abs().max(), (len(p), i)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_preemption_on_the_gpu_reproduces_the_same_tokens(tmp_path, dtype):
+    """So few pages that running requests are preempted and recomputed, decode steps replayed as graphs in
+    between: greedy and seeded tokens are those of a run with plenty of pages. A recomputed request meets other
+    batch sizes and portions than before, hence other kernels; the tokens stay the same because the kernels
+    that serve one shape of product agree to the bit (and none of these logits is a near-tie)."""
+    from lmsf_amd.engine import EngineArgs, LLMEngine
+    from lmsf_amd.sampling import SamplingParams
+    folder, cfg = make_model_folder(tmp_path, "B", dtype=dtype)
+    results = []
+    for pages in (96, 12):
+        engine = LLMEngine(EngineArgs(model=folder, dtype=dtype, block_size=16, num_gpu_blocks_override=pages,
+                                      max_num_seqs=8, prefill_chunk_size=32, max_num_batched_tokens=64))
+        for i, n in enumerate((60, 33, 18, 5)):
+            engine.add_request(i, random_tokens(n, cfg.vocab_size, 70 + i),
+                               SamplingParams(temperature=0.0 if i % 2 == 0 else 0.9, max_tokens=40, ignore_eos=True,
+                                              seed=500 + i))
+        done = {}
+        while engine.has_unfinished_requests():
+            for out in engine.step():
+                if out.finished:
+                    done[out.request_id] = out
+        results.append(({i: done[i].outputs[0].token_ids for i in done}, engine.stats["preemptions"]))
+        engine.core.storage.manager.check_invariants()
+        assert engine.core.storage.manager.num_free_pages(0) == pages
+    assert results[1][1] > 0, "the small pool was meant to force a preemption"
+    assert results[0][0] == results[1][0]
+
+
 def test_temperature_sampling_seeded(tmp_path):
     from lmsf_amd import LLM, SamplingParams
     folder, cfg = make_model_folder(tmp_path, "B")
