@@ -95,6 +95,16 @@ __device__ __forceinline__ void partial_sum_value4(const LmsfPartialSum& p, int 
   }
 }
 
+// What a fused QKV product needs for its rotary-embedding-and-cache-write epilogue beside its own arguments.
+struct RopeCacheArgs {
+  const int* positions;    // [M]
+  const float* table;      // [max_pos, d] = [cos(d/2) | sin(d/2)]
+  const int* slots;        // [M]: page * page_size + offset of the token in the cache, negative: not stored
+  bf16_t* k_pages;         // [pages, nkv, page_size, d]
+  bf16_t* v_pages;         // [pages, nkv, d, page_size]
+  int nh, nkv, d, ps;
+};
+
 // 16-byte vectors: 4 floats or 8 bfloat16
 template <typename T> struct Vec16;
 template <> struct Vec16<float> {

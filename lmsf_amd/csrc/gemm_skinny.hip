@@ -47,16 +47,6 @@ struct SkinnyTile {
   static constexpr int STEPS = KC / 32;                     // MFMA steps per chunk
 };
 
-// What the rotary epilogue needs beside the product's own arguments.
-struct RopeCacheArgs {
-  const int* positions;    // [M]
-  const float* table;      // [max_pos, d] = [cos(d/2) | sin(d/2)]
-  const int* slots;        // [M]: page * page_size + offset of the token in the cache, negative: not stored
-  bf16_t* k_pages;         // [pages, nkv, page_size, d]
-  bf16_t* v_pages;         // [pages, nkv, d, page_size]
-  int nh, nkv, d, ps;
-};
-
 // ACT: 0 none (plain linear layer), 1 silu-gated, 2 gelu-gated, 3 rotary embedding and cache write
 template <int MT, int KC, int NW, typename TOut, int ACT>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ x, long ldx,

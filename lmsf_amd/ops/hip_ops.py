@@ -50,6 +50,7 @@ class HipOps:
         self.use_library_gemm = True   # bfloat16 matrix products of many rows go to the BLAS library
         self.prefill_attention_variant = 0   # 0: keys and values staged in LDS; 1: fetched by every wave for itself
         self.decode_attention_splits = 0     # 0: chosen from the batch and the context; n: at most n splits of the keys
+        self.gemv_max_rows = 2               # products of up to this many rows stream W without the matrix cores (0: never)
         self.skinny_variant = 0        # tiling of the few-rows kernel (0: default; others for tuning)
         self.skinny_max_rows = 16      # rows up to which the few-rows kernel beats the library (measured)
 
@@ -233,6 +234,12 @@ class HipOps:
                     or v_pages.dtype != torch.bfloat16:
                 raise ValueError("v_pages must be contiguous bfloat16 [%d, %d, %d, %d]" % (num_pages, nkv, d, ps))
             y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+            if M <= self.gemv_max_rows and self._gemv_ok(M, K):
+                self._check(self.lib.lmsf_gemv_qkv_rope_cache(
+                    _ptr(x), x.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(y), y.stride(0), M, K,
+                    _ptr(positions), _ptr(table), table.shape[0], _ptr(slots), _ptr(k_pages), _ptr(v_pages), num_pages,
+                    nh, nkv, d, ps, self._stream()))
+                return y
             self._check(self.lib.lmsf_gemm_qkv_rope_cache(
                 _ptr(x), x.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(y), y.stride(0), M, K,
                 _ptr(positions), _ptr(table), table.shape[0], _ptr(slots), _ptr(k_pages), _ptr(v_pages), num_pages,
@@ -434,6 +441,14 @@ class HipOps:
         both_bf16 = x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
         if both_bf16 and self.skinny_max_rows < M <= 64 and self._mid_ok(x, weight):
             return self._linear_mid(x, weight, bias, 0, out_dtype, pending_ok and out_dtype == torch.bfloat16)
+        if both_bf16 and 0 < M <= min(1, self.gemv_max_rows) and self._skinny_ok(x, weight) and self._gemv_ok(M, K) \
+                and N * K <= 2 ** 28:
+            # one row: a pure stream of W (with two rows only the fused forms gain; the LM head's matrix is large
+            # enough for the few-rows kernel to reach the same rate, so it stays there)
+            y = torch.empty((M, N), dtype=out_dtype, device=x.device)
+            self._check(self.lib.lmsf_gemv(_ptr(x), x.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(y),
+                                           _code(out_dtype), y.stride(0), M, N, K, 0, self._stream()))
+            return y
         if both_bf16 and self._skinny_ok(x, weight):
             # few rows: the weight-streaming kernel. It also serves float32 output (logits), which the
             # library does not offer, for any number of rows, 64 at a time.
@@ -476,6 +491,10 @@ class HipOps:
             if bias is not None and (bias.shape != (2 * I,) or bias.dtype != weight.dtype or not bias.is_contiguous()):
                 raise ValueError("linear_gated: bias must be [%d] of the weight's dtype" % (2 * I))
             y = torch.empty((M, I), dtype=x.dtype, device=x.device)
+            if M <= self.gemv_max_rows and self._gemv_ok(M, x.shape[1]):
+                self._check(self.lib.lmsf_gemv(_ptr(x), x.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(y),
+                                               BF16, y.stride(0), M, I, x.shape[1], kinds[kind], self._stream()))
+                return y
             self._check(self.lib.lmsf_gemm_skinny(
                 _ptr(x), x.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(y), BF16, y.stride(0), M, I,
                 x.shape[1], self.skinny_variant, kinds[kind], self._stream()))
@@ -515,6 +534,11 @@ class HipOps:
                                            _code(out_dtype), y.stride(0), M, N, K, act, splits, _ptr(scratch),
                                            self._stream()))
         return y
+
+    @staticmethod
+    def _gemv_ok(M: int, K: int) -> bool:
+        """The one-or-two-rows kernel keeps x in LDS."""
+        return M * K * 2 <= 128 * 1024
 
     @staticmethod
     def _skinny_ok(x: torch.Tensor, weight: torch.Tensor) -> bool:

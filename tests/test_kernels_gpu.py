@@ -335,7 +335,8 @@ def test_linear_gated(ops, ref, M, I, K, kind, bias):
 
 
 @pytest.mark.parametrize("M,H,nh,nkv,d,ps", [(1, 128, 8, 1, 32, 16), (8, 4096, 32, 8, 128, 16), (16, 80, 3, 3, 64, 8),
-                                             (5, 256, 4, 2, 96, 4)])
+                                             (5, 256, 4, 2, 96, 4), (2, 4096, 32, 8, 128, 16), (1, 5000, 5, 5, 64, 8),
+                                             (2, 640, 6, 2, 32, 4)])
 @pytest.mark.parametrize("bias", [False, True])
 def test_qkv_rope_cache_fused_equals_the_three_steps(ops, ref, M, H, nh, nkv, d, ps, bias):
     """With few rows the rotation and the cache write are the epilogue of the QKV product; the result must be
@@ -356,7 +357,8 @@ def test_qkv_rope_cache_fused_equals_the_three_steps(ops, ref, M, H, nh, nkv, d,
     k1, v1 = dev(torch.zeros(pages, nkv, ps, d).bfloat16()), dev(torch.zeros(pages, nkv, d, ps).bfloat16())
     k2, v2, k3, v3 = k1.clone(), v1.clone(), k1.clone(), v1.clone()
     fused = ops.qkv_rope_cache(x, w, b, nh, nkv, d, pos, table, d, True, slots, k1, v1)
-    steps = ops.linear(x, w, b)
+    # (two rows: the fused form streams W without the matrix cores, the plain product does so row by row)
+    steps = ops.linear(x, w, b) if M != 2 else torch.cat([ops.linear(x[m:m + 1], w, b) for m in range(M)])
     ops.rope_cache_write(steps, nh, nkv, d, pos, table, d, True, slots, k2, v2)
     assert torch.equal(fused, steps) and torch.equal(k1, k2) and torch.equal(v1, v2)
     plain = ref.qkv_rope_cache(x, w, b, nh, nkv, d, pos, table, d, True, slots, k3, v3)
@@ -439,6 +441,41 @@ def test_qkv_rope_cache_from_partial_sums(ops, ref, M, H, nh, nkv, d, ps, rot, n
     c = ops.linear(x, w, b)
     ops.rope_cache_write(c, nh, nkv, d, pos, None, 0, True, slots, k5, v5)
     assert torch.equal(a, c) and torch.equal(k4, k5) and torch.equal(v4, v5)
+
+
+@pytest.mark.parametrize("M", [1, 2])
+@pytest.mark.parametrize("N,K", [(1000, 128), (331, 80), (4096, 4096), (520, 14336), (77, 5000), (64, 4608)])
+@pytest.mark.parametrize("bias", [False, True])
+def test_products_of_one_or_two_rows(ops, ref, M, N, K, bias):
+    """One or two rows stream W without the matrix cores (a wave per row of W, x in LDS, K in pieces of 4,096
+    with the last piece partial): plain with both output types, gated, and the fused QKV form, against the
+    plain formulas and against the few-rows kernel, which adds up K in another order."""
+    g = torch.Generator().manual_seed(N + K + M)
+    x = dev(torch.randn(M, K, generator=g).bfloat16())
+    w = dev((torch.randn(2 * N, K, generator=g) * K ** -0.5).bfloat16())
+    b = dev(torch.randn(2 * N, generator=g).bfloat16()) if bias else None
+    assert ops.gemv_max_rows >= 2
+    try:
+        for out_dtype in (torch.bfloat16, torch.float32):
+            b1 = b[:N] if bias else None
+            want = ref.linear(x, w[:N], b1, torch.float32)
+            ops.gemv_max_rows = 2
+            a = ops.linear(x, w[:N], b1, out_dtype=out_dtype)
+            ops.gemv_max_rows = 0
+            c = ops.linear(x, w[:N], b1, out_dtype=out_dtype)
+            t = (2e-2 if out_dtype == torch.bfloat16 else 2e-3) * max(1.0, want.abs().max().item())
+            assert a.dtype == out_dtype and (a.float() - want).abs().max().item() <= t
+            assert (a.float() - c.float()).abs().max().item() <= t
+        for kind in ("silu", "gelu"):
+            want = ref.linear_gated(x, w, b, kind).float()
+            ops.gemv_max_rows = 2
+            a = ops.linear_gated(x, w, b, kind)
+            # the bits of product (one row: the same kernel without epilogue), rounding, activation kernel
+            steps = ops.gated_act(torch.cat([ops.linear(x[m:m + 1], w, b) for m in range(M)]), kind)
+            assert torch.equal(a, steps)
+            assert (a.float() - want).abs().max().item() <= 2e-2 * max(1.0, want.abs().max().item())
+    finally:
+        ops.gemv_max_rows = 2
 
 
 def test_linear_mixed_storage(ops, ref):
