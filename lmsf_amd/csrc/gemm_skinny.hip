@@ -48,7 +48,7 @@ struct SkinnyTile {
 };
 
 // ACT: 0 none (plain linear layer), 1 silu-gated, 2 gelu-gated, 3 rotary embedding and cache write
-template <int MT, int KC, int NW, typename TOut, int ACT>
+template <int MT, int KC, int NW, typename TOut, int ACT, int DEPTH>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ x, long ldx,
                                                               const bf16_t* __restrict__ W, long ldw,
                                                               const bf16_t* __restrict__ bias, TOut* __restrict__ y,
@@ -93,11 +93,12 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __re
     for (int mt = 0; mt < MT; ++mt) acc[wt][mt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 
   const int nchunks = (K + KC - 1) / KC;
-  u32x4_t wreg[WT][T::LOADS], xreg[MT][T::LOADS];
+  // DEPTH chunks per wave are in flight: while chunk c is multiplied, c + NW .. c + DEPTH * NW are on their way
+  u32x4_t wreg[DEPTH][WT][T::LOADS], xreg[DEPTH][MT][T::LOADS];
 
   // K is a multiple of 8, so a 16-byte piece is inside or outside the row as a whole; a piece outside
   // is read from the start of the row instead and multiplied by nothing (its x piece is zeroed)
-#define SKINNY_FETCH(chunk)                                                                     \
+#define SKINNY_FETCH(buf, chunk)                                                                \
   {                                                                                             \
     const int k_ = (chunk) * KC;                                                                \
     const bool ok_ = (k_ + lcol) < K;                                                           \
@@ -105,45 +106,50 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __re
     const unsigned keep_ = ok_ ? 0xffffffffu : 0u;                                              \
     _Pragma("unroll") for (int i = 0; i < T::LOADS; ++i) {                                      \
       _Pragma("unroll") for (int wt = 0; wt < WT; ++wt) {                                       \
-        wreg[wt][i] = *reinterpret_cast<const u32x4_t*>(W + woff[wt][i] + kk_);                 \
+        wreg[buf][wt][i] = *reinterpret_cast<const u32x4_t*>(W + woff[wt][i] + kk_);            \
       }                                                                                         \
       _Pragma("unroll") for (int mt = 0; mt < MT; ++mt) {                                       \
-        xreg[mt][i] = *reinterpret_cast<const u32x4_t*>(x + xoff[mt][i] + kk_) & keep_;         \
+        xreg[buf][mt][i] = *reinterpret_cast<const u32x4_t*>(x + xoff[mt][i] + kk_) & keep_;    \
       }                                                                                         \
     }                                                                                           \
   }
 
-  // Every fetch is unconditional (a wave without a next chunk fetches its current one again, from
+  // Every fetch is unconditional (a wave without a further chunk fetches its current one again, from
   // cache), which keeps the staged pieces in registers across the loop.
   int c = wave;
-  SKINNY_FETCH(c < nchunks ? c : 0);
+#pragma unroll
+  for (int b = 0; b < DEPTH; ++b) SKINNY_FETCH(b, c + b * NW < nchunks ? c + b * NW : 0);
   while (c < nchunks) {
-    // registers -> LDS (load layout)
 #pragma unroll
-    for (int i = 0; i < T::LOADS; ++i) {
-      const int off = (lrow + i * T::ROWS_PER_LOAD) * T::ROW_BYTES + lcol * 2;
+    for (int b = 0; b < DEPTH; ++b) {
+      if (c >= nchunks) break;
+      // registers -> LDS (load layout)
 #pragma unroll
-      for (int wt = 0; wt < WT; ++wt) *reinterpret_cast<u32x4_t*>(my + wt * T::TILE_BYTES + off) = wreg[wt][i];
+      for (int i = 0; i < T::LOADS; ++i) {
+        const int off = (lrow + i * T::ROWS_PER_LOAD) * T::ROW_BYTES + lcol * 2;
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) *reinterpret_cast<u32x4_t*>(my + (WT + mt) * T::TILE_BYTES + off) = xreg[mt][i];
-    }
-    const int next = c + NW;
-    SKINNY_FETCH(next < nchunks ? next : c);
-    // LDS -> operands (MFMA layout), multiply
+        for (int wt = 0; wt < WT; ++wt) *reinterpret_cast<u32x4_t*>(my + wt * T::TILE_BYTES + off) = wreg[b][wt][i];
 #pragma unroll
-    for (int s = 0; s < T::STEPS; ++s) {
-      const int off = fr * T::ROW_BYTES + s * 64 + fg * 16;
-      bf16x8_t a[WT];
-#pragma unroll
-      for (int wt = 0; wt < WT; ++wt) a[wt] = *reinterpret_cast<const bf16x8_t*>(my + wt * T::TILE_BYTES + off);
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        const bf16x8_t b = *reinterpret_cast<const bf16x8_t*>(my + (WT + mt) * T::TILE_BYTES + off);
-#pragma unroll
-        for (int wt = 0; wt < WT; ++wt) acc[wt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[wt], b, acc[wt][mt], 0, 0, 0);
+        for (int mt = 0; mt < MT; ++mt) *reinterpret_cast<u32x4_t*>(my + (WT + mt) * T::TILE_BYTES + off) = xreg[b][mt][i];
       }
+      const int ahead = c + DEPTH * NW;
+      SKINNY_FETCH(b, ahead < nchunks ? ahead : c);
+      // LDS -> operands (MFMA layout), multiply
+#pragma unroll
+      for (int s = 0; s < T::STEPS; ++s) {
+        const int off = fr * T::ROW_BYTES + s * 64 + fg * 16;
+        bf16x8_t a[WT];
+#pragma unroll
+        for (int wt = 0; wt < WT; ++wt) a[wt] = *reinterpret_cast<const bf16x8_t*>(my + wt * T::TILE_BYTES + off);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          const bf16x8_t bb = *reinterpret_cast<const bf16x8_t*>(my + (WT + mt) * T::TILE_BYTES + off);
+#pragma unroll
+          for (int wt = 0; wt < WT; ++wt) acc[wt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[wt], bb, acc[wt][mt], 0, 0, 0);
+        }
+      }
+      c += NW;
     }
-    c = next;
   }
 #undef SKINNY_FETCH
 
@@ -230,7 +236,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __re
   }
 }
 
-template <int MT, int KC, int NW, typename TOut, int ACT>
+template <int MT, int KC, int NW, typename TOut, int ACT, int DEPTH = 1>
 static int launch_skinny(const void* x, long ldx, const void* W, long ldw, const void* bias, void* y, long ldy, int M,
                          int N, int K, hipStream_t stream, RopeCacheArgs rc = RopeCacheArgs()) {
   using T = SkinnyTile<KC>;
@@ -238,7 +244,7 @@ static int launch_skinny(const void* x, long ldx, const void* W, long ldw, const
   const size_t stage = (size_t)NW * (WT + MT) * T::TILE_BYTES;
   const size_t red = (size_t)NW * WT * MT * 64 * 4 * sizeof(float);
   const size_t smem = stage > red ? stage : red;
-  auto kernel = gemm_skinny_kernel<MT, KC, NW, TOut, ACT>;
+  auto kernel = gemm_skinny_kernel<MT, KC, NW, TOut, ACT, DEPTH>;
   static bool configured = false;   // per instantiation
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -281,8 +287,12 @@ extern "C" int lmsf_gemm_skinny(const void* x, long ldx, const void* W, long ldw
   rc = act == 1 ? launch_skinny<MT_, KC_, NW_, bf16_t, 1>(x, ldx, W, ldw, bias, y, ldy, M, N, K, stream)       \
                 : launch_skinny<MT_, KC_, NW_, bf16_t, 2>(x, ldx, W, ldw, bias, y, ldy, M, N, K, stream)
     if (mt == 1) {
+      // 8 waves with two chunks each in flight: measured 3 % ahead of 16 waves with one (deeper: slower)
       if (variant == 1) SKG(1, 128, 8);
-      else SKG(1, 64, 16);
+      else if (variant == 3) SKG(1, 64, 16);
+      else   // (variant 2 of the plain product splits K over 8 waves as well: the same order of summation)
+        rc = act == 1 ? launch_skinny<1, 64, 8, bf16_t, 1, 2>(x, ldx, W, ldw, bias, y, ldy, M, N, K, stream)
+                      : launch_skinny<1, 64, 8, bf16_t, 2, 2>(x, ldx, W, ldw, bias, y, ldy, M, N, K, stream);
     } else if (mt == 2) {
       SKG(2, 64, 16);
     } else if (mt == 3) {

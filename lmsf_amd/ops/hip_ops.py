@@ -477,7 +477,8 @@ class HipOps:
         [M, I] in x's dtype. With up to 64 bfloat16 rows the activation is the epilogue of the weight-streaming
         product; otherwise the product and the activation kernel run one after the other. Both ways round
         the two products to the storage type before the activation, so they give the same bits wherever
-        they add up K in the same order."""
+        they add up K in the same order (the default tilings of the fused and the plain product do not: they
+        split K over 8 and over 16 waves)."""
         if weight.dim() != 2 or weight.shape[0] % 2 != 0:
             raise ValueError("linear_gated: weight must be [2 I, K]")
         kinds = {"silu": 1, "gelu": 2}

@@ -324,6 +324,15 @@ def test_linear_gated(ops, ref, M, I, K, kind, bias):
     two = ops.gated_act(ops.linear(x, w, b), kind)
     assert fused.shape == (M, I) and fused.dtype == torch.bfloat16
     if M <= 16 or K <= 512:
+        if 2 < M <= 16:
+            # the default tilings split K over 8 waves (gated) and 16 (plain): equal up to a rounding of the
+            # sums; with the plain product's 8-wave tiling the order of summation is the same and so are the bits
+            assert (fused.float() - two.float()).abs().max().item() <= 2e-2 * max(1.0, two.float().abs().max().item())
+            ops.skinny_variant = 2
+            try:
+                fused, two = ops.linear_gated(x, w, b, kind), ops.gated_act(ops.linear(x, w, b), kind)
+            finally:
+                ops.skinny_variant = 0
         assert torch.equal(fused, two)           # the same order of summation in both
     else:
         # more than 16 rows and a long K: the two may split K differently, which moves a sum by a rounding
