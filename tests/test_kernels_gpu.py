@@ -212,6 +212,23 @@ def test_paged_attention_matrix_core_kernels(ops, ref, shape, window):
     assert torch.allclose(c.float(), b.float(), **tol(torch.bfloat16)), (c.float() - b.float()).abs().max()
 
 
+@pytest.mark.parametrize("shape", MFMA_SHAPES)
+@pytest.mark.parametrize("variant,splits", [(1, 1), (0, 3), (1, 64)])
+def test_matrix_core_attention_other_ways_of_cutting_the_work(ops, ref, shape, variant, splits):
+    """The forms that the planner picks only for other workloads: every wave fetching keys and values for itself
+    (prefill), the keys of a single token in one part, in three, in as many as there are 128-key chunks."""
+    nh, nkv, d, ps, seg_lens, ctx_lens = shape
+    q, kp, vp, bt, seg, pos = _paged_case(torch.bfloat16, nh, nkv, d, ps, seg_lens, ctx_lens, seed=7 * nh + d, spike=True)
+    scale = 1.0 / math.sqrt(d)
+    b = ref.paged_attention(q, kp, vp, bt, seg, pos, nh, nkv, d, scale, 0)
+    ops.prefill_attention_variant, ops.decode_attention_splits = variant, splits
+    try:
+        a = ops.paged_attention(q, kp, vp, bt, seg, pos, nh, nkv, d, scale, 0, kernel="mfma")
+    finally:
+        ops.prefill_attention_variant, ops.decode_attention_splits = 0, 0
+    assert torch.allclose(a.float(), b.float(), **tol(torch.bfloat16)), (a.float() - b.float()).abs().max()
+
+
 def test_matrix_core_attention_refuses_what_it_cannot_do(ops):
     q, kp, vp, bt, seg, pos = _paged_case(torch.bfloat16, 2, 1, 24, 16, [3], [3], seed=1)
     with pytest.raises(ValueError, match="multiple of 16"):
