@@ -11,6 +11,14 @@
 // of that reader's rate, which is why these one or two rows get a kernel of their own.
 // The reference leaves these products to cuBLASLt (tops/src/cublas.rs:29-114).
 //
+// Two more forms take the kernels between two products of a decoder block into the products themselves,
+// where that costs nothing: ACT 4 adds the result, rounded to bfloat16 as a product would store it, to the
+// float32 residual stream in place (every element of the stream belongs to one wave); XN makes x from the
+// stream on the way into LDS, x = bf16(stream * rsqrt(mean(stream^2) + eps) * (w + offset)): every workgroup
+// does the whole row's statistics for itself (a few KB from L2, while its first rows of W are on their way).
+// The addition and the norm are then no kernels of their own (vllm/kernels/layernorm_kernels.cu:41-68 in the
+// reference).
+//
 // A "unit" is what one wave produces: ACT 0: output n (one row of W); ACT 1, 2: output n of the gated form
 // (rows n and N + n: gate and up); ACT 3: the rotation pair (i, i + d/2) of one head of the fused QKV
 // projection (rows head * d + i and head * d + i + d/2).
@@ -20,6 +28,7 @@ typedef __bf16 gemv_bf16x2_t __attribute__((ext_vector_type(2)));
 
 #define GEMV_WAVES 8
 #define GEMV_UNROLL 8   // 16-byte pieces per lane in flight per row: 8 x 512 = 4,096 elements of K
+#define GEMV_XN_MAX_K 8192   // the longest row whose float32 values a workgroup keeps in registers while it sums their squares
 
 // A wave's work is a list of pieces: for each of its units, for each of the unit's rows (one, or two with an
 // epilogue that joins two rows), the row's K in pieces of GEMV_UNROLL x 512 elements. The loads of the next
@@ -29,14 +38,24 @@ struct GemvCursor {
   int unit, row, kb;
 };
 
-template <int NX, int ACT, typename TOut>
+// x as the RMSNorm of the float32 stream (XN): stream [M, K] with row stride ld, weight [K] bfloat16
+struct GemvNorm {
+  const float* stream;
+  long ld;
+  const bf16_t* weight;
+  float eps, offset;
+};
+
+template <int NX, int ACT, typename TOut, bool XN>
 __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_kernel(const bf16_t* __restrict__ x, long ldx,
                                                                const bf16_t* __restrict__ W, long ldw,
                                                                const bf16_t* __restrict__ bias, TOut* __restrict__ y,
-                                                               long ldy, int N, int K, int n_units, RopeCacheArgs rc) {
-  constexpr int ROWS = ACT == 0 ? 1 : 2;
+                                                               long ldy, int N, int K, int n_units, RopeCacheArgs rc,
+                                                               GemvNorm nm) {
+  constexpr int ROWS = (ACT == 0 || ACT == 4) ? 1 : 2;
   extern __shared__ __align__(16) unsigned char lds_raw[];
   bf16_t* xs = reinterpret_cast<bf16_t*>(lds_raw);             // [NX][K]
+  __shared__ float norm_red[GEMV_WAVES][NX];
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
   const int half = rc.d / 2;
   const int unit_step = (int)(gridDim.x * GEMV_WAVES);
@@ -115,6 +134,9 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_kernel(const bf16_t* __r
       }
       if (ACT == 0) {
         y[(long)m * ldy + n] = from_f32<TOut>(a);
+      } else if (ACT == 4) {
+        float* st = reinterpret_cast<float*>(y) + (long)m * ldy + n;   // this form's output is the float32 stream
+        *st += bf16_to_f32(f32_to_bf16(a));
       } else if (ACT == 1 || ACT == 2) {
         // the two products are rounded to the storage type before the activation, as the unfused path stores them
         const float g = bf16_to_f32(f32_to_bf16(a)), u = bf16_to_f32(f32_to_bf16(b));
@@ -158,10 +180,57 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_kernel(const bf16_t* __r
 
   GemvCursor cur = {(int)(blockIdx.x * GEMV_WAVES) + wave, 0, 0};
   uint4 wa[GEMV_UNROLL], wb[GEMV_UNROLL];
-  if (cur.unit < n_units) fetch(cur, wa);
-  for (int i = tid; i < NX * (K / 8); i += GEMV_WAVES * 64) {
-    const int m = i / (K / 8), p = i - m * (K / 8);
-    *reinterpret_cast<uint4*>(xs + (long)m * K + p * 8) = *reinterpret_cast<const uint4*>(x + (long)m * ldx + p * 8);
+  if (XN) {
+    // the stream first (loads come back in the order they were asked for, and these come from L2), then the
+    // first piece of W, then the statistics and the normalised x
+    constexpr int XP = GEMV_XN_MAX_K / (GEMV_WAVES * 64 * 4);   // float4 pieces of a row per thread
+    float4 sv[NX][XP];
+    float ss[NX];
+#pragma unroll
+    for (int m = 0; m < NX; ++m) {
+#pragma unroll
+      for (int j = 0; j < XP; ++j) {
+        const int k = (j * GEMV_WAVES * 64 + tid) * 4;
+        sv[m][j] = k < K ? *reinterpret_cast<const float4*>(nm.stream + (long)m * nm.ld + k) : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+    }
+    if (cur.unit < n_units) fetch(cur, wa);
+#pragma unroll
+    for (int m = 0; m < NX; ++m) {
+      ss[m] = 0.f;
+#pragma unroll
+      for (int j = 0; j < XP; ++j)
+        ss[m] += sv[m][j].x * sv[m][j].x + sv[m][j].y * sv[m][j].y + sv[m][j].z * sv[m][j].z + sv[m][j].w * sv[m][j].w;
+      ss[m] = wave_sum(ss[m]);
+      if (lane == 0) norm_red[wave][m] = ss[m];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int m = 0; m < NX; ++m) {
+      float tot = 0.f;
+#pragma unroll
+      for (int w2 = 0; w2 < GEMV_WAVES; ++w2) tot += norm_red[w2][m];
+      const float inv = rsqrtf(tot / (float)K + nm.eps);
+#pragma unroll
+      for (int j = 0; j < XP; ++j) {
+        const int k = (j * GEMV_WAVES * 64 + tid) * 4;
+        if (k < K) {
+          const uint2 wv = *reinterpret_cast<const uint2*>(nm.weight + k);
+          uint2 o;
+          o.x = pack2_bf16(sv[m][j].x * inv * (__uint_as_float(wv.x << 16) + nm.offset),
+                           sv[m][j].y * inv * (__uint_as_float(wv.x & 0xffff0000u) + nm.offset));
+          o.y = pack2_bf16(sv[m][j].z * inv * (__uint_as_float(wv.y << 16) + nm.offset),
+                           sv[m][j].w * inv * (__uint_as_float(wv.y & 0xffff0000u) + nm.offset));
+          *reinterpret_cast<uint2*>(xs + (long)m * K + k) = o;
+        }
+      }
+    }
+  } else {
+    if (cur.unit < n_units) fetch(cur, wa);
+    for (int i = tid; i < NX * (K / 8); i += GEMV_WAVES * 64) {
+      const int m = i / (K / 8), p = i - m * (K / 8);
+      *reinterpret_cast<uint4*>(xs + (long)m * K + p * 8) = *reinterpret_cast<const uint4*>(x + (long)m * ldx + p * 8);
+    }
   }
   __syncthreads();
   // one piece per half of the loop body, the two register sets taking turns
@@ -182,11 +251,12 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_kernel(const bf16_t* __r
 #undef GEMV_HALF
 }
 
-template <int NX, int ACT, typename TOut>
+template <int NX, int ACT, typename TOut, bool XN = false>
 static int launch_gemv(const void* x, long ldx, const void* W, long ldw, const void* bias, void* y, long ldy, int N,
-                       int K, int n_units, hipStream_t stream, RopeCacheArgs rc = RopeCacheArgs()) {
+                       int K, int n_units, hipStream_t stream, RopeCacheArgs rc = RopeCacheArgs(),
+                       GemvNorm nm = GemvNorm()) {
   const size_t smem = (size_t)NX * K * sizeof(bf16_t);
-  auto kernel = gemv_kernel<NX, ACT, TOut>;
+  auto kernel = gemv_kernel<NX, ACT, TOut, XN>;
   static size_t configured = 0;   // per instantiation: the largest LDS size asked for so far
   if (smem > configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -201,7 +271,7 @@ static int launch_gemv(const void* x, long ldx, const void* W, long ldw, const v
   long blocks = ((long)n_units + GEMV_WAVES - 1) / GEMV_WAVES;
   if (blocks > 2048) blocks = 2048;
   hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(GEMV_WAVES * 64), smem, stream, (const bf16_t*)x, ldx,
-                     (const bf16_t*)W, ldw, (const bf16_t*)bias, (TOut*)y, ldy, N, K, n_units, rc);
+                     (const bf16_t*)W, ldw, (const bf16_t*)bias, (TOut*)y, ldy, N, K, n_units, rc, nm);
   return 0;
 }
 
@@ -261,5 +331,79 @@ extern "C" int lmsf_gemv_qkv_rope_cache(const void* x, long ldx, const void* W, 
                  : launch_gemv<2, 3, bf16_t>(x, ldx, W, ldw, bias, y, ldy, (int)N, K, n_units, stream, rc);
   if (r) return r;
   LMSF_LAUNCH_CHECK("gemv_qkv_rope_cache");
+  return 0;
+}
+
+static int gemv_norm_check(const char* who, const void* stream_f32, long ld, const void* norm_weight, int M, int K) {
+  LMSF_CHECK(stream_f32 && norm_weight, "%s: null pointer", who);
+  LMSF_CHECK(K % 4 == 0 && K <= GEMV_XN_MAX_K, "%s: K=%d must be a multiple of 4, at most %d", who, K, GEMV_XN_MAX_K);
+  LMSF_CHECK(ld >= K && ld % 4 == 0 && lmsf_aligned16(stream_f32) && ((uintptr_t)norm_weight & 7) == 0,
+             "%s: the stream must be 16-byte aligned with a row stride that is a multiple of 4, the norm's weight 8-byte aligned", who);
+  (void)M;
+  return 0;
+}
+
+// y += bf16(x W^T + bias): y is the float32 residual stream [M, N] with row stride ldy, updated in place; the
+// product is rounded to bfloat16 first, as it is where it is stored before it is added. x, W as in lmsf_gemv.
+extern "C" int lmsf_gemv_add(const void* x, long ldx, const void* W, long ldw, const void* bias, void* y, long ldy,
+                             int M, int N, int K, hipStream_t stream) {
+  if (int rc = gemv_check("gemv_add", x, ldx, W, ldw, M, N, K)) return rc;
+  LMSF_CHECK(y != nullptr && ldy >= N, "gemv_add: bad output");
+  if (M == 0) return 0;
+  int r = M == 1 ? launch_gemv<1, 4, float>(x, ldx, W, ldw, bias, y, ldy, N, K, N, stream)
+                 : launch_gemv<2, 4, float>(x, ldx, W, ldw, bias, y, ldy, N, K, N, stream);
+  if (r) return r;
+  LMSF_LAUNCH_CHECK("gemv_add");
+  return 0;
+}
+
+// lmsf_gemv with x = bf16(s * rsqrt(mean(s^2) + eps) * (norm_weight + weight_offset)) made from the float32
+// stream s [M, K] (row stride ld) inside the kernel; norm_weight [K] bfloat16; y bfloat16. K <= 8192.
+extern "C" int lmsf_gemv_normed(const void* stream_f32, long ld, const void* norm_weight, float eps,
+                                float weight_offset, const void* W, long ldw, const void* bias, void* y, long ldy,
+                                int M, int N, int K, int act, hipStream_t stream) {
+  if (int rc = gemv_norm_check("gemv_normed", stream_f32, ld, norm_weight, M, K)) return rc;
+  if (int rc = gemv_check("gemv_normed", W, ldw, W, ldw, M, N, K)) return rc;
+  LMSF_CHECK(y != nullptr && ldy >= N, "gemv_normed: bad output");
+  LMSF_CHECK(act >= 0 && act <= 2, "gemv_normed: unknown activation %d", act);
+  if (M == 0) return 0;
+  GemvNorm nm = {(const float*)stream_f32, ld, (const bf16_t*)norm_weight, eps, weight_offset};
+  int r;
+#define GV(NX_)                                                                                                       \
+  r = act == 1   ? launch_gemv<NX_, 1, bf16_t, true>(nullptr, 0, W, ldw, bias, y, ldy, N, K, N, stream, RopeCacheArgs(), nm) \
+      : act == 2 ? launch_gemv<NX_, 2, bf16_t, true>(nullptr, 0, W, ldw, bias, y, ldy, N, K, N, stream, RopeCacheArgs(), nm) \
+                 : launch_gemv<NX_, 0, bf16_t, true>(nullptr, 0, W, ldw, bias, y, ldy, N, K, N, stream, RopeCacheArgs(), nm)
+  if (M == 1) GV(1); else GV(2);
+#undef GV
+  if (r) return r;
+  LMSF_LAUNCH_CHECK("gemv_normed");
+  return 0;
+}
+
+// lmsf_gemv_qkv_rope_cache with x made from the float32 stream as in lmsf_gemv_normed.
+extern "C" int lmsf_gemv_normed_qkv_rope_cache(const void* stream_f32, long ld, const void* norm_weight, float eps,
+                                               float weight_offset, const void* W, long ldw, const void* bias,
+                                               void* y, long ldy, int M, int K, const int* positions,
+                                               const float* table, int max_pos, const int* slots, void* k_pages,
+                                               void* v_pages, long num_pages, int nh, int nkv, int d, int ps,
+                                               hipStream_t stream) {
+  LMSF_CHECK(y && positions && table && slots && k_pages && v_pages, "gemv_normed_qkv_rope_cache: null pointer");
+  LMSF_CHECK(nh > 0 && nkv > 0 && d >= 2 && d % 2 == 0, "gemv_normed_qkv_rope_cache: head size %d must be even", d);
+  const long N = (long)(nh + 2 * nkv) * d;
+  if (int rc = gemv_norm_check("gemv_normed_qkv_rope_cache", stream_f32, ld, norm_weight, M, K)) return rc;
+  if (int rc = gemv_check("gemv_normed_qkv_rope_cache", W, ldw, W, ldw, M, N, K)) return rc;
+  LMSF_CHECK(ldy >= N, "gemv_normed_qkv_rope_cache: row stride of y below %ld", N);
+  LMSF_CHECK(ps > 0 && num_pages > 0 && max_pos > 0, "gemv_normed_qkv_rope_cache: bad page geometry or empty table");
+  if (M == 0) return 0;
+  RopeCacheArgs rc;
+  rc.positions = positions; rc.table = table; rc.slots = slots;
+  rc.k_pages = (bf16_t*)k_pages; rc.v_pages = (bf16_t*)v_pages;
+  rc.nh = nh; rc.nkv = nkv; rc.d = d; rc.ps = ps;
+  GemvNorm nm = {(const float*)stream_f32, ld, (const bf16_t*)norm_weight, eps, weight_offset};
+  const int n_units = (int)(N / 2);
+  int r = M == 1 ? launch_gemv<1, 3, bf16_t, true>(nullptr, 0, W, ldw, bias, y, ldy, (int)N, K, n_units, stream, rc, nm)
+                 : launch_gemv<2, 3, bf16_t, true>(nullptr, 0, W, ldw, bias, y, ldy, (int)N, K, n_units, stream, rc, nm);
+  if (r) return r;
+  LMSF_LAUNCH_CHECK("gemv_normed_qkv_rope_cache");
   return 0;
 }

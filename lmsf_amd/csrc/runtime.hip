@@ -16,7 +16,7 @@ void lmsf_set_error(const char* fmt, ...) {
 extern "C" const char* lmsf_last_error() { return g_last_error; }
 
 // ABI version of the entry points; the Python side refuses a library that reports another.
-extern "C" int lmsf_abi_version() { return 13; }
+extern "C" int lmsf_abi_version() { return 14; }
 
 // Name of the architecture the current device reports, e.g. "gfx950:sramecc+:xnack-".
 extern "C" int lmsf_device_arch(char* out, int cap) {

@@ -28,3 +28,51 @@ class PendingProduct:
     @property
     def device(self) -> torch.device:
         return self.partials.device
+
+
+class DeferredLinear:
+    """A bfloat16 product x weight^T + bias [M, N] of one or two rows that has not been started: the norm
+    that takes it as its branch runs it as a product that adds its result, rounded to bfloat16, straight
+    into the float32 residual stream, so that the addition is no kernel of its own. Made and taken by the
+    same operations as ``PendingProduct``."""
+
+    __slots__ = ("x", "weight", "bias", "dtype")
+
+    def __init__(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], dtype: torch.dtype):
+        self.x = x
+        self.weight = weight
+        self.bias = bias
+        self.dtype = dtype
+
+    @property
+    def shape(self) -> Tuple[int, int]:
+        return (self.x.shape[0], self.weight.shape[0])
+
+    @property
+    def device(self) -> torch.device:
+        return self.x.device
+
+
+class NormedStream:
+    """The RMSNorm of the float32 residual stream [M, H], M one or two, not computed yet: the product that
+    takes it (``HipOps.qkv_rope_cache``, ``HipOps.linear_gated``) normalises the row while it brings it into
+    LDS. ``HipOps.add_rms_norm(..., defer_ok=True)`` makes one; the stream must not change before the
+    product has run. ``HipOps.materialize`` runs the norm."""
+
+    __slots__ = ("stream", "weight", "eps", "weight_offset", "dtype")
+
+    def __init__(self, stream: torch.Tensor, weight: torch.Tensor, eps: float, weight_offset: float,
+                 dtype: torch.dtype):
+        self.stream = stream
+        self.weight = weight
+        self.eps = eps
+        self.weight_offset = weight_offset
+        self.dtype = dtype
+
+    @property
+    def shape(self) -> Tuple[int, int]:
+        return tuple(self.stream.shape)
+
+    @property
+    def device(self) -> torch.device:
+        return self.stream.device

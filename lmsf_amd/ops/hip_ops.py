@@ -11,7 +11,7 @@ from typing import Optional
 import torch
 
 from . import library
-from .handles import PendingProduct
+from .handles import DeferredLinear, NormedStream, PendingProduct
 
 F32 = 0
 BF16 = 1
@@ -50,6 +50,7 @@ class HipOps:
         self.use_library_gemm = True   # bfloat16 matrix products of many rows go to the BLAS library
         self.prefill_attention_variant = 0   # 0: keys and values staged in LDS; 1: fetched by every wave for itself
         self.decode_attention_splits = 0     # 0: chosen from the batch and the context; n: at most n splits of the keys
+        self.fuse_stream_rows = 1            # with up to this many rows the residual addition and the norm run inside the products (0: never)
         self.gemv_max_rows = 2               # products of up to this many rows stream W without the matrix cores (0: never)
         self.skinny_variant = 0        # tiling of the few-rows kernel (0: default; others for tuning)
         self.skinny_max_rows = 16      # rows up to which the few-rows kernel beats the library (measured)
@@ -107,15 +108,35 @@ class HipOps:
 
     def add_rms_norm(self, branch: Optional[torch.Tensor], residual: Optional[torch.Tensor], weight: torch.Tensor,
                      eps: float, out_dtype: torch.dtype, rows: Optional[torch.Tensor] = None,
-                     weight_offset: float = 0.0) -> torch.Tensor:
+                     weight_offset: float = 0.0, defer_ok: bool = False):
         """out = rms_norm(branch + residual) * (weight + weight_offset).
 
         ``residual`` (float32 [N, H]) is updated to the sum in place when both operands are given
         and ``rows`` is None. ``rows`` (int32 [R]) selects input rows; the output then has R rows.
-        ``branch`` may be a ``PendingProduct``: its partial sums are added up on the way in.
+        ``branch`` may be a ``PendingProduct``: its partial sums are added up on the way in; or a
+        ``DeferredLinear``, which then runs as a product that adds into ``residual``. With ``defer_ok``
+        the caller takes a ``NormedStream`` as well (one or two rows, nothing left to add).
         """
         if isinstance(branch, PendingProduct):
             return self._add_rms_norm_pending(branch, residual, weight, eps, out_dtype, rows, weight_offset)
+        if isinstance(branch, DeferredLinear):
+            if (rows is None and residual is not None and residual.dtype == torch.float32 and residual.is_contiguous()
+                    and tuple(residual.shape) == branch.shape):
+                self._dev(branch.x, branch.weight, branch.bias, residual)
+                M, N = branch.shape
+                self._check(self.lib.lmsf_gemv_add(_ptr(branch.x), branch.x.stride(0), _ptr(branch.weight),
+                                                   branch.weight.stride(0), _ptr(branch.bias), _ptr(residual),
+                                                   residual.stride(0), M, N, branch.x.shape[1], self._stream()))
+                branch = None
+            else:
+                branch = self.materialize(branch)
+        if (defer_ok and branch is None and rows is None and residual is not None and out_dtype == torch.bfloat16
+                and 0 < residual.shape[0] <= min(self.fuse_stream_rows, self.gemv_max_rows)
+                and residual.dtype == torch.float32 and residual.dim() == 2 and residual.is_contiguous()
+                and weight.dtype == torch.bfloat16 and weight.is_contiguous() and weight.shape == (residual.shape[1],)
+                and residual.shape[1] % 8 == 0 and residual.shape[1] <= 8192 and residual.data_ptr() % 16 == 0
+                and weight.data_ptr() % 8 == 0):
+            return NormedStream(residual, weight, float(eps), float(weight_offset), out_dtype)
         self._dev(branch, residual, weight, rows)
         ref = branch if branch is not None else residual
         if ref is None:
@@ -159,7 +180,12 @@ class HipOps:
         return out
 
     def materialize(self, y):
-        """The tensor behind ``y``: ``y`` itself, or the finished sum of a ``PendingProduct``."""
+        """The tensor behind ``y``: ``y`` itself, the finished sum of a ``PendingProduct``, the product of a
+        ``DeferredLinear`` or the norm of a ``NormedStream``."""
+        if isinstance(y, DeferredLinear):
+            return self.linear(y.x, y.weight, y.bias, out_dtype=y.dtype)
+        if isinstance(y, NormedStream):
+            return self.add_rms_norm(None, y.stream, y.weight, y.eps, y.dtype, weight_offset=y.weight_offset)
         if not isinstance(y, PendingProduct):
             return y
         M, N = y.shape
@@ -207,32 +233,53 @@ class HipOps:
             q, k, v, _code(qkv.dtype), N, qkv.stride(0), _ptr(positions), _ptr(table), rot_dim, 1 if neox else 0,
             max_pos, _ptr(slots), _ptr(k_pages), _ptr(v_pages), num_pages, nh, nkv, d, ps, self._stream()))
 
+    def _check_qkv_fused(self, bias, weight, N, table, d, positions, slots, M, k_pages, v_pages, nkv):
+        """Operand checks of the fused QKV forms; returns (pages, page size)."""
+        if bias is not None and (bias.shape != (N,) or bias.dtype != weight.dtype or not bias.is_contiguous()):
+            raise ValueError("qkv_rope_cache: bias must be [%d] of the weight's dtype" % N)
+        if table.dtype != torch.float32 or table.dim() != 2 or table.shape[1] != d or not table.is_contiguous():
+            raise ValueError("rotary table must be contiguous float32 [max_pos, %d]" % d)
+        self._i32(positions, "positions", M)
+        self._i32(slots, "slots", M)
+        if k_pages.dim() != 4 or k_pages.shape[1] != nkv or k_pages.shape[3] != d or not k_pages.is_contiguous():
+            raise ValueError("k_pages must be contiguous [pages, %d, page_size, %d]" % (nkv, d))
+        num_pages, ps = k_pages.shape[0], k_pages.shape[2]
+        if v_pages is None or tuple(v_pages.shape) != (num_pages, nkv, d, ps) or not v_pages.is_contiguous() \
+                or v_pages.dtype != torch.bfloat16:
+            raise ValueError("v_pages must be contiguous bfloat16 [%d, %d, %d, %d]" % (num_pages, nkv, d, ps))
+        return num_pages, ps
+
     def qkv_rope_cache(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], nh: int, nkv: int,
                        d: int, positions: torch.Tensor, table: Optional[torch.Tensor], rot_dim: int, neox: bool,
                        slots: Optional[torch.Tensor], k_pages: Optional[torch.Tensor],
                        v_pages: Optional[torch.Tensor]) -> torch.Tensor:
         """The fused QKV projection, the rotation of its q and k heads and the write of k and v into the
         pages: ``linear`` followed by ``rope_cache_write``, with the same results. With few bfloat16 rows and
-        a NeoX rotation over the whole head, the rotation and the write are the product's epilogue."""
+        a NeoX rotation over the whole head, the rotation and the write are the product's epilogue. ``x`` may
+        be a ``NormedStream``."""
         M, K = x.shape
         N = (nh + 2 * nkv) * d
+        if isinstance(x, NormedStream):
+            if not (table is not None and slots is not None and neox and rot_dim == d and d % 32 == 0
+                    and weight.dtype == torch.bfloat16 and tuple(weight.shape) == (N, K) and weight.stride(1) == 1
+                    and weight.stride(0) % 8 == 0 and weight.data_ptr() % 16 == 0 and self._gemv_ok(M, K)
+                    and k_pages is not None and k_pages.dtype == torch.bfloat16):
+                return self.qkv_rope_cache(self.materialize(x), weight, bias, nh, nkv, d, positions, table, rot_dim,
+                                           neox, slots, k_pages, v_pages)
+            self._dev(x.stream, x.weight, weight, bias, positions, table, slots, k_pages, v_pages)
+            num_pages, ps = self._check_qkv_fused(bias, weight, N, table, d, positions, slots, M, k_pages, v_pages, nkv)
+            y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+            self._check(self.lib.lmsf_gemv_normed_qkv_rope_cache(
+                _ptr(x.stream), x.stream.stride(0), _ptr(x.weight), x.eps, x.weight_offset, _ptr(weight),
+                weight.stride(0), _ptr(bias), _ptr(y), y.stride(0), M, K, _ptr(positions), _ptr(table), table.shape[0],
+                _ptr(slots), _ptr(k_pages), _ptr(v_pages), num_pages, nh, nkv, d, ps, self._stream()))
+            return y
         if (table is not None and slots is not None and neox and rot_dim == d and d % 32 == 0
                 and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and 0 < M <= self.skinny_max_rows
                 and tuple(weight.shape) == (N, K) and x.stride(1) == 1 and weight.stride(1) == 1
                 and self._skinny_ok(x, weight) and k_pages is not None and k_pages.dtype == torch.bfloat16):
             self._dev(x, weight, bias, positions, table, slots, k_pages, v_pages)
-            if bias is not None and (bias.shape != (N,) or bias.dtype != weight.dtype or not bias.is_contiguous()):
-                raise ValueError("qkv_rope_cache: bias must be [%d] of the weight's dtype" % N)
-            if table.dtype != torch.float32 or table.dim() != 2 or table.shape[1] != d or not table.is_contiguous():
-                raise ValueError("rotary table must be contiguous float32 [max_pos, %d]" % d)
-            self._i32(positions, "positions", M)
-            self._i32(slots, "slots", M)
-            if k_pages.dim() != 4 or k_pages.shape[1] != nkv or k_pages.shape[3] != d or not k_pages.is_contiguous():
-                raise ValueError("k_pages must be contiguous [pages, %d, page_size, %d]" % (nkv, d))
-            num_pages, ps = k_pages.shape[0], k_pages.shape[2]
-            if v_pages is None or tuple(v_pages.shape) != (num_pages, nkv, d, ps) or not v_pages.is_contiguous() \
-                    or v_pages.dtype != torch.bfloat16:
-                raise ValueError("v_pages must be contiguous bfloat16 [%d, %d, %d, %d]" % (num_pages, nkv, d, ps))
+            num_pages, ps = self._check_qkv_fused(bias, weight, N, table, d, positions, slots, M, k_pages, v_pages, nkv)
             y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
             if M <= self.gemv_max_rows and self._gemv_ok(M, K):
                 self._check(self.lib.lmsf_gemv_qkv_rope_cache(
@@ -245,7 +292,7 @@ class HipOps:
                 _ptr(positions), _ptr(table), table.shape[0], _ptr(slots), _ptr(k_pages), _ptr(v_pages), num_pages,
                 nh, nkv, d, ps, self.skinny_variant, self._stream()))
             return y
-        y = self.linear(x, weight, bias, pending_ok=True)
+        y = self.linear(x, weight, bias, pending_ok=M > self.fuse_stream_rows)
         if isinstance(y, PendingProduct):
             # 17 to 64 rows with K split: the rotation and the cache write add up the partial sums themselves
             if (table is None and slots is None) or tuple(weight.shape) != (N, K):
@@ -441,6 +488,9 @@ class HipOps:
         both_bf16 = x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
         if both_bf16 and self.skinny_max_rows < M <= 64 and self._mid_ok(x, weight):
             return self._linear_mid(x, weight, bias, 0, out_dtype, pending_ok and out_dtype == torch.bfloat16)
+        if (pending_ok and both_bf16 and out_dtype == torch.bfloat16 and self._skinny_ok(x, weight)
+                and 0 < M <= min(self.fuse_stream_rows, self.gemv_max_rows) and self._gemv_ok(M, K)):
+            return DeferredLinear(x, weight, bias, out_dtype)
         if both_bf16 and 0 < M <= min(1, self.gemv_max_rows) and self._skinny_ok(x, weight) and self._gemv_ok(M, K) \
                 and N * K <= 2 ** 28:
             # one row: a pure stream of W (with two rows only the fused forms gain; the LM head's matrix is large
@@ -485,6 +535,19 @@ class HipOps:
         if kind not in kinds:
             raise ValueError("unknown activation %r (known: %s)" % (kind, ", ".join(kinds)))
         M, I = x.shape[0], weight.shape[0] // 2
+        if isinstance(x, NormedStream):
+            K = x.shape[1]
+            if not (weight.dtype == torch.bfloat16 and weight.shape[1] == K and weight.stride(1) == 1
+                    and weight.stride(0) % 8 == 0 and weight.data_ptr() % 16 == 0 and self._gemv_ok(M, K)):
+                return self.linear_gated(self.materialize(x), weight, bias, kind)
+            self._dev(x.stream, x.weight, weight, bias)
+            if bias is not None and (bias.shape != (2 * I,) or bias.dtype != weight.dtype or not bias.is_contiguous()):
+                raise ValueError("linear_gated: bias must be [%d] of the weight's dtype" % (2 * I))
+            y = torch.empty((M, I), dtype=torch.bfloat16, device=x.device)
+            self._check(self.lib.lmsf_gemv_normed(_ptr(x.stream), x.stream.stride(0), _ptr(x.weight), x.eps,
+                                                  x.weight_offset, _ptr(weight), weight.stride(0), _ptr(bias), _ptr(y),
+                                                  y.stride(0), M, I, K, kinds[kind], self._stream()))
+            return y
         if (x.dim() == 2 and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and 0 < M <= self.skinny_max_rows
                 and x.shape[1] == weight.shape[1] and x.stride(1) == 1 and weight.stride(1) == 1
                 and self._skinny_ok(x, weight)):

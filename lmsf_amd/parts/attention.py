@@ -50,6 +50,11 @@ class PagedAttention(Mixer):
 
     may_return_pending = True
 
+    @property
+    def accepts_normed(self) -> bool:
+        # the fused projection takes the norm into itself; an encoding that acts on the projections needs h
+        return self.position is None or hasattr(self.position, "rotary_table")
+
     def forward(self, h: torch.Tensor, ctx, binding: CacheBinding, pending_ok: bool = False):
         ops = self.rt.ops
         group = ctx.groups[binding.group]

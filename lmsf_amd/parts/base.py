@@ -139,6 +139,13 @@ class Part:
     may_return_pending = False
     accepts_pending = False
 
+    # A norm whose ``forward_add`` takes ``defer_ok=True`` and may then return the norm not yet computed
+    # (ops.handles.NormedStream) sets ``may_defer``; a mixer or feed-forward whose ``forward`` takes such an
+    # ``h`` (it hands it to ``rt.ops.qkv_rope_cache`` or ``rt.ops.linear_gated``, or calls ``rt.ops.materialize``
+    # first) sets ``accepts_normed``. A block asks for a deferred norm only where both say so.
+    may_defer = False
+    accepts_normed = False
+
     def __init__(self, prefix: str, rt: Runtime):
         self.prefix = prefix
         self.rt = rt
@@ -162,7 +169,8 @@ class Part:
 class Norm(Part):
     """forward(x): norm of x [N, H] in the runtime dtype.
     forward_add(branch, residual): residual (float32, in place) += branch; returns norm(residual).
-    branch None: returns norm(residual). rows: compute only these rows (residual untouched)."""
+    branch None: returns norm(residual). rows: compute only these rows (residual untouched).
+    A norm with ``may_defer`` also takes ``defer_ok``."""
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         raise NotImplementedError

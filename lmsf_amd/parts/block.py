@@ -14,7 +14,8 @@ class PreNormResidualBlock(Block):
     the norm that follows it (vllm/kernels/layernorm_kernels.cu:41-68): the block receives the
     previous block's output not yet added, and returns its feed-forward output not yet added.
     Where the norm that follows accepts it, the o and down products may stay unfinished
-    (``PendingProduct``) and the norm's kernel adds up their partial sums.
+    (``PendingProduct``) and the norm's kernel adds up their partial sums; where a norm may defer
+    its work and the part after it takes that, the norm runs inside that part's first product.
     """
 
     graph_safe = True
@@ -27,13 +28,19 @@ class PreNormResidualBlock(Block):
 
     def forward(self, branch: Optional[torch.Tensor], residual: torch.Tensor, ctx,
                 binding: CacheBinding) -> torch.Tensor:
-        post = self.norms["post_mixer"]
-        h = self.norms["input"].forward_add(branch, residual)
+        first, post = self.norms["input"], self.norms["post_mixer"]
+        if first.may_defer and self.mixer.accepts_normed:
+            h = first.forward_add(branch, residual, defer_ok=True)
+        else:
+            h = first.forward_add(branch, residual)
         if self.mixer.may_return_pending and post.accepts_pending:
             a = self.mixer.forward(h, ctx, binding, pending_ok=True)
         else:
             a = self.mixer.forward(h, ctx, binding)
-        h = post.forward_add(a, residual)
+        if post.may_defer and self.feed_forward.accepts_normed:
+            h = post.forward_add(a, residual, defer_ok=True)
+        else:
+            h = post.forward_add(a, residual)
         if self.feed_forward.may_return_pending and self.pending_output_ok:
             return self.feed_forward.forward(h, pending_ok=True)
         return self.feed_forward.forward(h)

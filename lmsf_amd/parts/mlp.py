@@ -30,6 +30,7 @@ class GatedMLP(FeedForward):
         return [self.gate_up, self.down]
 
     may_return_pending = True
+    accepts_normed = True
 
     def forward(self, h: torch.Tensor, pending_ok: bool = False):
         a = self.rt.ops.linear_gated(h, self.gate_up.weight, self.gate_up.bias, self.activation)

@@ -16,6 +16,7 @@ from .base import Norm, Runtime, TensorDecl, register_part
 class RMSNorm(Norm):
     graph_safe = True
     accepts_pending = True
+    may_defer = True
 
     def __init__(self, prefix: str, rt: Runtime, size: int, eps: float, weight_offset: float = 0.0,
                  weight_name: str = "weight"):
@@ -38,6 +39,9 @@ class RMSNorm(Norm):
                                         weight_offset=self.weight_offset)
 
     def forward_add(self, branch: Optional[torch.Tensor], residual: torch.Tensor,
-                    rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+                    rows: Optional[torch.Tensor] = None, defer_ok: bool = False):
+        if defer_ok:
+            return self.rt.ops.add_rms_norm(branch, residual, self.weight, self.eps, self.rt.dtype, rows=rows,
+                                            weight_offset=self.weight_offset, defer_ok=True)
         return self.rt.ops.add_rms_norm(branch, residual, self.weight, self.eps, self.rt.dtype, rows=rows,
                                         weight_offset=self.weight_offset)

@@ -62,7 +62,7 @@ class TorchOps:
     def bad_token_seen(self):
         return False
 
-    def add_rms_norm(self, branch, residual, weight, eps, out_dtype, rows=None, weight_offset=0.0):
+    def add_rms_norm(self, branch, residual, weight, eps, out_dtype, rows=None, weight_offset=0.0, defer_ok=False):
         x = None
         if branch is not None:
             x = branch.to(torch.float32)
