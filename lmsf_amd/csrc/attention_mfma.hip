@@ -732,14 +732,20 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
 }
 
 // out[tok, head, :] = sum_s 2^(m_s - M) o_s / sum_s 2^(m_s - M) l_s over the splits that have keys.
-__global__ __launch_bounds__(256) void attn_decode_reduce_kernel(
+// One workgroup of 256 threads per (token, head): d / 4 lanes hold four output elements each, and the
+// 256 / (d / 4) groups of such lanes take every G-th split, so that the loads of many splits are in flight at
+// once (with 64 splits a single loop over them costs more than the attention itself); the groups' sums are
+// added in a fixed order.
+#define REDUCE_THREADS 256
+#define REDUCE_SERIAL_SPLITS 16   // up to this many splits a thread per output element that loops over them is faster
+__global__ __launch_bounds__(256) void attn_decode_reduce_serial_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, bf16_t* __restrict__ out, long out_stride,
     const int* __restrict__ tok_idx, const int* __restrict__ pos, int nh, int d, int window, int chunk, int n_splits) {
   const int i_tok = blockIdx.x, head = blockIdx.y;
   const int tok = tok_idx ? tok_idx[i_tok] : i_tok;
   const int p = pos[tok];
   const int lo = window > 0 ? max(0, p - window + 1) : 0;
-  const int s0 = ((lo / 32) * 32) / chunk, s1 = min(n_splits - 1, p / chunk);   // splits s0 .. s1 have keys
+  const int s0 = ((lo / 32) * 32) / chunk, s1 = min(n_splits - 1, p / chunk);
   const long base = ((long)i_tok * nh + head) * n_splits;
   float M = -INFINITY;
   for (int s = s0; s <= s1; ++s) M = fmaxf(M, part_ml[(base + s) * 2]);
@@ -750,6 +756,55 @@ __global__ __launch_bounds__(256) void attn_decode_reduce_kernel(
     float o = 0.f;
     for (int s = s0; s <= s1; ++s) o += exp2f(part_ml[(base + s) * 2] - M) * part_o[(base + s) * d + dv];
     out[(long)tok * out_stride + (long)head * d + dv] = f32_to_bf16(o * inv);
+  }
+}
+
+__global__ __launch_bounds__(REDUCE_THREADS) void attn_decode_reduce_kernel(
+    const float* __restrict__ part_o, const float* __restrict__ part_ml, bf16_t* __restrict__ out, long out_stride,
+    const int* __restrict__ tok_idx, const int* __restrict__ pos, int nh, int d, int window, int chunk, int n_splits) {
+  __shared__ float red_max[REDUCE_THREADS / 64];
+  __shared__ __align__(16) float red_o[REDUCE_THREADS * 4];   // [G][d], G * d <= 1024
+  __shared__ float red_l[REDUCE_THREADS];
+  const int i_tok = blockIdx.x, head = blockIdx.y, tid = threadIdx.x;
+  const int tok = tok_idx ? tok_idx[i_tok] : i_tok;
+  const int p = pos[tok];
+  const int lo = window > 0 ? max(0, p - window + 1) : 0;
+  const int s0 = ((lo / 32) * 32) / chunk, s1 = min(n_splits - 1, p / chunk);   // splits s0 .. s1 have keys
+  const long base = ((long)i_tok * nh + head) * n_splits;
+  float M = -INFINITY;
+  for (int s = s0 + tid; s <= s1; s += REDUCE_THREADS) M = fmaxf(M, part_ml[(base + s) * 2]);
+  M = wave_max(M);
+  if ((tid & 63) == 0) red_max[tid >> 6] = M;
+  __syncthreads();
+  M = fmaxf(fmaxf(red_max[0], red_max[1]), fmaxf(red_max[2], red_max[3]));
+  const int L = d / 4, G = REDUCE_THREADS / L;   // d is a multiple of 16, at most 256: G >= 4
+  const int g = tid / L, lane = tid - g * L;
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  float ls = 0.f;
+  if (g < G) {
+#pragma unroll 4
+    for (int s = s0 + g; s <= s1; s += G) {
+      const float2 ml = *reinterpret_cast<const float2*>(part_ml + (base + s) * 2);
+      const float4 o = *reinterpret_cast<const float4*>(part_o + (base + s) * d + lane * 4);
+      const float w = exp2f(ml.x - M);
+      ls += w * ml.y;
+      acc.x += w * o.x; acc.y += w * o.y; acc.z += w * o.z; acc.w += w * o.w;
+    }
+    *reinterpret_cast<float4*>(red_o + (g * d + lane * 4)) = acc;
+    if (lane == 0) red_l[g] = ls;
+  }
+  __syncthreads();
+  if (g == 0) {
+    for (int gg = 1; gg < G; ++gg) {
+      const float4 o = *reinterpret_cast<const float4*>(red_o + (gg * d + lane * 4));
+      acc.x += o.x; acc.y += o.y; acc.z += o.z; acc.w += o.w;
+      ls += red_l[gg];
+    }
+    const float inv = 1.0f / ls;
+    uint2 packed;
+    packed.x = pack2_bf16(acc.x * inv, acc.y * inv);
+    packed.y = pack2_bf16(acc.z * inv, acc.w * inv);
+    *reinterpret_cast<uint2*>(out + (long)tok * out_stride + (long)head * d + lane * 4) = packed;
   }
 }
 
@@ -885,7 +940,7 @@ extern "C" int lmsf_paged_attention_decode_mfma(const void* q, long q_stride, vo
   if (int rc = check_common("paged_attention_decode", q, out, k_pages, v_pages, block_tables, seg, pos, q_stride,
                             out_stride, num_pages, btw, nh, nkv, d, ps, window))
     return rc;
-  LMSF_CHECK(n >= 0 && scratch != nullptr, "paged_attention_decode: bad arguments");
+  LMSF_CHECK(n >= 0 && scratch != nullptr && lmsf_aligned16(scratch), "paged_attention_decode: bad arguments (scratch must be 16-byte aligned)");
   LMSF_CHECK(chunk > 0 && chunk % 128 == 0 && n_splits > 0 && n_splits <= 65535,
              "paged_attention_decode: chunk %d must be a positive multiple of 128 and splits %d in [1, 65535]", chunk,
              n_splits);
@@ -916,8 +971,11 @@ extern "C" int lmsf_paged_attention_decode_mfma(const void* q, long q_stride, vo
   if (rc) return rc;
   LMSF_LAUNCH_CHECK("paged_attention_decode");
   if (n_splits == 1) return 0;
-  int threads = (d + 63) / 64 * 64;
-  hipLaunchKernelGGL(attn_decode_reduce_kernel, dim3(n, nh), dim3(threads), 0, stream, part_o, part_ml, (bf16_t*)out,
+  if (n_splits <= REDUCE_SERIAL_SPLITS)
+    hipLaunchKernelGGL(attn_decode_reduce_serial_kernel, dim3(n, nh), dim3((d + 63) / 64 * 64), 0, stream, part_o,
+                       part_ml, (bf16_t*)out, out_stride, tok_idx, pos, nh, d, window, chunk, n_splits);
+  else
+    hipLaunchKernelGGL(attn_decode_reduce_kernel, dim3(n, nh), dim3(REDUCE_THREADS), 0, stream, part_o, part_ml, (bf16_t*)out,
                      out_stride, tok_idx, pos, nh, d, window, chunk, n_splits);
   LMSF_LAUNCH_CHECK("paged_attention_decode_reduce");
   return 0;

@@ -229,6 +229,24 @@ def test_matrix_core_attention_other_ways_of_cutting_the_work(ops, ref, shape, v
     assert torch.allclose(a.float(), b.float(), **tol(torch.bfloat16)), (a.float() - b.float()).abs().max()
 
 
+@pytest.mark.parametrize("nh,nkv,d,ps", [(4, 2, 16, 8), (5, 5, 48, 16), (6, 3, 80, 4), (8, 2, 128, 16), (2, 1, 256, 32), (3, 1, 112, 16)])
+@pytest.mark.parametrize("window", [0, 700])
+def test_decode_attention_reduction_over_many_splits(ops, ref, nh, nkv, d, ps, window):
+    """More than 16 splits of a long context are added up by groups of lanes that take every G-th split (up to
+    16: one loop per output element); requests of other lengths in the same call use fewer of the splits, and a
+    window leaves the first ones without keys."""
+    ctx_lens = [2500, 1, 2300, 130]
+    q, kp, vp, bt, seg, pos = _paged_case(torch.bfloat16, nh, nkv, d, ps, [1, 1, 1, 1], ctx_lens, seed=nh + d, spike=True)
+    scale = 1.0 / math.sqrt(d)
+    b = ref.paged_attention(q, kp, vp, bt, seg, pos, nh, nkv, d, scale, window)
+    ops.decode_attention_splits = 64
+    try:
+        a = ops.paged_attention(q, kp, vp, bt, seg, pos, nh, nkv, d, scale, window, kernel="mfma")
+    finally:
+        ops.decode_attention_splits = 0
+    assert torch.allclose(a.float(), b.float(), **tol(torch.bfloat16)), (a.float() - b.float()).abs().max()
+
+
 def test_matrix_core_attention_refuses_what_it_cannot_do(ops):
     q, kp, vp, bt, seg, pos = _paged_case(torch.bfloat16, 2, 1, 24, 16, [3], [3], seed=1)
     with pytest.raises(ValueError, match="multiple of 16"):
