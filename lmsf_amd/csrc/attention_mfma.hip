@@ -280,12 +280,15 @@ __device__ __forceinline__ unsigned lds_address(const void* p) {
 // operands in a stage) is worked out before the loop, pages are powers of two (shifts, no divisions), the
 // mask is only applied in steps that touch the diagonal or the window's edge, and the accumulators are
 // only rescaled when a row's maximum has moved.
+// How far (in powers of two) a row's scores may rise above the reference of its exponentials before the
+// accumulators are rescaled: 2^24 times a few thousand keys times the values stays far inside float32.
+#define PREFILL_LAZY_LOG2 24.0f
 template <int DPAD, int NQB, int STAGES>
 __global__ __launch_bounds__(256) void attn_prefill_dma_kernel(
     const bf16_t* __restrict__ q, long q_stride, bf16_t* __restrict__ out, long out_stride,
     const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages, const int* __restrict__ block_tables,
     int btw, const int* __restrict__ tiles, const int* __restrict__ seg, const int* __restrict__ pos, int nh, int nkv,
-    int d, int ps_log2, float scale_log2, int window, int HB, int n_hb, int bt_cap) {
+    int d, int ps_log2, float scale_log2, int window, int HB, int n_hb, int bt_cap, int n_cus) {
   constexpr int DS = DPAD / 32, DV = DPAD / 16;
   constexpr int PR = DPAD / 8;                   // 16-byte pieces per K row
   constexpr bool PR_POW2 = (PR & (PR - 1)) == 0;
@@ -294,10 +297,20 @@ __global__ __launch_bounds__(256) void attn_prefill_dma_kernel(
   constexpr int LPW = DPAD / 32;                 // transfers per wave and stage (DPAD / 8 in all)
   extern __shared__ __align__(16) unsigned char lds_raw[];   // [STAGES][STAGE], then the block table
   int* lds_bt = reinterpret_cast<int*>(lds_raw + STAGES * STAGE);
-  const int tile = blockIdx.x;
-  const int kvh = blockIdx.y / n_hb, hb = blockIdx.y - kvh * n_hb;
+  // Which (tile, kv head, block of heads) this workgroup takes. The caller lists the tiles with the most keys
+  // first, and workgroups start in the order of their index, so long tiles start first and short ones fill the
+  // gaps. When all workgroups fit on the chip at once, two to a compute unit, what counts is which two share
+  // one: workgroup n and workgroup n + n_cus do when the workgroups are placed in order, so the second n_cus take
+  // the items from the light end, and the longest tile is paired with the shortest. Items of one tile differ in
+  // the kv head, so that neighbours in the order (which go to different dies) read different keys and values,
+  // and each die keeps to few kv heads.
+  const int n_y = nkv * n_hb, n_items = gridDim.x;
+  int item = blockIdx.x;
+  if (n_items <= 2 * n_cus && item >= n_cus) item = n_items - 1 - (item - n_cus);
+  const int tile = item / n_y, y = item - tile * n_y;
+  const int kvh = y / n_hb, hb = y - kvh * n_hb;
   const int n_rep = nh / nkv;
-  const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, c = l & 15, g = l >> 4;
+  const int tid = threadIdx.x, w = __builtin_amdgcn_readfirstlane(tid >> 6), l = tid & 63, c = l & 15, g = l >> 4;
   const int t0 = tiles[2 * tile], ntok = tiles[2 * tile + 1];
   const int* bt = block_tables + (long)seg[t0] * btw;
   const int ps = 1 << ps_log2, pm = ps - 1;
@@ -360,11 +373,13 @@ __global__ __launch_bounds__(256) void attn_prefill_dma_kernel(
   }
 
   // what this lane moves in every step: transfer i of the wave covers pieces j * 64 .. j * 64 + 63 of a stage,
-  // j = w + 4 i; the first DPAD / 16 transfers are the K tile, the others the V^T tile
-  const long page_stride = (long)nkv * d << ps_log2;   // elements per page, K and V alike
-  int t_key[LPW], t_mul[LPW];
-  long t_fixed[LPW];
-  const bf16_t* t_base[LPW];
+  // j = w + 4 i; the first DPAD / 16 transfers are the K tile, the others the V^T tile. A step starts at a
+  // multiple of 32 keys and pages are powers of two, so a key's block and its place in the page are each a
+  // part that is the same for the whole wave (from the step) plus a part that never changes (from the lane).
+  const unsigned page_stride = (unsigned)(nkv * d) << ps_log2;   // elements per page, K and V alike
+  int t_blk[LPW];              // the lane's part of the block index
+  int t_mul[LPW];              // elements per key within a page: d for K, 1 for V^T (the same for the wave)
+  const bf16_t* t_base[LPW];   // the pages plus everything of the offset that never changes
 #pragma unroll
   for (int i = 0; i < LPW; ++i) {
     const int j = w + 4 * i;
@@ -379,20 +394,18 @@ __global__ __launch_bounds__(256) void attn_prefill_dma_kernel(
         if (col >= PR) col -= PR;
       }
       if (col * 8 >= d) col = 0;                   // beyond the head: any finite data, the query is zero there
-      t_key[i] = row;
+      t_blk[i] = row >> ps_log2;
       t_mul[i] = d;
-      t_fixed[i] = ((long)kvh * d << ps_log2) + col * 8;
-      t_base[i] = k_pages;
+      t_base[i] = k_pages + (((long)kvh * d << ps_log2) + col * 8 + (long)(row & pm) * d);
     } else {
       const int P = (j - DPAD / 16) * 64 + l;
       int dv = P >> 2;
       const int slot = P & 3;
       const int piece = (slot - (dv >> 2)) & 3;
-      if (dv >= d) dv = 0;                         // rows beyond the head are never read
-      t_key[i] = piece * 8;
+      if (dv >= d) dv = 0;                         // rows beyond the head: any finite data, their results are dropped
+      t_blk[i] = (piece * 8) >> ps_log2;
       t_mul[i] = 1;
-      t_fixed[i] = ((long)(kvh * d + dv) << ps_log2);
-      t_base[i] = v_pages;
+      t_base[i] = v_pages + (((long)(kvh * d + dv) << ps_log2) + ((piece * 8) & pm));
     }
   }
   // where this lane reads its operands in a stage (bytes)
@@ -425,12 +438,12 @@ __global__ __launch_bounds__(256) void attn_prefill_dma_kernel(
 
   // this wave's transfers of the step that starts at key kb, into the stage at byte ``stage_byte``
   auto issue = [&](int kb, int stage_byte) {
+    const int blk_step = (kb >> ps_log2) - blk0, in_page = kb & pm;   // the step's parts, the same for the wave
 #pragma unroll
     for (int i = 0; i < LPW; ++i) {
-      const int key = kb + t_key[i];
-      int blk = (key >> ps_log2) - blk0;
-      blk = min(blk, n_blk - 1);                   // keys beyond the last block are masked: any valid page
-      const long off = (long)lds_bt[blk] * page_stride + t_fixed[i] + (key & pm) * t_mul[i];
+      const int blk = min(blk_step + t_blk[i], n_blk - 1);   // keys beyond the last block are masked: any valid page
+      const unsigned long long off =
+          (unsigned long long)(unsigned)lds_bt[blk] * page_stride + (unsigned)(in_page * t_mul[i]);
       global_to_lds_16(t_base[i] + off, __builtin_amdgcn_readfirstlane(lds_address(lds_raw) + stage_byte +
                                                                        (w + 4 * i) * 1024));
     }
@@ -467,6 +480,13 @@ __global__ __launch_bounds__(256) void attn_prefill_dma_kernel(
           st[b][j] = a;
         }
       }
+      // the V^T fragments are asked for now and used after the softmax, which covers their way from LDS
+      Frag8 vf[DV];
+#pragma unroll
+      for (int v = 0; v < DV; ++v) {
+        vf[v].h[0] = *reinterpret_cast<const uint2*>(st_base + voff0 + v * 1024);
+        vf[v].h[1] = *reinterpret_cast<const uint2*>(st_base + voff1 + v * 1024);
+      }
       const bool need_mask = kbase + 31 > wminpos || kbase < wmaxlo;   // the same for the whole wave
       Frag8 pf[NQB];
 #pragma unroll
@@ -485,10 +505,15 @@ __global__ __launch_bounds__(256) void attn_prefill_dma_kernel(
         }
         float mx = fmaxf(fmaxf(fmaxf(r[0], r[1]), fmaxf(r[2], r[3])), fmaxf(fmaxf(r[4], r[5]), fmaxf(r[6], r[7])));
         mx = max_over_lane_groups(mx);
-        const float m_new = fmaxf(m[j], mx * scale_log2);      // the scale is positive
-        if (__any(m_new > m[j])) {
-          // rows whose maximum moved rescale what they have; the others multiply by one
-          const float corr = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m[j] - m_new);
+        // m is the reference the exponentials are taken against, not the running maximum: any reference gives
+        // the same softmax as long as nothing overflows, and bfloat16 probabilities and float32 sums have room
+        // for 2^LAZY above it. So the accumulators (which the matrix cores hold where other instructions cannot
+        // reach them without copies) are rescaled only when a row's scores rise that far above its reference,
+        // which after a row's first step happens almost never.
+        const float cand = mx * scale_log2;                    // the scale is positive
+        if (__builtin_expect(__any(cand > m[j] + PREFILL_LAZY_LOG2), 0)) {
+          const float m_new = cand > m[j] + PREFILL_LAZY_LOG2 ? cand : m[j];
+          const float corr = (m[j] == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m[j] - m_new);   // nothing summed yet: keep
           lsum[j] *= corr;
 #pragma unroll
           for (int v = 0; v < DV; ++v) acc[v][j] *= corr;
@@ -509,15 +534,9 @@ __global__ __launch_bounds__(256) void attn_prefill_dma_kernel(
         pf[j].w[3] = pack2_bf16(pv[6], pv[7]);
       }
 #pragma unroll
-      for (int v = 0; v < DV; ++v) {
-        if (v * 16 < d) {
-          Frag8 vf;
-          vf.h[0] = *reinterpret_cast<const uint2*>(st_base + voff0 + v * 1024);
-          vf.h[1] = *reinterpret_cast<const uint2*>(st_base + voff1 + v * 1024);
+      for (int v = 0; v < DV; ++v)
 #pragma unroll
-          for (int j = 0; j < NQB; ++j) acc[v][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[j].v, acc[v][j], 0, 0, 0);
-        }
-      }
+        for (int j = 0; j < NQB; ++j) acc[v][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[v].v, pf[j].v, acc[v][j], 0, 0, 0);
     }
     consume = consume + STAGE == STAGES * STAGE ? 0 : consume + STAGE;
   }
@@ -567,9 +586,9 @@ static int launch_prefill_dma(dim3 grid, hipStream_t stream, const bf16_t* q, lo
     }
     configured = true;
   }
-  hipLaunchKernelGGL(kernel, grid, dim3(256), smem, stream, q, q_stride, out, out_stride, k_pages, v_pages,
+  hipLaunchKernelGGL(kernel, dim3(grid.x * grid.y), dim3(256), smem, stream, q, q_stride, out, out_stride, k_pages, v_pages,
                      block_tables, btw, tiles, seg, pos, nh, nkv, d, ps_log2, scale_log2, window, HB, n_hb,
-                     PREFILL_BT_CAP);
+                     PREFILL_BT_CAP, lmsf_compute_units());
   return 0;
 }
 

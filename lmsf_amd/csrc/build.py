@@ -30,6 +30,11 @@ HIPCC_FLAGS = [
     "-ffp-contract=fast", "-Wno-unused-command-line-argument", "-Wno-unknown-warning-option",
 ]
 
+# Per source: the attention kernels rescale their accumulators with ordinary multiplications now and then, and
+# with the accumulators in the registers that only the matrix cores reach the compiler copies all of them to and
+# fro in every step of the loop; this keeps them where both can work on them.
+EXTRA_FLAGS = {"attention_mfma.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
+
 
 def sources() -> List[str]:
     return sorted(f for f in os.listdir(CSRC_DIR) if f.endswith(".hip"))
@@ -46,6 +51,7 @@ def source_digest() -> str:
         with open(os.path.join(CSRC_DIR, name), "rb") as f:
             h.update(f.read())
     h.update(" ".join(HIPCC_FLAGS).encode())
+    h.update(repr(sorted(EXTRA_FLAGS.items())).encode())
     return h.hexdigest()
 
 
@@ -116,7 +122,7 @@ def build(verbose: bool = True, jobs: Optional[int] = None) -> str:
 
     def compile_one(name: str):
         obj = os.path.join(obj_dir, name[:-4] + ".o")
-        cmd = [hipcc] + HIPCC_FLAGS + ["-I", CSRC_DIR, "-c", os.path.join(CSRC_DIR, name), "-o", obj]
+        cmd = [hipcc] + HIPCC_FLAGS + EXTRA_FLAGS.get(name, []) + ["-I", CSRC_DIR, "-c", os.path.join(CSRC_DIR, name), "-o", obj]
         proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
         return name, obj, proc.returncode, proc.stdout
 

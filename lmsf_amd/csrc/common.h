@@ -21,6 +21,7 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 
 void lmsf_set_error(const char* fmt, ...);
+int lmsf_compute_units();   // of the current device
 
 #define LMSF_CHECK(cond, ...)            \
   do {                                   \

@@ -18,6 +18,19 @@ extern "C" const char* lmsf_last_error() { return g_last_error; }
 // ABI version of the entry points; the Python side refuses a library that reports another.
 extern "C" int lmsf_abi_version() { return 14; }
 
+// Compute units of the current device (asked once per device; 0 if the device cannot be asked).
+int lmsf_compute_units() {
+  static int cached[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) n = 0;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}
+
 // Name of the architecture the current device reports, e.g. "gfx950:sramecc+:xnack-".
 extern "C" int lmsf_device_arch(char* out, int cap) {
   int dev = 0;

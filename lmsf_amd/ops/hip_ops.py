@@ -415,6 +415,7 @@ class HipOps:
             if key in aux:
                 return aux[key]
             lens, starts, max_context = batch.host_seg_lens, batch.host_seg_starts, batch.max_context
+            first_pos = batch.host_seg_first_pos
             if batch.replayed or batch.all_single:
                 plan = _AttentionPlan(None, 0, None, batch.n_tokens, max_context)
                 aux[key] = plan
@@ -427,15 +428,20 @@ class HipOps:
                     starts.append(i)
                     lens.append(0)
                 lens[-1] += 1
-            max_context = int(pos.max().item()) + 1
+            pos_h = pos.tolist()
+            max_context = max(pos_h) + 1
+            first_pos = [pos_h[st] for st in starts]
             aux, key = None, None
-        tiles, single = [], []
-        for st, n in zip(starts, lens):
+        by_keys, single = [], []
+        for st, n, p0 in zip(starts, lens, first_pos):
             if n == 1:
                 single.append(st)
             else:
                 for t in range(0, n, tq):
-                    tiles.extend((st + t, min(tq, n - t)))
+                    by_keys.append((p0 + t + min(tq, n - t), st + t, min(tq, n - t)))
+        # the tiles with the most keys first: the prefill kernel starts its workgroups in this order
+        by_keys.sort(key=lambda e: -e[0])
+        tiles = [x for e in by_keys for x in e[1:]]
         dev = seg.device
         if len(single) == len(lens):
             plan = _AttentionPlan(None, 0, None, len(single), max_context)
