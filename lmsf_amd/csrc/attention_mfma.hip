@@ -252,11 +252,15 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
 // and no registers are held by data in flight. One barrier per step.
 //
 // A stage holds the K tile [32 keys][DPAD] and the V^T tile [DPAD][32 keys], both without padding (the
-// transfer writes lane after lane). Bank conflicts of the operand reads are avoided by choosing which
-// piece each lane fetches: 16-byte piece ``col`` of K row ``row`` lies in slot col xor (row mod PR) of its row
-// where a row has a power of two of pieces (measured: full rate; the rotation (col - row) mod PR, used for the
-// other head sizes, loses 40 % of the rate when two workgroups share a compute unit), piece ``p`` of V^T row
-// ``dv`` in slot (p + dv / 4) mod 4. The request's block table is copied to LDS first,
+// transfer writes lane after lane). In the product K Q^T the 16 rows of block b are the keys
+// 8 (r / 4) + 4 b + r % 4 and not 16 b + r: a lane's eight scores (four of each block) are then eight keys in
+// a row, 8 g .. 8 g + 7, which is the order the second product wants, and a V^T fragment is one 16-byte read.
+// Bank conflicts of the operand reads are avoided by choosing which piece each lane fetches: eight lanes in
+// a row are served together and must differ in address bits 4 to 6. 16-byte piece ``col`` of K row ``row``
+// lies in slot col xor row_lane(row) of its row, row_lane being the lane that reads the row, where a row has
+// a power of two of pieces (measured: full rate; the rotation (col - row_lane) mod PR, used for the other head
+// sizes, loses 40 % of the rate when two workgroups share a compute unit), piece ``p`` of V^T row ``dv`` in
+// slot (p + dv / 2) mod 4. The request's block table is copied to LDS first,
 // so that no address waits for a lookup in global memory. Needs pages of 8, 16, 32, ... tokens.
 //
 // The transfer instruction is written as inline assembly: through the compiler's builtin every LDS read
@@ -271,6 +275,8 @@ __device__ __forceinline__ void global_to_lds_16(const void* src, unsigned lds_b
                : "memory", "m0");
 }
 #pragma clang diagnostic pop
+// c = lane % 16 of the lane that reads K row ``row`` (0 .. 31) of a stage; both blocks of 16 rows give 0 .. 15
+__device__ __forceinline__ int row_lane(int row) { return ((row >> 3) << 2) | (row & 3); }
 __device__ __forceinline__ unsigned lds_address(const void* p) {
   return (unsigned)(size_t)(__attribute__((address_space(3))) const unsigned char*)p;
 }
@@ -386,11 +392,12 @@ __global__ __launch_bounds__(256) void attn_prefill_dma_kernel(
     if (j < DPAD / 16) {
       const int P = j * 64 + l;
       const int row = P / PR, slot = P - row * PR;
+      const int rz = PR == 4 ? (row_lane(row) >> 1) & 3 : row_lane(row);
       int col;
       if (PR_POW2) {
-        col = slot ^ (row & (PR - 1));
+        col = slot ^ (rz & (PR - 1));
       } else {
-        col = slot + row % PR;
+        col = slot + rz % PR;
         if (col >= PR) col -= PR;
       }
       if (col * 8 >= d) col = 0;                   // beyond the head: any finite data, the query is zero there
@@ -401,7 +408,7 @@ __global__ __launch_bounds__(256) void attn_prefill_dma_kernel(
       const int P = (j - DPAD / 16) * 64 + l;
       int dv = P >> 2;
       const int slot = P & 3;
-      const int piece = (slot - (dv >> 2)) & 3;
+      const int piece = (slot - (dv >> 1)) & 3;
       if (dv >= d) dv = 0;                         // rows beyond the head: any finite data, their results are dropped
       t_blk[i] = (piece * 8) >> ps_log2;
       t_mul[i] = 1;
@@ -414,19 +421,18 @@ __global__ __launch_bounds__(256) void attn_prefill_dma_kernel(
   for (int b = 0; b < 2; ++b)
 #pragma unroll
     for (int s = 0; s < DS; ++s) {
-      const int row = b * 16 + c;
+      const int row = (c >> 2) * 8 + b * 4 + (c & 3);   // row_lane(row) == c
+      const int rz = PR == 4 ? (c >> 1) & 3 : c;
       int slot;
       if (PR_POW2) {
-        slot = (s * 4 + g) ^ (row & (PR - 1));
+        slot = (s * 4 + g) ^ (rz & (PR - 1));
       } else {
-        slot = s * 4 + g - row % PR;
+        slot = s * 4 + g - rz % PR;
         if (slot < 0) slot += PR;
       }
       koff[b][s] = (row * PR + slot) * 16;
     }
-  const int vrot = (g >> 1) + (c >> 2);            // (piece + dv / 4) mod 4 with dv = 16 v + c
-  const int voff0 = KTILE + c * 64 + (g & 1) * 8 + (vrot & 3) * 16;
-  const int voff1 = KTILE + c * 64 + (g & 1) * 8 + ((vrot + 2) & 3) * 16;
+  const int voff = KTILE + c * 64 + ((g + (c >> 1)) & 3) * 16;   // piece g of V^T row 16 v + c
 
   // The query fragments are pinned here, so that the compiler waits for their loads now and not, with a
   // wait for everything in flight, inside the loop.
@@ -484,8 +490,7 @@ __global__ __launch_bounds__(256) void attn_prefill_dma_kernel(
       Frag8 vf[DV];
 #pragma unroll
       for (int v = 0; v < DV; ++v) {
-        vf[v].h[0] = *reinterpret_cast<const uint2*>(st_base + voff0 + v * 1024);
-        vf[v].h[1] = *reinterpret_cast<const uint2*>(st_base + voff1 + v * 1024);
+        vf[v].q = *reinterpret_cast<const uint4*>(st_base + voff + v * 1024);
       }
       const bool need_mask = kbase + 31 > wminpos || kbase < wmaxlo;   // the same for the whole wave
       Frag8 pf[NQB];
@@ -499,7 +504,7 @@ __global__ __launch_bounds__(256) void attn_prefill_dma_kernel(
         if (need_mask) {
 #pragma unroll
           for (int e = 0; e < 8; ++e) {
-            const int key = kbase + (e >> 2) * 16 + g * 4 + (e & 3);
+            const int key = kbase + g * 8 + e;
             if (key > rpos[j] || key < rlo[j]) r[e] = -INFINITY;
           }
         }
