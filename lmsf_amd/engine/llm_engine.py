@@ -6,7 +6,7 @@ samples and applies the stop rules. ``LLM.generate`` is the convenience loop aro
 """
 import hashlib
 import time
-from typing import Any, Dict, Hashable, List, Optional, Sequence as Seq
+from typing import Any, Dict, Hashable, List, Optional, Sequence as Seq, Set, Union
 
 import torch
 
@@ -15,6 +15,7 @@ from ..sampling.sampler import Sampler, SamplingRow
 from .args import EngineArgs
 from .batch import StepEntry
 from .core import EngineCore, load_engine_core
+from .detokenizer import IncrementalDetokenizer, load_tokenizer
 from .outputs import RequestOutput
 from .scheduler import Scheduler, SchedulerConfig, StepPlan
 from .sequence import Sequence, SequenceState
@@ -35,6 +36,7 @@ class LLMEngine:
                                    self.core.storage.manager)
         self.sampler = Sampler(self.core.rt.ops, self.core.rt.device)
         self.eos_token_ids = set(self.core.config.eos_token_ids)
+        self.tokenizer = None if args.skip_tokenizer_init else load_tokenizer(args.model)
         self._arrivals = 0
         self._requests: Dict[Hashable, Sequence] = {}
         self.stats = {"steps": 0, "tokens": 0, "generated_tokens": 0, "preemptions": 0}
@@ -45,13 +47,31 @@ class LLMEngine:
 
     # ------------------------------------------------------------------ requests
 
-    def add_request(self, request_id: Hashable, prompt_token_ids: Seq[int],
-                    sampling_params: Optional[SamplingParams] = None) -> None:
-        """core/src/engine/llm_engine.rs:136-169, on token ids."""
+    def add_request(self, request_id: Hashable, prompt: Union[str, Seq[int], None],
+                    sampling_params: Optional[SamplingParams] = None,
+                    prompt_token_ids: Optional[Seq[int]] = None) -> None:
+        """core/src/engine/llm_engine.rs:136-169: ``prompt`` is text, encoded with the model folder's
+        tokenizer unless ``prompt_token_ids`` brings the ids; a list of token ids in its place is
+        taken as the ids."""
         if request_id in self._requests:
             raise ValueError("request id %r is already in use" % (request_id,))
         params = sampling_params or SamplingParams()
         params.verify()
+        text: Optional[str] = None
+        if isinstance(prompt, str):
+            text = prompt
+            if prompt_token_ids is None:
+                if self.tokenizer is None:
+                    raise ValueError("request %r: a text prompt needs %s/tokenizer.json; give token ids instead"
+                                     % (request_id, self.args.model or "<model>"))
+                prompt_token_ids = self.tokenizer.encode(prompt, add_special_tokens=True)
+        elif prompt_token_ids is None:
+            prompt_token_ids = prompt
+        if prompt_token_ids is None:
+            raise ValueError("request %r has no prompt" % (request_id,))
+        if params.stop and self.tokenizer is None:
+            raise ValueError("request %r: stop strings need %s/tokenizer.json; use stop_token_ids"
+                             % (request_id, self.args.model or "<model>"))
         ids = [int(t) for t in prompt_token_ids]
         V = self.core.config.vocab_size
         if not ids:
@@ -63,7 +83,9 @@ class LLMEngine:
         if seed is None:
             h = hashlib.sha256(("%d:%d" % (self.args.seed, self._arrivals)).encode()).digest()
             seed = int.from_bytes(h[:8], "little")
-        seq = Sequence(request_id, ids, params, self._arrivals, seed)
+        seq = Sequence(request_id, ids, params, self._arrivals, seed, prompt=text)
+        if self.tokenizer is not None:
+            seq.detokenizer = IncrementalDetokenizer(self.tokenizer, len(ids), params.skip_special_tokens)
         self._arrivals += 1
         self._requests[request_id] = seq
         self.scheduler.add(seq)
@@ -113,51 +135,67 @@ class LLMEngine:
             seq.output_token_ids.append(tok)
             if seq.metrics.first_token_time is None:
                 seq.metrics.first_token_time = now
-            self._check_stop(seq)
+            piece = ""
+            if seq.detokenizer is not None:
+                piece = seq.detokenizer.step(seq.prompt_token_ids + seq.output_token_ids)
+                seq.output_text += piece
+            before = len(seq.output_text)
+            check_stop(seq, self.core.max_model_len, self.eos_token_ids)
+            if len(seq.output_text) < before:       # a stop string was cut off the end
+                piece = piece[:max(0, len(piece) - (before - len(seq.output_text)))]
             if seq.state.finished:
                 seq.metrics.finished_time = now
                 self.scheduler.finish(seq)
                 self._requests.pop(seq.request_id, None)
-            outputs.append(RequestOutput.from_sequence(seq, tok))
+            outputs.append(RequestOutput.from_sequence(seq, tok, piece))
         self.stats["generated_tokens"] += len(sampled)
         self.stats["tokens"] += plan.num_tokens
         return outputs
 
-    def _check_stop(self, seq: Sequence) -> None:
-        """The reference's order without stop strings (core/src/engine/llm_engine.rs:221-258):
-        stop_token_ids, longer than max_model_len, max_tokens reached, EOS unless ignore_eos."""
-        p = seq.params
-        last = seq.last_token_id
-        if p.stop_token_ids and last in p.stop_token_ids:
+
+def check_stop(seq: Sequence, max_model_len: int, eos_token_ids: Set[int]) -> None:
+    """The reference's rules in its order (core/src/engine/llm_engine.rs:221-258): the text ends with a
+    stop string (which is cut off unless ``include_stop_str_in_output``), stop_token_ids, longer than
+    max_model_len, max_tokens reached, EOS unless ignore_eos."""
+    p = seq.params
+    last = seq.last_token_id
+    for stop in p.stop:
+        if seq.output_text.endswith(stop):
+            if not p.include_stop_str_in_output:
+                seq.output_text = seq.output_text[:len(seq.output_text) - len(stop)]
             seq.state = SequenceState.FINISHED_STOPPED
-        elif seq.length > self.core.max_model_len:
-            seq.state = SequenceState.FINISHED_LENGTH_CAPPED
-        elif len(seq.output_token_ids) >= p.max_tokens:
-            seq.state = SequenceState.FINISHED_LENGTH_CAPPED
-        elif not p.ignore_eos and last in self.eos_token_ids:
-            seq.state = SequenceState.FINISHED_STOPPED
-        elif seq.length >= self.core.max_model_len:
-            # the next token would have no position left
-            seq.state = SequenceState.FINISHED_LENGTH_CAPPED
+            return
+    if p.stop_token_ids and last in p.stop_token_ids:
+        seq.state = SequenceState.FINISHED_STOPPED
+    elif seq.length > max_model_len:
+        seq.state = SequenceState.FINISHED_LENGTH_CAPPED
+    elif len(seq.output_token_ids) >= p.max_tokens:
+        seq.state = SequenceState.FINISHED_LENGTH_CAPPED
+    elif not p.ignore_eos and last in eos_token_ids:
+        seq.state = SequenceState.FINISHED_STOPPED
+    elif seq.length >= max_model_len:
+        # the next token would have no position left
+        seq.state = SequenceState.FINISHED_LENGTH_CAPPED
 
 
 class LLM:
     """``LLM(model=..., **engine options).generate(prompts, sampling_params)``: every prompt a list of
-    token ids; returns one finished RequestOutput per prompt, in the order given."""
+    token ids, or text if the model folder has a tokenizer.json; returns one finished RequestOutput per
+    prompt, in the order given."""
 
     def __init__(self, model: str, **kwargs):
         self.engine = LLMEngine(EngineArgs(model=model, **kwargs))
         self._next_id = 0
 
-    def generate(self, prompt_token_ids: Seq[Seq[int]], sampling_params=None) -> List[RequestOutput]:
+    def generate(self, prompts: Seq[Union[str, Seq[int]]], sampling_params=None) -> List[RequestOutput]:
         if sampling_params is None or isinstance(sampling_params, SamplingParams):
-            params_list = [sampling_params] * len(prompt_token_ids)
+            params_list = [sampling_params] * len(prompts)
         else:
             params_list = list(sampling_params)
-            if len(params_list) != len(prompt_token_ids):
+            if len(params_list) != len(prompts):
                 raise ValueError("one SamplingParams per prompt, or one for all")
         ids = []
-        for prompt, params in zip(prompt_token_ids, params_list):
+        for prompt, params in zip(prompts, params_list):
             rid = self._next_id
             self._next_id += 1
             # every request gets its own copy: verify() may normalise fields

@@ -8,7 +8,7 @@ States and finish reasons follow core/src/common/sequence.rs:36-64.
 import enum
 import time
 from dataclasses import dataclass, field
-from typing import Hashable, List, Optional
+from typing import Any, Hashable, List, Optional
 
 from ..sampling.params import SamplingParams
 
@@ -54,6 +54,9 @@ class Sequence:
     num_computed: int = 0                  # tokens whose keys and values are in the cache
     num_preemptions: int = 0
     metrics: RequestMetrics = field(default_factory=lambda: RequestMetrics(time.monotonic()))
+    prompt: Optional[str] = None           # the prompt's text, if the request came as text
+    output_text: str = ""                  # text of the generated tokens (engines with a tokenizer)
+    detokenizer: Any = None                # engine.detokenizer.IncrementalDetokenizer
 
     @property
     def length(self) -> int:

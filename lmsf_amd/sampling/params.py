@@ -1,9 +1,10 @@
 """SamplingParams with the reference's names, defaults and checks
 (core/src/common/sampling_params.rs:29-80 fields and defaults, :166-298 verify).
 
-Options that need several sequences per request (n, best_of, beam search) or a tokenizer (stop
-strings) or log-probabilities are accepted only at their defaults: this engine keeps one sequence
-per request and works on token ids. ``seed`` is an addition: a request with a seed draws the same
+Options that need several sequences per request (n, best_of, beam search) or log-probabilities are
+accepted only at their defaults: this engine keeps one sequence per request. Stop strings need the
+model folder's tokenizer; the engine refuses them at ``add_request`` if it has none. ``seed`` is an
+addition: a request with a seed draws the same
 tokens whatever else is in the batch; without one the engine derives a seed from its own --seed and
 the request's arrival number.
 """
@@ -81,8 +82,10 @@ class SamplingParams:
         if abs(self.length_penalty - 1.0) > SAMPLING_EPS:
             raise ValueError("length_penalty is not effective and must be the default value of 1.0 when not "
                              "using beam search.")
-        if self.stop:
-            raise ValueError("stop strings need a tokenizer, which this engine does not have; use stop_token_ids.")
+        if isinstance(self.stop, str):
+            self.stop = [self.stop]
+        if any(not isinstance(x, str) or not x for x in self.stop):
+            raise ValueError("stop must be a list of non-empty strings.")
         if self.logprobs is not None or self.prompt_logprobs is not None:
             raise ValueError("logprobs and prompt_logprobs are not supported; trace replay gives the logits.")
         if self.stop_token_ids is not None and any(int(t) < 0 for t in self.stop_token_ids):

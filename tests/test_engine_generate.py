@@ -120,7 +120,7 @@ def test_sampling_params_follow_the_reference():
     for bad in (dict(n=2), dict(best_of=3), dict(use_beam_search=True), dict(temperature=-1.0), dict(top_p=0.0),
                 dict(top_p=1.5), dict(top_k=0), dict(top_k=-2), dict(min_p=2.0), dict(max_tokens=0),
                 dict(presence_penalty=3.0), dict(frequency_penalty=-3.0), dict(repetition_penalty=2.5),
-                dict(stop=["x"]), dict(logprobs=1), dict(length_penalty=2.0), dict(early_stopping=True)):
+                dict(stop=[""]), dict(logprobs=1), dict(length_penalty=2.0), dict(early_stopping=True)):
         with pytest.raises(ValueError):
             SamplingParams(**bad)
     p = SamplingParams(temperature=0.0, top_k=5, top_p=0.5, min_p=0.1)

@@ -103,3 +103,29 @@ def test_command_line(tmp_path):
     lines = proc.stdout.strip().splitlines()
     assert [int(t) for t in lines[0].split()] == plain_greedy_generate(cfg_dict, w, prompt, 8)
     assert lines[-1].startswith("cost ")
+
+
+def test_command_line_with_text(tmp_path):
+    """The reference's example takes its prompt as text: with a tokenizer.json in the folder the command line
+    does too, prints text, and a stop string ends the output."""
+    pytest.importorskip("tokenizers")
+    from test_text import write_word_tokenizer
+    from lmsf_amd.engine.detokenizer import Tokenizer
+    folder, cfg = make_model_folder(tmp_path, "A")
+    tok = Tokenizer(write_word_tokenizer(folder, n_words=cfg.vocab_size))
+    cfg_dict, w = read_model_folder(folder)
+    text = "to be or not to be ,"
+    want = plain_greedy_generate(cfg_dict, w, tok.encode(text), 8)
+    base = [os.path.join(ROOT, "bin", "lmsf_generate"), "--model", folder, "--dtype", "float32",
+            "--gpu-memory-utilization", "0.5", "--block-size", "8", "--max-model-len", "64", "--prompt", text,
+            "--temperature", "0", "--max-tokens", "8", "--ignore-eos"]
+    proc = subprocess.run(base, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    lines = proc.stdout.splitlines()
+    assert lines[0] == " " + tok.decode(want) and lines[-1].startswith("cost ")
+    stop = tok.decode(want[2:3])
+    first = [tok.decode([t]) for t in want].index(stop)
+    proc = subprocess.run(base + ["--stop", stop], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-3000:]
+    assert proc.stdout.splitlines()[0].split() == tok.decode(want[:first]).split()
+    assert ("to gen %d tokens" % (first + 1)) in proc.stdout
