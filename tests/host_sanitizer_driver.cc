@@ -1,0 +1,218 @@
+// Drives the C API of the host library (cache manager, scheduler, step metadata) the way the engine does,
+// over a random workload that reaches admission, portions, decoding, preemption, refusal, capping, abort and
+// the error paths. Built with -fsanitize=address,undefined by tests/test_host_sanitizers.py: what it checks is
+// what the sanitizers and the library's own check_invariants find. Test code only.
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <map>
+#include <vector>
+
+extern "C" {
+int lmsf_host_abi_version();
+const char* lmsf_host_last_error();
+int lmsf_pool_create(int num_pages, void** out);
+void lmsf_pool_destroy(void* pool);
+int lmsf_pool_num_free(void* pool);
+int lmsf_pool_allocate(void* pool, int* page);
+int lmsf_pool_release(void* pool, int page);
+int lmsf_cm_create(int n_groups, const int* page_size, const int* num_pages, const int* window, int num_state_slots,
+                   void** out);
+void lmsf_cm_destroy(void* cm);
+int lmsf_cm_has_request(void* cm, int64_t rid);
+int lmsf_cm_num_free_state_slots(void* cm);
+int lmsf_cm_num_free_pages(void* cm, int group, int* out);
+int lmsf_cm_request_info(void* cm, int64_t rid, int64_t* info);
+int lmsf_cm_block_table(void* cm, int64_t rid, int group, int* out, int cap, int* len, int* first_live);
+int lmsf_cm_live_requests(void* cm, int64_t* out, int cap, int* count);
+int lmsf_cm_append(void* cm, int64_t rid, int64_t n_new, int64_t* start);
+int lmsf_cm_free_request(void* cm, int64_t rid);
+int lmsf_cm_slot_mapping(void* cm, int64_t rid, int group, int64_t start, int64_t n, int* out);
+int lmsf_cm_check_invariants(void* cm);
+int lmsf_cm_begin_step(void* cm, int S, const int64_t* rids, const int* lens, int64_t* starts, unsigned char* added);
+int lmsf_cm_abort_step(void* cm, int S, const int64_t* rids, const unsigned char* added);
+int lmsf_cm_commit_step(void* cm, int S, const int64_t* rids);
+int lmsf_cm_step_widths(void* cm, int S, const int64_t* rids, int* widths);
+int lmsf_step_layout(int64_t N, int64_t S, int64_t R, int G, const int* widths, int64_t* offsets, int64_t* total);
+int lmsf_cm_fill_step(void* cm, int S, const int64_t* rids, const int64_t* starts, const int* lens, const int* widths,
+                      const int64_t* offsets, int32_t* buffer);
+int lmsf_sched_create(void* cm, int64_t max_num_batched_tokens, int max_num_seqs, int64_t max_model_len,
+                      int64_t prefill_chunk_size, double watermark, void** out);
+void lmsf_sched_destroy(void* s);
+int lmsf_sched_add(void* s, int64_t id, int64_t arrival, int64_t length);
+int lmsf_sched_set_progress(void* s, int n, const int64_t* ids, const int64_t* lengths, const int64_t* computed);
+int lmsf_sched_abort(void* s, int64_t id, int* found);
+int lmsf_sched_finish(void* s, int64_t id);
+int lmsf_sched_schedule(void* s, int* counts);
+int lmsf_sched_plan(void* s, int64_t* ids, int64_t* starts, int64_t* n_tokens, int* samples, int64_t* preempted,
+                    int64_t* ignored, int64_t* capped);
+int lmsf_sched_queue(void* s, int which, int64_t* out, int cap, int* count);
+int64_t lmsf_sched_num_preemptions(void* s);
+}
+
+#define MUST(call)                                                                              \
+  do {                                                                                          \
+    int rc_ = (call);                                                                           \
+    if (rc_ != 0) {                                                                             \
+      std::fprintf(stderr, "%s:%d: %s -> %d: %s\n", __FILE__, __LINE__, #call, rc_, lmsf_host_last_error()); \
+      return 1;                                                                                 \
+    }                                                                                           \
+  } while (0)
+#define MUST_FAIL(call, want)                                                                   \
+  do {                                                                                          \
+    int rc_ = (call);                                                                           \
+    if (rc_ != (want)) {                                                                        \
+      std::fprintf(stderr, "%s:%d: %s -> %d, expected %d\n", __FILE__, __LINE__, #call, rc_, (want)); \
+      return 1;                                                                                 \
+    }                                                                                           \
+  } while (0)
+
+struct Seq {
+  int64_t length, computed, target;   // target: the length at which the driver finishes it
+};
+
+static uint64_t rng_state = 12345;
+static uint32_t rnd(uint32_t n) {
+  rng_state = rng_state * 6364136223846793005ull + 1442695040888963407ull;
+  return (uint32_t)(rng_state >> 33) % n;
+}
+
+int main(int argc, char** argv) {
+  if (argc > 1) rng_state = std::strtoull(argv[1], nullptr, 10);
+  if (lmsf_host_abi_version() < 1) return 1;
+
+  // the pool alone, with its error paths
+  void* pool = nullptr;
+  MUST(lmsf_pool_create(3, &pool));
+  int page = -1, p2 = -1, p3 = -1;
+  MUST(lmsf_pool_allocate(pool, &page));
+  MUST(lmsf_pool_allocate(pool, &p2));
+  MUST(lmsf_pool_allocate(pool, &p3));
+  MUST_FAIL(lmsf_pool_allocate(pool, &p3), 2);     // out of pages
+  MUST(lmsf_pool_release(pool, p2));
+  MUST_FAIL(lmsf_pool_release(pool, p2), 1);       // freed twice
+  MUST_FAIL(lmsf_pool_release(pool, 99), 1);       // never held
+  if (lmsf_pool_num_free(pool) != 1) return 1;
+  lmsf_pool_destroy(pool);
+
+  // two groups: all keys in pages of 8, a window of 24 keys in pages of 16; few pages, few slots
+  const int page_size[2] = {8, 16}, num_pages[2] = {20, 12}, window[2] = {0, 24};   // 160 tokens: fewer than the model allows
+  void* cm = nullptr;
+  MUST(lmsf_cm_create(2, page_size, num_pages, window, 6, &cm));
+  void* sched = nullptr;
+  MUST(lmsf_sched_create(cm, 48, 5, 200, 16, 0.01, &sched));
+
+  int64_t start = 0, info[8] = {0};
+  MUST_FAIL(lmsf_cm_append(cm, 777, 3, &start), 1);          // unknown request
+  MUST_FAIL(lmsf_cm_free_request(cm, 777), 1);
+  MUST_FAIL(lmsf_cm_request_info(cm, 777, info), 1);
+
+  std::map<int64_t, Seq> live;
+  int64_t next_id = 1, arrival = 0, steps = 0, finished = 0, ignored_n = 0, capped_n = 0, aborted = 0;
+  std::vector<int32_t> buffer;
+  for (int it = 0; it < 600 || !live.empty(); ++it) {
+    if (it < 600 && rnd(3) == 0) {
+      const int64_t id = next_id++;
+      int64_t len = 1 + rnd(60);
+      if (rnd(20) == 0) len = 120 + rnd(100);      // some too long for the model or for the pool, some that outgrow the pool
+      MUST(lmsf_sched_add(sched, id, arrival++, len));
+      live[id] = Seq{len, 0, len + 1 + (int64_t)rnd(40)};
+    }
+    if (!live.empty() && rnd(25) == 0) {           // abort a request, wherever it is
+      auto pick = live.begin();
+      std::advance(pick, rnd((uint32_t)live.size()));
+      int found = 0;
+      MUST(lmsf_sched_abort(sched, pick->first, &found));
+      if (!found) return 1;
+      live.erase(pick);
+      ++aborted;
+    }
+    if (live.empty()) continue;
+    std::vector<int64_t> ids, lens, comp;
+    for (auto& kv : live) {
+      ids.push_back(kv.first);
+      lens.push_back(kv.second.length);
+      comp.push_back(kv.second.computed);
+    }
+    MUST(lmsf_sched_set_progress(sched, (int)ids.size(), ids.data(), lens.data(), comp.data()));
+    int counts[4] = {0, 0, 0, 0};
+    MUST(lmsf_sched_schedule(sched, counts));
+    const int ns = counts[0];
+    std::vector<int64_t> sid(ns + 1), sstart(ns + 1), stok(ns + 1), pre(counts[1] + 1), ign(counts[2] + 1), cap(counts[3] + 1);
+    std::vector<int> samples(ns + 1);
+    MUST(lmsf_sched_plan(sched, sid.data(), sstart.data(), stok.data(), samples.data(), pre.data(), ign.data(), cap.data()));
+    for (int i = 0; i < counts[1]; ++i) live[pre[i]].computed = 0;
+    for (int i = 0; i < counts[2]; ++i) { live.erase(ign[i]); ++ignored_n; }
+    for (int i = 0; i < counts[3]; ++i) { live.erase(cap[i]); ++capped_n; }
+    if (ns == 0) {
+      MUST(lmsf_cm_check_invariants(cm));
+      continue;
+    }
+    // the executor's part: take the pages, write the step's metadata, commit
+    std::vector<int> n_new(ns);
+    int64_t N = 0, R = 0;
+    for (int i = 0; i < ns; ++i) {
+      n_new[i] = (int)stok[i];
+      N += stok[i];
+      R += samples[i];
+      if (sstart[i] != live[sid[i]].computed) {
+        std::fprintf(stderr, "request %ld planned from %ld but has %ld computed\n", (long)sid[i], (long)sstart[i],
+                     (long)live[sid[i]].computed);
+        return 1;
+      }
+    }
+    if (N > 48) return 1;                            // the token budget
+    std::vector<int64_t> starts(ns);
+    std::vector<unsigned char> added(ns);
+    MUST(lmsf_cm_begin_step(cm, ns, sid.data(), n_new.data(), starts.data(), added.data()));
+    if (rnd(15) == 0) {                              // a step that fails after it took its pages
+      MUST(lmsf_cm_abort_step(cm, ns, sid.data(), added.data()));
+      MUST(lmsf_cm_check_invariants(cm));
+      continue;
+    }
+    int widths[2] = {0, 0};
+    MUST(lmsf_cm_step_widths(cm, ns, sid.data(), widths));
+    int64_t offsets[32] = {0}, total = 0;
+    MUST(lmsf_step_layout(N, ns, R, 2, widths, offsets, &total));
+    buffer.assign((size_t)total, -7);
+    MUST(lmsf_cm_fill_step(cm, ns, sid.data(), starts.data(), n_new.data(), widths, offsets, buffer.data()));
+    std::vector<int> slots((size_t)stok[0]);
+    MUST(lmsf_cm_slot_mapping(cm, sid[0], 0, starts[0], stok[0], slots.data()));
+    for (int s : slots)
+      if (s < 0 || s >= 20 * 8) return 1;
+    int table[64], len = 0, first_live = 0;
+    MUST(lmsf_cm_block_table(cm, sid[0], 1, table, 64, &len, &first_live));
+    MUST(lmsf_cm_commit_step(cm, ns, sid.data()));
+    ++steps;
+    for (int i = 0; i < ns; ++i) {
+      Seq& s = live[sid[i]];
+      s.computed += stok[i];
+      if (samples[i]) {
+        s.length += 1;
+        if (s.length >= s.target || s.length >= 200) {
+          MUST(lmsf_sched_finish(sched, sid[i]));
+          live.erase(sid[i]);
+          ++finished;
+        }
+      }
+    }
+    MUST(lmsf_cm_check_invariants(cm));
+    if (it > 100000) {
+      std::fprintf(stderr, "the workload does not drain\n");
+      return 1;
+    }
+  }
+  int free0 = 0, free1 = 0, count = 0;
+  MUST(lmsf_cm_num_free_pages(cm, 0, &free0));
+  MUST(lmsf_cm_num_free_pages(cm, 1, &free1));
+  MUST(lmsf_cm_live_requests(cm, nullptr, 0, &count));
+  if (free0 != 20 || free1 != 12 || count != 0 || lmsf_cm_num_free_state_slots(cm) != 6) {
+    std::fprintf(stderr, "left over: %d %d pages free, %d requests\n", free0, free1, count);
+    return 1;
+  }
+  std::printf("OK steps=%ld finished=%ld ignored=%ld capped=%ld aborted=%ld preemptions=%ld\n", (long)steps,
+              (long)finished, (long)ignored_n, (long)capped_n, (long)aborted, (long)lmsf_sched_num_preemptions(sched));
+  lmsf_sched_destroy(sched);
+  lmsf_cm_destroy(cm);
+  return 0;
+}
