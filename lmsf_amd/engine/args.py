@@ -2,8 +2,8 @@
 (core/src/common/config.rs:9-87), as a dataclass and as command-line flags.
 
 Options of the reference that have no meaning here are still accepted, so that its command lines
-run: --swap-space, --max-paddings, --threads, --chat-template, --log-dir, --alsologtostderr are
-parsed and unused (as --threads and --chat-template are in the reference); --tp, --pp must be 1
+run: --swap-space, --max-paddings, --threads, --chat-template are parsed and unused (as --threads and
+--chat-template are in the reference); --log-dir and --alsologtostderr switch on the engine's log; --tp, --pp must be 1
 and --quantization must be absent, or the engine refuses to start.
 """
 import argparse
@@ -71,8 +71,8 @@ class EngineArgs:
         a("--pp", dest="pipeline_parallel_size", type=int, default=1, help="number of pipeline stages (1)")
         a("--tp", dest="tensor_parallel_size", type=int, default=1, help="number of tensor parallel replicas (1)")
         a("--threads", type=int, default=4, help="(unused)")
-        a("--log-dir", default=None, help="log dir (unused)")
-        a("--alsologtostderr", action="store_true", help="print log into stderr (unused)")
+        a("--log-dir", default=None, help="log dir (lmsf.log in it, a new file every day)")
+        a("--alsologtostderr", action="store_true", help="print log into stderr")
         a("--load-format", default="auto", choices=["auto", "random"],
           help="auto: the folder's safetensors; random: random weights for the folder's config.json")
         a("--prefill-chunk-size", type=int, default=None, help="longest portion of a prompt in one step")

@@ -16,6 +16,7 @@ from .args import EngineArgs
 from .batch import StepEntry
 from .core import EngineCore, load_engine_core
 from .detokenizer import IncrementalDetokenizer, load_tokenizer
+from .metrics import Metrics, init_logging
 from .outputs import RequestOutput
 from .scheduler import Scheduler, SchedulerConfig, StepPlan
 from .sequence import Sequence, SequenceState
@@ -40,6 +41,11 @@ class LLMEngine:
         self._arrivals = 0
         self._requests: Dict[Hashable, Sequence] = {}
         self.stats = {"steps": 0, "tokens": 0, "generated_tokens": 0, "preemptions": 0}
+        # --log-dir / --alsologtostderr as in the reference (common/src/tracing.rs:1-22): without either the
+        # engine does not log; the metrics are kept either way and reported once a minute where there is a log
+        self.logger = init_logging(args.log_dir, args.alsologtostderr) if (args.log_dir or args.alsologtostderr) else None
+        self.metrics = Metrics(logger=self.logger)
+        self.last_step: Dict[str, Any] = {}
 
     @classmethod
     def from_engine_args(cls, args: EngineArgs) -> "LLMEngine":
@@ -89,6 +95,8 @@ class LLMEngine:
         self._arrivals += 1
         self._requests[request_id] = seq
         self.scheduler.add(seq)
+        self.metrics.counter("llm.prompt_recv")                   # core/src/engine/llm_engine.rs:794-795
+        self.metrics.gauge("llm.alive_prompt", len(self._requests))
 
     def abort_request(self, request_id: Hashable) -> None:
         """core/src/engine/llm_engine.rs:171-178."""
@@ -108,6 +116,7 @@ class LLMEngine:
     def step(self) -> List[RequestOutput]:
         """Schedule, run the model once, sample, apply the stop rules
         (core/src/engine/llm_engine.rs:536-582)."""
+        t_start = time.monotonic()
         plan: StepPlan = self.scheduler.schedule()
         outputs: List[RequestOutput] = []
         now = time.monotonic()
@@ -150,7 +159,33 @@ class LLMEngine:
             outputs.append(RequestOutput.from_sequence(seq, tok, piece))
         self.stats["generated_tokens"] += len(sampled)
         self.stats["tokens"] += plan.num_tokens
+        self._record_step(plan, len(sampled), outputs, t_start)
         return outputs
+
+    def _record_step(self, plan: StepPlan, n_sampled: int, outputs: List[RequestOutput], t_start: float) -> None:
+        """What the step did, for ``last_step`` and the metrics."""
+        now = time.monotonic()
+        decode = sum(1 for s in plan.scheduled if s.n_tokens == 1 and s.samples and s.start > 0)
+        m = self.metrics
+        self.last_step = {"tokens": plan.num_tokens, "decode_tokens": decode, "prefill_tokens": plan.num_tokens - decode,
+                          "sequences": len(plan.scheduled), "sampled": n_sampled, "preempted": len(plan.preempted),
+                          "free_pages": self.core.storage.manager.num_free_pages(0) if self.core.storage.manager.groups else 0,
+                          "ms": (now - t_start) * 1e3}
+        m.counter("llm.steps")
+        m.counter("llm.tokens", plan.num_tokens)
+        m.counter("llm.generated_tokens", n_sampled)
+        m.counter("llm.preemptions", len(plan.preempted))
+        m.gauge("llm.alive_prompt", len(self._requests))
+        m.gauge("llm.free_pages", self.last_step["free_pages"])
+        m.histogram("llm.step_ms", self.last_step["ms"])
+        m.histogram("llm.step_tokens", plan.num_tokens)
+        for out in outputs:
+            if out.finished and out.metrics is not None and out.metrics.finished_time is not None:
+                t = out.metrics
+                m.histogram("llm.request_s", t.finished_time - t.arrival_time)
+                if t.first_token_time is not None:
+                    m.histogram("llm.first_token_s", t.first_token_time - t.arrival_time)
+        m.maybe_report(now)
 
 
 def check_stop(seq: Sequence, max_model_len: int, eos_token_ids: Set[int]) -> None:
