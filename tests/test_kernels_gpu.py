@@ -247,6 +247,36 @@ def test_decode_attention_reduction_over_many_splits(ops, ref, nh, nkv, d, ps, w
     assert torch.allclose(a.float(), b.float(), **tol(torch.bfloat16)), (a.float() - b.float()).abs().max()
 
 
+@pytest.mark.parametrize("nh,nkv,d,ps", [(8, 2, 128, 16), (4, 4, 64, 8), (6, 2, 80, 16)])
+@pytest.mark.parametrize("trend", ["rising", "falling", "jump"])
+def test_prefill_attention_moves_its_reference_when_scores_run_away(ops, ref, nh, nkv, d, ps, trend):
+    """The prefill kernel takes its exponentials against a reference that it moves only when a row's scores have
+    risen 2^24 above it. Keys whose scores rise steadily, fall steadily, or jump once by far more than that
+    (in units of log2: hundreds) must give the plain result: every key a multiple of one direction that all
+    queries share, so that the score of key j is the multiple."""
+    T = 200
+    g = torch.Generator().manual_seed(nh * d + len(trend))
+    q, kp, vp, bt, seg, pos = _paged_case(torch.bfloat16, nh, nkv, d, ps, [T], [T], seed=5)
+    u = torch.randn(d, generator=g)
+    u = u / u.norm()
+    scale = 1.0 / math.sqrt(d)
+    # score of key j for every query = 8 * amp[j] * scale^-1 * scale = 8 amp[j] (natural log units)
+    amp = {"rising": torch.linspace(-40.0, 40.0, T), "falling": torch.linspace(40.0, -40.0, T),
+           "jump": torch.cat([torch.full((T // 2,), -30.0), torch.full((T - T // 2,), 30.0)])}[trend]
+    qn = torch.zeros(T, nh * d + 8)
+    for h in range(nh):
+        qn[:, h * d:(h + 1) * d] = 8.0 * u / scale ** 0.5
+    kn = kp.float().cpu()
+    for j in range(T):
+        page, off = int(bt[0, j // ps]), j % ps
+        kn[page, :, off, :] = (amp[j] * u / scale ** 0.5) + 0.05 * torch.randn(nkv, d, generator=g)
+    q, kp = dev(qn.bfloat16()), dev(kn.bfloat16())
+    b = ref.paged_attention(q, kp, vp, bt, seg, pos, nh, nkv, d, scale, 0)
+    a = ops.paged_attention(q, kp, vp, bt, seg, pos, nh, nkv, d, scale, 0, kernel="mfma")
+    assert torch.isfinite(a.float()).all()
+    assert torch.allclose(a.float(), b.float(), **tol(torch.bfloat16)), (a.float() - b.float()).abs().max()
+
+
 def test_matrix_core_attention_refuses_what_it_cannot_do(ops):
     q, kp, vp, bt, seg, pos = _paged_case(torch.bfloat16, 2, 1, 24, 16, [3], [3], seed=1)
     with pytest.raises(ValueError, match="multiple of 16"):
