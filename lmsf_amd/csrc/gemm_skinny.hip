@@ -31,6 +31,15 @@
 // would do this afterwards (vllm/kernels/pos_encoding_kernels.cu:38-77 and cache_kernels.cu:190-232 in the
 // reference) and its launch are gone from a decode step.
 //
+// Norm around the products (ACT == 4 and SCALED, up to 16 rows). An RMSNorm between two products is
+// x' = r * inv(r) * w with inv(r) = rsqrt(mean(r^2) + eps) one number per row, so inv can be taken out of the
+// product that follows: (r * w * inv) W^T = inv * ((r * w) W^T). The product before the norm (o, down:
+// ACT == 4) adds its rounded result to the float32 stream r in place and writes bf16(r * w) for the next
+// product and, per 16 columns, the sum of r^2; the product after it (SCALED: the gated and the rotary form)
+// adds up those sums while its first weights are on their way and multiplies its rows by inv before the bias.
+// The norm and the addition are then no kernel of their own (vllm/kernels/layernorm_kernels.cu:41-68 in the
+// reference); the values differ from the kernel's only in where the rounding to bfloat16 falls.
+//
 // MFMA: v_mfma_f32_16x16x32_bf16, A = W tile (16 rows x 32 k), B = x tile (32 k x 16 tokens), D[n][m]:
 // lane l holds token m = l % 16 and the four outputs n = (l / 16) * 4 .. + 3.
 #include "common.h"
@@ -47,14 +56,32 @@ struct SkinnyTile {
   static constexpr int STEPS = KC / 32;                     // MFMA steps per chunk
 };
 
-// ACT: 0 none (plain linear layer), 1 silu-gated, 2 gelu-gated, 3 rotary embedding and cache write
-template <int MT, int KC, int NW, typename TOut, int ACT, int DEPTH>
+// What the forms around a norm take beside the product's operands.
+struct NormAroundArgs {
+  // ACT == 4: the product before the norm
+  float* stream;              // [M, N] float32 residual stream, updated in place
+  long ld_stream;
+  const bf16_t* norm_weight;  // [N] of the norm that follows
+  float weight_offset;
+  float* sumsq_out;           // [ceil(N / 16)][16]: sums of stream^2 over 16 columns, per row (rows >= M: 0)
+  // SCALED: the product after the norm (its x is the bf16(stream * w) written above)
+  const float* sumsq_in;      // [in_tiles][16]
+  int in_tiles;
+  float eps;
+  int H;                      // columns of the stream: the mean is over these
+};
+
+// ACT: 0 none (plain linear layer), 1 silu-gated, 2 gelu-gated, 3 rotary embedding and cache write,
+// 4 add to the stream and prepare the norm that follows (y receives bf16(stream * w))
+template <int MT, int KC, int NW, typename TOut, int ACT, int DEPTH, bool SCALED>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ x, long ldx,
                                                               const bf16_t* __restrict__ W, long ldw,
                                                               const bf16_t* __restrict__ bias, TOut* __restrict__ y,
-                                                              long ldy, int M, int N, int K, RopeCacheArgs rc) {
+                                                              long ldy, int M, int N, int K, RopeCacheArgs rc,
+                                                              NormAroundArgs na) {
   using T = SkinnyTile<KC>;
-  constexpr int WT = ACT ? 2 : 1;   // W tiles per chunk: gate and up, the two halves of a head, or one
+  constexpr int WT = (ACT >= 1 && ACT <= 3) ? 2 : 1;   // W tiles per chunk: gate and up, the two halves of a head, or one
+  static_assert(!(SCALED || ACT == 4) || MT == 1, "the forms around a norm take up to 16 rows");
   extern __shared__ __align__(16) unsigned char lds[];
   const int tid = threadIdx.x;
   const int wave = tid / 64, lane = tid % 64;
@@ -116,9 +143,29 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __re
 
   // Every fetch is unconditional (a wave without a further chunk fetches its current one again, from
   // cache), which keeps the staged pieces in registers across the loop.
+  // SCALED: this thread's share of the sums of squares (row tid % 16). Loads come back in the order they were
+  // asked for: these go first and are added up once the first weights have been asked for, so that waiting
+  // for them does not wait for the weights.
+  constexpr int SQ_HELD = 8;
+  float sq_held[SQ_HELD];
+  if (SCALED) {
+#pragma unroll
+    for (int i = 0; i < SQ_HELD; ++i) {
+      const int e = tid + i * NW * 64;
+      sq_held[i] = e < na.in_tiles * 16 ? na.sumsq_in[e] : 0.f;
+    }
+  }
   int c = wave;
 #pragma unroll
   for (int b = 0; b < DEPTH; ++b) SKINNY_FETCH(b, c + b * NW < nchunks ? c + b * NW : 0);
+  float ssq = 0.f;
+  if (SCALED) {
+#pragma unroll
+    for (int i = 0; i < SQ_HELD; ++i) ssq += sq_held[i];
+    for (int e = tid + SQ_HELD * NW * 64; e < na.in_tiles * 16; e += NW * 64) ssq += na.sumsq_in[e];   // wider streams
+    ssq += __shfl_xor(ssq, 16, 64);
+    ssq += __shfl_xor(ssq, 32, 64);
+  }
   while (c < nchunks) {
 #pragma unroll
     for (int b = 0; b < DEPTH; ++b) {
@@ -156,11 +203,13 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __re
   // add the waves' partial sums in wave order
   __syncthreads();
   float* red = reinterpret_cast<float*>(lds);   // [NW][WT][MT][64 lanes][4]
+  float* extra = red + (size_t)NW * WT * MT * 256;   // SCALED: [NW][16] sums of squares; ACT 4: [256] squares
 #pragma unroll
   for (int wt = 0; wt < WT; ++wt)
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
       *reinterpret_cast<f32x4_t*>(red + ((((size_t)wave * WT + wt) * MT + mt) * 64 + lane) * 4) = acc[wt][mt];
+  if (SCALED && lane < 16) extra[wave * 16 + lane] = ssq;
   __syncthreads();
   for (int e = tid; e < MT * 256; e += NW * 64) {
     const int mt = e / 256, l = (e % 256) / 4, j = e % 4;
@@ -172,6 +221,29 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __re
       for (int w = 0; w < NW; ++w) sum[wt] += red[((((size_t)w * WT + wt) * MT + mt) * 64 + l) * 4 + j];
     }
     const int n = n0 + (l / 16) * 4 + j, m = mt * 16 + l % 16;
+    if (SCALED) {
+      float total = 0.f;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) total += extra[w * 16 + (l % 16)];
+      const float inv = rsqrtf(total / (float)na.H + na.eps);
+#pragma unroll
+      for (int wt = 0; wt < WT; ++wt) sum[wt] *= inv;
+    }
+    if (ACT == 4) {
+      // (MT == 1: thread e holds element e of the tile, row m = l % 16, column n)
+      float sq = 0.f;
+      if (n < N && m < M) {
+        float r = sum[0];
+        if (bias) r += bf16_to_f32(bias[n]);
+        float* st = na.stream + (long)m * na.ld_stream + n;
+        const float v = *st + bf16_to_f32(f32_to_bf16(r));   // the product rounded as it is where it is stored first
+        *st = v;
+        reinterpret_cast<bf16_t*>(y)[(long)m * ldy + n] = f32_to_bf16(v * (bf16_to_f32(na.norm_weight[n]) + na.weight_offset));
+        sq = v * v;
+      }
+      extra[e] = sq;
+      continue;
+    }
     if (ACT == 3) {
       if (m >= M) continue;
       float a = sum[0], b = sum[WT - 1];
@@ -234,17 +306,30 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __re
       y[(long)m * ldy + n] = from_f32<TOut>(r);
     }
   }
+  if (ACT == 4) {
+    // the tile's sum of squares per row, in a fixed order: element e = 4 l + j is row l % 16
+    __syncthreads();
+    if (tid < 16) {
+      float t = 0.f;
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) t += extra[(g * 16 + tid) * 4 + j];
+      na.sumsq_out[(long)blockIdx.x * 16 + tid] = t;
+    }
+  }
 }
 
-template <int MT, int KC, int NW, typename TOut, int ACT, int DEPTH = 1>
+template <int MT, int KC, int NW, typename TOut, int ACT, int DEPTH = 1, bool SCALED = false>
 static int launch_skinny(const void* x, long ldx, const void* W, long ldw, const void* bias, void* y, long ldy, int M,
-                         int N, int K, hipStream_t stream, RopeCacheArgs rc = RopeCacheArgs()) {
+                         int N, int K, hipStream_t stream, RopeCacheArgs rc = RopeCacheArgs(),
+                         NormAroundArgs na = NormAroundArgs()) {
   using T = SkinnyTile<KC>;
-  constexpr int WT = ACT ? 2 : 1;
+  constexpr int WT = (ACT >= 1 && ACT <= 3) ? 2 : 1;
   const size_t stage = (size_t)NW * (WT + MT) * T::TILE_BYTES;
-  const size_t red = (size_t)NW * WT * MT * 64 * 4 * sizeof(float);
+  const size_t red = (size_t)NW * WT * MT * 64 * 4 * sizeof(float) + ((SCALED || ACT == 4) ? 256 * sizeof(float) : 0);
   const size_t smem = stage > red ? stage : red;
-  auto kernel = gemm_skinny_kernel<MT, KC, NW, TOut, ACT, DEPTH>;
+  auto kernel = gemm_skinny_kernel<MT, KC, NW, TOut, ACT, DEPTH, SCALED>;
   static bool configured = false;   // per instantiation
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -258,7 +343,7 @@ static int launch_skinny(const void* x, long ldx, const void* W, long ldw, const
   // the gated form has a workgroup per 16 outputs, the rotary form one per 32 rows of W, the plain one per 16
   const int blocks = ACT == 3 ? N / 32 : (N + 15) / 16;
   hipLaunchKernelGGL(kernel, dim3(blocks), dim3(NW * 64), smem, stream, (const bf16_t*)x, ldx, (const bf16_t*)W, ldw,
-                     (const bf16_t*)bias, (TOut*)y, ldy, M, N, K, rc);
+                     (const bf16_t*)bias, (TOut*)y, ldy, M, N, K, rc, na);
   return 0;
 }
 
@@ -357,5 +442,99 @@ extern "C" int lmsf_gemm_qkv_rope_cache(const void* x, long ldx, const void* W, 
     r = launch_skinny<1, 64, 16, bf16_t, 3>(x, ldx, W, ldw, bias, y, ldy, M, (int)N, K, stream, rc);
   if (r) return r;
   LMSF_LAUNCH_CHECK("gemm_qkv_rope_cache");
+  return 0;
+}
+
+// The forms around a norm (up to 16 rows; see the top of the file).
+
+// The product before the norm: stream [M, N] float32 += bf16(x W^T + bias) in place; xw [M, N] = bf16(stream *
+// (norm_weight + weight_offset)); sumsq [ceil(N / 16)][16] = per 16 columns and row the sum of stream^2.
+extern "C" int lmsf_gemm_skinny_add_norm(const void* x, long ldx, const void* W, long ldw, const void* bias,
+                                         void* stream_f32, long ld_stream, const void* norm_weight,
+                                         float weight_offset, void* xw, long ld_xw, float* sumsq, int M, int N, int K,
+                                         int variant, hipStream_t stream) {
+  LMSF_CHECK(x && W && stream_f32 && norm_weight && xw && sumsq, "gemm_skinny_add_norm: null pointer");
+  LMSF_CHECK(M >= 0 && M <= 16, "gemm_skinny_add_norm: M=%d outside [0, 16]", M);
+  LMSF_CHECK(N > 0 && K > 0 && K % 8 == 0, "gemm_skinny_add_norm: K=%d must be a positive multiple of 8 (N=%d)", K, N);
+  LMSF_CHECK(ldx >= K && ldw >= K && ld_stream >= N && ld_xw >= N && ldx % 8 == 0 && ldw % 8 == 0,
+             "gemm_skinny_add_norm: row strides must cover the rows and those of x and W be multiples of 8");
+  LMSF_CHECK(lmsf_aligned16(x) && lmsf_aligned16(W), "gemm_skinny_add_norm: x and W must be 16-byte aligned");
+  if (M == 0) return 0;
+  NormAroundArgs na = NormAroundArgs();
+  na.stream = (float*)stream_f32; na.ld_stream = ld_stream;
+  na.norm_weight = (const bf16_t*)norm_weight; na.weight_offset = weight_offset;
+  na.sumsq_out = sumsq;
+  int r;
+  if (variant == 2)
+    r = launch_skinny<1, 64, 8, bf16_t, 4>(x, ldx, W, ldw, bias, xw, ld_xw, M, N, K, stream, RopeCacheArgs(), na);
+  else
+    r = launch_skinny<1, 64, 16, bf16_t, 4>(x, ldx, W, ldw, bias, xw, ld_xw, M, N, K, stream, RopeCacheArgs(), na);
+  if (r) return r;
+  LMSF_LAUNCH_CHECK("gemm_skinny_add_norm");
+  return 0;
+}
+
+static int scaled_check(const char* who, const float* sumsq, int in_tiles, int H) {
+  LMSF_CHECK(sumsq != nullptr && in_tiles > 0 && H > 0 && in_tiles == (H + 15) / 16,
+             "%s: %d sums of squares do not cover %d columns", who, in_tiles, H);
+  return 0;
+}
+
+// lmsf_gemm_skinny's gated form (act 1 silu, 2 gelu) after a norm: x [M, K] is bf16(stream * w) as written by
+// lmsf_gemm_skinny_add_norm, sumsq [in_tiles][16] its sums of squares; the two products' rows are multiplied
+// by rsqrt(sum / H + eps) before bias and activation. K == H.
+extern "C" int lmsf_gemm_skinny_scaled(const void* x, long ldx, const void* W, long ldw, const void* bias, void* y,
+                                       long ldy, int M, int N, int K, int act, const float* sumsq, int in_tiles,
+                                       float eps, int variant, hipStream_t stream) {
+  LMSF_CHECK(x && W && y, "gemm_skinny_scaled: null pointer");
+  LMSF_CHECK(M >= 0 && M <= 16, "gemm_skinny_scaled: M=%d outside [0, 16]", M);
+  LMSF_CHECK(N > 0 && K > 0 && K % 8 == 0, "gemm_skinny_scaled: K=%d must be a positive multiple of 8 (N=%d)", K, N);
+  LMSF_CHECK(ldx >= K && ldw >= K && ldy >= N && ldx % 8 == 0 && ldw % 8 == 0,
+             "gemm_skinny_scaled: row strides must cover K and be multiples of 8");
+  LMSF_CHECK(lmsf_aligned16(x) && lmsf_aligned16(W), "gemm_skinny_scaled: x and W must be 16-byte aligned");
+  LMSF_CHECK(act == 1 || act == 2, "gemm_skinny_scaled: activation %d (1 silu, 2 gelu)", act);
+  if (int rc = scaled_check("gemm_skinny_scaled", sumsq, in_tiles, K)) return rc;
+  if (M == 0) return 0;
+  NormAroundArgs na = NormAroundArgs();
+  na.sumsq_in = sumsq; na.in_tiles = in_tiles; na.eps = eps; na.H = K;
+  int r;
+  if (variant == 3)
+    r = act == 1 ? launch_skinny<1, 64, 16, bf16_t, 1, 1, true>(x, ldx, W, ldw, bias, y, ldy, M, N, K, stream, RopeCacheArgs(), na)
+                 : launch_skinny<1, 64, 16, bf16_t, 2, 1, true>(x, ldx, W, ldw, bias, y, ldy, M, N, K, stream, RopeCacheArgs(), na);
+  else
+    r = act == 1 ? launch_skinny<1, 64, 8, bf16_t, 1, 2, true>(x, ldx, W, ldw, bias, y, ldy, M, N, K, stream, RopeCacheArgs(), na)
+                 : launch_skinny<1, 64, 8, bf16_t, 2, 2, true>(x, ldx, W, ldw, bias, y, ldy, M, N, K, stream, RopeCacheArgs(), na);
+  if (r) return r;
+  LMSF_LAUNCH_CHECK("gemm_skinny_scaled");
+  return 0;
+}
+
+// lmsf_gemm_qkv_rope_cache after a norm: x and sumsq as in lmsf_gemm_skinny_scaled.
+extern "C" int lmsf_gemm_qkv_rope_cache_scaled(const void* x, long ldx, const void* W, long ldw, const void* bias,
+                                               void* y, long ldy, int M, int K, const int* positions,
+                                               const float* table, int max_pos, const int* slots, void* k_pages,
+                                               void* v_pages, long num_pages, int nh, int nkv, int d, int ps,
+                                               const float* sumsq, int in_tiles, float eps, hipStream_t stream) {
+  LMSF_CHECK(x && W && y && positions && table && slots && k_pages && v_pages, "gemm_qkv_rope_cache_scaled: null pointer");
+  LMSF_CHECK(M >= 0 && M <= 16, "gemm_qkv_rope_cache_scaled: M=%d outside [0, 16]", M);
+  LMSF_CHECK(nh > 0 && nkv > 0 && d >= 32 && d % 32 == 0, "gemm_qkv_rope_cache_scaled: head size %d must be a multiple of 32", d);
+  const long N = (long)(nh + 2 * nkv) * d;
+  LMSF_CHECK(N / 32 <= 2147483647L, "gemm_qkv_rope_cache_scaled: too many rows");
+  LMSF_CHECK(K > 0 && K % 8 == 0, "gemm_qkv_rope_cache_scaled: K=%d must be a positive multiple of 8", K);
+  LMSF_CHECK(ldx >= K && ldw >= K && ldy >= N && ldx % 8 == 0 && ldw % 8 == 0,
+             "gemm_qkv_rope_cache_scaled: row strides must cover K and be multiples of 8");
+  LMSF_CHECK(lmsf_aligned16(x) && lmsf_aligned16(W), "gemm_qkv_rope_cache_scaled: x and W must be 16-byte aligned");
+  LMSF_CHECK(ps > 0 && num_pages > 0 && max_pos > 0, "gemm_qkv_rope_cache_scaled: bad page geometry or empty table");
+  if (int rc = scaled_check("gemm_qkv_rope_cache_scaled", sumsq, in_tiles, K)) return rc;
+  if (M == 0) return 0;
+  RopeCacheArgs rc;
+  rc.positions = positions; rc.table = table; rc.slots = slots;
+  rc.k_pages = (bf16_t*)k_pages; rc.v_pages = (bf16_t*)v_pages;
+  rc.nh = nh; rc.nkv = nkv; rc.d = d; rc.ps = ps;
+  NormAroundArgs na = NormAroundArgs();
+  na.sumsq_in = sumsq; na.in_tiles = in_tiles; na.eps = eps; na.H = K;
+  int r = launch_skinny<1, 64, 16, bf16_t, 3, 1, true>(x, ldx, W, ldw, bias, y, ldy, M, (int)N, K, stream, rc, na);
+  if (r) return r;
+  LMSF_LAUNCH_CHECK("gemm_qkv_rope_cache_scaled");
   return 0;
 }

@@ -76,3 +76,34 @@ class NormedStream:
     @property
     def device(self) -> torch.device:
         return self.stream.device
+
+
+class ScaledRows:
+    """The RMSNorm of the float32 residual stream [M, H], M up to 16, with its row factor still to come:
+    ``xw`` is bf16(stream * (w + offset)) and ``sumsq`` [H / 16 tiles][16 rows] holds the sums of stream^2
+    over 16 columns each, both written by the product before the norm
+    (``HipOps.add_rms_norm(DeferredLinear, ..., defer_ok=True)``). The product that takes it
+    (``HipOps.qkv_rope_cache``, ``HipOps.linear_gated``) multiplies its rows by rsqrt(sum / H + eps), which
+    is the same product as with the normalised rows up to where the rounding falls. ``HipOps.materialize``
+    runs the norm kernel on the stream instead."""
+
+    __slots__ = ("xw", "sumsq", "tiles", "stream", "weight", "eps", "weight_offset", "dtype")
+
+    def __init__(self, xw: torch.Tensor, sumsq: torch.Tensor, tiles: int, stream: torch.Tensor, weight: torch.Tensor,
+                 eps: float, weight_offset: float, dtype: torch.dtype):
+        self.xw = xw
+        self.sumsq = sumsq
+        self.tiles = tiles
+        self.stream = stream
+        self.weight = weight
+        self.eps = eps
+        self.weight_offset = weight_offset
+        self.dtype = dtype
+
+    @property
+    def shape(self) -> Tuple[int, int]:
+        return tuple(self.xw.shape)
+
+    @property
+    def device(self) -> torch.device:
+        return self.xw.device

@@ -11,7 +11,7 @@ from typing import Optional
 import torch
 
 from . import library
-from .handles import DeferredLinear, NormedStream, PendingProduct
+from .handles import DeferredLinear, NormedStream, PendingProduct, ScaledRows
 
 F32 = 0
 BF16 = 1
@@ -50,6 +50,7 @@ class HipOps:
         self.use_library_gemm = True   # bfloat16 matrix products of many rows go to the BLAS library
         self.prefill_attention_variant = 0   # 0: keys and values staged in LDS; 1: fetched by every wave for itself
         self.decode_attention_splits = 0     # 0: chosen from the batch and the context; n: at most n splits of the keys
+        self.fuse_norm_rows = 16             # with up to this many rows (beyond fuse_stream_rows) the products around a norm do its work (0: never)
         self.fuse_stream_rows = 1            # with up to this many rows the residual addition and the norm run inside the products (0: never)
         self.gemv_max_rows = 2               # products of up to this many rows stream W without the matrix cores (0: never)
         self.skinny_variant = 0        # tiling of the few-rows kernel (0: default; others for tuning)
@@ -120,14 +121,28 @@ class HipOps:
         if isinstance(branch, PendingProduct):
             return self._add_rms_norm_pending(branch, residual, weight, eps, out_dtype, rows, weight_offset)
         if isinstance(branch, DeferredLinear):
-            if (rows is None and residual is not None and residual.dtype == torch.float32 and residual.is_contiguous()
-                    and tuple(residual.shape) == branch.shape):
+            M, N = branch.shape
+            fits = (rows is None and residual is not None and residual.dtype == torch.float32
+                    and residual.is_contiguous() and tuple(residual.shape) == branch.shape)
+            if fits and M <= min(self.fuse_stream_rows, self.gemv_max_rows) and self._gemv_ok(M, branch.x.shape[1]):
                 self._dev(branch.x, branch.weight, branch.bias, residual)
-                M, N = branch.shape
                 self._check(self.lib.lmsf_gemv_add(_ptr(branch.x), branch.x.stride(0), _ptr(branch.weight),
                                                    branch.weight.stride(0), _ptr(branch.bias), _ptr(residual),
                                                    residual.stride(0), M, N, branch.x.shape[1], self._stream()))
                 branch = None
+            elif (fits and defer_ok and M <= min(self.fuse_norm_rows, self.skinny_max_rows, 16)
+                  and out_dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and weight.is_contiguous()
+                  and weight.shape == (N,)):
+                # the product adds into the stream and leaves stream * w and the sums of squares for the next one
+                self._dev(branch.x, branch.weight, branch.bias, residual, weight)
+                tiles = -(-N // 16)
+                xw = torch.empty((M, N), dtype=torch.bfloat16, device=residual.device)
+                sumsq = torch.empty(tiles * 16, dtype=torch.float32, device=residual.device)
+                self._check(self.lib.lmsf_gemm_skinny_add_norm(
+                    _ptr(branch.x), branch.x.stride(0), _ptr(branch.weight), branch.weight.stride(0), _ptr(branch.bias),
+                    _ptr(residual), residual.stride(0), _ptr(weight), float(weight_offset), _ptr(xw), xw.stride(0),
+                    _ptr(sumsq), M, N, branch.x.shape[1], self.skinny_variant, self._stream()))
+                return ScaledRows(xw, sumsq, tiles, residual, weight, float(eps), float(weight_offset), out_dtype)
             else:
                 branch = self.materialize(branch)
         if (defer_ok and branch is None and rows is None and residual is not None and out_dtype == torch.bfloat16
@@ -184,7 +199,7 @@ class HipOps:
         ``DeferredLinear`` or the norm of a ``NormedStream``."""
         if isinstance(y, DeferredLinear):
             return self.linear(y.x, y.weight, y.bias, out_dtype=y.dtype)
-        if isinstance(y, NormedStream):
+        if isinstance(y, (NormedStream, ScaledRows)):
             return self.add_rms_norm(None, y.stream, y.weight, y.eps, y.dtype, weight_offset=y.weight_offset)
         if not isinstance(y, PendingProduct):
             return y
@@ -259,6 +274,20 @@ class HipOps:
         be a ``NormedStream``."""
         M, K = x.shape
         N = (nh + 2 * nkv) * d
+        if isinstance(x, ScaledRows):
+            if not (table is not None and slots is not None and neox and rot_dim == d and d % 32 == 0
+                    and weight.dtype == torch.bfloat16 and tuple(weight.shape) == (N, K) and weight.stride(1) == 1
+                    and self._skinny_ok(x.xw, weight) and k_pages is not None and k_pages.dtype == torch.bfloat16):
+                return self.qkv_rope_cache(self.materialize(x), weight, bias, nh, nkv, d, positions, table, rot_dim,
+                                           neox, slots, k_pages, v_pages)
+            self._dev(x.xw, x.sumsq, weight, bias, positions, table, slots, k_pages, v_pages)
+            num_pages, ps = self._check_qkv_fused(bias, weight, N, table, d, positions, slots, M, k_pages, v_pages, nkv)
+            y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+            self._check(self.lib.lmsf_gemm_qkv_rope_cache_scaled(
+                _ptr(x.xw), x.xw.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(y), y.stride(0), M, K,
+                _ptr(positions), _ptr(table), table.shape[0], _ptr(slots), _ptr(k_pages), _ptr(v_pages), num_pages,
+                nh, nkv, d, ps, _ptr(x.sumsq), x.tiles, x.eps, self._stream()))
+            return y
         if isinstance(x, NormedStream):
             if not (table is not None and slots is not None and neox and rot_dim == d and d % 32 == 0
                     and weight.dtype == torch.bfloat16 and tuple(weight.shape) == (N, K) and weight.stride(1) == 1
@@ -292,7 +321,7 @@ class HipOps:
                 _ptr(positions), _ptr(table), table.shape[0], _ptr(slots), _ptr(k_pages), _ptr(v_pages), num_pages,
                 nh, nkv, d, ps, self.skinny_variant, self._stream()))
             return y
-        y = self.linear(x, weight, bias, pending_ok=M > self.fuse_stream_rows)
+        y = self.linear(x, weight, bias, pending_ok=M > max(self.fuse_stream_rows, self.fuse_norm_rows, self.skinny_max_rows))
         if isinstance(y, PendingProduct):
             # 17 to 64 rows with K split: the rotation and the cache write add up the partial sums themselves
             if (table is None and slots is None) or tuple(weight.shape) != (N, K):
@@ -494,9 +523,10 @@ class HipOps:
         both_bf16 = x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
         if both_bf16 and self.skinny_max_rows < M <= 64 and self._mid_ok(x, weight):
             return self._linear_mid(x, weight, bias, 0, out_dtype, pending_ok and out_dtype == torch.bfloat16)
-        if (pending_ok and both_bf16 and out_dtype == torch.bfloat16 and self._skinny_ok(x, weight)
-                and 0 < M <= min(self.fuse_stream_rows, self.gemv_max_rows) and self._gemv_ok(M, K)):
-            return DeferredLinear(x, weight, bias, out_dtype)
+        if pending_ok and both_bf16 and out_dtype == torch.bfloat16 and self._skinny_ok(x, weight) and M > 0:
+            if (M <= min(self.fuse_stream_rows, self.gemv_max_rows) and self._gemv_ok(M, K)) \
+                    or M <= min(self.fuse_norm_rows, self.skinny_max_rows, 16):
+                return DeferredLinear(x, weight, bias, out_dtype)
         if both_bf16 and 0 < M <= min(1, self.gemv_max_rows) and self._skinny_ok(x, weight) and self._gemv_ok(M, K) \
                 and N * K <= 2 ** 28:
             # one row: a pure stream of W (with two rows only the fused forms gain; the LM head's matrix is large
@@ -541,6 +571,19 @@ class HipOps:
         if kind not in kinds:
             raise ValueError("unknown activation %r (known: %s)" % (kind, ", ".join(kinds)))
         M, I = x.shape[0], weight.shape[0] // 2
+        if isinstance(x, ScaledRows):
+            K = x.shape[1]
+            if not (weight.dtype == torch.bfloat16 and weight.shape[1] == K and weight.stride(1) == 1
+                    and self._skinny_ok(x.xw, weight)):
+                return self.linear_gated(self.materialize(x), weight, bias, kind)
+            self._dev(x.xw, x.sumsq, weight, bias)
+            if bias is not None and (bias.shape != (2 * I,) or bias.dtype != weight.dtype or not bias.is_contiguous()):
+                raise ValueError("linear_gated: bias must be [%d] of the weight's dtype" % (2 * I))
+            y = torch.empty((M, I), dtype=torch.bfloat16, device=x.device)
+            self._check(self.lib.lmsf_gemm_skinny_scaled(
+                _ptr(x.xw), x.xw.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(y), y.stride(0), M, I, K,
+                kinds[kind], _ptr(x.sumsq), x.tiles, x.eps, self.skinny_variant, self._stream()))
+            return y
         if isinstance(x, NormedStream):
             K = x.shape[1]
             if not (weight.dtype == torch.bfloat16 and weight.shape[1] == K and weight.stride(1) == 1

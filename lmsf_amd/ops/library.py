@@ -9,7 +9,7 @@ from typing import Optional
 
 from ..csrc import build as _build
 
-ABI_VERSION = 14
+ABI_VERSION = 15
 
 _lib: Optional[ctypes.CDLL] = None
 _lib_path: Optional[str] = None
@@ -41,6 +41,12 @@ _SIGNATURES = {
     "lmsf_gemm_skinny": (c_int, [_P, c_long, _P, c_long, _P, _P, c_int, c_long, c_int, c_int, c_int, c_int, c_int, _P]),
     "lmsf_gemm_qkv_rope_cache": (c_int, [_P, c_long, _P, c_long, _P, _P, c_long, c_int, c_int, _P, _P, c_int, _P, _P, _P,
                                          c_long, c_int, c_int, c_int, c_int, c_int, _P]),
+    "lmsf_gemm_skinny_add_norm": (c_int, [_P, c_long, _P, c_long, _P, _P, c_long, _P, c_float, _P, c_long, _P, c_int,
+                                          c_int, c_int, c_int, _P]),
+    "lmsf_gemm_skinny_scaled": (c_int, [_P, c_long, _P, c_long, _P, _P, c_long, c_int, c_int, c_int, c_int, _P, c_int,
+                                        c_float, c_int, _P]),
+    "lmsf_gemm_qkv_rope_cache_scaled": (c_int, [_P, c_long, _P, c_long, _P, _P, c_long, c_int, c_int, _P, _P, c_int, _P,
+                                                _P, _P, c_long, c_int, c_int, c_int, c_int, _P, c_int, c_float, _P]),
     "lmsf_gemv": (c_int, [_P, c_long, _P, c_long, _P, _P, c_int, c_long, c_int, c_int, c_int, c_int, _P]),
     "lmsf_gemv_qkv_rope_cache": (c_int, [_P, c_long, _P, c_long, _P, _P, c_long, c_int, c_int, _P, _P, c_int, _P, _P, _P,
                                          c_long, c_int, c_int, c_int, c_int, _P]),

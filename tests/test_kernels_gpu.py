@@ -636,6 +636,80 @@ def _addition_and_norm_inside(ops, ref, M, H, K, nh, nkv, d, I, bias, DeferredLi
     assert torch.is_tensor(ops.add_rms_norm(None, r1, nw.float(), 1e-5, torch.float32, defer_ok=True))
 
 
+@pytest.mark.parametrize("M", [2, 8, 16])
+@pytest.mark.parametrize("H,K,nh,nkv,d,I", [(4096, 4096, 32, 8, 128, 1024), (1000, 14336, 5, 5, 64, 331), (80, 128, 3, 1, 32, 77),
+                                            (8200, 256, 2, 2, 64, 96)])
+@pytest.mark.parametrize("bias", [False, True])
+def test_norm_done_by_the_products_around_it(ops, ref, M, H, K, nh, nkv, d, I, bias):
+    """With 2 to 16 rows the product before a norm adds its rounded result into the float32 stream and leaves
+    bf16(stream * w) and the sums of squares per 16 columns; the product after it multiplies its rows by
+    rsqrt(sum / H + eps). The stream gets the bits of product, then addition; the products agree with the norm
+    kernel's path up to where the rounding to bfloat16 falls."""
+    from lmsf_amd.ops.handles import DeferredLinear, ScaledRows
+    g = torch.Generator().manual_seed(M + H + K)
+    x = dev(torch.randn(M, K, generator=g).bfloat16())
+    w = dev((torch.randn(H, K, generator=g) * K ** -0.5).bfloat16())
+    b = dev(torch.randn(H, generator=g).bfloat16()) if bias else None
+    nw = dev(torch.randn(H, generator=g).bfloat16())
+    res0 = dev(torch.randn(M, H, generator=g) * 3.0)
+    p = ops.linear(x, w, b, pending_ok=True)
+    assert isinstance(p, DeferredLinear) and p.shape == (M, H)
+    y = ops.linear(x, w, b)
+    assert torch.equal(ops.materialize(p), y)
+    r1, r2 = res0.clone(), res0.clone()
+    h = ops.add_rms_norm(p, r1, nw, 1e-5, torch.bfloat16, weight_offset=0.25, defer_ok=True)
+    c = ops.add_rms_norm(y, r2, nw, 1e-5, torch.bfloat16, weight_offset=0.25)
+    assert torch.equal(r1, r2) and not torch.equal(r1, res0)
+    assert isinstance(h, ScaledRows) and h.shape == (M, H) and h.stream is r1 and h.tiles == -(-H // 16)
+    # what it holds: stream * w rounded, and sums of squares that add up to the rows' own
+    assert torch.equal(h.xw, (r1 * (nw.float() + 0.25)).bfloat16())
+    sums = h.sumsq.view(h.tiles, 16).sum(0)
+    want_sums = (r1.double() ** 2).sum(1)
+    assert torch.allclose(sums[:M].double(), want_sums, rtol=1e-5) and (M == 16 or float(sums[M:].abs().max()) == 0.0)
+    assert torch.equal(ops.materialize(h), c)
+    want_h = ref.add_rms_norm(y, res0.clone(), nw, 1e-5, torch.bfloat16, weight_offset=0.25)
+    wg = dev((torch.randn(2 * I, H, generator=g) * H ** -0.5).bfloat16())
+    bg = dev(torch.randn(2 * I, generator=g).bfloat16()) if bias else None
+    for kind in ("silu", "gelu"):
+        a = ops.linear_gated(h, wg, bg, kind)
+        want = ref.linear_gated(want_h, wg, bg, kind).float()
+        t = 2e-2 * max(1.0, want.abs().max().item())
+        assert a.shape == (M, I) and (a.float() - want).abs().max().item() <= t
+        assert (a.float() - ops.linear_gated(c, wg, bg, kind).float()).abs().max().item() <= t
+    N = (nh + 2 * nkv) * d
+    wq = dev((torch.randn(N, H, generator=g) * H ** -0.5).bfloat16())
+    bq = dev(torch.randn(N, generator=g).bfloat16()) if bias else None
+    max_pos, pages, ps = 50, 5, 8
+    pos = dev(torch.randint(0, max_pos, (M,), generator=g, dtype=torch.int32))
+    ang = torch.arange(max_pos, dtype=torch.float32)[:, None] * torch.rand(d // 2, generator=g)[None, :]
+    table = dev(torch.cat([ang.cos(), ang.sin()], dim=1).contiguous())
+    slots = torch.randperm(pages * ps, generator=g)[:M].to(torch.int32)
+    slots[1] = -1
+    slots = dev(slots)
+    k1, v1 = dev(torch.zeros(pages, nkv, ps, d).bfloat16()), dev(torch.zeros(pages, nkv, d, ps).bfloat16())
+    k2, v2 = k1.clone(), v1.clone()
+    a = ops.qkv_rope_cache(h, wq, bq, nh, nkv, d, pos, table, d, True, slots, k1, v1)
+    want = ref.qkv_rope_cache(want_h, wq, bq, nh, nkv, d, pos, table, d, True, slots, k2, v2)
+    t = 2e-2 * max(1.0, want.float().abs().max().item())
+    assert (a.float() - want.float()).abs().max().item() <= t
+    assert (k1.float() - k2.float()).abs().max().item() <= t and (v1.float() - v2.float()).abs().max().item() <= t
+    assert k1.float().abs().sum().item() > 0
+    # what the fused forms do not take sees the norm kernel's output: GPT-J pairing
+    k3, v3, k4, v4 = k1.clone().zero_(), v1.clone().zero_(), k1.clone().zero_(), v1.clone().zero_()
+    a = ops.qkv_rope_cache(h, wq, bq, nh, nkv, d, pos, table[:, :d // 2].contiguous(), d // 2, False, slots, k3, v3)
+    e = ops.qkv_rope_cache(c, wq, bq, nh, nkv, d, pos, table[:, :d // 2].contiguous(), d // 2, False, slots, k4, v4)
+    assert torch.equal(a, e) and torch.equal(k3, k4)
+    # the caller that does not take it, selected rows, a float32 norm weight: the norm kernel
+    r3 = res0.clone()
+    assert torch.equal(ops.add_rms_norm(p, r3, nw, 1e-5, torch.bfloat16, weight_offset=0.25), c) and torch.equal(r3, r1)
+    rows = dev(torch.tensor([M - 1], dtype=torch.int32))
+    r4 = res0.clone()
+    a = ops.add_rms_norm(p, r4, nw, 1e-5, torch.bfloat16, rows=rows, weight_offset=0.25, defer_ok=True)
+    assert torch.is_tensor(a) and torch.equal(a, c[M - 1:]) and torch.equal(r4, res0)
+    r5 = res0.clone()
+    assert torch.is_tensor(ops.add_rms_norm(p, r5, nw.float(), 1e-5, torch.bfloat16, weight_offset=0.25, defer_ok=True))
+
+
 def test_linear_mixed_storage(ops, ref):
     """A weight stored in 32 bits stays so and still multiplies bfloat16 activations."""
     g = torch.Generator().manual_seed(5)
