@@ -11,13 +11,11 @@
 // of that reader's rate, which is why these one or two rows get a kernel of their own.
 // The reference leaves these products to cuBLASLt (tops/src/cublas.rs:29-114).
 //
-// Two more forms take the kernels between two products of a decoder block into the products themselves,
-// where that costs nothing: ACT 4 adds the result, rounded to bfloat16 as a product would store it, to the
-// float32 residual stream in place (every element of the stream belongs to one wave); XN makes x from the
-// stream on the way into LDS, x = bf16(stream * rsqrt(mean(stream^2) + eps) * (w + offset)): every workgroup
-// does the whole row's statistics for itself (a few KB from L2, while its first rows of W are on their way).
-// The addition and the norm are then no kernels of their own (vllm/kernels/layernorm_kernels.cu:41-68 in the
-// reference).
+// Two more forms take the kernels between two products of a decoder block into the products themselves:
+// ACT 4 adds the result, rounded to bfloat16 as a product would store it, to the float32 residual stream in
+// place (every element of the stream belongs to one wave), and can write what the norm that follows needs;
+// SC takes that norm's row factor out of the product (see GemvNorm). The addition and the norm are then no
+// kernels of their own (vllm/kernels/layernorm_kernels.cu:41-68 in the reference).
 //
 // A "unit" is what one wave produces: ACT 0: output n (one row of W); ACT 1, 2: output n of the gated form
 // (rows n and N + n: gate and up); ACT 3: the rotation pair (i, i + d/2) of one head of the fused QKV
@@ -28,7 +26,6 @@ typedef __bf16 gemv_bf16x2_t __attribute__((ext_vector_type(2)));
 
 #define GEMV_WAVES 8
 #define GEMV_UNROLL 8   // 16-byte pieces per lane in flight per row: 8 x 512 = 4,096 elements of K
-#define GEMV_XN_MAX_K 8192   // the longest row whose float32 values a workgroup keeps in registers while it sums their squares
 
 // A wave's work is a list of pieces: for each of its units, for each of the unit's rows (one, or two with an
 // epilogue that joins two rows), the row's K in pieces of GEMV_UNROLL x 512 elements. The loads of the next
@@ -38,15 +35,22 @@ struct GemvCursor {
   int unit, row, kb;
 };
 
-// x as the RMSNorm of the float32 stream (XN): stream [M, K] with row stride ld, weight [K] bfloat16
+// The forms around a norm: ACT 4 with xw_out also writes bf16(stream * (weight + offset)) for the next product
+// and, per workgroup and row, the sum of the squares of the stream's elements it produced (sumsq_out
+// [workgroups][NX]); SC multiplies its rows by rsqrt(sum of sumsq_in / K + eps) before the bias, its x being
+// that bf16(stream * w): RMSNorm is r * inv(r) * w with one inv per row, and (r * w * inv) W^T =
+// inv * ((r * w) W^T).
 struct GemvNorm {
-  const float* stream;
-  long ld;
-  const bf16_t* weight;
+  const bf16_t* weight;   // [N] of the norm that follows (ACT 4)
   float eps, offset;
+  bf16_t* xw_out;
+  long ld_xw;
+  float* sumsq_out;
+  const float* sumsq_in;
+  int n_partials;
 };
 
-template <int NX, int ACT, typename TOut, bool XN>
+template <int NX, int ACT, typename TOut, bool SC>
 __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_kernel(const bf16_t* __restrict__ x, long ldx,
                                                                const bf16_t* __restrict__ W, long ldw,
                                                                const bf16_t* __restrict__ bias, TOut* __restrict__ y,
@@ -114,6 +118,13 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_kernel(const bf16_t* __r
     if (c.row == 0) multiply_into(acc0, c, wv);
     else multiply_into(acc1, c, wv);
   };
+  float inv_rms[NX];   // SC: the rows' factors
+  float sq_acc[NX];    // ACT 4 with xw_out: squares of what this wave added to the stream
+#pragma unroll
+  for (int m = 0; m < NX; ++m) {
+    inv_rms[m] = 1.f;
+    sq_acc[m] = 0.f;
+  }
   // the unit's rows are complete: add the lanes' sums, apply the epilogue, store
   auto finish = [&](int unit) {
     float p[NX], q[NX];
@@ -121,6 +132,10 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_kernel(const bf16_t* __r
     for (int m = 0; m < NX; ++m) {
       p[m] = wave_sum(acc0[m]);
       q[m] = ROWS == 2 ? wave_sum(acc1[m]) : 0.f;
+      if (SC) {
+        p[m] *= inv_rms[m];
+        q[m] *= inv_rms[m];
+      }
     }
     if (lane != 0) return;
     GemvCursor c0 = {unit, 0, 0}, c1 = {unit, ROWS - 1, 0};
@@ -136,7 +151,12 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_kernel(const bf16_t* __r
         y[(long)m * ldy + n] = from_f32<TOut>(a);
       } else if (ACT == 4) {
         float* st = reinterpret_cast<float*>(y) + (long)m * ldy + n;   // this form's output is the float32 stream
-        *st += bf16_to_f32(f32_to_bf16(a));
+        const float v = *st + bf16_to_f32(f32_to_bf16(a));
+        *st = v;
+        if (nm.xw_out) {
+          nm.xw_out[(long)m * nm.ld_xw + n] = f32_to_bf16(v * (bf16_to_f32(nm.weight[n]) + nm.offset));
+          sq_acc[m] += v * v;
+        }
       } else if (ACT == 1 || ACT == 2) {
         // the two products are rounded to the storage type before the activation, as the unfused path stores them
         const float g = bf16_to_f32(f32_to_bf16(a)), u = bf16_to_f32(f32_to_bf16(b));
@@ -180,59 +200,40 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_kernel(const bf16_t* __r
 
   GemvCursor cur = {(int)(blockIdx.x * GEMV_WAVES) + wave, 0, 0};
   uint4 wa[GEMV_UNROLL], wb[GEMV_UNROLL];
-  if (XN) {
-    // the stream first (loads come back in the order they were asked for, and these come from L2), then the
-    // first piece of W, then the statistics and the normalised x
-    constexpr int XP = GEMV_XN_MAX_K / (GEMV_WAVES * 64 * 4);   // float4 pieces of a row per thread
-    float4 sv[NX][XP];
-    float ss[NX];
+  {
+    float part[NX];
+    if (SC) {
+      // this thread's share of the sums of squares, asked for first (loads come back in order)
 #pragma unroll
-    for (int m = 0; m < NX; ++m) {
+      for (int m = 0; m < NX; ++m) part[m] = 0.f;
+      for (int i = tid; i < nm.n_partials; i += GEMV_WAVES * 64) {
 #pragma unroll
-      for (int j = 0; j < XP; ++j) {
-        const int k = (j * GEMV_WAVES * 64 + tid) * 4;
-        sv[m][j] = k < K ? *reinterpret_cast<const float4*>(nm.stream + (long)m * nm.ld + k) : make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int m = 0; m < NX; ++m) part[m] += nm.sumsq_in[(long)i * NX + m];
       }
     }
-    if (cur.unit < n_units) fetch(cur, wa);
-#pragma unroll
-    for (int m = 0; m < NX; ++m) {
-      ss[m] = 0.f;
-#pragma unroll
-      for (int j = 0; j < XP; ++j)
-        ss[m] += sv[m][j].x * sv[m][j].x + sv[m][j].y * sv[m][j].y + sv[m][j].z * sv[m][j].z + sv[m][j].w * sv[m][j].w;
-      ss[m] = wave_sum(ss[m]);
-      if (lane == 0) norm_red[wave][m] = ss[m];
-    }
-    __syncthreads();
-#pragma unroll
-    for (int m = 0; m < NX; ++m) {
-      float tot = 0.f;
-#pragma unroll
-      for (int w2 = 0; w2 < GEMV_WAVES; ++w2) tot += norm_red[w2][m];
-      const float inv = rsqrtf(tot / (float)K + nm.eps);
-#pragma unroll
-      for (int j = 0; j < XP; ++j) {
-        const int k = (j * GEMV_WAVES * 64 + tid) * 4;
-        if (k < K) {
-          const uint2 wv = *reinterpret_cast<const uint2*>(nm.weight + k);
-          uint2 o;
-          o.x = pack2_bf16(sv[m][j].x * inv * (__uint_as_float(wv.x << 16) + nm.offset),
-                           sv[m][j].y * inv * (__uint_as_float(wv.x & 0xffff0000u) + nm.offset));
-          o.y = pack2_bf16(sv[m][j].z * inv * (__uint_as_float(wv.y << 16) + nm.offset),
-                           sv[m][j].w * inv * (__uint_as_float(wv.y & 0xffff0000u) + nm.offset));
-          *reinterpret_cast<uint2*>(xs + (long)m * K + k) = o;
-        }
-      }
-    }
-  } else {
     if (cur.unit < n_units) fetch(cur, wa);
     for (int i = tid; i < NX * (K / 8); i += GEMV_WAVES * 64) {
       const int m = i / (K / 8), p = i - m * (K / 8);
       *reinterpret_cast<uint4*>(xs + (long)m * K + p * 8) = *reinterpret_cast<const uint4*>(x + (long)m * ldx + p * 8);
     }
+    if (SC) {
+#pragma unroll
+      for (int m = 0; m < NX; ++m) {
+        const float t = wave_sum(part[m]);
+        if (lane == 0) norm_red[wave][m] = t;
+      }
+    }
   }
   __syncthreads();
+  if (SC) {
+#pragma unroll
+    for (int m = 0; m < NX; ++m) {
+      float tot = 0.f;
+#pragma unroll
+      for (int w2 = 0; w2 < GEMV_WAVES; ++w2) tot += norm_red[w2][m];
+      inv_rms[m] = rsqrtf(tot / (float)K + nm.eps);
+    }
+  }
   // one piece per half of the loop body, the two register sets taking turns
 #define GEMV_HALF(mine, other)                                                       \
   {                                                                                  \
@@ -249,14 +250,34 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_kernel(const bf16_t* __r
     GEMV_HALF(wb, wa);
   }
 #undef GEMV_HALF
+  if (ACT == 4 && nm.sumsq_out) {
+    // the workgroup's sums of squares, the waves' in wave order (every wave comes here, with or without units)
+    if (lane == 0) {
+#pragma unroll
+      for (int m = 0; m < NX; ++m) norm_red[wave][m] = sq_acc[m];
+    }
+    __syncthreads();
+    if (tid < NX) {
+      float t = 0.f;
+#pragma unroll
+      for (int w2 = 0; w2 < GEMV_WAVES; ++w2) t += norm_red[w2][tid];
+      nm.sumsq_out[(long)blockIdx.x * NX + tid] = t;
+    }
+  }
 }
 
-template <int NX, int ACT, typename TOut, bool XN = false>
+// workgroups of a launch over n_units units: every wave takes one unit at a time
+static long gemv_blocks(long n_units) {
+  long blocks = (n_units + GEMV_WAVES - 1) / GEMV_WAVES;
+  return blocks > 2048 ? 2048 : blocks;
+}
+
+template <int NX, int ACT, typename TOut, bool SC = false>
 static int launch_gemv(const void* x, long ldx, const void* W, long ldw, const void* bias, void* y, long ldy, int N,
                        int K, int n_units, hipStream_t stream, RopeCacheArgs rc = RopeCacheArgs(),
                        GemvNorm nm = GemvNorm()) {
   const size_t smem = (size_t)NX * K * sizeof(bf16_t);
-  auto kernel = gemv_kernel<NX, ACT, TOut, XN>;
+  auto kernel = gemv_kernel<NX, ACT, TOut, SC>;
   static size_t configured = 0;   // per instantiation: the largest LDS size asked for so far
   if (smem > configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -267,9 +288,7 @@ static int launch_gemv(const void* x, long ldx, const void* W, long ldw, const v
     }
     configured = smem;
   }
-  // every wave takes one unit at a time; at most 8 workgroups per compute unit's worth of them
-  long blocks = ((long)n_units + GEMV_WAVES - 1) / GEMV_WAVES;
-  if (blocks > 2048) blocks = 2048;
+  const long blocks = gemv_blocks(n_units);   // at most 8 workgroups per compute unit's worth of them
   hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(GEMV_WAVES * 64), smem, stream, (const bf16_t*)x, ldx,
                      (const bf16_t*)W, ldw, (const bf16_t*)bias, (TOut*)y, ldy, N, K, n_units, rc, nm);
   return 0;
@@ -334,15 +353,6 @@ extern "C" int lmsf_gemv_qkv_rope_cache(const void* x, long ldx, const void* W, 
   return 0;
 }
 
-static int gemv_norm_check(const char* who, const void* stream_f32, long ld, const void* norm_weight, int M, int K) {
-  LMSF_CHECK(stream_f32 && norm_weight, "%s: null pointer", who);
-  LMSF_CHECK(K % 4 == 0 && K <= GEMV_XN_MAX_K, "%s: K=%d must be a multiple of 4, at most %d", who, K, GEMV_XN_MAX_K);
-  LMSF_CHECK(ld >= K && ld % 4 == 0 && lmsf_aligned16(stream_f32) && ((uintptr_t)norm_weight & 7) == 0,
-             "%s: the stream must be 16-byte aligned with a row stride that is a multiple of 4, the norm's weight 8-byte aligned", who);
-  (void)M;
-  return 0;
-}
-
 // y += bf16(x W^T + bias): y is the float32 residual stream [M, N] with row stride ldy, updated in place; the
 // product is rounded to bfloat16 first, as it is where it is stored before it is added. x, W as in lmsf_gemv.
 extern "C" int lmsf_gemv_add(const void* x, long ldx, const void* W, long ldw, const void* bias, void* y, long ldy,
@@ -357,53 +367,76 @@ extern "C" int lmsf_gemv_add(const void* x, long ldx, const void* W, long ldw, c
   return 0;
 }
 
-// lmsf_gemv with x = bf16(s * rsqrt(mean(s^2) + eps) * (norm_weight + weight_offset)) made from the float32
-// stream s [M, K] (row stride ld) inside the kernel; norm_weight [K] bfloat16; y bfloat16. K <= 8192.
-extern "C" int lmsf_gemv_normed(const void* stream_f32, long ld, const void* norm_weight, float eps,
-                                float weight_offset, const void* W, long ldw, const void* bias, void* y, long ldy,
-                                int M, int N, int K, int act, hipStream_t stream) {
-  if (int rc = gemv_norm_check("gemv_normed", stream_f32, ld, norm_weight, M, K)) return rc;
-  if (int rc = gemv_check("gemv_normed", W, ldw, W, ldw, M, N, K)) return rc;
-  LMSF_CHECK(y != nullptr && ldy >= N, "gemv_normed: bad output");
-  LMSF_CHECK(act >= 0 && act <= 2, "gemv_normed: unknown activation %d", act);
+// The forms around a norm for one or two rows (see GemvNorm).
+
+// Workgroups, and so sums of squares per row, of lmsf_gemv_add_norm with N outputs.
+extern "C" int lmsf_gemv_partials(int N) { return (int)gemv_blocks(N); }
+
+// lmsf_gemv_add that also writes xw [M, N] = bf16(stream * (norm_weight + weight_offset)) and
+// sumsq [lmsf_gemv_partials(N)][M]: per workgroup and row the sum of the squares of the stream's elements
+// that the workgroup produced.
+extern "C" int lmsf_gemv_add_norm(const void* x, long ldx, const void* W, long ldw, const void* bias, void* y,
+                                  long ldy, const void* norm_weight, float weight_offset, void* xw, long ld_xw,
+                                  float* sumsq, int M, int N, int K, hipStream_t stream) {
+  if (int rc = gemv_check("gemv_add_norm", x, ldx, W, ldw, M, N, K)) return rc;
+  LMSF_CHECK(y != nullptr && ldy >= N && norm_weight && xw && ld_xw >= N && sumsq, "gemv_add_norm: bad output");
   if (M == 0) return 0;
-  GemvNorm nm = {(const float*)stream_f32, ld, (const bf16_t*)norm_weight, eps, weight_offset};
-  int r;
-#define GV(NX_)                                                                                                       \
-  r = act == 1   ? launch_gemv<NX_, 1, bf16_t, true>(nullptr, 0, W, ldw, bias, y, ldy, N, K, N, stream, RopeCacheArgs(), nm) \
-      : act == 2 ? launch_gemv<NX_, 2, bf16_t, true>(nullptr, 0, W, ldw, bias, y, ldy, N, K, N, stream, RopeCacheArgs(), nm) \
-                 : launch_gemv<NX_, 0, bf16_t, true>(nullptr, 0, W, ldw, bias, y, ldy, N, K, N, stream, RopeCacheArgs(), nm)
-  if (M == 1) GV(1); else GV(2);
-#undef GV
+  GemvNorm nm = GemvNorm();
+  nm.weight = (const bf16_t*)norm_weight; nm.offset = weight_offset;
+  nm.xw_out = (bf16_t*)xw; nm.ld_xw = ld_xw; nm.sumsq_out = sumsq;
+  int r = M == 1 ? launch_gemv<1, 4, float>(x, ldx, W, ldw, bias, y, ldy, N, K, N, stream, RopeCacheArgs(), nm)
+                 : launch_gemv<2, 4, float>(x, ldx, W, ldw, bias, y, ldy, N, K, N, stream, RopeCacheArgs(), nm);
   if (r) return r;
-  LMSF_LAUNCH_CHECK("gemv_normed");
+  LMSF_LAUNCH_CHECK("gemv_add_norm");
   return 0;
 }
 
-// lmsf_gemv_qkv_rope_cache with x made from the float32 stream as in lmsf_gemv_normed.
-extern "C" int lmsf_gemv_normed_qkv_rope_cache(const void* stream_f32, long ld, const void* norm_weight, float eps,
-                                               float weight_offset, const void* W, long ldw, const void* bias,
+// lmsf_gemv's gated forms (act 1 silu, 2 gelu) after a norm: x is the xw of lmsf_gemv_add_norm, sumsq its sums
+// ([n_partials][M]); rows are multiplied by rsqrt(sum / K + eps) before bias and activation.
+extern "C" int lmsf_gemv_scaled(const void* x, long ldx, const void* W, long ldw, const void* bias, void* y, long ldy,
+                                int M, int N, int K, int act, const float* sumsq, int n_partials, float eps,
+                                hipStream_t stream) {
+  if (int rc = gemv_check("gemv_scaled", x, ldx, W, ldw, M, N, K)) return rc;
+  LMSF_CHECK(y != nullptr && ldy >= N && sumsq && n_partials > 0, "gemv_scaled: bad output or sums");
+  LMSF_CHECK(act == 1 || act == 2, "gemv_scaled: activation %d (1 silu, 2 gelu)", act);
+  if (M == 0) return 0;
+  GemvNorm nm = GemvNorm();
+  nm.sumsq_in = sumsq; nm.n_partials = n_partials; nm.eps = eps;
+  int r;
+#define GV(NX_)                                                                                                          \
+  r = act == 1 ? launch_gemv<NX_, 1, bf16_t, true>(x, ldx, W, ldw, bias, y, ldy, N, K, N, stream, RopeCacheArgs(), nm) \
+               : launch_gemv<NX_, 2, bf16_t, true>(x, ldx, W, ldw, bias, y, ldy, N, K, N, stream, RopeCacheArgs(), nm)
+  if (M == 1) GV(1); else GV(2);
+#undef GV
+  if (r) return r;
+  LMSF_LAUNCH_CHECK("gemv_scaled");
+  return 0;
+}
+
+// lmsf_gemv_qkv_rope_cache after a norm: x and sumsq as in lmsf_gemv_scaled.
+extern "C" int lmsf_gemv_scaled_qkv_rope_cache(const void* x, long ldx, const void* W, long ldw, const void* bias,
                                                void* y, long ldy, int M, int K, const int* positions,
                                                const float* table, int max_pos, const int* slots, void* k_pages,
                                                void* v_pages, long num_pages, int nh, int nkv, int d, int ps,
-                                               hipStream_t stream) {
-  LMSF_CHECK(y && positions && table && slots && k_pages && v_pages, "gemv_normed_qkv_rope_cache: null pointer");
-  LMSF_CHECK(nh > 0 && nkv > 0 && d >= 2 && d % 2 == 0, "gemv_normed_qkv_rope_cache: head size %d must be even", d);
+                                               const float* sumsq, int n_partials, float eps, hipStream_t stream) {
+  LMSF_CHECK(y && positions && table && slots && k_pages && v_pages, "gemv_scaled_qkv_rope_cache: null pointer");
+  LMSF_CHECK(nh > 0 && nkv > 0 && d >= 2 && d % 2 == 0, "gemv_scaled_qkv_rope_cache: head size %d must be even", d);
   const long N = (long)(nh + 2 * nkv) * d;
-  if (int rc = gemv_norm_check("gemv_normed_qkv_rope_cache", stream_f32, ld, norm_weight, M, K)) return rc;
-  if (int rc = gemv_check("gemv_normed_qkv_rope_cache", W, ldw, W, ldw, M, N, K)) return rc;
-  LMSF_CHECK(ldy >= N, "gemv_normed_qkv_rope_cache: row stride of y below %ld", N);
-  LMSF_CHECK(ps > 0 && num_pages > 0 && max_pos > 0, "gemv_normed_qkv_rope_cache: bad page geometry or empty table");
+  if (int rc = gemv_check("gemv_scaled_qkv_rope_cache", x, ldx, W, ldw, M, N, K)) return rc;
+  LMSF_CHECK(ldy >= N, "gemv_scaled_qkv_rope_cache: row stride of y below %ld", N);
+  LMSF_CHECK(ps > 0 && num_pages > 0 && max_pos > 0, "gemv_scaled_qkv_rope_cache: bad page geometry or empty table");
+  LMSF_CHECK(sumsq && n_partials > 0, "gemv_scaled_qkv_rope_cache: no sums of squares");
   if (M == 0) return 0;
   RopeCacheArgs rc;
   rc.positions = positions; rc.table = table; rc.slots = slots;
   rc.k_pages = (bf16_t*)k_pages; rc.v_pages = (bf16_t*)v_pages;
   rc.nh = nh; rc.nkv = nkv; rc.d = d; rc.ps = ps;
-  GemvNorm nm = {(const float*)stream_f32, ld, (const bf16_t*)norm_weight, eps, weight_offset};
+  GemvNorm nm = GemvNorm();
+  nm.sumsq_in = sumsq; nm.n_partials = n_partials; nm.eps = eps;
   const int n_units = (int)(N / 2);
-  int r = M == 1 ? launch_gemv<1, 3, bf16_t, true>(nullptr, 0, W, ldw, bias, y, ldy, (int)N, K, n_units, stream, rc, nm)
-                 : launch_gemv<2, 3, bf16_t, true>(nullptr, 0, W, ldw, bias, y, ldy, (int)N, K, n_units, stream, rc, nm);
+  int r = M == 1 ? launch_gemv<1, 3, bf16_t, true>(x, ldx, W, ldw, bias, y, ldy, (int)N, K, n_units, stream, rc, nm)
+                 : launch_gemv<2, 3, bf16_t, true>(x, ldx, W, ldw, bias, y, ldy, (int)N, K, n_units, stream, rc, nm);
   if (r) return r;
-  LMSF_LAUNCH_CHECK("gemv_normed_qkv_rope_cache");
+  LMSF_LAUNCH_CHECK("gemv_scaled_qkv_rope_cache");
   return 0;
 }

@@ -53,47 +53,25 @@ class DeferredLinear:
         return self.x.device
 
 
-class NormedStream:
-    """The RMSNorm of the float32 residual stream [M, H], M one or two, not computed yet: the product that
-    takes it (``HipOps.qkv_rope_cache``, ``HipOps.linear_gated``) normalises the row while it brings it into
-    LDS. ``HipOps.add_rms_norm(..., defer_ok=True)`` makes one; the stream must not change before the
-    product has run. ``HipOps.materialize`` runs the norm."""
-
-    __slots__ = ("stream", "weight", "eps", "weight_offset", "dtype")
-
-    def __init__(self, stream: torch.Tensor, weight: torch.Tensor, eps: float, weight_offset: float,
-                 dtype: torch.dtype):
-        self.stream = stream
-        self.weight = weight
-        self.eps = eps
-        self.weight_offset = weight_offset
-        self.dtype = dtype
-
-    @property
-    def shape(self) -> Tuple[int, int]:
-        return tuple(self.stream.shape)
-
-    @property
-    def device(self) -> torch.device:
-        return self.stream.device
-
-
 class ScaledRows:
-    """The RMSNorm of the float32 residual stream [M, H], M up to 16, with its row factor still to come:
-    ``xw`` is bf16(stream * (w + offset)) and ``sumsq`` [H / 16 tiles][16 rows] holds the sums of stream^2
-    over 16 columns each, both written by the product before the norm
+    """The RMSNorm of the float32 residual stream [M, H], M up to 16, with its row factor still to come
+    (RMSNorm is r * inv(r) * w with one inv per row, and (r * w * inv) W^T = inv * ((r * w) W^T)):
+    ``xw`` is bf16(stream * (w + offset)) and ``sumsq`` [tiles][rows_per_tile] holds sums of stream^2 over a
+    part of the columns each (16 columns, or what a workgroup produced), both written by the product before
+    the norm
     (``HipOps.add_rms_norm(DeferredLinear, ..., defer_ok=True)``). The product that takes it
     (``HipOps.qkv_rope_cache``, ``HipOps.linear_gated``) multiplies its rows by rsqrt(sum / H + eps), which
     is the same product as with the normalised rows up to where the rounding falls. ``HipOps.materialize``
     runs the norm kernel on the stream instead."""
 
-    __slots__ = ("xw", "sumsq", "tiles", "stream", "weight", "eps", "weight_offset", "dtype")
+    __slots__ = ("xw", "sumsq", "tiles", "rows_per_tile", "stream", "weight", "eps", "weight_offset", "dtype")
 
-    def __init__(self, xw: torch.Tensor, sumsq: torch.Tensor, tiles: int, stream: torch.Tensor, weight: torch.Tensor,
-                 eps: float, weight_offset: float, dtype: torch.dtype):
+    def __init__(self, xw: torch.Tensor, sumsq: torch.Tensor, tiles: int, rows_per_tile: int, stream: torch.Tensor,
+                 weight: torch.Tensor, eps: float, weight_offset: float, dtype: torch.dtype):
         self.xw = xw
         self.sumsq = sumsq
         self.tiles = tiles
+        self.rows_per_tile = rows_per_tile   # 16: written by the few-rows product; M: by the one-or-two-rows product
         self.stream = stream
         self.weight = weight
         self.eps = eps

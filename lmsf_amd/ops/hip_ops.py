@@ -11,7 +11,7 @@ from typing import Optional
 import torch
 
 from . import library
-from .handles import DeferredLinear, NormedStream, PendingProduct, ScaledRows
+from .handles import DeferredLinear, PendingProduct, ScaledRows
 
 F32 = 0
 BF16 = 1
@@ -116,7 +116,7 @@ class HipOps:
         and ``rows`` is None. ``rows`` (int32 [R]) selects input rows; the output then has R rows.
         ``branch`` may be a ``PendingProduct``: its partial sums are added up on the way in; or a
         ``DeferredLinear``, which then runs as a product that adds into ``residual``. With ``defer_ok``
-        the caller takes a ``NormedStream`` as well (one or two rows, nothing left to add).
+        the caller takes a ``ScaledRows`` as well (up to 16 rows, after a ``DeferredLinear``).
         """
         if isinstance(branch, PendingProduct):
             return self._add_rms_norm_pending(branch, residual, weight, eps, out_dtype, rows, weight_offset)
@@ -124,15 +124,27 @@ class HipOps:
             M, N = branch.shape
             fits = (rows is None and residual is not None and residual.dtype == torch.float32
                     and residual.is_contiguous() and tuple(residual.shape) == branch.shape)
+            norm_ok = (defer_ok and out_dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
+                       and weight.is_contiguous() and weight.shape == (N,))
+            if (fits and norm_ok and M <= min(self.fuse_stream_rows, self.gemv_max_rows)
+                    and self._gemv_ok(M, branch.x.shape[1]) and self._gemv_ok(M, N)):
+                # the product adds into the stream and leaves stream * w and its workgroups' sums of squares
+                self._dev(branch.x, branch.weight, branch.bias, residual, weight)
+                parts = self.lib.lmsf_gemv_partials(N)
+                xw = torch.empty((M, N), dtype=torch.bfloat16, device=residual.device)
+                sumsq = torch.empty(parts * M, dtype=torch.float32, device=residual.device)
+                self._check(self.lib.lmsf_gemv_add_norm(
+                    _ptr(branch.x), branch.x.stride(0), _ptr(branch.weight), branch.weight.stride(0), _ptr(branch.bias),
+                    _ptr(residual), residual.stride(0), _ptr(weight), float(weight_offset), _ptr(xw), xw.stride(0),
+                    _ptr(sumsq), M, N, branch.x.shape[1], self._stream()))
+                return ScaledRows(xw, sumsq, parts, M, residual, weight, float(eps), float(weight_offset), out_dtype)
             if fits and M <= min(self.fuse_stream_rows, self.gemv_max_rows) and self._gemv_ok(M, branch.x.shape[1]):
                 self._dev(branch.x, branch.weight, branch.bias, residual)
                 self._check(self.lib.lmsf_gemv_add(_ptr(branch.x), branch.x.stride(0), _ptr(branch.weight),
                                                    branch.weight.stride(0), _ptr(branch.bias), _ptr(residual),
                                                    residual.stride(0), M, N, branch.x.shape[1], self._stream()))
                 branch = None
-            elif (fits and defer_ok and M <= min(self.fuse_norm_rows, self.skinny_max_rows, 16)
-                  and out_dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and weight.is_contiguous()
-                  and weight.shape == (N,)):
+            elif fits and norm_ok and M <= min(self.fuse_norm_rows, self.skinny_max_rows, 16):
                 # the product adds into the stream and leaves stream * w and the sums of squares for the next one
                 self._dev(branch.x, branch.weight, branch.bias, residual, weight)
                 tiles = -(-N // 16)
@@ -142,16 +154,9 @@ class HipOps:
                     _ptr(branch.x), branch.x.stride(0), _ptr(branch.weight), branch.weight.stride(0), _ptr(branch.bias),
                     _ptr(residual), residual.stride(0), _ptr(weight), float(weight_offset), _ptr(xw), xw.stride(0),
                     _ptr(sumsq), M, N, branch.x.shape[1], self.skinny_variant, self._stream()))
-                return ScaledRows(xw, sumsq, tiles, residual, weight, float(eps), float(weight_offset), out_dtype)
+                return ScaledRows(xw, sumsq, tiles, 16, residual, weight, float(eps), float(weight_offset), out_dtype)
             else:
                 branch = self.materialize(branch)
-        if (defer_ok and branch is None and rows is None and residual is not None and out_dtype == torch.bfloat16
-                and 0 < residual.shape[0] <= min(self.fuse_stream_rows, self.gemv_max_rows)
-                and residual.dtype == torch.float32 and residual.dim() == 2 and residual.is_contiguous()
-                and weight.dtype == torch.bfloat16 and weight.is_contiguous() and weight.shape == (residual.shape[1],)
-                and residual.shape[1] % 8 == 0 and residual.shape[1] <= 8192 and residual.data_ptr() % 16 == 0
-                and weight.data_ptr() % 8 == 0):
-            return NormedStream(residual, weight, float(eps), float(weight_offset), out_dtype)
         self._dev(branch, residual, weight, rows)
         ref = branch if branch is not None else residual
         if ref is None:
@@ -196,10 +201,10 @@ class HipOps:
 
     def materialize(self, y):
         """The tensor behind ``y``: ``y`` itself, the finished sum of a ``PendingProduct``, the product of a
-        ``DeferredLinear`` or the norm of a ``NormedStream``."""
+        ``DeferredLinear`` or the norm of a ``ScaledRows``."""
         if isinstance(y, DeferredLinear):
             return self.linear(y.x, y.weight, y.bias, out_dtype=y.dtype)
-        if isinstance(y, (NormedStream, ScaledRows)):
+        if isinstance(y, ScaledRows):
             return self.add_rms_norm(None, y.stream, y.weight, y.eps, y.dtype, weight_offset=y.weight_offset)
         if not isinstance(y, PendingProduct):
             return y
@@ -271,37 +276,29 @@ class HipOps:
         """The fused QKV projection, the rotation of its q and k heads and the write of k and v into the
         pages: ``linear`` followed by ``rope_cache_write``, with the same results. With few bfloat16 rows and
         a NeoX rotation over the whole head, the rotation and the write are the product's epilogue. ``x`` may
-        be a ``NormedStream``."""
+        be a ``ScaledRows``."""
         M, K = x.shape
         N = (nh + 2 * nkv) * d
         if isinstance(x, ScaledRows):
             if not (table is not None and slots is not None and neox and rot_dim == d and d % 32 == 0
                     and weight.dtype == torch.bfloat16 and tuple(weight.shape) == (N, K) and weight.stride(1) == 1
-                    and self._skinny_ok(x.xw, weight) and k_pages is not None and k_pages.dtype == torch.bfloat16):
+                    and self._skinny_ok(x.xw, weight) and k_pages is not None and k_pages.dtype == torch.bfloat16
+                    and (x.rows_per_tile == 16 or self._gemv_ok(M, K))):
                 return self.qkv_rope_cache(self.materialize(x), weight, bias, nh, nkv, d, positions, table, rot_dim,
                                            neox, slots, k_pages, v_pages)
             self._dev(x.xw, x.sumsq, weight, bias, positions, table, slots, k_pages, v_pages)
             num_pages, ps = self._check_qkv_fused(bias, weight, N, table, d, positions, slots, M, k_pages, v_pages, nkv)
             y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+            if x.rows_per_tile != 16:
+                self._check(self.lib.lmsf_gemv_scaled_qkv_rope_cache(
+                    _ptr(x.xw), x.xw.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(y), y.stride(0), M, K,
+                    _ptr(positions), _ptr(table), table.shape[0], _ptr(slots), _ptr(k_pages), _ptr(v_pages), num_pages,
+                    nh, nkv, d, ps, _ptr(x.sumsq), x.tiles, x.eps, self._stream()))
+                return y
             self._check(self.lib.lmsf_gemm_qkv_rope_cache_scaled(
                 _ptr(x.xw), x.xw.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(y), y.stride(0), M, K,
                 _ptr(positions), _ptr(table), table.shape[0], _ptr(slots), _ptr(k_pages), _ptr(v_pages), num_pages,
                 nh, nkv, d, ps, _ptr(x.sumsq), x.tiles, x.eps, self._stream()))
-            return y
-        if isinstance(x, NormedStream):
-            if not (table is not None and slots is not None and neox and rot_dim == d and d % 32 == 0
-                    and weight.dtype == torch.bfloat16 and tuple(weight.shape) == (N, K) and weight.stride(1) == 1
-                    and weight.stride(0) % 8 == 0 and weight.data_ptr() % 16 == 0 and self._gemv_ok(M, K)
-                    and k_pages is not None and k_pages.dtype == torch.bfloat16):
-                return self.qkv_rope_cache(self.materialize(x), weight, bias, nh, nkv, d, positions, table, rot_dim,
-                                           neox, slots, k_pages, v_pages)
-            self._dev(x.stream, x.weight, weight, bias, positions, table, slots, k_pages, v_pages)
-            num_pages, ps = self._check_qkv_fused(bias, weight, N, table, d, positions, slots, M, k_pages, v_pages, nkv)
-            y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
-            self._check(self.lib.lmsf_gemv_normed_qkv_rope_cache(
-                _ptr(x.stream), x.stream.stride(0), _ptr(x.weight), x.eps, x.weight_offset, _ptr(weight),
-                weight.stride(0), _ptr(bias), _ptr(y), y.stride(0), M, K, _ptr(positions), _ptr(table), table.shape[0],
-                _ptr(slots), _ptr(k_pages), _ptr(v_pages), num_pages, nh, nkv, d, ps, self._stream()))
             return y
         if (table is not None and slots is not None and neox and rot_dim == d and d % 32 == 0
                 and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and 0 < M <= self.skinny_max_rows
@@ -574,28 +571,20 @@ class HipOps:
         if isinstance(x, ScaledRows):
             K = x.shape[1]
             if not (weight.dtype == torch.bfloat16 and weight.shape[1] == K and weight.stride(1) == 1
-                    and self._skinny_ok(x.xw, weight)):
+                    and self._skinny_ok(x.xw, weight) and (x.rows_per_tile == 16 or self._gemv_ok(M, K))):
                 return self.linear_gated(self.materialize(x), weight, bias, kind)
             self._dev(x.xw, x.sumsq, weight, bias)
             if bias is not None and (bias.shape != (2 * I,) or bias.dtype != weight.dtype or not bias.is_contiguous()):
                 raise ValueError("linear_gated: bias must be [%d] of the weight's dtype" % (2 * I))
             y = torch.empty((M, I), dtype=torch.bfloat16, device=x.device)
+            if x.rows_per_tile != 16:
+                self._check(self.lib.lmsf_gemv_scaled(
+                    _ptr(x.xw), x.xw.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(y), y.stride(0), M, I, K,
+                    kinds[kind], _ptr(x.sumsq), x.tiles, x.eps, self._stream()))
+                return y
             self._check(self.lib.lmsf_gemm_skinny_scaled(
                 _ptr(x.xw), x.xw.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(y), y.stride(0), M, I, K,
                 kinds[kind], _ptr(x.sumsq), x.tiles, x.eps, self.skinny_variant, self._stream()))
-            return y
-        if isinstance(x, NormedStream):
-            K = x.shape[1]
-            if not (weight.dtype == torch.bfloat16 and weight.shape[1] == K and weight.stride(1) == 1
-                    and weight.stride(0) % 8 == 0 and weight.data_ptr() % 16 == 0 and self._gemv_ok(M, K)):
-                return self.linear_gated(self.materialize(x), weight, bias, kind)
-            self._dev(x.stream, x.weight, weight, bias)
-            if bias is not None and (bias.shape != (2 * I,) or bias.dtype != weight.dtype or not bias.is_contiguous()):
-                raise ValueError("linear_gated: bias must be [%d] of the weight's dtype" % (2 * I))
-            y = torch.empty((M, I), dtype=torch.bfloat16, device=x.device)
-            self._check(self.lib.lmsf_gemv_normed(_ptr(x.stream), x.stream.stride(0), _ptr(x.weight), x.eps,
-                                                  x.weight_offset, _ptr(weight), weight.stride(0), _ptr(bias), _ptr(y),
-                                                  y.stride(0), M, I, K, kinds[kind], self._stream()))
             return y
         if (x.dim() == 2 and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and 0 < M <= self.skinny_max_rows
                 and x.shape[1] == weight.shape[1] and x.stride(1) == 1 and weight.stride(1) == 1

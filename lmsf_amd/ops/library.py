@@ -9,7 +9,7 @@ from typing import Optional
 
 from ..csrc import build as _build
 
-ABI_VERSION = 15
+ABI_VERSION = 17
 
 _lib: Optional[ctypes.CDLL] = None
 _lib_path: Optional[str] = None
@@ -51,11 +51,13 @@ _SIGNATURES = {
     "lmsf_gemv_qkv_rope_cache": (c_int, [_P, c_long, _P, c_long, _P, _P, c_long, c_int, c_int, _P, _P, c_int, _P, _P, _P,
                                          c_long, c_int, c_int, c_int, c_int, _P]),
     "lmsf_gemv_add": (c_int, [_P, c_long, _P, c_long, _P, _P, c_long, c_int, c_int, c_int, _P]),
-    "lmsf_gemv_normed": (c_int, [_P, c_long, _P, c_float, c_float, _P, c_long, _P, _P, c_long, c_int, c_int, c_int,
-                                 c_int, _P]),
-    "lmsf_gemv_normed_qkv_rope_cache": (c_int, [_P, c_long, _P, c_float, c_float, _P, c_long, _P, _P, c_long, c_int,
-                                                c_int, _P, _P, c_int, _P, _P, _P, c_long, c_int, c_int, c_int, c_int,
-                                                _P]),
+    "lmsf_gemv_partials": (c_int, [c_int]),
+    "lmsf_gemv_add_norm": (c_int, [_P, c_long, _P, c_long, _P, _P, c_long, _P, c_float, _P, c_long, _P, c_int, c_int,
+                                   c_int, _P]),
+    "lmsf_gemv_scaled": (c_int, [_P, c_long, _P, c_long, _P, _P, c_long, c_int, c_int, c_int, c_int, _P, c_int, c_float,
+                                 _P]),
+    "lmsf_gemv_scaled_qkv_rope_cache": (c_int, [_P, c_long, _P, c_long, _P, _P, c_long, c_int, c_int, _P, _P, c_int, _P,
+                                                _P, _P, c_long, c_int, c_int, c_int, c_int, _P, c_int, c_float, _P]),
     "lmsf_gemm_mid_splits": (c_int, [c_int, c_int, c_int, c_int]),
     "lmsf_gemm_mid_scratch_floats": (c_long, [c_int, c_int, c_int, c_int]),
     "lmsf_gemm_mid": (c_int, [_P, c_long, _P, c_long, _P, _P, c_int, c_long, c_int, c_int, c_int, c_int, c_int, _P, _P]),

@@ -140,7 +140,7 @@ class Part:
     accepts_pending = False
 
     # A norm whose ``forward_add`` takes ``defer_ok=True`` and may then return the norm not yet computed
-    # (ops.handles.NormedStream) sets ``may_defer``; a mixer or feed-forward whose ``forward`` takes such an
+    # (ops.handles.ScaledRows) sets ``may_defer``; a mixer or feed-forward whose ``forward`` takes such an
     # ``h`` (it hands it to ``rt.ops.qkv_rope_cache`` or ``rt.ops.linear_gated``, or calls ``rt.ops.materialize``
     # first) sets ``accepts_normed``. A block asks for a deferred norm only where both say so.
     may_defer = False
