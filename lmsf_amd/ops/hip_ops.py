@@ -121,42 +121,9 @@ class HipOps:
         if isinstance(branch, PendingProduct):
             return self._add_rms_norm_pending(branch, residual, weight, eps, out_dtype, rows, weight_offset)
         if isinstance(branch, DeferredLinear):
-            M, N = branch.shape
-            fits = (rows is None and residual is not None and residual.dtype == torch.float32
-                    and residual.is_contiguous() and tuple(residual.shape) == branch.shape)
-            norm_ok = (defer_ok and out_dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
-                       and weight.is_contiguous() and weight.shape == (N,))
-            if (fits and norm_ok and M <= min(self.fuse_stream_rows, self.gemv_max_rows)
-                    and self._gemv_ok(M, branch.x.shape[1]) and self._gemv_ok(M, N)):
-                # the product adds into the stream and leaves stream * w and its workgroups' sums of squares
-                self._dev(branch.x, branch.weight, branch.bias, residual, weight)
-                parts = self.lib.lmsf_gemv_partials(N)
-                xw = torch.empty((M, N), dtype=torch.bfloat16, device=residual.device)
-                sumsq = torch.empty(parts * M, dtype=torch.float32, device=residual.device)
-                self._check(self.lib.lmsf_gemv_add_norm(
-                    _ptr(branch.x), branch.x.stride(0), _ptr(branch.weight), branch.weight.stride(0), _ptr(branch.bias),
-                    _ptr(residual), residual.stride(0), _ptr(weight), float(weight_offset), _ptr(xw), xw.stride(0),
-                    _ptr(sumsq), M, N, branch.x.shape[1], self._stream()))
-                return ScaledRows(xw, sumsq, parts, M, residual, weight, float(eps), float(weight_offset), out_dtype)
-            if fits and M <= min(self.fuse_stream_rows, self.gemv_max_rows) and self._gemv_ok(M, branch.x.shape[1]):
-                self._dev(branch.x, branch.weight, branch.bias, residual)
-                self._check(self.lib.lmsf_gemv_add(_ptr(branch.x), branch.x.stride(0), _ptr(branch.weight),
-                                                   branch.weight.stride(0), _ptr(branch.bias), _ptr(residual),
-                                                   residual.stride(0), M, N, branch.x.shape[1], self._stream()))
-                branch = None
-            elif fits and norm_ok and M <= min(self.fuse_norm_rows, self.skinny_max_rows, 16):
-                # the product adds into the stream and leaves stream * w and the sums of squares for the next one
-                self._dev(branch.x, branch.weight, branch.bias, residual, weight)
-                tiles = -(-N // 16)
-                xw = torch.empty((M, N), dtype=torch.bfloat16, device=residual.device)
-                sumsq = torch.empty(tiles * 16, dtype=torch.float32, device=residual.device)
-                self._check(self.lib.lmsf_gemm_skinny_add_norm(
-                    _ptr(branch.x), branch.x.stride(0), _ptr(branch.weight), branch.weight.stride(0), _ptr(branch.bias),
-                    _ptr(residual), residual.stride(0), _ptr(weight), float(weight_offset), _ptr(xw), xw.stride(0),
-                    _ptr(sumsq), M, N, branch.x.shape[1], self.skinny_variant, self._stream()))
-                return ScaledRows(xw, sumsq, tiles, 16, residual, weight, float(eps), float(weight_offset), out_dtype)
-            else:
-                branch = self.materialize(branch)
+            handle, branch = self._run_deferred(branch, residual, weight, eps, out_dtype, rows, weight_offset, defer_ok)
+            if handle is not None:
+                return handle
         self._dev(branch, residual, weight, rows)
         ref = branch if branch is not None else residual
         if ref is None:
@@ -178,6 +145,47 @@ class HipOps:
             _code(weight.dtype), _ptr(out), _code(out_dtype), _ptr(rows), n_out, H, float(eps),
             float(weight_offset), self._stream()))
         return out
+
+    def _run_deferred(self, branch: DeferredLinear, residual: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
+                      out_dtype: torch.dtype, rows: Optional[torch.Tensor], weight_offset: float, defer_ok: bool):
+        """Runs the product that ``branch`` stands for, in the form that leaves the norm the least to do.
+        Returns (handle, branch): a ``ScaledRows`` if the product did the norm's preparation as well (then the
+        norm is done), else None and what is left to add: nothing if the product added into the stream itself,
+        the product's tensor otherwise."""
+        M, N = branch.shape
+        K = branch.x.shape[1]
+        fits = (rows is None and residual is not None and residual.dtype == torch.float32
+                and residual.is_contiguous() and tuple(residual.shape) == branch.shape)
+        prepares = (fits and defer_ok and out_dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
+                    and weight.is_contiguous() and weight.shape == (N,))
+        one_or_two = fits and M <= min(self.fuse_stream_rows, self.gemv_max_rows) and self._gemv_ok(M, K)
+        operands = (_ptr(branch.x), branch.x.stride(0), _ptr(branch.weight), branch.weight.stride(0), _ptr(branch.bias))
+        if prepares and one_or_two and self._gemv_ok(M, N):
+            # adds into the stream, leaves stream * w and its workgroups' sums of squares
+            self._dev(branch.x, branch.weight, branch.bias, residual, weight)
+            parts = self.lib.lmsf_gemv_partials(N)
+            xw = torch.empty((M, N), dtype=torch.bfloat16, device=residual.device)
+            sumsq = torch.empty(parts * M, dtype=torch.float32, device=residual.device)
+            self._check(self.lib.lmsf_gemv_add_norm(*operands, _ptr(residual), residual.stride(0), _ptr(weight),
+                                                    float(weight_offset), _ptr(xw), xw.stride(0), _ptr(sumsq), M, N, K,
+                                                    self._stream()))
+            return ScaledRows(xw, sumsq, parts, M, residual, weight, float(eps), float(weight_offset), out_dtype), None
+        if prepares and M <= min(self.fuse_norm_rows, self.skinny_max_rows, 16) and not one_or_two:
+            # the same from the few-rows kernel: sums of squares per 16 columns
+            self._dev(branch.x, branch.weight, branch.bias, residual, weight)
+            tiles = -(-N // 16)
+            xw = torch.empty((M, N), dtype=torch.bfloat16, device=residual.device)
+            sumsq = torch.empty(tiles * 16, dtype=torch.float32, device=residual.device)
+            self._check(self.lib.lmsf_gemm_skinny_add_norm(*operands, _ptr(residual), residual.stride(0), _ptr(weight),
+                                                           float(weight_offset), _ptr(xw), xw.stride(0), _ptr(sumsq), M,
+                                                           N, K, self.skinny_variant, self._stream()))
+            return ScaledRows(xw, sumsq, tiles, 16, residual, weight, float(eps), float(weight_offset), out_dtype), None
+        if one_or_two:
+            # adds into the stream; the norm kernel follows
+            self._dev(branch.x, branch.weight, branch.bias, residual)
+            self._check(self.lib.lmsf_gemv_add(*operands, _ptr(residual), residual.stride(0), M, N, K, self._stream()))
+            return None, None
+        return None, self.materialize(branch)
 
     def _add_rms_norm_pending(self, branch: PendingProduct, residual: Optional[torch.Tensor], weight: torch.Tensor,
                               eps: float, out_dtype: torch.dtype, rows: Optional[torch.Tensor],
