@@ -641,6 +641,16 @@ def _norm_done_by_the_products(ops, ref, M, H, K, nh, nkv, d, I, bias, gemv):
     assert torch.is_tensor(ops.add_rms_norm(p, r5, nw.float(), 1e-5, torch.bfloat16, weight_offset=0.25, defer_ok=True))
 
 
+def test_split_heuristic_counts_the_gated_forms_extra_kernel(ops):
+    """Splitting K fills the chip when there are few rows of W, at the price of partial sums and, for the gated
+    form, a kernel that adds them up: at a feed-forward's sizes (224 workgroups without a split) that price is
+    never worth it, at an o projection's (64 workgroups) it always is."""
+    for M in (17, 18, 24, 32, 64):
+        assert ops.lib.lmsf_gemm_mid_splits(M, 14336, 4096, 1) == 1
+        assert ops.lib.lmsf_gemm_mid_splits(M, 4096, 4096, 0) >= 4
+        assert ops.lib.lmsf_gemm_mid_splits(M, 4096, 14336, 0) >= 4
+
+
 def test_linear_mixed_storage(ops, ref):
     """A weight stored in 32 bits stays so and still multiplies bfloat16 activations."""
     g = torch.Generator().manual_seed(5)
