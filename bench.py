@@ -222,7 +222,8 @@ def main():
     full_layers = cfg["num_hidden_layers"]
     if args.layers:
         cfg["num_hidden_layers"] = args.layers
-    engine = make_engine(cfg, args, max_num_seqs=64, dtype=args.dtype)
+    point_batches = [] if args.skip_points else [int(x) for x in args.points.split(",") if x]
+    engine = make_engine(cfg, args, max_num_seqs=max([64, args.batch] + point_batches), dtype=args.dtype)
     wbytes = weight_bytes(engine)
     kv_per_token = 2 * cfg["num_key_value_heads"] * cfg["head_dim"] * cfg["num_hidden_layers"] * \
         (2 if args.dtype == "bfloat16" else 4)
@@ -235,7 +236,7 @@ def main():
 
     points = {}
     if not args.skip_points:
-        for b in [int(x) for x in args.points.split(",") if x]:
+        for b in point_batches:
             k = max(16, args.steps // 2)
             d, _ = decode_run(engine, b, args.prompt_len, k, args.warmup, seed=2 + b)
             points["decode_b%d" % b] = round(b * k / d, 1)

@@ -1,6 +1,6 @@
-// Linear layer for 17 to 64 rows (decoding at larger batches): y[M, N] = x[M, K] W[N, K]^T (+ bias),
-// bfloat16 inputs, float32 accumulation on the matrix cores, bfloat16 output; optionally the gated
-// activation of a feed-forward as epilogue.
+// Linear layer for 17 to 128 rows (decoding at larger batches): y[M, N] = x[M, K] W[N, K]^T (+ bias),
+// bfloat16 inputs, float32 accumulation on the matrix cores, bfloat16 output; up to 64 rows optionally with
+// the gated activation of a feed-forward as epilogue (beyond that its stages do not fit LDS).
 //
 // The product is still a stream of the weight matrix, but with this many rows the activations are no
 // longer negligible: a workgroup that owns 16 rows of W reads four times as many bytes of x as of W. Here
@@ -56,7 +56,7 @@ __device__ __forceinline__ void mid_store4(float* p, const float* o) {
 #define MID_STAGES 5
 #define MID_TILE 2048
 
-// MT: tiles of 16 rows of x (2 or 4). ACT: 0 none, 1 silu-gated, 2 gelu-gated (W = [gate rows; up rows], N
+// MT: tiles of 16 rows of x (2, 4, 6 or 8). ACT: 0 none, 1 silu-gated, 2 gelu-gated (W = [gate rows; up rows], N
 // outputs). PARTIAL: write float32 partial sums of this workgroup's part of K instead of the result.
 template <int MT, int ACT, bool PARTIAL, typename TOut>
 __global__ __launch_bounds__(256) void gemm_mid_kernel(const bf16_t* __restrict__ x, long ldx,
@@ -251,14 +251,14 @@ extern "C" long lmsf_gemm_mid_scratch_floats(int M, int N, int n_split, int act)
 }
 
 // x [M, K] bfloat16 (row stride ldx), W [N, K] (act 0) or [2 N, K] (act 1 silu, 2 gelu: gate rows first),
-// bias [N] or [2 N] or null, y [M, N] of out_dtype (float32 only without activation). Needs 1 <= M <= 64, K a multiple of 64, N a multiple of 4,
+// bias [N] or [2 N] or null, y [M, N] of out_dtype (float32 only without activation). Needs 1 <= M <= 128 (64 with an activation), K a multiple of 64, N a multiple of 4,
 // 16-byte aligned x and W, row strides of x and W that are multiples of 8 and of y of 4; anything else is
 // refused. n_split: parts of K that go to different workgroups (lmsf_gemm_mid_splits proposes a number);
 // scratch: lmsf_gemm_mid_scratch_floats floats (may be null when that is 0).
 static int mid_check(const void* x, long ldx, const void* W, long ldw, int M, int N, int K, int n_split,
-                     const float* scratch) {
+                     const float* scratch, int act = 0) {
   LMSF_CHECK(x && W, "gemm_mid: null pointer");
-  LMSF_CHECK(M >= 0 && M <= 64, "gemm_mid: M=%d outside [0, 64]", M);
+  LMSF_CHECK(M >= 0 && M <= (act ? 64 : 128), "gemm_mid: M=%d outside [0, %d]", M, act ? 64 : 128);
   LMSF_CHECK(N > 0 && N % 4 == 0 && K > 0 && K % 64 == 0, "gemm_mid: N=%d must be a multiple of 4 and K=%d of 64", N, K);
   LMSF_CHECK(ldx >= K && ldw >= K && ldx % 8 == 0 && ldw % 8 == 0,
              "gemm_mid: row strides of x and W must cover the rows and be multiples of 8");
@@ -279,11 +279,15 @@ static int mid_product(const bf16_t* xb, long ldx, const bf16_t* Wb, long ldw, c
            ? launch_mid<MT_, ACT_, true, T_>(grid, stream, xb, ldx, Wb, ldw, bb, (T_*)y, ldy, scratch, M, N, K, n_split) \
            : launch_mid<MT_, ACT_, false, T_>(grid, stream, xb, ldx, Wb, ldw, bb, (T_*)y, ldy, scratch, M, N, K, n_split)
   if (out_dtype == LMSF_F32) {
-    if (M <= 32) MID(2, 0, float); else MID(4, 0, float);
+    if (M <= 32) MID(2, 0, float); else if (M <= 64) MID(4, 0, float); else if (M <= 96) MID(6, 0, float); else MID(8, 0, float);
   } else if (M <= 32) {
     if (act == 0) MID(2, 0, bf16_t); else if (act == 1) MID(2, 1, bf16_t); else MID(2, 2, bf16_t);
-  } else {
+  } else if (M <= 64) {
     if (act == 0) MID(4, 0, bf16_t); else if (act == 1) MID(4, 1, bf16_t); else MID(4, 2, bf16_t);
+  } else if (M <= 96) {
+    MID(6, 0, bf16_t);
+  } else {
+    MID(8, 0, bf16_t);
   }
 #undef MID
   if (rc) return rc;
@@ -308,10 +312,10 @@ static int mid_reduce(const float* scratch, const bf16_t* bb, void* y, int out_d
 extern "C" int lmsf_gemm_mid(const void* x, long ldx, const void* W, long ldw, const void* bias, void* y,
                              int out_dtype, long ldy, int M, int N, int K, int act, int n_split, float* scratch,
                              hipStream_t stream) {
-  if (int rc = mid_check(x, ldx, W, ldw, M, N, K, M == 0 ? 1 : n_split, scratch)) return rc;
+  LMSF_CHECK(act >= 0 && act <= 2, "gemm_mid: unknown activation %d", act);
+  if (int rc = mid_check(x, ldx, W, ldw, M, N, K, M == 0 ? 1 : n_split, scratch, act)) return rc;
   LMSF_CHECK(y != nullptr && lmsf_aligned16(y) && ldy >= N && ldy % 4 == 0,
              "gemm_mid: y must be 16-byte aligned with a row stride that covers N and is a multiple of 4");
-  LMSF_CHECK(act >= 0 && act <= 2, "gemm_mid: unknown activation %d", act);
   LMSF_CHECK(out_dtype == LMSF_BF16 || (out_dtype == LMSF_F32 && act == 0),
              "gemm_mid: output is bfloat16, or float32 without activation");
   if (M == 0) return 0;

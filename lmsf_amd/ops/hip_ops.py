@@ -54,6 +54,8 @@ class HipOps:
         self.fuse_stream_rows = 1            # with up to this many rows the residual addition and the norm run inside the products (0: never)
         self.gemv_max_rows = 2               # products of up to this many rows stream W without the matrix cores (0: never)
         self.skinny_variant = 0        # tiling of the few-rows kernel (0: default; others for tuning)
+        self.mid_wide_max_cols = 8192  # beyond 64 rows only products of up to this many columns: the library is good at the wide ones (measured)
+        self.mid_max_rows = 128        # rows up to which the 17-and-more-rows kernel beats the library (64 with the gated activation)
         self.skinny_max_rows = 16      # rows up to which the few-rows kernel beats the library (measured)
 
     # ------------------------------------------------------------------ helpers
@@ -526,7 +528,8 @@ class HipOps:
             raise ValueError("linear: bias must be [%d] of the weight's dtype" % N)
         out_dtype = out_dtype or x.dtype
         both_bf16 = x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
-        if both_bf16 and self.skinny_max_rows < M <= 64 and self._mid_ok(x, weight):
+        if (both_bf16 and self.skinny_max_rows < M <= self.mid_max_rows and self._mid_ok(x, weight)
+                and (M <= 64 or N <= self.mid_wide_max_cols or out_dtype == torch.float32)):
             return self._linear_mid(x, weight, bias, 0, out_dtype, pending_ok and out_dtype == torch.bfloat16)
         if pending_ok and both_bf16 and out_dtype == torch.bfloat16 and self._skinny_ok(x, weight) and M > 0:
             if (M <= min(self.fuse_stream_rows, self.gemv_max_rows) and self._gemv_ok(M, K)) \
@@ -540,9 +543,17 @@ class HipOps:
             self._check(self.lib.lmsf_gemv(_ptr(x), x.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(y),
                                            _code(out_dtype), y.stride(0), M, N, K, 0, self._stream()))
             return y
+        if both_bf16 and out_dtype == torch.float32 and M > self.mid_max_rows and self._mid_ok(x, weight):
+            # float32 output (logits) for many rows, which the library does not offer: as many rows at a time
+            # as the kernel above takes
+            y = torch.empty((M, N), dtype=out_dtype, device=x.device)
+            for r0 in range(0, M, self.mid_max_rows):
+                rows = min(self.mid_max_rows, M - r0)
+                y[r0:r0 + rows] = self.linear(x[r0:r0 + rows], weight, bias, out_dtype=out_dtype)
+            return y
         if both_bf16 and self._skinny_ok(x, weight):
-            # few rows: the weight-streaming kernel. It also serves float32 output (logits), which the
-            # library does not offer, for any number of rows, 64 at a time.
+            # few rows: the weight-streaming kernel. It also serves float32 output where the kernels above
+            # do not take the operands, for any number of rows, 64 at a time.
             limit = self.skinny_max_rows if out_dtype == torch.bfloat16 else 64
             if M <= limit or out_dtype == torch.float32:
                 y = torch.empty((M, N), dtype=out_dtype, device=x.device)

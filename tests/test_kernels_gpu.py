@@ -359,7 +359,9 @@ def test_linear_float32_is_exact_float32(ops, M, N, K, bias):
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 1000, 128), (7, 331, 80), (64, 640, 352), (65, 512, 176), (300, 1024, 512),
-                                   (17, 328, 128), (33, 4096, 4096), (64, 6144, 4096), (48, 1000, 14336), (64, 4096, 1024)])
+                                   (17, 328, 128), (33, 4096, 4096), (64, 6144, 4096), (48, 1000, 14336), (64, 4096, 1024),
+                                   (65, 4096, 4096), (96, 1000, 14336), (97, 328, 128), (128, 6144, 4096), (127, 4096, 1024),
+                                   (200, 1000, 1024)])
 @pytest.mark.parametrize("bias", [False, True])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
 def test_linear_bfloat16(ops, ref, M, N, K, bias, out_dtype):
@@ -446,7 +448,8 @@ def test_qkv_rope_cache_fused_equals_the_three_steps(ops, ref, M, H, nh, nkv, d,
     assert (a.float() - c.float()).abs().max().item() <= 2e-2 * scale and (k4.float() - k5.float()).abs().max().item() <= 2e-2 * scale
 
 
-@pytest.mark.parametrize("M,N,K", [(17, 256, 1024), (40, 4096, 4096), (64, 80, 1280), (33, 1000, 2048)])
+@pytest.mark.parametrize("M,N,K", [(17, 256, 1024), (40, 4096, 4096), (64, 80, 1280), (33, 1000, 2048), (65, 256, 1024),
+                                   (100, 4096, 4096), (128, 80, 1280)])
 @pytest.mark.parametrize("bias", [False, True])
 def test_unfinished_product_is_finished_by_the_norm(ops, ref, M, N, K, bias):
     """A product of 17 to 64 rows whose K is split may stay as partial sums; the norm that takes it as its
@@ -479,7 +482,8 @@ def test_unfinished_product_is_finished_by_the_norm(ops, ref, M, N, K, bias):
 
 
 @pytest.mark.parametrize("M,H,nh,nkv,d,ps,rot,neox", [(17, 1024, 8, 2, 64, 16, 64, True), (64, 4096, 32, 8, 128, 16, 128, True),
-                                                      (40, 1024, 6, 3, 48, 8, 24, False), (33, 1280, 5, 5, 80, 4, 80, False)])
+                                                      (40, 1024, 6, 3, 48, 8, 24, False), (33, 1280, 5, 5, 80, 4, 80, False),
+                                                      (100, 4096, 32, 8, 128, 16, 128, True), (128, 1024, 6, 3, 48, 8, 24, False)])
 @pytest.mark.parametrize("bias", [False, True])
 def test_qkv_rope_cache_from_partial_sums(ops, ref, M, H, nh, nkv, d, ps, rot, neox, bias):
     """With 17 to 64 rows the QKV product splits K, and the rotation kernel adds up the partial sums before it
