@@ -9,6 +9,15 @@
 // keyed by (seed of the request, number of the draw, vocabulary index): the token does not depend
 // on what else is in the batch.
 //
+// A bisection step over the whole vocabulary costs a pass over the row; 32 of them per cut are most of a
+// millisecond at 128,256 entries. With a top-k of up to 1,024 the row is passed over twice instead: the k-th
+// largest of the 1,024 threads' own maxima is a value that at least k entries reach, so everything the cuts
+// can keep is among the entries that reach it; those (a few times k) are gathered in LDS, and the cuts and
+// the draw work on them alone. Top-p without a top-k does the same from a value below which top-p removes
+// everything whatever the rest of the row is; it gains where the distribution is peaked. Masses are added up there as integers (exp scaled by 2^32), so that the
+// order in which the entries were gathered does not show. Rows without any cut draw over the whole
+// vocabulary, split over several workgroups a row like the greedy search.
+//
 // Cut rules (ties at a cut value are kept together):
 //   top-k : keep x >= k-th largest value                         (sampler.rs:170-178)
 //   top-p : keep x whose mass of strictly larger values is < p   (sampler.rs:180-197: ascending
@@ -79,6 +88,47 @@ __device__ __forceinline__ int block_argmax(float v, int idx, float* redv, int* 
   return bi;
 }
 
+__device__ __forceinline__ float key_value(uint32_t key) {
+  return __uint_as_float((key & 0x80000000u) ? (key & 0x7fffffffu) : ~key);
+}
+
+#define SAMP_CAND 8192   // entries the small-top-k path gathers in LDS (keys, then indices)
+
+// The largest c with at least ``need`` of keys[0 .. n) >= c (the need-th largest key); every thread gets it.
+__device__ __forceinline__ uint32_t lds_kth_largest(const uint32_t* keys, int n, unsigned long long need,
+                                                    unsigned long long* redu) {
+  uint32_t cur = 0u;
+  for (int bit = 31; bit >= 0; --bit) {
+    const uint32_t cand = cur | (1u << bit);
+    unsigned long long cnt = 0;
+    for (int j = threadIdx.x; j < n; j += SAMP_THREADS) cnt += keys[j] >= cand ? 1u : 0u;
+    cnt = block_sum_u64(cnt, redu);
+    if (cnt >= need) cur = cand;
+  }
+  return cur;
+}
+
+// exp(x - mx) for x <= mx as an integer: 2^32 at the maximum
+__device__ __forceinline__ unsigned long long mass_fixed(float x, float mx) {
+  return (unsigned long long)(expf(x - mx) * 4294967296.0f);
+}
+
+// f(i, row[i]) for this thread's entries i = tid, tid + SAMP_THREADS, ..., in ascending order, eight loads in
+// flight at a time: one workgroup passes over a row of half a megabyte, and with a load per wave and trip the
+// pass is as slow as the loads' latency.
+template <typename F>
+__device__ __forceinline__ void for_each_entry(const float* __restrict__ row, int V, F f) {
+  int i = threadIdx.x;
+  for (; i + 7 * SAMP_THREADS < V; i += 8 * SAMP_THREADS) {
+    float x[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) x[u] = row[i + u * SAMP_THREADS];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) f(i + u * SAMP_THREADS, x[u]);
+  }
+  for (; i < V; i += SAMP_THREADS) f(i, row[i]);
+}
+
 // One workgroup per row. temperature < 1e-5 means greedy (core/src/common/sampling_params.rs:156-163).
 __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(
     const float* __restrict__ logits, long ld, int V, const float* __restrict__ temperature,
@@ -95,75 +145,146 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(
   if (greedy) {
     float bv = -INFINITY;
     int bi = 0x7fffffff;
-    for (int i = tid; i < V; i += SAMP_THREADS) {
-      const float x = row[i];
+    for_each_entry(row, V, [&](int i, float x) {
       if (x > bv) { bv = x; bi = i; }  // ascending i per thread: the first maximum wins
-    }
+    });
     const int best = block_argmax(bv, bi, redf, redi);
     if (tid == 0) out[r] = best < V ? best : 0;
     return;
   }
 
+  extern __shared__ __align__(16) uint32_t cand_keys[];   // [SAMP_CAND] keys, [SAMP_CAND] indices, [SAMP_THREADS] maxima
+  uint32_t* cand_idx = cand_keys + SAMP_CAND;
+  uint32_t* thread_max = cand_idx + SAMP_CAND;
+  __shared__ unsigned int n_cand;
   const float invT = 1.0f / T;
   float mx = -INFINITY;
-  for (int i = tid; i < V; i += SAMP_THREADS) mx = fmaxf(mx, row[i] * invT);
+  for_each_entry(row, V, [&](int, float x) { mx = fmaxf(mx, x * invT); });
+  thread_max[tid] = order_key(mx);   // (-inf for a thread without entries: below every entry)
   mx = block_max(mx, redf);
+  const unsigned long long seed = seeds ? seeds[r] : 0ull;
+  const unsigned int draw = draws ? draws[r] : 0u;
+  const float p = top_p ? top_p[r] : 1.0f;
+  const float mp = min_p ? min_p[r] : 0.f;
+  const uint32_t kmax = order_key(mx);
 
   uint32_t cut = 0u;  // keep order_key(x) >= cut
   const int k = top_k ? top_k[r] : -1;
+  const bool small_k = k > 0 && k < V && k <= SAMP_THREADS;
+  const bool p_alone = p < 1.0f && !(k > 0 && k < V);
+  if (small_k || p_alone) {
+    // A value below which nothing can be kept. Top-k: at least k entries reach the k-th largest of the threads'
+    // maxima. Top-p alone: entries whose exp(x - max) is below (1 - p) / V add up to less than 1 - p, which
+    // is at most (1 - p) of the whole mass (the maximum alone contributes 1): top-p removes them all. With a
+    // peaked distribution, as a model's, few entries are above either.
+    const uint32_t floor_key = small_k ? lds_kth_largest(thread_max, SAMP_THREADS, (unsigned long long)k, redu)
+                                       : order_key(mx + logf((1.0f - p) / (float)V));
+    if (tid == 0) n_cand = 0u;
+    __syncthreads();
+    unsigned long long z_all = 0;   // top-p alone: the mass of every entry
+    for_each_entry(row, V, [&](int i, float xr) {
+      const float x = xr * invT;
+      const uint32_t key = order_key(x);
+      if (p_alone) z_all += mass_fixed(x, mx);
+      if (key >= floor_key) {
+        const unsigned int at = atomicAdd(&n_cand, 1u);
+        if (at < SAMP_CAND) {
+          cand_keys[at] = key;
+          cand_idx[at] = (uint32_t)i;
+        }
+      }
+    });
+    __syncthreads();
+    const int n = (int)n_cand;
+    if (n <= SAMP_CAND) {      // (more: a flat distribution, or thousands of equal values; the passes below take those)
+      cut = small_k ? lds_kth_largest(cand_keys, n, (unsigned long long)k, redu) : floor_key;
+      if (p < 1.0f) {
+        unsigned long long z = 0;
+        if (p_alone) {
+          z = z_all;
+        } else {
+          for (int j = tid; j < n; j += SAMP_THREADS)
+            if (cand_keys[j] >= cut) z += mass_fixed(key_value(cand_keys[j]), mx);
+        }
+        z = block_sum_u64(z, redu);
+        const unsigned long long target = (unsigned long long)((double)p * (double)z);
+        uint32_t cur = 0u;
+        for (int bit = 31; bit >= 0; --bit) {
+          const uint32_t c = cur | (1u << bit);
+          unsigned long long mass = 0;
+          for (int j = tid; j < n; j += SAMP_THREADS)
+            if (cand_keys[j] >= c && cand_keys[j] >= cut) mass += mass_fixed(key_value(cand_keys[j]), mx);
+          mass = block_sum_u64(mass, redu);
+          if (mass >= target) cur = c;
+        }
+        if (cur > cut) cut = cur;
+      }
+      if (mp > 0.f) {
+        const uint32_t c = order_key(mx + logf(mp));
+        if (c > cut) cut = c;
+      }
+      if (cut > kmax) cut = kmax;
+      float bv = -INFINITY;
+      int bi = 0x7fffffff;
+      for (int j = tid; j < n; j += SAMP_THREADS) {
+        if (cand_keys[j] < cut) continue;
+        const int i = (int)cand_idx[j];
+        const float y = key_value(cand_keys[j]) + gumbel_noise(seed, draw, (uint32_t)i);
+        if (y > bv || (y == bv && i < bi)) { bv = y; bi = i; }
+      }
+      const int best = block_argmax(bv, bi, redf, redi);
+      if (tid == 0) out[r] = best < V ? best : 0;
+      return;
+    }
+  }
   if (k > 0 && k < V) {
     uint32_t cur = 0u;
     for (int bit = 31; bit >= 0; --bit) {
       const uint32_t cand = cur | (1u << bit);
       unsigned long long cnt = 0;
-      for (int i = tid; i < V; i += SAMP_THREADS) cnt += order_key(row[i] * invT) >= cand ? 1u : 0u;
+      for_each_entry(row, V, [&](int, float x) { cnt += order_key(x * invT) >= cand ? 1u : 0u; });
       cnt = block_sum_u64(cnt, redu);
       if (cnt >= (unsigned long long)k) cur = cand;
     }
     cut = cur;
   }
-  const float p = top_p ? top_p[r] : 1.0f;
   if (p < 1.0f) {
     float z = 0.f;
-    for (int i = tid; i < V; i += SAMP_THREADS) {
-      const float x = row[i] * invT;
+    for_each_entry(row, V, [&](int, float xr) {
+      const float x = xr * invT;
       if (order_key(x) >= cut) z += expf(x - mx);
-    }
+    });
     z = block_sum(z, redf);
     const float target = p * z;
     uint32_t cur = 0u;
     for (int bit = 31; bit >= 0; --bit) {
       const uint32_t cand = cur | (1u << bit);
       float mass = 0.f;
-      for (int i = tid; i < V; i += SAMP_THREADS) {
-        const float x = row[i] * invT;
+      for_each_entry(row, V, [&](int, float xr) {
+        const float x = xr * invT;
         const uint32_t key = order_key(x);
         if (key >= cand && key >= cut) mass += expf(x - mx);
-      }
+      });
       mass = block_sum(mass, redf);
       if (mass >= target) cur = cand;
     }
     if (cur > cut) cut = cur;
   }
-  const float mp = min_p ? min_p[r] : 0.f;
   if (mp > 0.f) {
     const uint32_t c = order_key(mx + logf(mp));
     if (c > cut) cut = c;
   }
   // the maximum is always kept, whatever rounding did to the cuts
-  const uint32_t kmax = order_key(mx);
   if (cut > kmax) cut = kmax;
 
-  const unsigned long long seed = seeds ? seeds[r] : 0ull;
-  const unsigned int draw = draws ? draws[r] : 0u;
   float bv = -INFINITY;
   int bi = 0x7fffffff;
-  for (int i = tid; i < V; i += SAMP_THREADS) {
-    const float x = row[i] * invT;
-    if (order_key(x) < cut) continue;
+  for_each_entry(row, V, [&](int i, float xr) {
+    const float x = xr * invT;
+    if (order_key(x) < cut) return;
     const float y = x + gumbel_noise(seed, draw, (uint32_t)i);
     if (y > bv) { bv = y; bi = i; }
-  }
+  });
   const int best = block_argmax(bv, bi, redf, redi);
   if (tid == 0) out[r] = best < V ? best : 0;
 }
@@ -192,6 +313,46 @@ __global__ __launch_bounds__(256) void argmax_partial_kernel(const float* __rest
     pval[r * ARGMAX_SPLIT + part] = best < V ? row[best] : -INFINITY;
   }
 }
+// The same with the draw's noise: rows without any cut (temperature only, or greedy where it is below 1e-5).
+__global__ __launch_bounds__(256) void noisy_argmax_partial_kernel(
+    const float* __restrict__ logits, long ld, int V, const float* __restrict__ temperature,
+    const unsigned long long* __restrict__ seeds, const unsigned int* __restrict__ draws, float* __restrict__ pval,
+    int* __restrict__ pidx) {
+  __shared__ float redf[16];
+  __shared__ int redi[16];
+  const int r = blockIdx.x, part = blockIdx.y, tid = threadIdx.x;
+  const int per = (V + ARGMAX_SPLIT - 1) / ARGMAX_SPLIT;
+  const int lo = part * per, hi = min(V, lo + per);
+  const float* row = logits + (long)r * ld;
+  const float T = temperature[r];
+  const bool greedy = T < 1e-5f;
+  const float invT = greedy ? 1.0f : 1.0f / T;
+  const unsigned long long seed = seeds ? seeds[r] : 0ull;
+  const unsigned int draw = draws ? draws[r] : 0u;
+  float bv = -INFINITY;
+  int bi = 0x7fffffff;
+  for (int i = lo + tid; i < hi; i += 256) {
+    const float x = row[i] * invT;
+    const float y = greedy ? x : x + gumbel_noise(seed, draw, (uint32_t)i);
+    if (y > bv) { bv = y; bi = i; }
+  }
+  // (the value is carried along: the last kernel compares the shares' best values, noise included)
+#pragma unroll
+  for (int o = LMSF_WAVE / 2; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(bv, o, LMSF_WAVE);
+    const int oi = __shfl_xor(bi, o, LMSF_WAVE);
+    if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+  }
+  const int w = tid / LMSF_WAVE, l = tid % LMSF_WAVE;
+  if (l == 0) { redf[w] = bv; redi[w] = bi; }
+  __syncthreads();
+  if (tid == 0) {
+    for (int i = 1; i < 256 / LMSF_WAVE; ++i)
+      if (redf[i] > bv || (redf[i] == bv && redi[i] < bi)) { bv = redf[i]; bi = redi[i]; }
+    pidx[r * ARGMAX_SPLIT + part] = bi;
+    pval[r * ARGMAX_SPLIT + part] = bv;
+  }
+}
 __global__ __launch_bounds__(64) void argmax_final_kernel(const float* __restrict__ pval, const int* __restrict__ pidx,
                                                           int V, int* __restrict__ out) {
   const int r = blockIdx.x, l = threadIdx.x;
@@ -211,8 +372,9 @@ extern "C" long lmsf_sample_scratch_elems(int R, int V) { return (V >= 16384 && 
 
 // logits [R, V] float32 with row stride ld. temperature/top_k/top_p/min_p/seeds/draws are per-row
 // device arrays; any of them may be null (greedy, no cut, seed 0, draw 0).
-// scratch (optional): lmsf_sample_scratch_elems(R, V) floats followed by as many ints; with it, and with
-// no temperature (all rows greedy), a large vocabulary is searched by several workgroups per row.
+// scratch (optional): lmsf_sample_scratch_elems(R, V) floats followed by as many ints; with it, a large
+// vocabulary is searched by several workgroups per row where no row has a cut: with no temperature (all rows
+// greedy), or with top_k, top_p and min_p all null.
 extern "C" int lmsf_sample(const float* logits, long ld, int R, int V, const float* temperature, const int* top_k,
                            const float* top_p, const float* min_p, const unsigned long long* seeds,
                            const unsigned int* draws, int* out, void* scratch, hipStream_t stream) {
@@ -228,7 +390,28 @@ extern "C" int lmsf_sample(const float* logits, long ld, int R, int V, const flo
     LMSF_LAUNCH_CHECK("sample (greedy)");
     return 0;
   }
-  hipLaunchKernelGGL(sample_kernel, dim3(R), dim3(SAMP_THREADS), 0, stream, logits, ld, V, temperature, top_k, top_p,
+  if (top_k == nullptr && top_p == nullptr && min_p == nullptr && scratch != nullptr && elems > 0) {
+    // no row has a cut: the draw over the whole vocabulary, several workgroups a row
+    float* pval = (float*)scratch;
+    int* pidx = (int*)(pval + elems);
+    hipLaunchKernelGGL(noisy_argmax_partial_kernel, dim3(R, ARGMAX_SPLIT), dim3(256), 0, stream, logits, ld, V,
+                       temperature, seeds, draws, pval, pidx);
+    hipLaunchKernelGGL(argmax_final_kernel, dim3(R), dim3(64), 0, stream, pval, pidx, V, out);
+    LMSF_LAUNCH_CHECK("sample (no cuts)");
+    return 0;
+  }
+  const size_t smem = (size_t)(2 * SAMP_CAND + SAMP_THREADS) * sizeof(uint32_t);
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(sample_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) {
+      lmsf_set_error("sample: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
+      return 2;
+    }
+    configured = true;
+  }
+  hipLaunchKernelGGL(sample_kernel, dim3(R), dim3(SAMP_THREADS), smem, stream, logits, ld, V, temperature, top_k, top_p,
                      min_p, seeds, draws, out);
   LMSF_LAUNCH_CHECK("sample");
   return 0;

@@ -687,7 +687,7 @@ class HipOps:
                 raise ValueError("sample: %s must be a contiguous %s tensor of %d elements" % (name, dt, R))
         out = torch.empty((R,), dtype=torch.int32, device=logits.device)
         scratch = None
-        if temperature is None:
+        if temperature is None or (top_k is None and top_p is None and min_p is None):
             elems = self.lib.lmsf_sample_scratch_elems(R, V)
             if elems:
                 scratch = torch.empty(2 * elems, dtype=torch.float32, device=logits.device)

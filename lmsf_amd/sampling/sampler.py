@@ -8,6 +8,7 @@ pipeline: one for the penalties (only when a request has any), one for everythin
 """
 from typing import List, Optional, Sequence
 
+import numpy as np
 import torch
 
 from .params import SamplingParams
@@ -32,6 +33,10 @@ class Sampler:
         self.ops = ops
         self.device = device
 
+    def _upload(self, words: "np.ndarray") -> torch.Tensor:
+        """One copy to the device for everything a call needs: int32 words, float32 values as their bits."""
+        return torch.from_numpy(words).to(self.device, non_blocking=False)
+
     def sample(self, logits: torch.Tensor, rows: Sequence[SamplingRow]) -> List[int]:
         """One token id per row of float32 ``logits`` [R, V]."""
         R = len(rows)
@@ -39,7 +44,6 @@ class Sampler:
             raise ValueError("%d rows of logits for %d requests" % (logits.shape[0], R))
         if R == 0:
             return []
-        dev = self.device
         if any(r.params.has_penalties for r in rows):
             logits = logits.clone()
             tokens: List[int] = []
@@ -53,26 +57,41 @@ class Sampler:
                 else:
                     plens.append(0)
                 offsets.append(len(tokens))
-            self.ops.apply_penalties(
-                logits,
-                torch.tensor(tokens or [0], dtype=torch.int32, device=dev),
-                torch.tensor(offsets, dtype=torch.int32, device=dev),
-                torch.tensor(plens, dtype=torch.int32, device=dev),
-                torch.tensor([r.params.presence_penalty for r in rows], dtype=torch.float32, device=dev),
-                torch.tensor([r.params.frequency_penalty for r in rows], dtype=torch.float32, device=dev),
-                torch.tensor([r.params.repetition_penalty for r in rows], dtype=torch.float32, device=dev))
+            T = max(len(tokens), 1)
+            # tokens | offsets | prompt lengths | presence | frequency | repetition, in one upload
+            words = np.zeros(T + (R + 1) + 4 * R, dtype=np.int32)
+            words[:len(tokens)] = tokens
+            words[T:T + R + 1] = offsets
+            at = T + R + 1
+            words[at:at + R] = plens
+            fl = words[at + R:].view(np.float32)
+            fl[0:R] = [r.params.presence_penalty for r in rows]
+            fl[R:2 * R] = [r.params.frequency_penalty for r in rows]
+            fl[2 * R:3 * R] = [r.params.repetition_penalty for r in rows]
+            d = self._upload(words)
+            f = d[at + R:].view(torch.float32)
+            self.ops.apply_penalties(logits, d[:T], d[T:T + R + 1], d[at:at + R], f[0:R], f[R:2 * R], f[2 * R:3 * R])
         if all(r.params.greedy for r in rows):
             out = self.ops.sample(logits)
         else:
-            out = self.ops.sample(
-                logits,
-                torch.tensor([0.0 if r.params.greedy else r.params.temperature for r in rows], dtype=torch.float32,
-                             device=dev),
-                torch.tensor([r.params.top_k for r in rows], dtype=torch.int32, device=dev),
-                torch.tensor([r.params.top_p for r in rows], dtype=torch.float32, device=dev),
-                torch.tensor([r.params.min_p for r in rows], dtype=torch.float32, device=dev),
-                torch.tensor([_to_i64(r.seed) for r in rows], dtype=torch.int64, device=dev),
-                torch.tensor([r.draw & 0x7FFFFFFF for r in rows], dtype=torch.int32, device=dev))
+            # seeds (two words each) | temperature | top_p | min_p | top_k | draws, in one upload
+            words = np.zeros(7 * R, dtype=np.int32)
+            words[:2 * R].view(np.int64)[:] = [_to_i64(r.seed) for r in rows]
+            fl = words[2 * R:5 * R].view(np.float32)
+            fl[0:R] = [0.0 if r.params.greedy else r.params.temperature for r in rows]
+            fl[R:2 * R] = [r.params.top_p for r in rows]
+            fl[2 * R:3 * R] = [r.params.min_p for r in rows]
+            words[5 * R:6 * R] = [r.params.top_k for r in rows]
+            words[6 * R:7 * R] = [r.draw & 0x7FFFFFFF for r in rows]
+            d = self._upload(words)
+            seeds = d[:2 * R].view(torch.int64)
+            fd = d[2 * R:5 * R].view(torch.float32)
+            temperature, draws = fd[0:R], d[6 * R:7 * R]
+            if all(r.params.top_k <= 0 and r.params.top_p >= 1.0 and r.params.min_p <= 0.0 for r in rows):
+                # no row cuts anything: the kernel can split a row over several workgroups
+                out = self.ops.sample(logits, temperature, None, None, None, seeds, draws)
+            else:
+                out = self.ops.sample(logits, temperature, d[5 * R:6 * R], fd[R:2 * R], fd[2 * R:3 * R], seeds, draws)
         return [int(t) for t in out.tolist()]
 
 

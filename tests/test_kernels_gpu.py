@@ -685,6 +685,27 @@ def test_sample_greedy_and_seeded(ops, ref, V):
         assert a.tolist() == b.tolist(), (draw, a.tolist(), b.tolist())
 
 
+@pytest.mark.parametrize("V", [1000, 128256])
+def test_sample_top_p_alone_on_peaked_and_flat_rows(ops, ref, V):
+    """Top-p without a top-k: peaked rows (few entries can be kept: they are gathered once) and flat rows (most
+    of the row can be kept: the passes over the whole row) give the plain sampler's tokens."""
+    g = torch.Generator().manual_seed(V + 1)
+    scales = [0.5, 2.0, 6.0, 9.0, 14.0, 9.0, 9.0, 0.0]
+    R = len(scales)
+    logits = torch.randn(R, V, generator=g) * torch.tensor(scales)[:, None]
+    logits[6, 3] = logits[6].max() + 30.0                  # one entry holds all the mass
+    lg = dev(logits)
+    temp = dev(torch.tensor([1.0, 0.8, 1.0, 1.2, 1.0, 0.6, 1.0, 1.0]))
+    top_p = dev(torch.tensor([0.9, 0.95, 0.9, 0.5, 0.999, 0.05, 0.9, 0.7]))
+    seeds = dev(torch.arange(100, 100 + R, dtype=torch.int64))
+    for draw in range(4):
+        draws = dev(torch.full((R,), draw, dtype=torch.int32))
+        a = ops.sample(lg, temp, None, top_p, None, seeds, draws)
+        b = ref.sample(lg, temp, None, top_p, None, seeds, draws)
+        assert a.tolist() == b.tolist(), (draw, a.tolist(), b.tolist())
+        assert a[6].item() == 3
+
+
 @pytest.mark.parametrize("V", [1000, 16384, 128256])
 def test_greedy_takes_the_first_of_equal_maxima(ops, V):
     g = torch.Generator().manual_seed(V)
