@@ -250,6 +250,18 @@ class CacheManager:
             _raise(self._lib, rc, "request %r" % (rid,))
         return int(info[1])
 
+    def tokens_held(self, rids: Sequence[Hashable]) -> np.ndarray:
+        """``num_tokens`` of every request of the list at once (0 for one that holds no cache)."""
+        S = len(rids)
+        get = self._handle_of.get
+        handles = np.fromiter((get(r, -1) for r in rids), dtype=np.int64, count=S)
+        known = (handles >= 0).astype(np.uint8)
+        held = np.zeros(max(S, 1), dtype=np.int64)
+        rc = self._lib.lmsf_cm_tokens_held(self._h, S, _ptr(handles), _ptr(known), _ptr(held))
+        if rc:
+            _raise(self._lib, rc)
+        return held[:S]
+
     def pages_needed(self, rid: Optional[Hashable], n_new: int, held_tokens: Optional[int] = None) -> List[int]:
         """New pages per group that appending ``n_new`` tokens would take. ``rid`` None (or unknown)
         counts for a request that holds nothing yet."""

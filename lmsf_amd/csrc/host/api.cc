@@ -27,7 +27,7 @@ static thread_local std::string g_error;
 
 extern "C" {
 
-int lmsf_host_abi_version() { return 1; }
+int lmsf_host_abi_version() { return 2; }
 const char* lmsf_host_last_error() { return g_error.c_str(); }
 
 // ---------------------------------------------------------------- a page pool alone
@@ -77,6 +77,18 @@ int lmsf_cm_request_info(void* cm, int64_t rid, int64_t* info) {
   info[0] = rc.state_slot;
   info[1] = rc.num_tokens;
   info[2] = rc.pending;
+  LMSF_API_END
+}
+// held[i] = tokens of rids[i] that are in the pages; 0 where known[i] is 0 or the request holds no cache.
+int lmsf_cm_tokens_held(void* cm, int S, const int64_t* rids, const unsigned char* known, int64_t* held) {
+  LMSF_API_BEGIN
+  CacheManager* m = static_cast<CacheManager*>(cm);
+  for (int i = 0; i < S; ++i) {
+    held[i] = 0;
+    if (known[i] && m->has_request(rids[i])) {
+      held[i] = m->request(rids[i]).num_tokens;
+    }
+  }
   LMSF_API_END
 }
 // Blocks of rid in group: their number into *len, first_live into *first_live, and the pages into out if cap allows.

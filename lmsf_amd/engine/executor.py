@@ -77,22 +77,28 @@ class ModelExecutor:
 
     def _validate(self, entries: Sequence[StepEntry]) -> None:
         seen = set()
+        V = self.vocab_size
         for e in entries:
             if e.request_id in seen:
                 raise StepError("request %r appears twice in one step" % (e.request_id,))
             seen.add(e.request_id)
             n = len(e.tokens)
-            for t in e.tokens:
-                if not (0 <= int(t) < self.vocab_size):
-                    raise StepError("request %r: token id %r outside the vocabulary of %d"
-                                    % (e.request_id, t, self.vocab_size))
+            if n == 1:
+                bad = not (0 <= int(e.tokens[0]) < V)
+            else:
+                ids = np.asarray(e.tokens, dtype=np.int64)
+                bad = bool(((ids < 0) | (ids >= V)).any())
+            if bad:
+                t = next(t for t in e.tokens if not (0 <= int(t) < V))
+                raise StepError("request %r: token id %r outside the vocabulary of %d" % (e.request_id, t, V))
             for w in e.want:
                 if not (0 <= int(w) < n):
                     raise StepError("request %r: wanted place %r outside its %d tokens" % (e.request_id, w, n))
-            held = self.manager.num_tokens(e.request_id) if self.manager.has_request(e.request_id) else 0
-            if held + n > self.max_model_len:
+        held = self.manager.tokens_held([e.request_id for e in entries])
+        for e, h in zip(entries, held.tolist()):
+            if h + len(e.tokens) > self.max_model_len:
                 raise StepError("request %r would hold %d tokens, more than max_model_len %d"
-                                % (e.request_id, held + n, self.max_model_len))
+                                % (e.request_id, h + len(e.tokens), self.max_model_len))
 
     def _build_context(self, entries: Sequence[StepEntry], handles: np.ndarray, starts_a: np.ndarray,
                        static: Optional["_StaticBatch"] = None) -> StepContext:
@@ -116,7 +122,12 @@ class ModelExecutor:
         R = int(logit_rows.shape[0])
         G = len(mgr.groups)
         widths = static.widths if static is not None else mgr.step_widths(handles)
-        offsets, raw_offsets, total = mgr.step_layout(N, S, R, widths)
+        if static is not None:
+            if static.layout is None:
+                static.layout = mgr.step_layout(N, S, R, widths)
+            offsets, raw_offsets, total = static.layout
+        else:
+            offsets, raw_offsets, total = mgr.step_layout(N, S, R, widths)
         if self._pinned is None or self._pinned.numel() < total:
             self._pinned = torch.empty(max(total, 4096), dtype=torch.int32,
                                        pin_memory=self.rt.device.type == "cuda")
@@ -138,8 +149,6 @@ class ModelExecutor:
             mgr.fill_step(handles, starts_a, lens, widths, raw_offsets, host_np)
         except CacheError as e:
             raise CacheError("%s (requests %s)" % (e, ", ".join(repr(x.request_id) for x in entries)))
-        seg_starts = section("seg_starts").tolist()
-        state_slots = section("state_slots").tolist()
         # the copy is synchronous: the staging buffer is free again when the next step fills it
         if static is not None:
             static.device_buffer.copy_(host, non_blocking=False)
@@ -156,6 +165,8 @@ class ModelExecutor:
             o, n = offsets[name]
             return dev[o:o + n]
 
+        seg_starts = section("seg_starts").tolist()
+        state_slots = section("state_slots").tolist()
         groups = [GroupView(slots=view("slots%d" % gi),
                             block_tables=view("tables%d" % gi).view(S, widths[gi]),
                             page_size=mgr.groups[gi].page_size) for gi in range(G)]
@@ -228,5 +239,6 @@ class _StaticBatch:
         self.max_context = int(max_context)
         self.device_buffer = device_buffer
         self.context: Optional[StepContext] = None
+        self.layout = None                 # the metadata buffer's sections: the same at every step of this kind
         self.graph = None
         self.logits: Optional[torch.Tensor] = None

@@ -157,28 +157,30 @@ class LLMEngine:
                 self.scheduler.finish(seq)
                 self._requests.pop(seq.request_id, None)
             outputs.append(RequestOutput.from_sequence(seq, tok, piece))
+        n_tokens = plan.num_tokens
         self.stats["generated_tokens"] += len(sampled)
-        self.stats["tokens"] += plan.num_tokens
-        self._record_step(plan, len(sampled), outputs, t_start)
+        self.stats["tokens"] += n_tokens
+        self._record_step(plan, n_tokens, len(sampled), outputs, t_start)
         return outputs
 
-    def _record_step(self, plan: StepPlan, n_sampled: int, outputs: List[RequestOutput], t_start: float) -> None:
+    def _record_step(self, plan: StepPlan, n_tokens: int, n_sampled: int, outputs: List[RequestOutput],
+                     t_start: float) -> None:
         """What the step did, for ``last_step`` and the metrics."""
         now = time.monotonic()
         decode = sum(1 for s in plan.scheduled if s.n_tokens == 1 and s.samples and s.start > 0)
         m = self.metrics
-        self.last_step = {"tokens": plan.num_tokens, "decode_tokens": decode, "prefill_tokens": plan.num_tokens - decode,
+        self.last_step = {"tokens": n_tokens, "decode_tokens": decode, "prefill_tokens": n_tokens - decode,
                           "sequences": len(plan.scheduled), "sampled": n_sampled, "preempted": len(plan.preempted),
                           "free_pages": self.core.storage.manager.num_free_pages(0) if self.core.storage.manager.groups else 0,
                           "ms": (now - t_start) * 1e3}
         m.counter("llm.steps")
-        m.counter("llm.tokens", plan.num_tokens)
+        m.counter("llm.tokens", n_tokens)
         m.counter("llm.generated_tokens", n_sampled)
         m.counter("llm.preemptions", len(plan.preempted))
         m.gauge("llm.alive_prompt", len(self._requests))
         m.gauge("llm.free_pages", self.last_step["free_pages"])
         m.histogram("llm.step_ms", self.last_step["ms"])
-        m.histogram("llm.step_tokens", plan.num_tokens)
+        m.histogram("llm.step_tokens", n_tokens)
         for out in outputs:
             if out.finished and out.metrics is not None and out.metrics.finished_time is not None:
                 t = out.metrics

@@ -23,14 +23,16 @@ class SequenceState(enum.Enum):
 
     @property
     def finished(self) -> bool:
-        return self in (SequenceState.FINISHED_STOPPED, SequenceState.FINISHED_LENGTH_CAPPED,
-                        SequenceState.FINISHED_ABORTED, SequenceState.FINISHED_IGNORED)
+        return self.value in _FINISH_REASONS
 
     @property
     def finish_reason(self) -> Optional[str]:
-        # core/src/common/sequence.rs:56-64
-        return {SequenceState.FINISHED_STOPPED: "stop", SequenceState.FINISHED_LENGTH_CAPPED: "length",
-                SequenceState.FINISHED_ABORTED: "abort", SequenceState.FINISHED_IGNORED: "length"}.get(self)
+        return _FINISH_REASONS.get(self.value)
+
+
+# core/src/common/sequence.rs:56-64
+_FINISH_REASONS = {"finished_stopped": "stop", "finished_length_capped": "length", "finished_aborted": "abort",
+                   "finished_ignored": "length"}
 
 
 @dataclass

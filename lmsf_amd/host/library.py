@@ -7,7 +7,7 @@ from typing import Optional
 
 from ..csrc import build as _build
 
-HOST_ABI_VERSION = 1
+HOST_ABI_VERSION = 2
 
 OK, CACHE_ERROR, OUT_OF_PAGES, VALUE_ERROR = 0, 1, 2, 3
 
@@ -34,6 +34,7 @@ _SIGNATURES = {
     "lmsf_cm_num_free_state_slots": (c_int, [_P]),
     "lmsf_cm_num_free_pages": (c_int, [_P, c_int, POINTER(c_int)]),
     "lmsf_cm_request_info": (c_int, [_P, c_int64, _P]),
+    "lmsf_cm_tokens_held": (c_int, [_P, c_int, _P, _P, _P]),
     "lmsf_cm_block_table": (c_int, [_P, c_int64, c_int, _P, c_int, POINTER(c_int), POINTER(c_int)]),
     "lmsf_cm_live_requests": (c_int, [_P, _P, c_int, POINTER(c_int)]),
     "lmsf_cm_pages_needed": (c_int, [_P, c_int, c_int64, c_int64, _P]),

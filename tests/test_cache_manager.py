@@ -38,6 +38,11 @@ def test_append_commit_and_tables():
     assert m.append("a", 1) == 8 and m.block_table("a", 0) == [0, 1, 2]    # position 8 opens a page
     m.commit("a")
     assert m.pages_needed("a", 3) == [0] and m.pages_needed("a", 4) == [1] and m.pages_needed(None, 9) == [3]
+    m.add_request("b")
+    m.append("b", 3)                                   # not committed: not yet in the pages
+    assert m.tokens_held(["a", "nobody", "b", "a"]).tolist() == [9, 0, 0, 9] and m.tokens_held([]).tolist() == []
+    m.commit("b")
+    assert m.tokens_held(["b"]).tolist() == [3]
     m.check_invariants()
 
 
