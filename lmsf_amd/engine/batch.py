@@ -42,6 +42,9 @@ class StepContext:
     logit_rows: torch.Tensor       # int32 [R]: flat indices whose logits are wanted
     n_logit_rows: int
     groups: List[GroupView]
+    # a step of single tokens: its tokens, the longest context first (int32 [N]); a kernel whose work grows with
+    # the context starts its workgroups in this order
+    longest_first: Optional[torch.Tensor] = None
     # host-side facts, for choosing kernels and for parts that loop over segments
     host_seg_starts: List[int] = field(default_factory=list)
     host_seg_lens: List[int] = field(default_factory=list)

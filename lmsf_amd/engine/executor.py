@@ -128,12 +128,18 @@ class ModelExecutor:
             offsets, raw_offsets, total = static.layout
         else:
             offsets, raw_offsets, total = mgr.step_layout(N, S, R, widths)
+        # a step of single tokens also carries its tokens ordered by context, the longest first, behind the
+        # sections the host library lays out
+        single = N == S
+        order_at, total = total, total + (_pad4(N) if single else 0)
         if self._pinned is None or self._pinned.numel() < total:
             self._pinned = torch.empty(max(total, 4096), dtype=torch.int32,
                                        pin_memory=self.rt.device.type == "cuda")
             self._pinned_np = self._pinned.numpy()
         host = self._pinned[:total]
         host_np = self._pinned_np
+        if single:
+            host_np[order_at:order_at + N] = np.argsort(-starts_a, kind="stable")
 
         def section(name: str) -> np.ndarray:
             o, n = offsets[name]
@@ -174,6 +180,7 @@ class ModelExecutor:
             n_tokens=N, n_segments=S, token_ids=view("token_ids"), positions=view("positions"),
             seg_of_token=view("seg_of"), seg_starts=view("seg_starts"), seg_first_pos=view("seg_first"),
             state_slots=view("state_slots"), logit_rows=view("logit_rows"), n_logit_rows=R, groups=groups,
+            longest_first=dev[order_at:order_at + N] if single else None,
             host_seg_starts=seg_starts, host_seg_lens=lens, host_seg_first_pos=list(starts),
             host_state_slots=list(state_slots), request_ids=[e.request_id for e in entries],
             max_seg_len=max(lens),
@@ -206,7 +213,7 @@ class ModelExecutor:
         if sb is None:
             widths = [-(-bucket // g.page_size) for g in self.manager.groups]
             _, _, total = self.manager.step_layout(B, B, B, widths)
-            sb = _StaticBatch(widths, torch.zeros(total, dtype=torch.int32, device=self.rt.device), bucket)
+            sb = _StaticBatch(widths, torch.zeros(total + _pad4(B), dtype=torch.int32, device=self.rt.device), bucket)
             self._static[(B, bucket)] = sb
         ctx = self._build_context(entries, handles, starts, static=sb)
         if sb.graph is None:
@@ -228,6 +235,10 @@ class ModelExecutor:
         if not wanted:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.rt.device)
         return logits[torch.tensor(wanted, device=self.rt.device)]
+
+
+def _pad4(n: int) -> int:
+    return (n + 3) // 4 * 4
 
 
 class _StaticBatch:

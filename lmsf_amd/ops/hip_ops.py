@@ -49,6 +49,7 @@ class HipOps:
         self._bad_flag = None
         self.use_library_gemm = True   # bfloat16 matrix products of many rows go to the BLAS library
         self.prefill_attention_variant = 0   # 0: keys and values staged in LDS; 1: fetched by every wave for itself
+        self.decode_attention_order = 0      # 0: chosen from the number of workgroups; 1: the tokens of a head start together; 2: the heads of a token
         self.decode_attention_splits = 0     # 0: chosen from the batch and the context; n: at most n splits of the keys
         self.fuse_norm_rows = 16             # with up to this many rows (beyond fuse_stream_rows) the products around a norm do its work (0: never)
         self.fuse_stream_rows = 1            # with up to this many rows the residual addition and the norm run inside the products (0: never)
@@ -437,7 +438,7 @@ class HipOps:
             self._check(self.lib.lmsf_paged_attention_decode_mfma(
                 _ptr(q), q.stride(0), _ptr(out), out.stride(0), *common, _ptr(plan.single_tokens), plan.n_single,
                 _ptr(seg), _ptr(pos), nh, nkv, d, ps, float(scale), int(window or 0), chunk, n_splits,
-                _ptr(scratch), self._stream()))
+                _ptr(scratch), self.decode_attention_order, self._stream()))
         return out
 
     def _attention_plan(self, batch, seg: torch.Tensor, pos: torch.Tensor, nh: int, nkv: int) -> "_AttentionPlan":
@@ -453,7 +454,7 @@ class HipOps:
             lens, starts, max_context = batch.host_seg_lens, batch.host_seg_starts, batch.max_context
             first_pos = batch.host_seg_first_pos
             if batch.replayed or batch.all_single:
-                plan = _AttentionPlan(None, 0, None, batch.n_tokens, max_context)
+                plan = _AttentionPlan(None, 0, getattr(batch, "longest_first", None), batch.n_tokens, max_context)
                 aux[key] = plan
                 return plan
         else:
@@ -471,13 +472,15 @@ class HipOps:
         by_keys, single = [], []
         for st, n, p0 in zip(starts, lens, first_pos):
             if n == 1:
-                single.append(st)
+                single.append((p0, st))
             else:
                 for t in range(0, n, tq):
                     by_keys.append((p0 + t + min(tq, n - t), st + t, min(tq, n - t)))
         # the tiles with the most keys first: the prefill kernel starts its workgroups in this order
         by_keys.sort(key=lambda e: -e[0])
         tiles = [x for e in by_keys for x in e[1:]]
+        # likewise the single tokens with the longest contexts first
+        single = [st for _, st in sorted(single, key=lambda e: -e[0])]
         dev = seg.device
         if len(single) == len(lens):
             plan = _AttentionPlan(None, 0, None, len(single), max_context)

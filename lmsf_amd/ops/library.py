@@ -9,7 +9,7 @@ from typing import Optional
 
 from ..csrc import build as _build
 
-ABI_VERSION = 17
+ABI_VERSION = 18
 
 _lib: Optional[ctypes.CDLL] = None
 _lib_path: Optional[str] = None
@@ -35,7 +35,8 @@ _SIGNATURES = {
                                                   c_int, c_int, c_int, c_int, c_float, c_int, c_int, _P]),
     "lmsf_attention_decode_scratch_floats": (c_long, [c_int, c_int, c_int, c_int]),
     "lmsf_paged_attention_decode_mfma": (c_int, [_P, c_long, _P, c_long, _P, _P, c_long, _P, c_int, _P, c_int, _P, _P,
-                                                 c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, _P, _P]),
+                                                 c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, _P, c_int,
+                                                 _P]),
     "lmsf_gated_act": (c_int, [_P, _P, c_int, c_int, c_int, c_long, c_int, _P]),
     "lmsf_gemm_plain": (c_int, [_P, c_int, c_long, _P, c_int, c_long, _P, _P, c_int, c_long, c_int, c_int, c_int, _P]),
     "lmsf_gemm_skinny": (c_int, [_P, c_long, _P, c_long, _P, _P, c_int, c_long, c_int, c_int, c_int, c_int, c_int, _P]),

@@ -229,6 +229,41 @@ def test_matrix_core_attention_other_ways_of_cutting_the_work(ops, ref, shape, v
     assert torch.allclose(a.float(), b.float(), **tol(torch.bfloat16)), (a.float() - b.float()).abs().max()
 
 
+@pytest.mark.parametrize("order", [1, 2])
+def test_decode_attention_in_a_given_order_of_tokens(ops, ref, order):
+    """A step of single tokens whose contexts differ, with the tokens listed longest context first and either
+    arrangement of the workgroups: the same result as in the order they come in."""
+    from types import SimpleNamespace
+    g = torch.Generator().manual_seed(21)
+    nh, nkv, d, ps, B = 6, 3, 48, 8, 19
+    lens = [int(x) for x in torch.randint(1, 300, (B,), generator=g)]
+    per = [-(-n // ps) for n in lens]
+    pages = sum(per) + 3
+    kp = dev(torch.randn(pages, nkv, ps, d, generator=g).to(torch.bfloat16))
+    vp = dev(torch.randn(pages, nkv, d, ps, generator=g).to(torch.bfloat16))
+    perm = torch.randperm(pages, generator=g).to(torch.int32)
+    bt = torch.zeros(B, max(per) + 2, dtype=torch.int32)
+    at = 0
+    for i, n in enumerate(per):
+        bt[i, :n] = perm[at:at + n]
+        at += n
+    q = dev(torch.randn(B, (nh + 2 * nkv) * d, generator=g).to(torch.bfloat16))
+    seg = dev(torch.arange(B, dtype=torch.int32))
+    pos = dev(torch.tensor([n - 1 for n in lens], dtype=torch.int32))
+    want = ref.paged_attention(q, kp, vp, dev(bt), seg, pos, nh, nkv, d, d ** -0.5)
+    batch = SimpleNamespace(aux={}, host_seg_lens=[1] * B, host_seg_starts=list(range(B + 1)),
+                            host_seg_first_pos=[n - 1 for n in lens], max_context=512, replayed=False, all_single=True,
+                            n_tokens=B, longest_first=torch.argsort(pos, descending=True, stable=True).to(torch.int32))
+    ops.decode_attention_order = order
+    try:
+        got = ops.paged_attention(q, kp, vp, dev(bt), seg, pos, nh, nkv, d, d ** -0.5, batch=batch, kernel="mfma")
+    finally:
+        ops.decode_attention_order = 0
+    assert torch.allclose(got.float(), want.float(), **tol(torch.bfloat16)), (got.float() - want.float()).abs().max()
+    plain = ops.paged_attention(q, kp, vp, dev(bt), seg, pos, nh, nkv, d, d ** -0.5, kernel="mfma")
+    assert torch.equal(got, plain)
+
+
 @pytest.mark.parametrize("nh,nkv,d,ps", [(4, 2, 16, 8), (5, 5, 48, 16), (6, 3, 80, 4), (8, 2, 128, 16), (2, 1, 256, 32), (3, 1, 112, 16)])
 @pytest.mark.parametrize("window", [0, 700])
 def test_decode_attention_reduction_over_many_splits(ops, ref, nh, nkv, d, ps, window):
