@@ -651,30 +651,21 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
   for (int v = 0; v < DV; ++v) acc[v] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, lsum = 0.f;
 
-  // Where this lane's keys and values of a step lie (four looks into the block table). The next step's are
-  // asked for right after this step's keys and values: a step then waits for memory once, not twice.
-  long kr[2], vo[2];
-  auto locate = [&](int kb, long* kr_, long* vo_) {
-    kr_[0] = k_row_offset(G, kb + c);
-    kr_[1] = k_row_offset(G, kb + 16 + c);
-    vo_[0] = v_col_offset(G, kb + 4 * g);
-    vo_[1] = v_col_offset(G, kb + 16 + 4 * g);
-  };
-  locate(c0 + w * 32, kr, vo);
   for (int kbase = c0 + w * 32; kbase < c1; kbase += 128) {
     Frag8 kf[2][DS];
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
+      const long kr = k_row_offset(G, kbase + b * 16 + c);
 #pragma unroll
       for (int s = 0; s < DS; ++s) {
         const int d0 = s * 32 + g * 8;
         if (d0 < d)
-          kf[b][s].q = *reinterpret_cast<const uint4*>(k_pages + kr[b] + d0);
+          kf[b][s].q = *reinterpret_cast<const uint4*>(k_pages + kr + d0);
         else
           kf[b][s].q = make_uint4(0, 0, 0, 0);
       }
     }
-    const long vo0 = vo[0], vo1 = vo[1];
+    const long vo0 = v_col_offset(G, kbase + 4 * g), vo1 = v_col_offset(G, kbase + 16 + 4 * g);
     Frag8 vf[DV];
 #pragma unroll
     for (int v = 0; v < DV; ++v) {
@@ -684,7 +675,6 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
         vf[v].h[1] = *reinterpret_cast<const uint2*>(v_pages + vo1 + dvo);
       }
     }
-    if (kbase + 128 < c1) locate(kbase + 128, kr, vo);
     float sv[8];
     float mx = -INFINITY;
 #pragma unroll
