@@ -233,3 +233,39 @@ def test_graph_replay_equals_eager(models, dtype):
             assert core.executor._static and all(sb.graph is not None for sb in core.executor._static.values())
     for rid in reqs:
         assert torch.equal(outs[0][rid], outs[1][rid]), rid
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_steps_of_many_requests_of_different_lengths(models, dtype):
+    """Twenty requests of 3 to 250 tokens: each prompt whole but for its last six tokens, then six steps that
+    decode all twenty at once, captured and replayed. From sixteen requests on the attention over the cache
+    takes the requests with the longest contexts first, in an order that changes from step to step; the logits
+    are the plain implementation's whatever the order."""
+    folder, cfg, w = models[("B", dtype)]
+    from lmsf_amd.engine import load_engine_core
+    V = cfg["vocab_size"]
+    lens = [3 + (37 * i * i + 11 * i) % 248 for i in range(20)]
+    assert len(set(lens)) > 15 and max(lens) > 200 and min(lens) < 12
+    reqs = {"m%d" % i: random_tokens(max(n, 8), V, 400 + i) for i, n in enumerate(lens)}
+    refs = {rid: plain_llama_forward(cfg, w, toks) for rid, toks in reqs.items()}
+    steps, n_step = [], 0
+    for rid, toks in reqs.items():
+        n = len(toks) - 6
+        steps.append({"step": n_step, "entries": [{"id": rid, "tokens": toks[:n], "want": list(range(n))}], "end": []})
+        n_step += 1
+    for k in range(6, 0, -1):
+        # the lengths' order changes under way: every second request is left out of the third step
+        ids = [rid for i, rid in enumerate(reqs) if not (k == 4 and i % 2)]
+        steps.append({"step": n_step, "entries": [{"id": rid, "tokens": [reqs[rid][len(reqs[rid]) - k - (1 if k <= 4 and int(rid[1:]) % 2 else 0)]],
+                                                   "want": [0]} for rid in ids], "end": []})
+        n_step += 1
+    # the requests left out once are one token behind: one more step for them
+    late = [rid for i, rid in enumerate(reqs) if i % 2]
+    steps.append({"step": n_step, "entries": [{"id": rid, "tokens": [reqs[rid][-1]], "want": [0]} for rid in late],
+                  "end": list(reqs)})
+    core = load_engine_core(folder, dtype=dtype, block_size=16, num_pages=sum(-(-len(t) // 16) for t in reqs.values()) + 2,
+                            max_num_seqs=32)
+    got = replay_in_process(core.executor, steps)
+    assert any(b >= 16 for (b, _bucket) in core.executor._static), "no decode step of sixteen or more was captured"
+    check(got, refs, dtype, "twenty requests")
+    core.storage.manager.check_invariants()
