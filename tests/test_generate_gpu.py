@@ -129,3 +129,52 @@ def test_command_line_with_text(tmp_path):
     assert proc.returncode == 0, proc.stderr[-3000:]
     assert proc.stdout.splitlines()[0].split() == tok.decode(want[:first]).split()
     assert ("to gen %d tokens" % (first + 1)) in proc.stdout
+
+
+@pytest.mark.parametrize("seed", [10011, 10013, 10022, 10036, 10040, 10042])
+def test_loads_drawn_at_random_generate_the_plain_tokens(tmp_path, seed):
+    """A load drawn at random: which model, how many requests of what lengths, how few pages, the prompt
+    portions, the token budget, the live requests allowed, requests that arrive while others run. Greedy in
+    float32: every request's tokens are the plain implementation's, however often it was preempted and
+    recomputed, and every page comes back. (The seeds are ones whose draw preempts 5 to 26 times.)"""
+    import random
+
+    from lmsf_amd.engine import EngineArgs, LLMEngine
+    from lmsf_amd.sampling import SamplingParams
+    rng = random.Random(seed)
+    which = rng.choice(["A", "B", "C"])
+    folder, cfg = make_model_folder(tmp_path, which, dtype="float32")
+    cfg_dict, w = read_model_folder(folder)
+    bs, top = TINY[which][2], cfg.max_position_embeddings
+    reqs = []
+    for i in range(rng.randint(3, 12)):
+        n, mt = rng.choice([1, 2, 5, 9, 17, 30, 47, 64, 90]), rng.choice([1, 2, 5, 12, 25])
+        reqs.append((random_tokens(min(n, top - mt - 1), cfg.vocab_size, (seed - 10000) * 100 + i), mt))
+    need_one = max(-(-(len(p) + mt) // bs) for p, mt in reqs)
+    pages = rng.choice([need_one + 1, need_one + 3, 2 * need_one, 64])
+    chunk = rng.choice([None, 8, 16, 32])
+    budget = rng.choice([32, 64, 128, 256])
+    engine = LLMEngine(EngineArgs(model=folder, dtype="float32", block_size=bs, num_gpu_blocks_override=pages,
+                                  max_num_seqs=rng.choice([2, 4, 8, 16]), prefill_chunk_size=chunk,
+                                  max_num_batched_tokens=budget, max_model_len=top))
+    pending = list(enumerate(reqs))
+    rng.shuffle(pending)
+    first = rng.randint(1, len(pending))
+    add = lambda i, p, mt: engine.add_request(i, p, SamplingParams(temperature=0.0, max_tokens=mt, ignore_eos=True))
+    for i, (p, mt) in pending[:first]:
+        add(i, p, mt)
+    later, done, steps = pending[first:], {}, 0
+    while engine.has_unfinished_requests() or later:
+        if later and (steps % 3 == 0 or not engine.has_unfinished_requests()):
+            i, (p, mt) = later.pop(0)
+            add(i, p, mt)
+        for out in engine.step():
+            if out.finished:
+                done[out.request_id] = out
+        steps += 1
+        assert steps < 5000, "the engine makes no progress"
+    engine.core.storage.manager.check_invariants()
+    assert engine.core.storage.manager.num_free_pages(0) == pages
+    assert engine.stats["preemptions"] >= 5
+    for i, (p, mt) in enumerate(reqs):
+        assert done[i].outputs[0].token_ids == plain_greedy_generate(cfg_dict, w, p, mt), (i, len(p), mt)
