@@ -29,8 +29,10 @@
 
 #define SAMP_THREADS 1024
 
+// (-0 and +0 compare equal as numbers and get one key)
 __device__ __forceinline__ uint32_t order_key(float f) {
-  const uint32_t b = __float_as_uint(f);
+  uint32_t b = __float_as_uint(f);
+  if (b == 0x80000000u) b = 0u;
   return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
 }
 
@@ -51,7 +53,9 @@ __device__ __forceinline__ uint32_t philox_first(uint32_t c0, uint32_t c1, uint3
 
 __device__ __forceinline__ float gumbel_noise(uint64_t seed, uint32_t draw, uint32_t index) {
   const uint32_t r = philox_first(index, draw, 0u, 0u, (uint32_t)seed, (uint32_t)(seed >> 32));
-  const float u = ((float)(r >> 8) + 0.5f) * (1.0f / 16777216.0f);  // in (0, 1)
+  // 23 bits: k + 0.5 is exact in float32 for k < 2^23, so u lies strictly inside (0, 1) and the noise is finite
+  // (with 24 bits the largest k + 0.5 rounds up to 2^24, u to 1 and the noise to +inf: that entry would win)
+  const float u = ((float)(r >> 9) + 0.5f) * (1.0f / 8388608.0f);
   return -logf(-logf(u));
 }
 

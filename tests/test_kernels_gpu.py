@@ -741,6 +741,48 @@ def test_sample_top_p_alone_on_peaked_and_flat_rows(ops, ref, V):
         assert a[6].item() == 3
 
 
+def test_sample_noise_is_finite(ops):
+    """The draw adds -log(-log(u)) to every entry; a u that rounds to 1 makes that +inf and its entry the
+    winner whatever its probability. One entry holds all the mass but 1e-8 here: over 2,000 draws of 128,256
+    entries each (where a u of 24 bits plus a half rounds to 1 fifteen times) it is drawn every time."""
+    V, R = 128256, 500
+    logits = torch.full((R, V), -30.0)
+    logits[:, 77] = 0.0
+    lg = dev(logits)
+    temp = dev(torch.ones(R))
+    seeds = dev(torch.arange(1000, 1000 + R, dtype=torch.int64))
+    for draw in range(4):
+        draws = dev(torch.full((R,), draw, dtype=torch.int32))
+        for cuts in (None, dev(torch.full((R,), 0.999))):          # the draw over the whole row, and the kernel with cuts
+            out = ops.sample(lg, temp, None, cuts, None, seeds, draws)
+            assert (out == 77).all(), (draw, cuts is not None, out[out != 77].tolist())
+
+
+@pytest.mark.parametrize("V", [50, 5000, 128256])
+def test_sample_takes_zeros_of_either_sign_as_equal(ops, ref, V):
+    """A row whose largest values are zeros of both signs (they compare equal): no cut separates them."""
+    g = torch.Generator().manual_seed(V)
+    R = 6
+    logits = torch.randn(R, V, generator=g) * 0.0                # +0 and -0 at random
+    logits[3:] -= torch.rand(3, V, generator=g).round() * 5.0     # about half of the entries far below the zeros
+    assert (logits == 0).any() and torch.signbit(logits[0]).any() and not torch.signbit(logits[0]).all()
+    lg = dev(logits)
+    temp = dev(torch.tensor([0.7, 1.0, 0.3, 0.7, 1.0, 1.5]))
+    top_k = dev(torch.tensor([1, 2, -1, 5, 1000, -1], dtype=torch.int32))
+    top_p = dev(torch.tensor([1.0, 0.9, 0.1, 0.5, 0.01, 0.9]))
+    min_p = dev(torch.tensor([0.0, 0.01, 0.0, 0.3, 0.0, 0.0]))
+    seeds = dev(torch.arange(40, 40 + R, dtype=torch.int64))
+    seen = set()
+    for draw in range(6):
+        draws = dev(torch.full((R,), draw, dtype=torch.int32))
+        a = ops.sample(lg, temp, top_k, top_p, min_p, seeds, draws)
+        b = ref.sample(lg, temp, top_k, top_p, min_p, seeds, draws)
+        assert a.tolist() == b.tolist(), (draw, a.tolist(), b.tolist())
+        assert all(logits[r, t] == 0 for r, t in enumerate(a.tolist()))
+        seen.add(bool(torch.signbit(logits[0, a[0]])))
+    assert seen == {True, False} or V == 50    # with top_k = 1 both kinds of zero are drawn
+
+
 @pytest.mark.parametrize("V", [1000, 16384, 128256])
 def test_greedy_takes_the_first_of_equal_maxima(ops, V):
     g = torch.Generator().manual_seed(V)

@@ -38,16 +38,18 @@ def _philox_first(c0, c1, k0, k1):
 
 
 def gumbel_noise(seed, draw, V):
-    """float32 [V]: -log(-log(u_i)), u_i = ((r_i >> 8) + 0.5) / 2^24."""
+    """float32 [V]: -log(-log(u_i)), u_i = ((r_i >> 9) + 0.5) / 2^23, strictly inside (0, 1)."""
     seed = int(seed) & 0xFFFFFFFFFFFFFFFF
     r = _philox_first(np.arange(V, dtype=np.uint64), int(draw) & 0xFFFFFFFF, seed & 0xFFFFFFFF, seed >> 32)
-    u = ((r >> np.uint64(8)).astype(np.float32) + np.float32(0.5)) * np.float32(1.0 / 16777216.0)
+    u = ((r >> np.uint64(9)).astype(np.float32) + np.float32(0.5)) * np.float32(1.0 / 8388608.0)
+    assert u.min() > 0.0 and u.max() < 1.0
     return torch.from_numpy(-np.log(-np.log(u))).to(torch.float32)
 
 
 def _order_key(x):
     """Order-preserving uint32 image of float32 values (as int64 tensor)."""
     b = x.contiguous().view(torch.int32).to(torch.int64) & 0xFFFFFFFF
+    b = torch.where(b == 0x80000000, torch.zeros_like(b), b)      # -0 and +0 are one value
     neg = (b & 0x80000000) != 0
     return torch.where(neg, (~b) & 0xFFFFFFFF, b | 0x80000000)
 
