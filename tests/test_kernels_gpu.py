@@ -741,6 +741,43 @@ def test_sample_top_p_alone_on_peaked_and_flat_rows(ops, ref, V):
         assert a[6].item() == 3
 
 
+@pytest.mark.parametrize("extreme", [False, True])
+def test_sample_rows_and_settings_drawn_at_random(ops, ref, extreme):
+    """Rows and settings drawn at random (vocabularies of 50 to 128,256, flat to peaked rows, many equal values,
+    one entry far above the rest; with ``extreme`` also masked entries, huge values and temperatures of 2e-5
+    to 50) give the plain sampler's tokens. A sweep like this is what found a noise value of +inf and zeros
+    of two signs with two keys."""
+    import random
+    for it in range(40):
+        rng = random.Random(it + (1000 if extreme else 0))
+        V = rng.choice([50, 777, 1000, 5000, 32000, 128256])
+        R = rng.choice([1, 3, 8])
+        g = torch.Generator().manual_seed(it)
+        scales = torch.tensor([rng.choice([0.0, 0.1, 1.0, 3.0, 8.0, 15.0]) for _ in range(R)])
+        logits = torch.randn(R, V, generator=g) * scales[:, None]
+        if rng.random() < 0.3:
+            logits = (logits * 4).round() / 4
+        if rng.random() < 0.3:
+            logits[0, rng.randrange(V)] += 40.0
+        if extreme:
+            if rng.random() < 0.5:
+                logits[torch.rand(R, V, generator=g) < 0.3] = float("-inf")
+                logits[:, rng.randrange(V)] = 1.0
+            if rng.random() < 0.3:
+                logits = logits * 1e4
+        temps = [0.0, 0.3, 0.7, 1.0, 1.5] + ([1e-4, 2e-5, 50.0] if extreme else [])
+        args = [dev(torch.tensor([rng.choice(temps) for _ in range(R)])),
+                dev(torch.tensor([rng.choice([-1, 1, 2, 5, 50, 1000, 1024, 1025, 5000]) for _ in range(R)], dtype=torch.int32)),
+                dev(torch.tensor([rng.choice([1.0, 0.99, 0.9, 0.5, 0.1, 0.01]) for _ in range(R)])),
+                dev(torch.tensor([rng.choice([0.0, 0.0, 0.01, 0.3]) for _ in range(R)])),
+                dev(torch.tensor([rng.randrange(2 ** 48) for _ in range(R)], dtype=torch.int64))]
+        lg = dev(logits)
+        for draw in range(2):
+            draws = dev(torch.full((R,), draw, dtype=torch.int32))
+            a, b = ops.sample(lg, *args, draws).tolist(), ref.sample(lg, *args, draws).tolist()
+            assert a == b, (it, draw, V, a, b, [t.tolist() for t in args[:4]])
+
+
 def test_sample_noise_is_finite(ops):
     """The draw adds -log(-log(u)) to every entry; a u that rounds to 1 makes that +inf and its entry the
     winner whatever its probability. One entry holds all the mass but 1e-8 here: over 2,000 draws of 128,256
