@@ -1,6 +1,6 @@
 // Linear layer for 17 to 128 rows (decoding at larger batches): y[M, N] = x[M, K] W[N, K]^T (+ bias),
-// bfloat16 inputs, float32 accumulation on the matrix cores, bfloat16 output; up to 64 rows optionally with
-// the gated activation of a feed-forward as epilogue (beyond that its stages do not fit LDS).
+// bfloat16 inputs, float32 accumulation on the matrix cores, bfloat16 or float32 output; up to 64 rows
+// optionally with the gated activation of a feed-forward as epilogue (beyond that its stages do not fit LDS).
 //
 // The product is still a stream of the weight matrix, but with this many rows the activations are no
 // longer negligible: a workgroup that owns 16 rows of W reads four times as many bytes of x as of W. Here
@@ -11,7 +11,7 @@
 // (tops/src/cublas.rs:29-114).
 //
 // Tiles of 64 k travel from global memory straight into LDS (global_load_lds_dwordx4: lane i of a wave
-// writes its 16 bytes at the wave's LDS base + 16 i), three steps ahead of the one being multiplied; each
+// writes its 16 bytes at the wave's LDS base + 16 i), four steps ahead of the one being multiplied; each
 // wave moves its own rows of W and a quarter of x. A tile is 16 rows of 128 bytes; the 16-byte piece c of
 // row r lies in slot (c + r) mod 8 of its row, which keeps the operand reads of a wave on distinct
 // banks without padding (the transfer cannot pad). One barrier per step.
