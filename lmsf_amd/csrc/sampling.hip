@@ -24,8 +24,11 @@
 //           cumulative sums <= 1 - p are removed, the largest always stays)
 //   min-p : keep x with prob >= min_p * max prob, i.e. x >= max + log(min_p)   (sampler.rs:305-325)
 #include "common.h"
+#include "no_alloc.h"
 
 #include <math.h>
+
+#include <mutex>
 
 #define SAMP_THREADS 1024
 
@@ -418,6 +421,54 @@ extern "C" int lmsf_sample(const float* logits, long ld, int R, int V, const flo
   hipLaunchKernelGGL(sample_kernel, dim3(R), dim3(SAMP_THREADS), smem, stream, logits, ld, V, temperature, top_k, top_p,
                      min_p, seeds, draws, out);
   LMSF_LAUNCH_CHECK("sample");
+  return 0;
+}
+
+// ---------------------------------------------------------------- greedy tokens without an allocation
+// The partial results of argmax_partial_kernel in a device array of the library's own (declared in
+// no_alloc.h). In host code the array's name is only a stand-in for the symbol; the address on the current
+// device comes from hipGetSymbolAddress and is kept per device.
+static __device__ __align__(256) unsigned char scratch[(size_t)LMSF_GREEDY_STATIC_MAX_ROWS * ARGMAX_SPLIT * 8];
+
+static std::mutex g_scratch_mutex;
+static void* g_scratch_ptr[64] = {nullptr};
+
+// Address of ``scratch`` on the current device, or null (error set).
+static void* greedy_static_scratch() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
+    lmsf_set_error("greedy_tokens_static: cannot tell the current device");
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* ptr = nullptr;
+    const hipError_t e = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ptr == nullptr) {
+      lmsf_set_error("greedy_tokens_static: hipGetSymbolAddress failed on device %d: %s", dev, hipGetErrorString(e));
+      return nullptr;
+    }
+    g_scratch_ptr[dev] = ptr;
+  }
+  return g_scratch_ptr[dev];
+}
+
+extern "C" int lmsf_greedy_tokens_static(const float* logits, long ld, int R, int V, int* out, hipStream_t stream) {
+  LMSF_CHECK(logits && out, "greedy_tokens_static: null pointer");
+  LMSF_CHECK(R >= 0 && V > 0 && ld >= V, "greedy_tokens_static: bad sizes R=%d V=%d ld=%ld", R, V, ld);
+  LMSF_CHECK(R <= LMSF_GREEDY_STATIC_MAX_ROWS,
+             "greedy_tokens_static: %d rows, the library's own buffer holds the partial results of %d at most", R,
+             LMSF_GREEDY_STATIC_MAX_ROWS);
+  if (R == 0) return 0;
+  void* ptr = greedy_static_scratch();
+  if (ptr == nullptr) return 2;
+  // values first, then indices, each R * ARGMAX_SPLIT entries: every entry is written by the first kernel
+  // before the second reads it, so the last call's contents do not matter
+  float* pval = (float*)ptr;
+  int* pidx = (int*)(pval + (size_t)R * ARGMAX_SPLIT);
+  hipLaunchKernelGGL(argmax_partial_kernel, dim3(R, ARGMAX_SPLIT), dim3(256), 0, stream, logits, ld, V, pval, pidx);
+  hipLaunchKernelGGL(argmax_final_kernel, dim3(R), dim3(64), 0, stream, pval, pidx, V, out);
+  LMSF_LAUNCH_CHECK("greedy_tokens_static");
   return 0;
 }
 

@@ -9,7 +9,7 @@ from typing import Optional
 
 from ..csrc import build as _build
 
-ABI_VERSION = 18
+ABI_VERSION = 19
 
 _lib: Optional[ctypes.CDLL] = None
 _lib_path: Optional[str] = None
@@ -70,6 +70,7 @@ _SIGNATURES = {
                                               c_long, c_int, c_int, c_int, c_int, _P]),
     "lmsf_sample": (c_int, [_P, c_long, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, _P, _P]),
     "lmsf_sample_scratch_elems": (c_long, [c_int, c_int]),
+    "lmsf_greedy_tokens_static": (c_int, [_P, c_long, c_int, c_int, _P, _P]),
     "lmsf_apply_penalties": (c_int, [_P, c_long, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, _P]),
 }
 
