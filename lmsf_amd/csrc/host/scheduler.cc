@@ -126,15 +126,19 @@ const StepPlan& Scheduler::schedule() {
 
   std::stable_sort(running_.begin(), running_.end(),
                    [&](int64_t a, int64_t b) { return seqs_.at(a).arrival < seqs_.at(b).arrival; });
-  std::deque<int64_t> todo(running_.begin(), running_.end());   // in arrival order; victims come from its end
-  while (!todo.empty()) {
-    const int64_t id = todo.front();
-    todo.pop_front();
-    if (budget <= 0) break;
+  // The running requests in arrival order, served in two passes: first every request that has one token to
+  // run (the decoding ones; core/src/sched/scheduler.rs:459-490 is the reference's decode pass), then the
+  // portions of prompts from what is left of the budget. A request that cannot get its pages makes the latest
+  // arrival behind it that this step has not served yet give up its pages; if there is none it is itself the
+  // one to yield.
+  const std::vector<int64_t> order(running_);
+  enum { kUnserved = 0, kServed = 1, kGone = 2 };
+  std::vector<char> mark(order.size(), kUnserved);
+  auto serve = [&](size_t i) {
+    const int64_t id = order[i];
     SeqInfo& s = seq(id);
     int64_t n = s.remaining();
     if (n > 1) n = chunk(std::min(n, budget));
-    bool dropped = false;
     while (!fits(&s, n, false)) {
       if (n > 1) {
         const int64_t room = std::min(room_tokens(&s, planned, nullptr), n - 1);   // a shorter portion may fit
@@ -143,30 +147,44 @@ const StepPlan& Scheduler::schedule() {
           continue;
         }
       }
-      if (!todo.empty()) {
-        const int64_t victim = todo.back();   // the latest arrival
-        todo.pop_back();
-        preempt(victim);
-      } else if (plan_.scheduled.empty()) {
+      size_t victim = order.size();
+      for (size_t j = order.size(); j-- > i + 1;)
+        if (mark[j] == kUnserved) { victim = j; break; }
+      if (victim < order.size()) {
+        mark[victim] = kGone;
+        preempt(order[victim]);
+        continue;
+      }
+      bool others = !plan_.scheduled.empty();
+      for (size_t j = 0; j < i && !others; ++j) others = mark[j] == kUnserved;
+      if (!others) {
         // alone and still no room: it can never continue
         remove_running(id);
         s.state = kFinishedLengthCapped;
         release(id);
         plan_.capped.push_back(id);
         forget(id);
-        dropped = true;
-        break;
-      } else {
+        mark[i] = kGone;
+      } else if (s.remaining() == 1) {
+        // a decoding request that is the latest arrival of those still unserved: it yields
+        mark[i] = kGone;
         preempt(id);
-        dropped = true;
-        break;
+      } else {
+        // a prompt with nobody behind it to take pages from: it keeps what it holds and waits for the requests
+        // that run in this step to finish or to yield
+        mark[i] = kServed;
       }
+      return;
     }
-    if (dropped) continue;
     take(&s, n);
     plan_.scheduled.push_back(Scheduled{id, s.num_computed, n, s.num_computed + n == s.length ? 1 : 0});
     budget -= n;
-  }
+    mark[i] = kServed;
+  };
+  for (size_t i = 0; i < order.size() && budget > 0; ++i)
+    if (mark[i] == kUnserved && seq(order[i]).remaining() == 1) serve(i);
+  for (size_t i = 0; i < order.size() && budget > 0; ++i)
+    if (mark[i] == kUnserved) serve(i);
 
   // admission, head of line only; nothing is admitted in a step that had to preempt
   while (!waiting_.empty() && plan_.preempted.empty() && budget > 0 && (int)running_.size() < config_.max_num_seqs) {

@@ -13,8 +13,10 @@
 // When pages run out:
 //  - a new request is not admitted while its first portion does not fit above the watermark (it waits);
 //  - a running request that cannot get the pages for its next tokens makes the latest-arrived running
-//    request give up everything it holds and go back to the front of the waiting queue, to be recomputed
-//    (prompt and tokens generated so far) later;
+//    request behind it that the step has not served yet give up everything it holds and go back to the front
+//    of the waiting queue, to be recomputed (prompt and tokens generated so far) later;
+//  - with nobody behind it, a decoding request yields in the same way itself, and a request in the middle of
+//    its prompt keeps what it holds and sits the step out (the requests that do run will finish or yield);
 //  - a request that is alone and still cannot continue can never continue: it is finished with reason
 //    "length";
 //  - a prompt that would not fit the whole pool even alone is ignored at admission (reason "length").

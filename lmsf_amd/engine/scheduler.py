@@ -7,14 +7,7 @@ what is different). This module is its Python face: it owns the ``Sequence`` obj
 sampling parameters), tells the library each request's length and progress before a plan is made, and
 writes the plan's consequences (state, progress, counters) back to them.
 
-What happens when pages run out:
-- a new request is not admitted while its first portion does not fit above the watermark (it waits);
-- a running request that cannot get the pages for its next tokens makes the latest-arrived running
-  request give up everything it holds and go back to the front of the waiting queue, to be
-  recomputed (prompt and tokens generated so far) later;
-- a request that is alone and still cannot continue can never continue: it is finished with
-  reason "length";
-- a prompt that would not fit the whole pool even alone is ignored at admission (reason "length").
+What happens when pages run out is written out once, at the top of ``lmsf_amd/csrc/host/scheduler.h``.
 """
 import ctypes
 import time

@@ -14,14 +14,7 @@ re-insertion at the front of the waiting queue, and prompts longer than the limi
 for every decoding request, then portions of prompts in arrival order, each at most
 ``prefill_chunk_size`` long.
 
-What happens when pages run out:
-- a new request is not admitted while its first portion does not fit above the watermark (it waits);
-- a running request that cannot get the pages for its next tokens makes the latest-arrived running
-  request give up everything it holds and go back to the front of the waiting queue, to be
-  recomputed (prompt and tokens generated so far) later;
-- a request that is alone and still cannot continue can never continue: it is finished with
-  reason "length";
-- a prompt that would not fit the whole pool even alone is ignored at admission (reason "length").
+What happens when pages run out is written out once, at the top of lmsf_amd/csrc/host/scheduler.h.
 """
 import time
 from collections import deque
@@ -140,41 +133,47 @@ class Scheduler:
                 planned[gi] += k
 
         self.running.sort(key=lambda s: s.arrival)
-        todo = list(self.running)                  # in arrival order; victims come from its end
-        while todo:
-            seq = todo.pop(0)
-            if budget <= 0:
-                break
-            n = seq.remaining
-            if n > 1:
-                n = min(n, budget, cfg.prefill_chunk_size or n)
+        # two passes over the running requests, each in arrival order: the decoding requests get their token
+        # first (core/src/sched/scheduler.rs:459-490), prompts are cut from the budget that is left
+        unserved = list(self.running)
+
+        def run_one(seq) -> None:
+            nonlocal budget
+            unserved.remove(seq)
+            decoding = seq.remaining == 1
+            n = 1 if decoding else min(seq.remaining, budget, cfg.prefill_chunk_size or seq.remaining)
             while not fits(seq.request_id, n):
                 if n > 1:
-                    # a shorter portion may fit
-                    room = min(self._room_tokens(seq, planned), n - 1)
+                    room = min(self._room_tokens(seq, planned), n - 1)      # a shorter portion may fit
                     if room >= 1:
                         n = room
                         continue
-                if todo:
-                    victim = todo.pop()            # the latest arrival
+                behind = [s for s in unserved if s.arrival > seq.arrival]
+                if behind:
+                    victim = max(behind, key=lambda s: s.arrival)           # the latest arrival
+                    unserved.remove(victim)
                     self._preempt(victim, plan)
-                elif not plan.scheduled:
+                    continue
+                if not plan.scheduled and not unserved:
                     # alone and still no room: it can never continue
                     self.running.remove(seq)
                     seq.state = SequenceState.FINISHED_LENGTH_CAPPED
                     self._release(seq)
                     plan.capped.append(seq)
-                    seq = None
-                    break
-                else:
+                elif decoding:
                     self._preempt(seq, plan)
-                    seq = None
-                    break
-            if seq is None:
-                continue
+                # else: a prompt with nobody behind it waits, keeping its pages
+                return
             take(seq.request_id, n)
             plan.scheduled.append(ScheduledSequence(seq, seq.num_computed, n, seq.num_computed + n == seq.length))
             budget -= n
+
+        for want_decoding in (True, False):
+            for seq in list(self.running):
+                if budget <= 0:
+                    break
+                if seq in unserved and (seq.remaining == 1 or not want_decoding):
+                    run_one(seq)
 
         # admission, head of line only; nothing is admitted in a step that had to preempt
         while self.waiting and not plan.preempted and budget > 0 and \

@@ -50,7 +50,7 @@ def test_fcfs_and_budget():
         [("a", 12, 1, True), ("b", 8, 4, True), ("c", 0, 3, True)]
 
 
-def test_prefill_chunk_size_and_decode_first():
+def test_prefill_chunk_size():
     sched, cache = make(num_pages=64, budget=16, chunk=5)
     a = seq("a", 11, 0)
     sched.add(a)
@@ -63,6 +63,60 @@ def test_prefill_chunk_size_and_decode_first():
     sched.add(seq("b", 9, 1))
     plan = sched.schedule()
     assert [(s.seq.request_id, s.n_tokens) for s in plan.scheduled] == [("a", 1), ("b", 5)]
+
+
+def test_decoding_requests_get_their_token_before_prompt_portions():
+    """An earlier arrival in the middle of a long prompt, a portion size of the whole budget, and a later
+    request that decodes: the decoder gets its token in every step and the prompt the rest."""
+    sched, cache = make(num_pages=64, budget=8, chunk=8, max_len=128)
+    sched.add(seq("short", 3, 1))
+    run_plan(sched, cache, sched.schedule())                  # short's prompt: it decodes from now on
+    long = seq("long", 40, 0)                                 # an earlier arrival number than short's
+    sched.add(long)
+    for step in range(5):
+        plan = sched.schedule()
+        got = [(s.seq.request_id, s.n_tokens) for s in plan.scheduled]
+        assert got == [("short", 1), ("long", 7)], (step, got)
+        assert plan.num_tokens <= 8
+        run_plan(sched, cache, plan)
+    assert long.num_computed == 35
+
+
+def test_a_decoder_without_pages_yields_to_an_earlier_prompt_and_a_prompt_without_pages_waits():
+    sched, cache = make(num_pages=4, page_size=4, budget=16, max_len=64)
+    old, new = seq("old", 12, 0), seq("new", 4, 1)
+    sched.add(old)
+    sched.add(new)
+    plan = sched.schedule()
+    assert [(s.seq.request_id, s.n_tokens) for s in plan.scheduled] == [("old", 12), ("new", 4)]
+    run_plan(sched, cache, plan)                              # all 4 pages are full
+    plan = sched.schedule()
+    # both decode and neither has a page: the later arrival gives its page up, the earlier takes it
+    assert [x.request_id for x in plan.preempted] == ["new"]
+    assert [(s.seq.request_id, s.n_tokens) for s in plan.scheduled] == [("old", 1)]
+    run_plan(sched, cache, plan)
+    cache.check_invariants()
+
+    # a prompt in its middle that finds no page while a later arrival decodes on its own page's slack keeps
+    # what it holds and sits the step out
+    sched, cache = make(num_pages=4, page_size=4, budget=7, chunk=6, max_len=64)
+    dec = seq("dec", 1, 1)
+    sched.add(dec)
+    run_plan(sched, cache, sched.schedule())                  # dec holds one page with one token
+    pro = seq("pro", 16, 0)
+    sched.add(pro)
+    for _ in range(2):                                        # 1 + 6 tokens a step: pro takes the other 3 pages
+        plan = sched.schedule()
+        run_plan(sched, cache, plan)
+    assert pro.num_computed == 12 and cache.num_free_pages(0) == 0
+    plan = sched.schedule()
+    assert [(s.seq.request_id, s.n_tokens) for s in plan.scheduled] == [("dec", 1)] and not plan.preempted
+    run_plan(sched, cache, plan)
+    assert cache.tokens_held(["pro"]).tolist() == [12]
+    # dec's page is full now: it is the latest arrival, so it yields, and pro goes on with its page
+    plan = sched.schedule()
+    assert [x.request_id for x in plan.preempted] == ["dec"]
+    assert [(s.seq.request_id, s.start, s.n_tokens) for s in plan.scheduled] == [("pro", 12, 4)]
 
 
 def test_too_long_prompt_is_ignored():
