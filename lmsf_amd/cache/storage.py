@@ -63,6 +63,7 @@ class CacheStorage:
         for g, n in zip(self.groups, num_pages):
             g.num_pages = int(n)
         self.num_state_slots = int(num_state_slots)
+        self.spare_state_slot = self.num_state_slots
         self.manager = CacheManager([GroupConfig(g.page_size, g.num_pages, g.spec.window) for g in self.groups],
                                     self.num_state_slots)
         bindings: List[CacheBinding] = []
@@ -81,7 +82,9 @@ class CacheStorage:
                     b.k_pages, b.v_pages = bindings[src].k_pages, bindings[src].v_pages
                     b.writes_cache = False
             if sspec is not None:
-                b.state = torch.zeros((max(1, self.num_state_slots),) + tuple(sspec.shape), dtype=sspec.dtype,
+                # one row more than there are slots: the spare one, for a padded batch's tokens that belong to
+                # no request
+                b.state = torch.zeros((self.num_state_slots + 1,) + tuple(sspec.shape), dtype=sspec.dtype,
                                       device=rt.device)
             bindings.append(b)
         self.bindings = bindings

@@ -7,7 +7,8 @@ produces logits: it takes pages for the new tokens, builds the flat batch, runs 
 exactly the tokens it was given, and commits them to the cache. Sampling is a separate call, so that
 trace replay can take the logits.
 """
-from typing import Dict, Hashable, Optional, Sequence, Tuple
+from collections import OrderedDict
+from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
 import numpy as np
 import torch
@@ -24,7 +25,7 @@ class StepError(ValueError):
 
 class ModelExecutor:
     def __init__(self, model, storage: CacheStorage, rt: Runtime, max_model_len: int, use_graphs: bool = True,
-                 max_graph_batch: int = 256):
+                 max_graph_batch: int = 256, max_graphs: int = 48):
         self.model = model
         self.storage = storage
         self.manager: CacheManager = storage.manager
@@ -36,12 +37,15 @@ class ModelExecutor:
         self.vocab_size = model.spec.vocab_size
         self._pinned: Optional[torch.Tensor] = None
         self._pinned_np: Optional[np.ndarray] = None
-        # steps of single tokens are captured as HIP graphs, one per batch size and context bucket
-        self.use_graphs = bool(use_graphs) and rt.device.type == "cuda" and \
-            all(getattr(p, "graph_safe", False) for p in model.parts())
+        # steps of single tokens run at a padded batch size and are captured as HIP graphs, one per padded
+        # size and context bucket, the least recently used dropped beyond max_graphs
+        self.pad_decode = all(getattr(p, "graph_safe", False) for p in model.parts())
+        self.use_graphs = bool(use_graphs) and rt.device.type == "cuda" and self.pad_decode
         self.max_graph_batch = int(max_graph_batch)
-        self._static: Dict[Tuple[int, int], "_StaticBatch"] = {}
+        self.max_graphs = int(max_graphs)
+        self._static: "OrderedDict[Tuple[int, int], _StaticBatch]" = OrderedDict()
         self._graph_pool = None
+        self._decode_logits: Optional[torch.Tensor] = None     # [rows, V]: every captured step writes here
 
     # ------------------------------------------------------------------ the step
 
@@ -58,8 +62,8 @@ class ModelExecutor:
         lens = [len(e.tokens) for e in entries]
         handles, starts, added = mgr.begin_step(rids, lens)      # OutOfPages: nothing was taken
         try:
-            if self.use_graphs and all(n == 1 for n in lens) and len(entries) <= self.max_graph_batch:
-                logits = self._graph_step(entries, handles, starts)
+            if self.pad_decode and all(n == 1 for n in lens) and len(entries) <= self.max_graph_batch:
+                logits = self._decode_step(entries, handles, starts)
             else:
                 logits = self.model.forward(self._build_context(entries, handles, starts))
         except Exception:
@@ -103,16 +107,19 @@ class ModelExecutor:
     def _build_context(self, entries: Sequence[StepEntry], handles: np.ndarray, starts_a: np.ndarray,
                        static: Optional["_StaticBatch"] = None) -> StepContext:
         """Flatten the entries into the step's device tensors. Everything goes through one pinned staging
-        buffer, which the host library fills, and one copy. With ``static`` (a decode step that replays a
-        captured graph) the copy goes into that batch's fixed device buffer, block tables padded to their
-        full width, and every token's logits are asked for."""
+        buffer, which the host library fills, and one copy. With ``static`` (a step of single tokens) the
+        batch is padded to that kind's size with tokens that store nothing (slot -1, position 0, a segment of
+        their own whose block table is all zeros, the spare state slot), the copy goes into its fixed device
+        buffer, block tables padded to their full width, and every token's logits are asked for."""
         mgr = self.manager
         S = len(entries)
         lens = [len(e.tokens) for e in entries]
         N = sum(lens)
         starts = starts_a.tolist()
+        Np = Sp = None
         if static is not None:
-            logit_rows = np.arange(N, dtype=np.int32)
+            Np = Sp = static.batch                      # N == S: single tokens
+            logit_rows = np.arange(Np, dtype=np.int32)
         else:
             seg_start, rows = 0, []
             for e, n in zip(entries, lens):
@@ -124,14 +131,15 @@ class ModelExecutor:
         widths = static.widths if static is not None else mgr.step_widths(handles)
         if static is not None:
             if static.layout is None:
-                static.layout = mgr.step_layout(N, S, R, widths)
+                static.layout = mgr.step_layout(Np, Sp, R, widths)
             offsets, raw_offsets, total = static.layout
         else:
             offsets, raw_offsets, total = mgr.step_layout(N, S, R, widths)
         # a step of single tokens also carries its tokens ordered by context, the longest first, behind the
         # sections the host library lays out
         single = N == S
-        order_at, total = total, total + (_pad4(N) if single else 0)
+        n_all = Np if static is not None else N
+        order_at, total = total, total + (_pad4(n_all) if single else 0)
         if self._pinned is None or self._pinned.numel() < total:
             self._pinned = torch.empty(max(total, 4096), dtype=torch.int32,
                                        pin_memory=self.rt.device.type == "cuda")
@@ -140,13 +148,15 @@ class ModelExecutor:
         host_np = self._pinned_np
         if single:
             host_np[order_at:order_at + N] = np.argsort(-starts_a, kind="stable")
+            if n_all > N:
+                host_np[order_at + N:order_at + n_all] = np.arange(N, n_all, dtype=np.int32)
 
         def section(name: str) -> np.ndarray:
             o, n = offsets[name]
             return host_np[o:o + n]
 
         if N == S:
-            section("token_ids")[:] = [e.tokens[0] for e in entries]
+            section("token_ids")[:N] = [e.tokens[0] for e in entries]
         else:
             section("token_ids")[:] = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in entries])
         if R:
@@ -155,6 +165,17 @@ class ModelExecutor:
             mgr.fill_step(handles, starts_a, lens, widths, raw_offsets, host_np)
         except CacheError as e:
             raise CacheError("%s (requests %s)" % (e, ", ".join(repr(x.request_id) for x in entries)))
+        if static is not None and Np > N:
+            pad = np.arange(N, Np, dtype=np.int32)
+            section("token_ids")[N:] = 0
+            section("positions")[N:] = 0
+            section("seg_of")[N:] = pad
+            section("seg_starts")[N:Np + 1] = np.arange(N, Np + 1, dtype=np.int32)
+            section("seg_first")[N:] = 0
+            section("state_slots")[N:] = self.storage.spare_state_slot
+            for gi in range(G):
+                section("slots%d" % gi)[N:] = -1
+                section("tables%d" % gi)[N * widths[gi]:] = 0
         # the copy is synchronous: the staging buffer is free again when the next step fills it
         if static is not None:
             static.device_buffer.copy_(host, non_blocking=False)
@@ -171,70 +192,112 @@ class ModelExecutor:
             o, n = offsets[name]
             return dev[o:o + n]
 
-        seg_starts = section("seg_starts").tolist()
-        state_slots = section("state_slots").tolist()
+        S_all = Sp if static is not None else S
+        if static is None:
+            seg_starts = section("seg_starts").tolist()
+            state_slots = section("state_slots").tolist()
+        else:
+            # a captured step is told nothing that changes from step to step
+            seg_starts, state_slots, lens, starts = list(range(S_all + 1)), [], [1] * S_all, []
         groups = [GroupView(slots=view("slots%d" % gi),
-                            block_tables=view("tables%d" % gi).view(S, widths[gi]),
+                            block_tables=view("tables%d" % gi).view(S_all, widths[gi]),
                             page_size=mgr.groups[gi].page_size) for gi in range(G)]
         return StepContext(
-            n_tokens=N, n_segments=S, token_ids=view("token_ids"), positions=view("positions"),
+            n_tokens=n_all, n_segments=S_all, token_ids=view("token_ids"), positions=view("positions"),
             seg_of_token=view("seg_of"), seg_starts=view("seg_starts"), seg_first_pos=view("seg_first"),
             state_slots=view("state_slots"), logit_rows=view("logit_rows"), n_logit_rows=R, groups=groups,
-            longest_first=dev[order_at:order_at + N] if single else None,
+            longest_first=dev[order_at:order_at + n_all] if single else None,
             host_seg_starts=seg_starts, host_seg_lens=lens, host_seg_first_pos=list(starts),
-            host_state_slots=list(state_slots), request_ids=[e.request_id for e in entries],
+            host_state_slots=list(state_slots),
+            request_ids=[e.request_id for e in entries] if static is None else [],
             max_seg_len=max(lens),
             max_context=(static.max_context if static is not None else
-                         self._context_bucket(max(starts) + 1) if all(n == 1 for n in lens) else
                          max(st + n for st, n in zip(starts, lens))),
             all_single=all(n == 1 for n in lens), replayed=static is not None)
 
     def _context_bucket(self, longest: int) -> int:
         """The longest context of a step of single tokens, rounded up to a power of two (at least 256, at
-        most the model's limit). Eager and replayed decode steps tell the parts this number instead of
-        the true one, so that both split the work alike and give the same bits."""
+        most the model's limit). The parts are told this number instead of the true one, so that every step
+        of a kind splits the work alike, captured or not."""
         bucket = 256
         while bucket < longest:
             bucket *= 2
         return min(bucket, self.max_model_len)
 
-    # ------------------------------------------------------------------ decode steps as HIP graphs
+    # ------------------------------------------------------------------ steps of single tokens
 
-    def _graph_step(self, entries: Sequence[StepEntry], handles: np.ndarray, starts: np.ndarray) -> torch.Tensor:
-        """A step of single tokens. The first step of a batch size and context bucket (the longest context
-        rounded up to a power of two) runs eagerly and is then captured as a HIP graph over a fixed
-        metadata buffer; later steps of that kind copy their metadata into the buffer and replay the
+    def _decode_step(self, entries: Sequence[StepEntry], handles: np.ndarray, starts: np.ndarray) -> torch.Tensor:
+        """A step of single tokens. Its batch is padded to one of a few sizes (``padded_batch``) and its
+        longest context rounded up to a power of two; what is left is a *kind* of step, whose metadata has a
+        fixed layout in a fixed device buffer. The first step of a kind runs kernel by kernel and is then
+        captured as a HIP graph; later steps of that kind copy their metadata into the buffer and replay the
         graph: one launch instead of hundreds. Inside a graph nothing may depend on the step's actual
         context lengths but through the device tensors, so the parts are told the bucket as the longest
-        context. The graph computes the logits of every token; the wanted rows are picked afterwards."""
+        context. Every kind writes the logits of all its tokens into one buffer shared by all kinds; the wanted
+        rows are picked from it afterwards. At most ``max_graphs`` kinds are kept, the least recently used is
+        dropped. Without graphs the same padded steps run kernel by kernel, to the same bits."""
         B = len(entries)
+        Bp = padded_batch(B, self.max_graph_batch)
         bucket = self._context_bucket(int(starts.max()) + 1)
-        sb = self._static.get((B, bucket))
+        sb = self._static.get((Bp, bucket))
         if sb is None:
             widths = [-(-bucket // g.page_size) for g in self.manager.groups]
-            _, _, total = self.manager.step_layout(B, B, B, widths)
-            sb = _StaticBatch(widths, torch.zeros(total + _pad4(B), dtype=torch.int32, device=self.rt.device), bucket)
-            self._static[(B, bucket)] = sb
+            _, _, total = self.manager.step_layout(Bp, Bp, Bp, widths)
+            sb = _StaticBatch(Bp, widths, torch.zeros(total + _pad4(Bp), dtype=torch.int32, device=self.rt.device),
+                              bucket)
+            self._static[(Bp, bucket)] = sb
+            while len(self._static) > self.max_graphs:
+                self._static.popitem(last=False)
+        else:
+            self._static.move_to_end((Bp, bucket))
+        if self._decode_logits is None:
+            rows = padded_batch(min(self.max_graph_batch, max(1, self.storage.num_state_slots)), self.max_graph_batch)
+            self._decode_logits = torch.empty((max(rows, Bp), self.vocab_size), dtype=torch.float32,
+                                              device=self.rt.device)
+        elif self._decode_logits.shape[0] < Bp:
+            # more live requests than state slots cannot be; a caller that builds such a step all the same gets
+            # a larger buffer, and the kinds captured so far, which write into the old one, are dropped
+            self._static = OrderedDict({(Bp, bucket): sb})
+            self._decode_logits = torch.empty((Bp, self.vocab_size), dtype=torch.float32, device=self.rt.device)
+        out = self._decode_logits[:Bp]
         ctx = self._build_context(entries, handles, starts, static=sb)
         if sb.graph is None:
             sb.context = ctx
-            logits = self.model.forward(ctx)                 # eager: this step's result, and the warm-up
-            torch.cuda.current_stream().synchronize()
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph, pool=self._graph_pool):
-                sb.logits = self.model.forward(ctx)
-            sb.graph = graph
-            if self._graph_pool is None:
-                self._graph_pool = graph.pool()
+            self.model.forward(ctx, logits_out=out)          # kernel by kernel: this step's result, and the warm-up
+            if self.use_graphs:
+                torch.cuda.current_stream().synchronize()
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph, pool=self._graph_pool):   # records, runs nothing: ``out`` stays
+                    self.model.forward(ctx, logits_out=out)
+                sb.graph = graph
+                if self._graph_pool is None:
+                    self._graph_pool = graph.pool()
         else:
             sb.graph.replay()
-            logits = sb.logits
+        # the rows go to the caller as a copy: the buffer is written again by the next step of single tokens
         wanted = [i for i, e in enumerate(entries) if len(e.want)]
         if len(wanted) == B:
-            return logits.clone()
+            return out[:B].clone()
         if not wanted:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.rt.device)
-        return logits[torch.tensor(wanted, device=self.rt.device)]
+        return out[torch.tensor(wanted, device=self.rt.device)]
+
+    def graph_memory_bytes(self) -> int:
+        """Device memory the captured steps hold beside the weights and the cache: the shared logits buffer and
+        the metadata buffers (the kernels' temporaries live in one pool that the graphs share)."""
+        total = 0 if self._decode_logits is None else self._decode_logits.numel() * 4
+        return total + sum(sb.device_buffer.numel() * 4 for sb in self._static.values())
+
+
+def padded_batch(batch: int, limit: int = 256) -> int:
+    """The size at which a step of ``batch`` single tokens runs: 1, 2, 4, 8, then multiples of 8."""
+    if batch <= 8:
+        size = 1
+        while size < batch:
+            size *= 2
+    else:
+        size = (batch + 7) // 8 * 8
+    return max(batch, min(size, limit))
 
 
 def _pad4(n: int) -> int:
@@ -242,14 +305,14 @@ def _pad4(n: int) -> int:
 
 
 class _StaticBatch:
-    """What a captured decode step of one batch size keeps: the fixed metadata buffer, the context whose
-    tensors are views into it, the graph and its output."""
+    """What a kind of decode step (padded batch size, context bucket) keeps: the fixed metadata buffer, the
+    context whose tensors are views into it, and the graph."""
 
-    def __init__(self, widths: Sequence[int], device_buffer: torch.Tensor, max_context: int):
+    def __init__(self, batch: int, widths: Sequence[int], device_buffer: torch.Tensor, max_context: int):
+        self.batch = int(batch)
         self.widths = list(widths)
         self.max_context = int(max_context)
         self.device_buffer = device_buffer
         self.context: Optional[StepContext] = None
         self.layout = None                 # the metadata buffer's sections: the same at every step of this kind
         self.graph = None
-        self.logits: Optional[torch.Tensor] = None

@@ -4,6 +4,7 @@ Embedding, the layers in the order of the schedule, final norm on the wanted row
 (core/src/model_executor/models/llama/llama.rs:397-476 is the reference's fixed version of this
 loop). The model holds no sizes of its own: everything comes from the spec.
 """
+import inspect
 from typing import Dict, List, Optional, Sequence, Tuple
 
 import torch
@@ -26,6 +27,7 @@ class DecoderModel:
                                           norms=norms))
         self.final_norm = build_part("norm", spec.final_norm, _prefix_of(spec.final_norm), rt)
         self.head = build_part("head", spec.head, _prefix_of(spec.head), rt)
+        self._head_takes_out = "out" in inspect.signature(self.head.forward).parameters
         self.schedule: Tuple[ScheduleEntry, ...] = tuple(spec.schedule)
         for i, e in enumerate(self.schedule):
             if not (0 <= e.layer < len(self.blocks)):
@@ -73,8 +75,9 @@ class DecoderModel:
 
     # ------------------------------------------------------------------ forward
 
-    def forward(self, ctx) -> torch.Tensor:
-        """Run the step's tokens; float32 logits [R, V] at ctx.logit_rows."""
+    def forward(self, ctx, logits_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Run the step's tokens; float32 logits [R, V] at ctx.logit_rows, in ``logits_out`` if one is given
+        (a head that does not take ``out`` gets its result copied there)."""
         residual = self.embedding.forward(ctx.token_ids)
         branch = None
         for e, binding in zip(self.schedule, self.bindings):
@@ -82,7 +85,11 @@ class DecoderModel:
         if ctx.n_logit_rows == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=residual.device)
         h = self.final_norm.forward_add(branch, residual, rows=ctx.logit_rows)
-        return self.head.forward(h)
+        if logits_out is None:
+            return self.head.forward(h)
+        if self._head_takes_out:
+            return self.head.forward(h, out=logits_out)
+        return logits_out.copy_(self.head.forward(h))
 
 
 def _prefix_of(spec) -> str:

@@ -523,10 +523,12 @@ class HipOps:
     # ------------------------------------------------------------------ matrix products
 
     def linear(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
-               out_dtype: Optional[torch.dtype] = None, pending_ok: bool = False):
+               out_dtype: Optional[torch.dtype] = None, pending_ok: bool = False,
+               out: Optional[torch.Tensor] = None):
         """y = x weight^T (+ bias); x [M, K], weight [N, K]; y [M, N] in ``out_dtype`` (default x's).
         With ``pending_ok`` the caller takes a ``PendingProduct`` as well, which comes back where the
-        product splits K over workgroups (17 to 64 rows, few columns).
+        product splits K over workgroups (17 to 64 rows, few columns). ``out``: a contiguous [M, N] tensor of
+        ``out_dtype`` that takes the result instead of a new one (not together with ``pending_ok``).
 
         float32 operands always run the float32 multiply-add kernel. bfloat16 products with bfloat16
         output and many rows go to the BLAS library, as the reference's do
@@ -542,10 +544,18 @@ class HipOps:
         if bias is not None and (bias.shape != (N,) or bias.dtype != weight.dtype or not bias.is_contiguous()):
             raise ValueError("linear: bias must be [%d] of the weight's dtype" % N)
         out_dtype = out_dtype or x.dtype
+        if out is not None:
+            if pending_ok or tuple(out.shape) != (M, N) or out.dtype != out_dtype or not out.is_contiguous() \
+                    or out.device != x.device:
+                raise ValueError("linear: out must be a contiguous [%d, %d] %s tensor on x's device" % (M, N, out_dtype))
+
+        def new():
+            return out if out is not None else torch.empty((M, N), dtype=out_dtype, device=x.device)
+
         both_bf16 = x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
         if (both_bf16 and self.skinny_max_rows < M <= self.mid_max_rows and self._mid_ok(x, weight)
                 and (M <= 64 or N <= self.mid_wide_max_cols or out_dtype == torch.float32)):
-            return self._linear_mid(x, weight, bias, 0, out_dtype, pending_ok and out_dtype == torch.bfloat16)
+            return self._linear_mid(x, weight, bias, 0, out_dtype, pending_ok and out_dtype == torch.bfloat16, out=out)
         if pending_ok and both_bf16 and out_dtype == torch.bfloat16 and self._skinny_ok(x, weight) and M > 0:
             if (M <= min(self.fuse_stream_rows, self.gemv_max_rows) and self._gemv_ok(M, K)) \
                     or M <= min(self.fuse_norm_rows, self.skinny_max_rows, 16):
@@ -554,14 +564,14 @@ class HipOps:
                 and N * K <= 2 ** 28:
             # one row: a pure stream of W (with two rows only the fused forms gain; the LM head's matrix is large
             # enough for the few-rows kernel to reach the same rate, so it stays there)
-            y = torch.empty((M, N), dtype=out_dtype, device=x.device)
+            y = new()
             self._check(self.lib.lmsf_gemv(_ptr(x), x.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(y),
                                            _code(out_dtype), y.stride(0), M, N, K, 0, self._stream()))
             return y
         if both_bf16 and out_dtype == torch.float32 and M > self.mid_max_rows and self._mid_ok(x, weight):
             # float32 output (logits) for many rows, which the library does not offer: as many rows at a time
             # as the kernel above takes
-            y = torch.empty((M, N), dtype=out_dtype, device=x.device)
+            y = new()
             for r0 in range(0, M, self.mid_max_rows):
                 rows = min(self.mid_max_rows, M - r0)
                 y[r0:r0 + rows] = self.linear(x[r0:r0 + rows], weight, bias, out_dtype=out_dtype)
@@ -571,7 +581,7 @@ class HipOps:
             # do not take the operands, for any number of rows, 64 at a time.
             limit = self.skinny_max_rows if out_dtype == torch.bfloat16 else 64
             if M <= limit or out_dtype == torch.float32:
-                y = torch.empty((M, N), dtype=out_dtype, device=x.device)
+                y = new()
                 for r0 in range(0, M, 64):
                     rows = min(64, M - r0)
                     xs, ys = x[r0:r0 + rows], y[r0:r0 + rows]
@@ -581,8 +591,10 @@ class HipOps:
                 return y
         if self.use_library_gemm and both_bf16 and M > self.skinny_max_rows:
             y = torch.nn.functional.linear(x, weight, bias)
+            if out is not None:
+                return out.copy_(y)
             return y if out_dtype == torch.bfloat16 else y.to(out_dtype)
-        y = torch.empty((M, N), dtype=out_dtype, device=x.device)
+        y = new()
         self._check(self.lib.lmsf_gemm_plain(_ptr(x), _code(x.dtype), x.stride(0), _ptr(weight), _code(weight.dtype),
                                              weight.stride(0), _ptr(bias), _ptr(y), _code(out_dtype), y.stride(0),
                                              M, N, K, self._stream()))
@@ -650,7 +662,8 @@ class HipOps:
                 and weight.data_ptr() % 16 == 0)
 
     def _linear_mid(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], act: int,
-                    out_dtype: torch.dtype = torch.bfloat16, pending_ok: bool = False):
+                    out_dtype: torch.dtype = torch.bfloat16, pending_ok: bool = False,
+                    out: Optional[torch.Tensor] = None):
         self._dev(x, weight, bias)
         M, K = x.shape
         N = weight.shape[0] // 2 if act else weight.shape[0]
@@ -665,7 +678,7 @@ class HipOps:
             return PendingProduct(partials, bias, out_dtype)
         floats = self.lib.lmsf_gemm_mid_scratch_floats(M, N, splits, act)
         scratch = torch.empty(floats, dtype=torch.float32, device=x.device) if floats else None
-        y = torch.empty((M, N), dtype=out_dtype, device=x.device)
+        y = out if out is not None else torch.empty((M, N), dtype=out_dtype, device=x.device)
         self._check(self.lib.lmsf_gemm_mid(_ptr(x), x.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(y),
                                            _code(out_dtype), y.stride(0), M, N, K, act, splits, _ptr(scratch),
                                            self._stream()))

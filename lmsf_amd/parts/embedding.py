@@ -62,6 +62,8 @@ class LMHead(Part):
         if self.bias_name:
             self.bias = fetch(self.bias_name).to(self.weight.dtype).contiguous()
 
-    def forward(self, h: torch.Tensor) -> torch.Tensor:
-        """[R, H] -> float32 logits [R, V]."""
+    def forward(self, h: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """[R, H] -> float32 logits [R, V], written into ``out`` if one is given."""
+        if out is not None:
+            return self.rt.ops.linear(h, self.weight, self.bias, out_dtype=torch.float32, out=out)
         return self.rt.ops.linear(h, self.weight, self.bias, out_dtype=torch.float32)

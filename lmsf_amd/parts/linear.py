@@ -43,19 +43,30 @@ class FusedLinear(Part):
                 out[self._name(sub, "bias")] = TensorDecl((rows,))
         return out
 
-    @staticmethod
-    def _cat(ts: List[torch.Tensor]) -> torch.Tensor:
-        if len(ts) == 1:
-            return ts[0].contiguous()
-        if any(t.dtype == torch.float32 for t in ts):
-            ts = [t.to(torch.float32) for t in ts]
-        return torch.cat(ts, dim=0).contiguous()
+    def _gather(self, fetch: Callable[[str], torch.Tensor], what: str) -> torch.Tensor:
+        """The sources' tensors as the row slices of one buffer, allocated once; every source is copied in
+        as it is read and dropped at once, so that beside the fused tensor only one source is alive at a time
+        (core/src/model_executor/layers/linear.rs:573-583, :603-622 copy into a zeroed buffer likewise). If
+        sources differ in element type the buffer takes the widest."""
+        if len(self.sources) == 1:
+            return fetch(self._name(self.sources[0][0], what)).contiguous()
+        out: Optional[torch.Tensor] = None
+        row = 0
+        for sub, rows in self.sources:
+            t = fetch(self._name(sub, what))
+            if out is None:
+                out = torch.empty((self.out_features,) + tuple(t.shape[1:]), dtype=t.dtype, device=t.device)
+            elif t.dtype != out.dtype and t.dtype == torch.float32:
+                out = out.to(torch.float32)
+            out[row:row + rows].copy_(t)
+            row += rows
+            del t
+        return out
 
     def load_weights(self, fetch: Callable[[str], torch.Tensor]) -> None:
-        self.weight = self._cat([fetch(self._name(sub, "weight")) for sub, _ in self.sources])
+        self.weight = self._gather(fetch, "weight")
         if self.has_bias:
-            b = self._cat([fetch(self._name(sub, "bias")) for sub, _ in self.sources])
-            self.bias = b.to(self.weight.dtype)
+            self.bias = self._gather(fetch, "bias").to(self.weight.dtype)
 
     def forward(self, x: torch.Tensor, out_dtype: Optional[torch.dtype] = None, pending_ok: bool = False):
         if pending_ok:

@@ -10,6 +10,7 @@ Element types: a tensor declared "float" is kept in bfloat16 in a bfloat16 run (
 converted) and converted to float32 in a float32 run; a tensor stored in 32 bits stays in 32 bits
 in either run. A tensor declared "int" becomes int32.
 """
+import warnings
 from typing import Callable, Dict, Iterable, List, Optional, Sequence, Tuple
 
 import torch
@@ -29,13 +30,18 @@ class WeightsError(ValueError):
         self.wrong_shape = list(wrong_shape)
 
 
-def collect_declarations(parts: Iterable[Part]) -> Dict[str, TensorDecl]:
+def collect_declarations(parts: Iterable[Part], shared: Optional[set] = None) -> Dict[str, TensorDecl]:
+    """Every declared tensor by name; ``shared`` (a set, if given) takes the names that more than one part
+    declares (tied weights)."""
     decls: Dict[str, TensorDecl] = {}
     for p in parts:
         for name, decl in p.checkpoint_tensors().items():
-            if name in decls and decls[name].shape != decl.shape:
-                raise ValueError("tensor %r is declared twice with shapes %s and %s"
-                                 % (name, decls[name].shape, decl.shape))
+            if name in decls:
+                if decls[name].shape != decl.shape:
+                    raise ValueError("tensor %r is declared twice with shapes %s and %s"
+                                     % (name, decls[name].shape, decl.shape))
+                if shared is not None:
+                    shared.add(name)
             decls[name] = decl
     return decls
 
@@ -81,7 +87,8 @@ def load_weights(parts: Sequence[Part], folder: str, device: torch.device, run_d
     """Check the checkpoint in ``folder`` against the parts' declarations, then hand every part its
     tensors on ``device``. A name declared by two parts (tied weights) is loaded once and shared."""
     parts = list(parts)
-    decls = collect_declarations(parts)
+    shared: set = set()
+    decls = collect_declarations(parts, shared)
     try:
         files = [SafetensorsFile(p) for p in list_weight_files(folder)]
     except SafetensorsError as e:
@@ -95,21 +102,32 @@ def load_weights(parts: Sequence[Part], folder: str, device: torch.device, run_d
                 entries[name] = (f, e)
         check_against_declarations(decls, {n: e.shape for n, (_, e) in entries.items()}, tolerated,
                                    where="checkpoint %r" % folder)
-        cache: Dict[str, torch.Tensor] = {}
+        cache: Dict[str, torch.Tensor] = {}      # only what several parts share: the rest belongs to its part
+        kept_wide: List[str] = []
 
         def fetch(name: str) -> torch.Tensor:
             if name not in decls:
                 raise KeyError("part asked for tensor %r that it did not declare" % name)
-            if name not in cache:
-                f, _ = entries[name]
-                try:
-                    cache[name] = _convert(f.read(name), decls[name], run_dtype).to(device)
-                except WeightsError as e:
-                    raise WeightsError("%s: %s" % (name, e))
-            return cache[name]
+            if name in cache:
+                return cache[name]
+            f, _ = entries[name]
+            try:
+                t = _convert(f.read(name), decls[name], run_dtype)
+            except WeightsError as e:
+                raise WeightsError("%s: %s" % (name, e))
+            if t.dtype == torch.float32 and run_dtype != torch.float32 and t.dim() >= 2:
+                kept_wide.append(name)
+            t = t.to(device)
+            if name in shared:
+                cache[name] = t
+            return t
 
         for p in parts:
             p.load_weights(fetch)
+        if kept_wide:
+            warnings.warn("%d matrices of %r are stored in 32 bits and stay so in this %s run (first: %s): their "
+                          "products run without the matrix cores and they take twice the memory; store the "
+                          "checkpoint in bfloat16 for speed" % (len(kept_wide), folder, run_dtype, kept_wide[0]))
     finally:
         for f in files:
             f.close()
@@ -118,19 +136,22 @@ def load_weights(parts: Sequence[Part], folder: str, device: torch.device, run_d
 def load_weights_from_generator(parts: Sequence[Part], make: Callable[[str, TensorDecl], torch.Tensor]) -> None:
     """Hand every part tensors made by ``make(name, declaration)`` (random weights on the device)."""
     parts = list(parts)
-    decls = collect_declarations(parts)
+    shared: set = set()
+    decls = collect_declarations(parts, shared)
     cache: Dict[str, torch.Tensor] = {}
 
     def fetch(name: str) -> torch.Tensor:
         if name not in decls:
             raise KeyError("part asked for tensor %r that it did not declare" % name)
-        if name not in cache:
-            t = make(name, decls[name])
-            if tuple(t.shape) != tuple(decls[name].shape):
-                raise WeightsError("generated tensor %r has shape %s, declared %s"
-                                   % (name, list(t.shape), list(decls[name].shape)))
+        if name in cache:
+            return cache[name]
+        t = make(name, decls[name])
+        if tuple(t.shape) != tuple(decls[name].shape):
+            raise WeightsError("generated tensor %r has shape %s, declared %s"
+                               % (name, list(t.shape), list(decls[name].shape)))
+        if name in shared:
             cache[name] = t
-        return cache[name]
+        return t
 
     for p in parts:
         p.load_weights(fetch)

@@ -93,3 +93,46 @@ def test_out_of_pages_takes_nothing(tmp_path):
     mgr.check_invariants()
     assert mgr.num_tokens("x") == 20 and not mgr.has_request("y")
     assert mgr.num_free_pages(0) == 1
+
+
+def test_padded_batch_sizes_are_few():
+    from lmsf_amd.engine.executor import padded_batch
+    sizes = sorted({padded_batch(b) for b in range(1, 257)})
+    assert sizes == [1, 2, 4, 8] + list(range(16, 257, 8))
+    assert all(padded_batch(b) >= b and padded_batch(b) < b + 8 for b in range(1, 257))
+    assert padded_batch(5, limit=6) == 6 and padded_batch(300, limit=256) == 300
+
+
+def test_kinds_of_decode_steps_stay_bounded_and_padding_changes_nothing(tmp_path):
+    """Steps of single tokens over a random sequence of batch sizes: the number of kinds the executor keeps
+    stays under its limit, all of them write into one logits buffer, and each request's logits are the plain
+    implementation's whatever the padding beside it was."""
+    import random
+    folder, cfg = make_model_folder(tmp_path, "A")
+    core = load_engine_core(folder, dtype="float32", block_size=8, num_pages=80, device="cpu", ops=TorchOps(),
+                            max_num_seqs=24)
+    cfg_dict, w = read_model_folder(folder)
+    ex = core.executor
+    ex.max_graphs = 3
+    assert ex.pad_decode and not ex.use_graphs
+    V = cfg_dict["vocab_size"]
+    toks = {i: random_tokens(20, V, 50 + i) for i in range(24)}
+    ref = {i: plain_llama_forward(cfg_dict, w, t) for i, t in toks.items()}
+    ex.step([StepEntry(i, t[:4], []) for i, t in toks.items()])
+    at = {i: 4 for i in toks}
+    rng = random.Random(1)
+    seen = set()
+    for _ in range(40):
+        ids = rng.sample([i for i in toks if at[i] < 20], k=min(rng.randint(1, 24), sum(a < 20 for a in at.values())))
+        out = ex.step([StepEntry(i, toks[i][at[i]:at[i] + 1], [0]) for i in ids])
+        seen.update(ex._static)
+        assert len(ex._static) <= 3
+        for row, i in zip(out, ids):
+            assert torch.allclose(row, ref[i][at[i]], atol=2e-5, rtol=1e-5), (i, at[i])
+            at[i] += 1
+        if all(a >= 20 for a in at.values()):
+            break
+    assert len(seen) > 3                     # more kinds came by than are kept
+    buffers = {sb.device_buffer.data_ptr() for sb in ex._static.values()}
+    assert len(buffers) == len(ex._static) and ex._decode_logits.shape[0] == 24
+    assert ex.graph_memory_bytes() >= ex._decode_logits.numel() * 4

@@ -484,10 +484,10 @@ def test_toy_parts_are_registered_built_and_stepped(toy_architecture, tmp_path):
                                                               w["toy.layers.0.ln2.weight"], cfg.rms_norm_eps),
                                              w["toy.layers.0.moe.router.weight"]), -1)[t].argmax()) for t in range(64)}
     assert len(used) > 1                                         # the routing does route
-    # the two runs of layer 0 have a state tensor each, one slot per live request; no pages for them
+    # the two runs of layer 0 have a state tensor each, one slot per live request and a spare one; no pages for them
     states = [b.state for b in core.storage.bindings]
     assert states[0] is not None and states[2] is not None and states[1] is None
-    assert states[0].data_ptr() != states[2].data_ptr() and tuple(states[0].shape) == (3, cfg.hidden_size + 1)
+    assert states[0].data_ptr() != states[2].data_ptr() and tuple(states[0].shape) == (3 + 1, cfg.hidden_size + 1)
     assert core.storage.entry_group == [None, 0, None]
     assert not core.executor.use_graphs                          # a part that does not declare itself graph-safe: eager
     from test_replay_gpu import check

@@ -186,3 +186,50 @@ def test_write_random_model_uses_the_requested_storage(tmp_path):
     assert all(v.dtype == torch.bfloat16 for v in t.values())
     with open(os.path.join(folder, "config.json")) as f:
         assert json.load(f)["torch_dtype"] == "bfloat16"
+
+
+def test_loading_keeps_one_source_tensor_alive_beside_the_weights(tmp_path):
+    """The fused products copy every checkpoint tensor into its rows of one buffer and drop it at once, and
+    the loader keeps nothing but tied tensors: while the model loads, at most one tensor that is not part of
+    the model is alive."""
+    import gc
+    import weakref
+    from lmsf_amd.weights.loader import load_weights_from_generator
+    folder, cfg = make_model_folder(tmp_path, "B")
+    raw = load_file(os.path.join(folder, "model.safetensors"))
+    model = cpu_model(cfg)
+    made = []                 # (name, weak reference) of everything handed out
+    most = [0]
+
+    def make(name, decl):
+        gc.collect()
+        alive = [n for n, r in made if r() is not None and not _is_model_tensor(model, r())]
+        most[0] = max(most[0], len(alive))
+        t = raw[name].clone()
+        made.append((name, weakref.ref(t)))
+        return t
+
+    load_weights_from_generator(model.parts(), make)
+    assert most[0] <= 1, most[0]
+    p = "model.layers.2.self_attn."
+    assert torch.equal(model.blocks[2].mixer.qkv.weight,
+                       torch.cat([raw[p + "q_proj.weight"], raw[p + "k_proj.weight"], raw[p + "v_proj.weight"]]))
+    # mixed storage: the buffer takes the widest element type
+    wide = cpu_model(cfg, torch.bfloat16)
+    load_weights_from_generator(wide.parts(), lambda n, d: raw[n].clone() if n.endswith("k_proj.weight")
+                                else raw[n].to(torch.bfloat16))
+    assert wide.blocks[0].mixer.qkv.weight.dtype == torch.float32
+    assert torch.equal(wide.blocks[0].mixer.qkv.weight[256:288], raw["model.layers.0.self_attn.k_proj.weight"])
+
+
+def _is_model_tensor(model, t):
+    return any(getattr(p, a, None) is not None and getattr(p, a).data_ptr() == t.data_ptr()
+               for p in model.parts() for a in ("weight", "bias"))
+
+
+def test_matrices_stored_in_32_bits_are_reported(tmp_path):
+    folder, cfg = make_model_folder(tmp_path, "A", dtype="float32")
+    m = cpu_model(cfg, torch.bfloat16)
+    with pytest.warns(UserWarning, match="stored in 32 bits"):
+        load_weights(m.parts(), folder, torch.device("cpu"), torch.bfloat16)
+    assert m.blocks[0].mixer.qkv.weight.dtype == torch.float32

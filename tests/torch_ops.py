@@ -155,11 +155,12 @@ class TorchOps:
     def linear_gated(self, x, weight, bias=None, kind="silu"):
         return self.gated_act(self.linear(x, weight, bias), kind)
 
-    def linear(self, x, weight, bias=None, out_dtype=None, pending_ok=False):
+    def linear(self, x, weight, bias=None, out_dtype=None, pending_ok=False, out=None):
         y = x.to(torch.float32) @ weight.to(torch.float32).t()
         if bias is not None:
             y = y + bias.to(torch.float32)
-        return y.to(out_dtype or x.dtype)
+        y = y.to(out_dtype or x.dtype)
+        return y if out is None else out.copy_(y)
 
     def materialize(self, y):
         return y
