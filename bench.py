@@ -51,9 +51,8 @@ def weight_bytes(engine):
     emb = engine.core.model.embedding.weight
     head = engine.core.model.head.weight
     for p in engine.core.model.parts():
-        for name in ("weight", "bias"):
-            t = getattr(p, name, None)
-            if t is None or t.data_ptr() in seen:
+        for t in p.tensors():
+            if t.data_ptr() in seen:
                 continue
             if t.data_ptr() == emb.data_ptr() and emb.data_ptr() != head.data_ptr():
                 continue

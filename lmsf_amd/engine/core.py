@@ -5,6 +5,7 @@ on top). Reference: Worker::from + Worker::init_cache (core/src/worker/model_wor
 the sizing of the cache from free device memory (:128-162).
 """
 import os
+import warnings
 from dataclasses import dataclass
 from typing import Any, Optional, Sequence
 
@@ -26,10 +27,14 @@ _DTYPES = {"float32": torch.float32, "float": torch.float32, "bfloat16": torch.b
 
 def resolve_dtype(name: Optional[str], config: ArchConfig) -> torch.dtype:
     """--dtype overrides config.json's torch_dtype (core/src/common/config.rs:181-186). float16
-    checkpoints run in bfloat16: the kernels have two element types, float32 and bfloat16."""
+    checkpoints run in bfloat16 (with a warning: three bits of every weight's mantissa go): the kernels
+    have two element types, float32 and bfloat16."""
     key = name if name not in (None, "auto") else config.torch_dtype
     if key not in _DTYPES:
         raise ValueError("dtype %r is not supported (float32, bfloat16)" % (key,))
+    if key in ("float16", "half"):
+        warnings.warn("dtype %s runs as bfloat16 here: weights stored in float16 are rounded to bfloat16's 8 bits "
+                      "of mantissa; use --dtype float32 to keep all of them" % key)
     return _DTYPES[key]
 
 
@@ -77,22 +82,36 @@ def profile_num_pages(model: DecoderModel, rt: Runtime, block_size: int, gpu_mem
     if not groups:
         return []
     es = 4 if rt.dtype == torch.float32 else 2
+    # what torch has freed but keeps (the loader's source tensors) goes back first, so that "used" is what is
+    # really held: the weights, the HIP context and the libraries' own buffers
+    torch.cuda.empty_cache()
     free, total = torch.cuda.mem_get_info(rt.device)
     spec = model.spec
-    widest = max((p.weight.shape[0] for p in model.parts() if getattr(p, "weight", None) is not None
-                  and p.weight.dim() == 2 and p.weight.shape[0] != spec.vocab_size), default=spec.hidden_size)
-    act = max_num_batched_tokens * (spec.hidden_size * 4 * 2 + widest * es * 3) \
+    mats = [t for p in model.parts() for t in p.tensors() if t.dim() == 2 and t.shape[0] != spec.vocab_size]
+    widest = max((t.shape[0] for t in mats), default=spec.hidden_size)
+    wes = max((t.element_size() for t in mats), default=es)       # matrices kept in 32 bits have 32-bit products
+    # one step's activations (float32 stream twice, three buffers of the widest product), the logits of every
+    # request three times over (the decode steps' shared buffer, the caller's copy, the sampler's scratch), and
+    # the metadata buffers and the kernels' pool of the captured decode steps
+    act = max_num_batched_tokens * (spec.hidden_size * 4 * 2 + widest * max(es, wes) * 3) \
         + max_num_seqs * spec.vocab_size * 4 * 3 + (512 << 20)
-    budget = int(total * gpu_memory_utilization) - (total - free) - act
+    return pages_for_budget(groups, int(total * gpu_memory_utilization) - (total - free) - act, es, block_size,
+                            max_num_batched_tokens, max_num_seqs, max_model_len)
+
+
+def pages_for_budget(groups, budget: int, elem_size: int, block_size: int, max_num_batched_tokens: int,
+                     max_num_seqs: int, max_model_len: int) -> Sequence[int]:
+    """Pages per cache group from ``budget`` bytes: a window group gets what its window can ever hold, the
+    groups that keep every key share the rest, the same number of pages each (their block tables run in step)."""
     counts = [0] * len(groups)
     for gi, g in enumerate(groups):
         if g.spec.window is not None:
             per_seq = (g.spec.window + max_num_batched_tokens) // block_size + 2
             counts[gi] = per_seq * max_num_seqs
-            budget -= counts[gi] * g.bytes_per_page(es)
+            budget -= counts[gi] * g.bytes_per_page(elem_size)
     full = [gi for gi, g in enumerate(groups) if g.spec.window is None]
     if full:
-        per_page_all = sum(groups[gi].bytes_per_page(es) for gi in full)
+        per_page_all = sum(groups[gi].bytes_per_page(elem_size) for gi in full)
         n = max(0, budget // per_page_all)
         n = min(n, max_num_seqs * (-(-max_model_len // block_size)) + 1)   # more can never be used
         for gi in full:

@@ -5,6 +5,11 @@ step function, cache manager and kernels that generation uses. The reference has
 it (its closest is the hand-driven step loop of example/examples/llm_engine_example.rs:65-151).
 
     trace_run --model DIR --dtype bfloat16|float32 --out DIR --max-tokens N
+              [--block-size B] [--num-gpu-blocks P] [--random CONFIG.json --seed S]
+
+``--random CONFIG.json`` stands in for ``--model``: the model of that configuration with random weights
+made from ``--seed`` (the engine's random-weights mode). ``--block-size`` is the page size in tokens
+(default 16); ``--num-gpu-blocks`` sets the number of pages instead of deriving it from ``--max-tokens``.
 
 Steps come on standard input, one JSON object a line:
 
@@ -19,11 +24,23 @@ step a line ``done <step>`` is printed and flushed.
 import argparse
 import json
 import os
+import shutil
 import sys
 import tempfile
 import time
 
-PAGE_SIZE = 16
+DEFAULT_PAGE_SIZE = 16
+
+
+def pages_for(max_tokens: int, page_size: int) -> int:
+    """Pages that hold ``max_tokens`` tokens of live requests when each request's count is rounded up to a
+    multiple of 64: with a page size that divides 64 that is max_tokens / page_size; otherwise every 64
+    tokens of a request may end in a page that is partly empty."""
+    if 64 % page_size == 0:
+        return -(-max_tokens // page_size)
+    if page_size % 64 == 0:
+        return -(-max_tokens // 64)          # each request rounds up to its own pages: at most one per 64 tokens
+    return -(-max_tokens // 64) * -(-64 // page_size)
 
 
 def _say(msg: str) -> None:
@@ -40,7 +57,13 @@ def _usable_home() -> None:
 
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(prog="trace_run", description=__doc__.split("\n\n")[0])
-    ap.add_argument("--model", required=True, help="folder with config.json and model.safetensors")
+    ap.add_argument("--model", default=None, help="folder with config.json and model.safetensors")
+    ap.add_argument("--random", default=None, metavar="CONFIG.json",
+                    help="instead of --model: this configuration with random weights")
+    ap.add_argument("--seed", type=int, default=0, help="seed of the random weights of --random")
+    ap.add_argument("--block-size", type=int, default=DEFAULT_PAGE_SIZE, help="tokens a page of the cache holds")
+    ap.add_argument("--num-gpu-blocks", type=int, default=None,
+                    help="pages of the cache pool (default: what --max-tokens needs)")
     ap.add_argument("--dtype", required=True, choices=["bfloat16", "float32"])
     ap.add_argument("--out", required=True, help="folder the logits files are written to")
     ap.add_argument("--max-tokens", type=int, required=True,
@@ -49,6 +72,10 @@ def main(argv=None) -> int:
     args = ap.parse_args(argv)
     if args.max_tokens <= 0:
         ap.error("--max-tokens must be > 0")
+    if (args.model is None) == (args.random is None):
+        ap.error("give --model DIR or --random CONFIG.json")
+    if args.block_size <= 0:
+        ap.error("--block-size must be > 0")
     _usable_home()
     os.makedirs(args.out, exist_ok=True)
     t0 = time.time()
@@ -58,12 +85,16 @@ def main(argv=None) -> int:
 
     from lmsf_amd.engine import StepEntry, load_engine_core
 
-    _say("torch ready after %.0f s; loading kernels and %s" % (time.time() - t0, args.model))
-    num_pages = -(-args.max_tokens // PAGE_SIZE)
-    core = load_engine_core(args.model, dtype=args.dtype, block_size=PAGE_SIZE, num_pages=num_pages,
-                            max_num_seqs=64, device=args.device)
+    model_dir, load_format = args.model, "auto"
+    if args.random is not None:
+        model_dir, load_format = tempfile.mkdtemp(prefix="lmsf_random_"), "random"
+        shutil.copyfile(args.random, os.path.join(model_dir, "config.json"))
+    _say("torch ready after %.0f s; loading kernels and %s" % (time.time() - t0, args.model or args.random))
+    num_pages = args.num_gpu_blocks if args.num_gpu_blocks else pages_for(args.max_tokens, args.block_size)
+    core = load_engine_core(model_dir, dtype=args.dtype, block_size=args.block_size, num_pages=num_pages,
+                            max_num_seqs=64, device=args.device, load_format=load_format, seed=args.seed)
     _say("model %s ready after %.0f s: %s, %d pages of %d tokens" % (
-        core.arch.name, time.time() - t0, args.dtype, num_pages, PAGE_SIZE))
+        core.arch.name, time.time() - t0, args.dtype, num_pages, args.block_size))
     executor = core.executor
     for line in sys.stdin:
         line = line.strip()

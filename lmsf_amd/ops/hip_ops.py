@@ -385,6 +385,15 @@ class HipOps:
 
     # ------------------------------------------------------------------ attention
 
+    @staticmethod
+    def check_head_dim(d: int) -> None:
+        """Raises if no attention kernel takes head size ``d``: the matrix-core kernels take multiples of 16
+        up to 256 (bfloat16), the general kernel multiples of 4 up to 256 (either dtype). Parts ask this when
+        they are built, before any weight is loaded."""
+        if d <= 0 or d % 4 != 0 or d > 256:
+            raise ValueError("head size %d is not supported by the attention kernels: they take multiples of 4 "
+                             "up to 256 (multiples of 16 on the matrix cores)" % d)
+
     def paged_attention(self, q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                         block_tables: torch.Tensor, seg: torch.Tensor, pos: torch.Tensor, nh: int, nkv: int, d: int,
                         scale: float, window: int = 0, batch=None, kernel: Optional[str] = None) -> torch.Tensor:

@@ -32,6 +32,9 @@ class PagedAttention(Mixer):
         if num_heads % num_kv_heads != 0:
             raise ValueError("num_heads %d is not a multiple of num_kv_heads %d" % (num_heads, num_kv_heads))
         self.nh, self.nkv, self.d = int(num_heads), int(num_kv_heads), int(head_dim)
+        check = getattr(rt.ops, "check_head_dim", None)
+        if check is not None:
+            check(self.d)          # a size no kernel takes is refused here, not at the first step
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.d)
         self.window = int(window) if window else None
         self.qkv = FusedLinear(prefix, rt, hidden_size,

@@ -160,6 +160,12 @@ class Part:
     def children(self) -> Sequence["Part"]:
         return ()
 
+    def tensors(self) -> Sequence[torch.Tensor]:
+        """The device tensors this part (not its children) holds after loading: what memory sizing and the
+        count of a step's bytes look at. The default finds ``weight`` and ``bias``; a part that keeps its
+        tensors elsewhere (a list of experts) returns them here."""
+        return [t for t in (getattr(self, "weight", None), getattr(self, "bias", None)) if isinstance(t, torch.Tensor)]
+
     def walk(self):
         yield self
         for c in self.children():

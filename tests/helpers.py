@@ -147,15 +147,15 @@ def replay_in_process(executor, steps):
     return {rid: torch.cat(parts) for rid, parts in got.items()}
 
 
-def replay_with_program(program, model_dir, dtype, steps, out_dir, max_tokens, vocab, timeout=600):
+def replay_with_program(program, model_dir, dtype, steps, out_dir, max_tokens, vocab, timeout=600, extra_args=()):
     """Run a trace through bin/trace_run as a child process; returns {request id: logits [len, V]}."""
     import subprocess
 
     import numpy as np
     os.makedirs(out_dir, exist_ok=True)
     text = "".join(json.dumps(st) + "\n" for st in steps)
-    proc = subprocess.run([program, "--model", model_dir, "--dtype", dtype, "--out", out_dir,
-                           "--max-tokens", str(max_tokens)], input=text, stdout=subprocess.PIPE,
+    proc = subprocess.run([program] + (["--model", model_dir] if model_dir else []) + ["--dtype", dtype, "--out", out_dir,
+                           "--max-tokens", str(max_tokens)] + list(extra_args), input=text, stdout=subprocess.PIPE,
                           stderr=subprocess.PIPE, text=True, timeout=timeout)
     if proc.returncode != 0:
         raise RuntimeError("trace_run failed (%d):\n%s" % (proc.returncode, proc.stderr[-4000:]))

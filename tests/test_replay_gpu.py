@@ -212,6 +212,42 @@ def test_trace_run_program(models, dtype, tmp_path):
     check(got, refs_cut, dtype, "trace_run mixed")
 
 
+def test_trace_run_with_another_page_size(models, tmp_path):
+    """Tiny A at its own page size of 8 through the program (--block-size), with so few pages that they are
+    used again."""
+    folder, cfg, w = models[("A", "float32")]
+    reqs = requests_for(cfg, "A")
+    refs = {rid: plain_llama_forward(cfg, w, toks) for rid, toks in reqs.items()}
+    max_tokens = 128 + 128
+    steps = trace_mixed(reqs, max_tokens, seed=3)
+    got = replay_with_program(TRACE_RUN, folder, "float32", steps, str(tmp_path / "out"), max_tokens, cfg["vocab_size"],
+                              extra_args=["--block-size", "8"])
+    check(got, refs, "float32", "trace_run, pages of 8")
+
+
+def test_trace_run_with_random_weights(tmp_path):
+    """--random CONFIG.json --seed: the same seed gives the same logits, another seed others, and cutting the
+    tokens differently changes nothing."""
+    import json
+    import numpy as np
+    from helpers import TINY
+    cfg = TINY["B"][0]
+    path = tmp_path / "cfg.json"
+    path.write_text(json.dumps(cfg))
+    toks = random_tokens(40, cfg["vocab_size"], 9)
+    whole = [{"step": 0, "entries": [{"id": "a", "tokens": toks, "want": [38, 39]}], "end": ["a"]}]
+    cut = [{"step": 0, "entries": [{"id": "a", "tokens": toks[:17], "want": []}], "end": []},
+           {"step": 1, "entries": [{"id": "a", "tokens": toks[17:39], "want": [21]}], "end": []},
+           {"step": 2, "entries": [{"id": "a", "tokens": toks[39:], "want": [0]}], "end": ["a"]}]
+
+    def run(steps, seed, name):
+        return replay_with_program(TRACE_RUN, None, "float32", steps, str(tmp_path / name), 64, cfg["vocab_size"],
+                                   extra_args=["--random", str(path), "--seed", str(seed), "--num-gpu-blocks", "5"])["a"]
+    a, b, c = run(whole, 1, "a"), run(cut, 1, "b"), run(whole, 2, "c")
+    assert torch.allclose(a, b, atol=3e-5) and not torch.allclose(a, c, atol=1e-3)
+    assert np.isfinite(a.numpy()).all()
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_graph_replay_equals_eager(models, dtype):
     """Decode steps are captured as HIP graphs and replayed. Every replay must give what the same step
@@ -269,3 +305,39 @@ def test_decode_steps_of_many_requests_of_different_lengths(models, dtype):
     assert any(b >= 16 for (b, _bucket) in core.executor._static), "no decode step of sixteen or more was captured"
     check(got, refs, dtype, "twenty requests")
     core.storage.manager.check_invariants()
+
+
+def test_float32_checkpoint_in_a_bfloat16_run(models):
+    """A checkpoint stored in 32 bits keeps its 32 bits in a bfloat16 run (with a warning): activations and cache
+    are bfloat16, the products run in float32 arithmetic, and the logits are the plain implementation's within
+    the bfloat16 bound, under portions and single tokens alike."""
+    folder, cfg, w = models[("B", "float32")]
+    from lmsf_amd.engine import load_engine_core
+    with pytest.warns(UserWarning, match="stored in 32 bits"):
+        core = load_engine_core(folder, dtype="bfloat16", block_size=16, num_pages=24, max_num_seqs=4)
+    assert core.model.blocks[0].mixer.qkv.weight.dtype == torch.float32
+    assert core.model.bindings[0].k_pages.dtype == torch.bfloat16
+    reqs = {"a": random_tokens(150, cfg["vocab_size"], 31), "b": random_tokens(40, cfg["vocab_size"], 32)}
+    refs = {rid: plain_llama_forward(cfg, w, toks) for rid, toks in reqs.items()}
+    check(replay_in_process(core.executor, trace_bulk_then_single(reqs)), refs, "bfloat16", "float32 weights, bulk then single")
+    check(replay_in_process(core.executor, trace_portions(reqs, seed=4)), refs, "bfloat16", "float32 weights, portions")
+
+
+def test_page_count_ignores_memory_that_torch_only_caches(models):
+    """Sizing the cache after a large tensor was freed: torch keeps the block, the page count must not."""
+    folder, cfg, w = models[("B", "bfloat16")]
+    from lmsf_amd.cache.storage import plan_groups
+    from lmsf_amd.engine import load_engine_core
+    from lmsf_amd.engine.core import profile_num_pages
+    core = load_engine_core(folder, dtype="bfloat16", block_size=16, num_pages=4, max_num_seqs=4)
+    big = torch.empty(24 << 30, dtype=torch.uint8, device="cuda:0")
+    del big
+    assert torch.cuda.memory_reserved() - torch.cuda.memory_allocated() > 20 << 30
+    seqs = 1 << 18
+    n = profile_num_pages(core.model, core.rt, 16, 0.5, 2048, seqs, 4096)[0]
+    free, total = torch.cuda.mem_get_info()
+    groups, _ = plan_groups(core.model.cache_requirements(), 16)
+    act = 2048 * (128 * 4 * 2 + 704 * 2 * 3) + seqs * 1000 * 4 * 3 + (512 << 20)
+    want = (int(total * 0.5) - (total - free) - act) / groups[0].bytes_per_page(2)
+    assert abs(n - want) / want < 0.02, (n, want)
+    assert torch.cuda.memory_reserved() - torch.cuda.memory_allocated() < 1 << 30
