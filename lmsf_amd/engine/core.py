@@ -124,7 +124,8 @@ def load_engine_core(model_dir: Optional[str], dtype: Optional[str] = None, bloc
                      gpu_memory_utilization: float = 0.9, max_num_seqs: int = 256,
                      max_num_batched_tokens: Optional[int] = None, device: str = "cuda:0",
                      ops: Any = None, load_format: str = "auto", seed: int = 0,
-                     config: Optional[ArchConfig] = None, enforce_eager: bool = False) -> EngineCore:
+                     config: Optional[ArchConfig] = None, enforce_eager: bool = False,
+                     use_program: bool = True) -> EngineCore:
     """``num_pages``: pages of every cache group (tests, replay); None sizes the pools from free memory."""
     if config is None:
         if model_dir is None:
@@ -163,5 +164,6 @@ def load_engine_core(model_dir: Optional[str], dtype: Optional[str] = None, bloc
     else:
         counts = [int(num_pages)] * len(groups)
     storage = CacheStorage(model, rt, block_size, counts, num_state_slots=max_num_seqs)
-    executor = ModelExecutor(model, storage, rt, max_model_len, use_graphs=not enforce_eager)
+    executor = ModelExecutor(model, storage, rt, max_model_len, use_graphs=not enforce_eager,
+                             use_program=use_program)
     return EngineCore(arch, config, rt, model, storage, executor, max_model_len, block_size)

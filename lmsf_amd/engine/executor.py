@@ -25,7 +25,7 @@ class StepError(ValueError):
 
 class ModelExecutor:
     def __init__(self, model, storage: CacheStorage, rt: Runtime, max_model_len: int, use_graphs: bool = True,
-                 max_graph_batch: int = 256, max_graphs: int = 48):
+                 max_graph_batch: int = 256, max_graphs: int = 48, use_program: bool = True):
         self.model = model
         self.storage = storage
         self.manager: CacheManager = storage.manager
@@ -46,6 +46,14 @@ class ModelExecutor:
         self._static: "OrderedDict[Tuple[int, int], _StaticBatch]" = OrderedDict()
         self._graph_pool = None
         self._decode_logits: Optional[torch.Tensor] = None     # [rows, V]: every captured step writes here
+        # the model's kernel calls recorded once and run from C++, a step a call; None where the model's parts
+        # do more with their activations than hand them to the kernels (then the parts run one by one)
+        self.program = None
+        self.use_program = bool(use_program) and rt.device.type == "cuda"
+        if self.use_program:
+            from ..ops.program import record_program
+            self.program = record_program(model, rt.ops)
+        self.program_steps = 0          # steps that the program ran
 
     # ------------------------------------------------------------------ the step
 
@@ -65,12 +73,48 @@ class ModelExecutor:
             if self.pad_decode and all(n == 1 for n in lens) and len(entries) <= self.max_graph_batch:
                 logits = self._decode_step(entries, handles, starts)
             else:
-                logits = self.model.forward(self._build_context(entries, handles, starts))
+                logits = self._forward(self._build_context(entries, handles, starts))
         except Exception:
             mgr.abort_step(rids, handles, added)
             raise
         mgr.commit_step(handles)
         return logits
+
+    def _forward(self, ctx: StepContext, logits_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """The model over the step: through the recorded program where there is one and it takes the step, else
+        part by part."""
+        prog = self.program
+        if prog is not None and prog.stale():
+            # somebody moved the kernels' switch points (tests, tuning): record again, and forget what was captured
+            from ..ops.program import record_program
+            prog = self.program = record_program(self.model, self.rt.ops)
+            self._static.clear()
+        if prog is not None:
+            from ..ops.hip_ops import _current_device, _raw_stream
+            R = ctx.n_logit_rows
+            out = logits_out
+            if out is None and R:
+                out = torch.empty((R, self.vocab_size), dtype=torch.float32, device=self.rt.device)
+            plan_ptr = ctx.aux.get("program_plan")
+            if ctx.all_single or plan_ptr is not None:
+                stream = _raw_stream(_current_device())
+                capturing = torch.cuda.is_current_stream_capturing()
+                nbytes = max(prog.workspace.numel() if prog.workspace is not None else 0, 32 << 20)
+                while True:
+                    if not capturing:
+                        prog.ensure_workspace(nbytes)
+                    if prog.run(ctx, out, plan_ptr, stream):
+                        self.program_steps += 1
+                        if out is None:
+                            return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.rt.device)
+                        return out
+                    if capturing or "too small" not in getattr(prog, "last_refusal", "") or nbytes >= (32 << 30):
+                        break
+                    nbytes *= 2
+                    self._static.clear()     # captured steps point into the workspace that is about to go
+        if logits_out is not None:
+            return self.model.forward(ctx, logits_out=logits_out)
+        return self.model.forward(ctx)
 
     def release(self, request_id: Hashable) -> None:
         """The request is finished: its pages and state slot go back."""
@@ -140,6 +184,11 @@ class ModelExecutor:
         single = N == S
         n_all = Np if static is not None else N
         order_at, total = total, total + (_pad4(n_all) if single else 0)
+        # a step that the recorded program may run carries its attention plan behind that
+        plan_at = plan_cap = 0
+        if self.program is not None and static is None and N != S and (N, R) not in self.program._refused:
+            plan_at, plan_cap = total, self.program.plan_capacity(N)
+            total += plan_cap
         if self._pinned is None or self._pinned.numel() < total:
             self._pinned = torch.empty(max(total, 4096), dtype=torch.int32,
                                        pin_memory=self.rt.device.type == "cuda")
@@ -176,6 +225,10 @@ class ModelExecutor:
             for gi in range(G):
                 section("slots%d" % gi)[N:] = -1
                 section("tables%d" % gi)[N * widths[gi]:] = 0
+        if plan_cap:
+            used = self.program.write_plan(lens, starts, host_np[plan_at:plan_at + plan_cap], plan_cap)
+            total = plan_at + _pad4(max(used, 1))
+            host = self._pinned[:total]
         # the copy is synchronous: the staging buffer is free again when the next step fills it
         if static is not None:
             static.device_buffer.copy_(host, non_blocking=False)
@@ -202,8 +255,9 @@ class ModelExecutor:
         groups = [GroupView(slots=view("slots%d" % gi),
                             block_tables=view("tables%d" % gi).view(S_all, widths[gi]),
                             page_size=mgr.groups[gi].page_size) for gi in range(G)]
+        aux = {"program_plan": dev.data_ptr() + 4 * plan_at} if plan_cap else {}
         return StepContext(
-            n_tokens=n_all, n_segments=S_all, token_ids=view("token_ids"), positions=view("positions"),
+            aux=aux, n_tokens=n_all, n_segments=S_all, token_ids=view("token_ids"), positions=view("positions"),
             seg_of_token=view("seg_of"), seg_starts=view("seg_starts"), seg_first_pos=view("seg_first"),
             state_slots=view("state_slots"), logit_rows=view("logit_rows"), n_logit_rows=R, groups=groups,
             longest_first=dev[order_at:order_at + n_all] if single else None,
@@ -263,12 +317,12 @@ class ModelExecutor:
         ctx = self._build_context(entries, handles, starts, static=sb)
         if sb.graph is None:
             sb.context = ctx
-            self.model.forward(ctx, logits_out=out)          # kernel by kernel: this step's result, and the warm-up
+            self._forward(ctx, logits_out=out)               # launched one by one: this step's result, and the warm-up
             if self.use_graphs:
                 torch.cuda.current_stream().synchronize()
                 graph = torch.cuda.CUDAGraph()
                 with torch.cuda.graph(graph, pool=self._graph_pool):   # records, runs nothing: ``out`` stays
-                    self.model.forward(ctx, logits_out=out)
+                    self._forward(ctx, logits_out=out)
                 sb.graph = graph
                 if self._graph_pool is None:
                     self._graph_pool = graph.pool()

@@ -58,9 +58,9 @@ def requests_for(cfg, which):
     return {"r%d" % i: random_tokens(min(n, top), V, 100 + i) for i, n in enumerate(lens)}
 
 
-def engine(folder, which, dtype, num_pages):
+def engine(folder, which, dtype, num_pages, **more):
     from lmsf_amd.engine import load_engine_core
-    return load_engine_core(folder, dtype=dtype, block_size=TINY[which][2], num_pages=num_pages, max_num_seqs=8)
+    return load_engine_core(folder, dtype=dtype, block_size=TINY[which][2], num_pages=num_pages, max_num_seqs=8, **more)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -99,9 +99,10 @@ def test_mixed_requests_with_page_reuse(models, which, dtype):
 
 def test_wide_model_leaves_products_unfinished(models, monkeypatch):
     """The wide configuration does reach the kernels that add up partial sums (a step of 40 tokens in
-    bfloat16): twice per layer the norm, once per layer the rotation; a step of 8 tokens reaches neither."""
+    bfloat16): twice per layer the norm, once per layer the rotation; a step of 8 tokens reaches neither. (Run
+    part by part: the recorded program makes the same choices in C++, where this test cannot count them.)"""
     folder, cfg, w = models[("W", "bfloat16")]
-    core = engine(folder, "W", "bfloat16", num_pages=8)
+    core = engine(folder, "W", "bfloat16", num_pages=8, use_program=False)
     ops = core.executor.rt.ops
     seen = {"norm": 0, "rope": 0}
     norm, rope = ops._add_rms_norm_pending, ops._rope_cache_write_pending
@@ -341,3 +342,30 @@ def test_page_count_ignores_memory_that_torch_only_caches(models):
     want = (int(total * 0.5) - (total - free) - act) / groups[0].bytes_per_page(2)
     assert abs(n - want) / want < 0.02, (n, want)
     assert torch.cuda.memory_reserved() - torch.cuda.memory_allocated() < 1 << 30
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("which", ["A", "B", "W"])
+def test_recorded_program_gives_the_bits_of_the_parts(models, which, dtype):
+    """The model's kernel calls recorded once and run from C++ (one call a step) against the same model run
+    part by part from Python: the same kernels with the same arguments, so the logits are equal bit for bit,
+    under portions, mixed steps with page reuse and single tokens."""
+    folder, cfg, w = models[(which, dtype)]
+    from lmsf_amd.engine import load_engine_core
+    reqs = requests_for(cfg, which)
+    longest = -(-max(len(t) for t in reqs.values()) // 64) * 64
+    traces = [trace_portions(reqs, seed=2), trace_mixed(reqs, longest + 128, seed=8), trace_bulk_then_single(reqs)]
+    bs = TINY[which][2]
+    outs = []
+    for use_program in (True, False):
+        core = load_engine_core(folder, dtype=dtype, block_size=bs, num_pages=(longest + 128) // bs, max_num_seqs=8,
+                                use_program=use_program, enforce_eager=True)
+        assert (core.executor.program is not None) == use_program
+        outs.append([replay_in_process(core.executor, steps) for steps in traces])
+        if use_program:
+            assert core.executor.program_steps > 20
+    for a, b in zip(*outs):
+        for rid in reqs:
+            assert torch.equal(a[rid], b[rid]), rid
+    refs = {rid: plain_llama_forward(cfg, w, toks) for rid, toks in reqs.items()}
+    check(outs[0][1], refs, dtype, "recorded program, mixed")
