@@ -4,10 +4,13 @@
 
 A step is one decode step of the whole engine (schedule, batch building, model, sampling) at
 batch 8: requests with 512-token random prompts are prefilled (untimed), W decode steps warm up,
-then exactly K decode steps are timed between device synchronisations. The same line carries the
-prefill of 2,048 tokens, the decode step's share of the HBM roofline, and decode at batch 1 and 64.
-Weights are random (N(0, 0.02), bfloat16, made on the device), token ids are seeded uniform-random.
-The reference publishes no numbers, so vs_baseline is null.
+then exactly K decode steps are timed between device synchronisations; every step is also timed by
+itself with HIP events and the median is reported. The same line carries the prefill of 2,048 tokens,
+the decode step's share of the HBM roofline with the machine's measured rates beside the published
+peaks, and ``points``: decode at batch 1, 64 and 128, at 8,000 tokens of context, a 512-token prompt,
+a mixed step (8 decoding requests beside a 32-token portion of a prompt) and continuous batching of
+64 requests at Llama-2-7B shape. Weights are random (N(0, 0.02), bfloat16, made on the device),
+token ids are seeded uniform-random. The reference publishes no numbers, so vs_baseline is null.
 """
 import argparse
 import json
@@ -81,15 +84,20 @@ def decode_run(engine, batch, prompt_len, steps, warmup, seed):
     for _ in range(warmup):
         engine.step()
     ctx0 = sum(s.length for s in engine.scheduler.running) / batch
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(steps):
+    for a, b in events:
+        a.record()
         outs = engine.step()
+        b.record()
         assert len(outs) == batch
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     for rid in ids:
         engine.abort_request(rid)
+    per_step = sorted(a.elapsed_time(b) for a, b in events)
+    decode_run.median_ms = per_step[len(per_step) // 2]
     return dt, ctx0 + steps / 2.0
 
 
@@ -113,6 +121,43 @@ def prefill_run(engine, n_tokens, reps, seed):
     return times[len(times) // 2]
 
 
+def mixed_step_run(engine, n_decoding, context, portion, reps, seed):
+    """A step of ``n_decoding`` single tokens (requests with ``context`` tokens behind them) beside a
+    ``portion``-token piece of a prompt, through the step function: (median milliseconds from call to
+    synchronised result, median milliseconds on the GPU by events)."""
+    import torch
+    from lmsf_amd.engine import StepEntry
+    rng = random.Random(seed)
+    V = engine.core.config.vocab_size
+    ex = engine.core.executor
+    ids = ["m%d" % i for i in range(n_decoding)]
+    for rid in ids:
+        ex.step([StepEntry(rid, [rng.randrange(V) for _ in range(context)], [])])
+    ex.step([StepEntry("mp", [rng.randrange(V) for _ in range(context)], [])])
+
+    def entries():
+        e = [StepEntry(rid, [rng.randrange(V)], [0]) for rid in ids]
+        e.append(StepEntry("mp", [rng.randrange(V) for _ in range(portion)], [portion - 1]))
+        return e
+    wall, gpu = [], []
+    for r in range(reps + 2):
+        e = entries()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        a.record()
+        ex.step(e)
+        b.record()
+        torch.cuda.synchronize()
+        if r >= 2:
+            wall.append((time.perf_counter() - t0) * 1e3)
+            gpu.append(a.elapsed_time(b))
+    for rid in ids + ["mp"]:
+        ex.release(rid)
+    wall.sort(), gpu.sort()
+    return wall[len(wall) // 2], gpu[len(gpu) // 2]
+
+
 LLAMA2_7B = dict(
     architectures=["LlamaForCausalLM"], model_type="llama", vocab_size=32000, hidden_size=4096,
     intermediate_size=11008, num_hidden_layers=32, num_attention_heads=32, num_key_value_heads=32, head_dim=128,
@@ -134,13 +179,13 @@ SHAPES = {"llama3-8b": ("Llama-3-8B", LLAMA3_8B), "llama2-7b": ("Llama-2-7B", LL
           "llama3.1-70b": ("Llama-3.1-70B", LLAMA31_70B)}
 
 
-def serve_run(args):
+def serve_run(args, emit=True):
     """Continuous batching at Llama-2-7B shape: 64 requests arrive at once, prompts of 128 to 2,048 random
     tokens, 128 generated tokens each, prompts cut into portions that run beside the decoding requests."""
     import torch
     from lmsf_amd.sampling import SamplingParams
     cfg = dict(LLAMA2_7B)
-    if args.layers:
+    if args.layers and emit:
         cfg["num_hidden_layers"] = args.layers
     engine = make_engine(cfg, args, max_num_seqs=64, dtype=args.dtype, prefill_chunk_size=args.prefill_chunk_size)
     rng = random.Random(7)
@@ -174,7 +219,9 @@ def serve_run(args):
                    "total_tok_per_s": round((prompt_tokens + out_tokens) / dt, 1), "seconds": round(dt, 3),
                    "preemptions": engine.stats["preemptions"]},
     }
-    print(json.dumps(line))
+    if emit:
+        print(json.dumps(line))
+    return line
 
 
 def prefill_flops(cfg, T):
@@ -206,7 +253,7 @@ def main():
     ap.add_argument("--prefill-chunk-size", type=int, default=1024, help="serve: longest portion of a prompt in a step")
     ap.add_argument("--shape", default="llama3-8b", choices=sorted(SHAPES),
                     help="decode: the model whose layer sizes are measured (default: the headline configuration)")
-    ap.add_argument("--points", default="1,64", help="decode: further batch sizes, comma separated")
+    ap.add_argument("--points", default="1,64,128", help="decode: further batch sizes, comma separated")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this engine runs on one GPU; --gpus %d is not supported" % args.gpus)
@@ -222,27 +269,55 @@ def main():
     if args.layers:
         cfg["num_hidden_layers"] = args.layers
     point_batches = [] if args.skip_points else [int(x) for x in args.points.split(",") if x]
-    engine = make_engine(cfg, args, max_num_seqs=max([64, args.batch] + point_batches), dtype=args.dtype)
+    max_seqs = max([64, args.batch] + point_batches)
+    engine = make_engine(cfg, args, max_num_seqs=max_seqs, dtype=args.dtype)
     wbytes = weight_bytes(engine)
     kv_per_token = 2 * cfg["num_key_value_heads"] * cfg["head_dim"] * cfg["num_hidden_layers"] * \
         (2 if args.dtype == "bfloat16" else 4)
 
+    measured = engine.core.rt.ops.measure()
+
     dt, mean_ctx = decode_run(engine, args.batch, args.prompt_len, args.steps, args.warmup, seed=1)
     ms_per_step = dt / args.steps * 1e3
+    median_ms = decode_run.median_ms
     value = args.batch * args.steps / dt
     step_bytes = wbytes + args.batch * mean_ctx * kv_per_token
     achieved = step_bytes / (dt / args.steps) / 1e9
 
-    points = {}
+    points = {"decode_b%d_median_ms" % args.batch: round(median_ms, 4)}
     if not args.skip_points:
         for b in point_batches:
             k = max(16, args.steps // 2)
-            d, _ = decode_run(engine, b, args.prompt_len, k, args.warmup, seed=2 + b)
+            d, ctx_b = decode_run(engine, b, args.prompt_len, k, args.warmup, seed=2 + b)
             points["decode_b%d" % b] = round(b * k / d, 1)
+            points["decode_b%d_hbm_frac" % b] = round((wbytes + b * ctx_b * kv_per_token) / (d / k) / HBM_BYTES_PER_S, 4)
+        long_ctx = min(8000, cfg["max_position_embeddings"] - 64)
+        for b in (1, 8):
+            d, ctx_b = decode_run(engine, b, long_ctx, 24, 4, seed=40 + b)
+            points["decode_b%d_ctx%d" % (b, long_ctx)] = round(b * 24 / d, 1)
+            points["decode_b%d_ctx%d_hbm_frac" % (b, long_ctx)] = round(
+                (wbytes + b * ctx_b * kv_per_token) / (d / 24) / HBM_BYTES_PER_S, 4)
+        wall_ms, gpu_ms = mixed_step_run(engine, 8, args.prompt_len, 32, reps=9, seed=5)
+        points["mixed_step_ms"] = round(wall_ms, 3)
+        points["mixed_step_gpu_ms"] = round(gpu_ms, 3)
 
     pt = prefill_run(engine, args.prefill_tokens, reps=5, seed=3)
     pflops = prefill_flops(cfg, args.prefill_tokens)
     peak = PEAK_FLOPS["bf16" if args.dtype == "bfloat16" else "fp32"]
+    if not args.skip_points:
+        p512 = prefill_run(engine, 512, reps=5, seed=4)
+        points["prefill_512_tok_s"] = round(512 / p512, 1)
+        points["prefill_512_frac"] = round(prefill_flops(cfg, 512) / p512 / peak, 4)
+        if args.shape == "llama3-8b" and args.dtype == "bfloat16":
+            # continuous batching at Llama-2-7B shape needs the memory: the first engine goes
+            del engine
+            import gc
+            gc.collect()
+            torch.cuda.empty_cache()
+            serve = serve_run(args, emit=False)
+            points["serve_tok_s"] = serve["value"]
+            points["serve_total_tok_s"] = serve["config"]["total_tok_per_s"]
+            points["serve_ms_per_step"] = serve["ms_per_step"]
 
     line = {
         "metric": "decode tok/s at batch %d (%s %s)" % (args.batch, shape_name, "bf16" if args.dtype == "bfloat16" else "fp32"),
@@ -261,7 +336,11 @@ def main():
         "prefill": {"value": round(args.prefill_tokens / pt, 1), "tokens": args.prefill_tokens,
                     "ms": round(pt * 1e3, 3), "frac": round(pflops / pt / peak, 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_BYTES_PER_S / 1e9, "unit": "GB/s",
-                     "frac": round(achieved / (HBM_BYTES_PER_S / 1e9), 4)},
+                     "frac": round(achieved / (HBM_BYTES_PER_S / 1e9), 4),
+                     "measured_read_GBps": round(measured["read_GBps"], 1),
+                     "measured_copy_GBps": round(measured["copy_GBps"], 1),
+                     "measured_mfma_bf16_TFLOPs": round(measured["mfma_bf16_TFLOPs"], 1),
+                     "nominal_mfma_bf16_TFLOPs": PEAK_FLOPS["bf16"] / 1e12},
         "points": points,
     }
     print(json.dumps(line))

@@ -755,6 +755,43 @@ class HipOps:
                                                   _ptr(repetition), self._stream()))
 
 
+    # ------------------------------------------------------------------ what the machine gives
+
+    def measure(self, nbytes: int = 4 << 30, reps: int = 5) -> dict:
+        """Measured rates of this GPU: reading and copying ``nbytes`` of device memory with plain kernels (GB/s,
+        a copy counted as bytes read plus bytes written) and the bfloat16 matrix-core instruction in a loop
+        without memory traffic (TFLOP/s). The best of ``reps`` runs each, timed with events."""
+        dev = torch.device("cuda", _current_device())
+        src = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+        src.random_(0, 255)
+        dst = torch.empty_like(src)
+        sink = torch.zeros(64, dtype=torch.float32, device=dev)
+
+        def timed(launch):
+            best = None
+            for _ in range(reps + 1):
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+                launch()
+                b.record()
+                b.synchronize()
+                ms = a.elapsed_time(b)
+                best = ms if best is None else min(best, ms)
+            return best * 1e-3
+
+        t_read = timed(lambda: self._check(self.lib.lmsf_measure_read(_ptr(src), nbytes, _ptr(sink), self._stream())))
+        t_copy = timed(lambda: self._check(self.lib.lmsf_measure_copy(_ptr(src), _ptr(dst), nbytes, self._stream())))
+        flops = [0.0]
+
+        def mfma():
+            flops[0] = self.lib.lmsf_measure_mfma(_ptr(sink), 4096, 256 * 8, self._stream())
+            if flops[0] == 0.0:
+                self._check(1)
+        t_mfma = timed(mfma)
+        return {"read_GBps": nbytes / t_read / 1e9, "copy_GBps": 2 * nbytes / t_copy / 1e9,
+                "mfma_bf16_TFLOPs": flops[0] / t_mfma / 1e12}
+
+
 class _AttentionPlan:
     __slots__ = ("tiles", "n_tiles", "single_tokens", "n_single", "max_context")
 

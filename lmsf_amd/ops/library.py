@@ -4,12 +4,12 @@ There is no fallback: if the library cannot be built or loaded, or reports anoth
 version, importing the kernels fails with the reason.
 """
 import ctypes
-from ctypes import c_char_p, c_float, c_int, c_long, c_void_p
+from ctypes import c_char_p, c_double, c_float, c_int, c_long, c_void_p
 from typing import Optional
 
 from ..csrc import build as _build
 
-ABI_VERSION = 19
+ABI_VERSION = 20
 
 _lib: Optional[ctypes.CDLL] = None
 _lib_path: Optional[str] = None
@@ -71,6 +71,9 @@ _SIGNATURES = {
     "lmsf_sample": (c_int, [_P, c_long, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, _P, _P]),
     "lmsf_sample_scratch_elems": (c_long, [c_int, c_int]),
     "lmsf_greedy_tokens_static": (c_int, [_P, c_long, c_int, c_int, _P, _P]),
+    "lmsf_measure_read": (c_int, [_P, c_long, _P, _P]),
+    "lmsf_measure_copy": (c_int, [_P, _P, c_long, _P]),
+    "lmsf_measure_mfma": (c_double, [_P, c_int, c_int, _P]),
     "lmsf_apply_penalties": (c_int, [_P, c_long, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, _P]),
 }
 

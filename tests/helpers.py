@@ -40,12 +40,12 @@ TINY_W = dict(
 TINY = {"A": (TINY_A, 0, 8), "B": (TINY_B, 1, 16), "C": (TINY_C, 2, 16), "W": (TINY_W, 3, 16)}   # config, seed, block size
 
 
-def make_model_folder(tmp_path, which, dtype="float32", seed=None):
+def make_model_folder(tmp_path, which, dtype="float32", seed=None, std=0.02):
     """Write config.json + model.safetensors of a tiny configuration; returns (folder, config)."""
     cfg_dict, default_seed, _ = TINY[which]
     cfg = LlamaConfig.from_dict(dict(cfg_dict, torch_dtype=dtype))
-    folder = os.path.join(str(tmp_path), "tiny_%s_%s" % (which, dtype))
-    write_random_model(folder, cfg, seed=default_seed if seed is None else seed, dtype=dtype)
+    folder = os.path.join(str(tmp_path), "tiny_%s_%s%s" % (which, dtype, "" if std == 0.02 else "_std%g" % std))
+    write_random_model(folder, cfg, seed=default_seed if seed is None else seed, dtype=dtype, std=std)
     return folder, cfg
 
 

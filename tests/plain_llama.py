@@ -241,7 +241,7 @@ def plain_llama_layer(cfg, w, prefix, stream, positions, inv_freq, window=None, 
     return stream + m, (k, v)
 
 
-def plain_llama_forward(cfg, w, token_ids, start_position=0, schedule=None, windows=None):
+def plain_llama_forward(cfg, w, token_ids, start_position=0, schedule=None, windows=None, last=None):
     """Logits [T, V] (float32) for every position of one whole sequence.
 
     core/src/model_executor/models/llama/llama.rs:397-476: embedding, the blocks in order,
@@ -254,6 +254,7 @@ def plain_llama_forward(cfg, w, token_ids, start_position=0, schedule=None, wind
     ``schedule`` is a list of (layer index, index of the earlier schedule entry whose keys and
     values are read, or None); default: every layer once, in order.
     ``windows`` maps a layer index to a sliding window length.
+    ``last``: only the logits of the last ``last`` positions (the head is the costly part of a wide model).
     """
     d = plain_head_dim(cfg)
     inv_freq = plain_rope_inv_freq(d, cfg.get("rope_theta", 10000.0), cfg.get("rope_scaling"))
@@ -269,6 +270,8 @@ def plain_llama_forward(cfg, w, token_ids, start_position=0, schedule=None, wind
                                        inv_freq, window=window,
                                        kv_from=None if src is None else kvs[src])
         kvs.append(kv)
+    if last is not None:
+        stream = stream[-last:]
     final = plain_rms_norm(stream, w["model.norm.weight"], cfg["rms_norm_eps"])
     head = w["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings", False) else w["lm_head.weight"]
     return plain_linear(final, head)

@@ -8,13 +8,20 @@ import os
 import pytest
 import torch
 
-from helpers import random_tokens, replay_in_process, trace_mixed, trace_whole
+from helpers import (random_tokens, replay_in_process, trace_bulk_then_single, trace_mixed, trace_portions,
+                     trace_whole)
 from lmsf_amd.config import LlamaConfig
 from lmsf_amd.weights import write_random_model
 from plain_llama import plain_llama_forward, read_model_folder
 from test_replay_gpu import check
 
 pytestmark = pytest.mark.gpu
+
+# At a width of 4,096 the usual N(0, 0.02) weights give the attention scores a spread of 0.02^2 * 4096 = 1.6:
+# attention is peaked in both layers, and the rounding of bfloat16 activations costs 1.2 % of the largest logit on
+# average and 1.7 % at most over these requests, the same for whole prompts as for every other way of cutting
+# (measured; the largest of 128,256 logits' errors). The bound leaves that half as much room again.
+BOUND = 2.5e-2
 
 FULL = dict(
     architectures=["LlamaForCausalLM"], model_type="llama", vocab_size=128256, hidden_size=4096,
@@ -42,12 +49,12 @@ def test_llama3_8b_layer_sizes_every_product_path(full_model):
             "d": random_tokens(9, V, 4)}
     refs = {rid: plain_llama_forward(cfg, w, toks) for rid, toks in reqs.items()}
     core = load_engine_core(folder, dtype="bfloat16", block_size=16, num_pages=24, max_num_seqs=8)
-    check(replay_in_process(core.executor, trace_whole(reqs)), refs, "bfloat16", "whole")
+    check(replay_in_process(core.executor, trace_whole(reqs)), refs, "bfloat16", "whole", BOUND)
     steps = trace_mixed(reqs, 24 * 16, seed=3)
     sizes = {len(e["tokens"]) for s in steps for e in s["entries"]}
     rows = {sum(len(e["tokens"]) for e in s["entries"]) for s in steps}
     assert 1 in sizes and any(17 <= r <= 64 for r in rows) and any(r <= 16 for r in rows)
-    check(replay_in_process(core.executor, steps), refs, "bfloat16", "mixed")
+    check(replay_in_process(core.executor, steps), refs, "bfloat16", "mixed", BOUND)
     core.storage.manager.check_invariants()
     assert core.storage.manager.num_free_pages(0) == 24
     # greedy tokens of the engine's sampler against the plain logits (ties aside: random weights have none)
@@ -67,3 +74,52 @@ def test_llama3_8b_layer_sizes_in_true_float32(full_model):
     steps = [{"step": i, "entries": [{"id": "x", "tokens": p, "want": list(range(len(p)))}],
               "end": ["x"] if i == len(parts) - 1 else []} for i, p in enumerate(parts)]
     check(replay_in_process(core.executor, steps), {"x": ref}, "float32", "float32 at full layer sizes")
+
+
+def test_llama3_8b_layer_sizes_bulk_then_single_and_portions(full_model):
+    """The other two ways of cutting at these sizes: most of a request in one step and its last 32 tokens one by
+    one (the one-row products with their fused norm, residual and rotary forms), and portions of changing size."""
+    from lmsf_amd.engine import load_engine_core
+    folder, cfg, w = full_model
+    V = cfg["vocab_size"]
+    reqs = {"a": random_tokens(90, V, 21), "b": random_tokens(37, V, 22)}
+    refs = {rid: plain_llama_forward(cfg, w, toks) for rid, toks in reqs.items()}
+    core = load_engine_core(folder, dtype="bfloat16", block_size=16, num_pages=8, max_num_seqs=4)
+    check(replay_in_process(core.executor, trace_bulk_then_single(reqs)), refs, "bfloat16", "bulk then single", BOUND)
+    check(replay_in_process(core.executor, trace_portions(reqs, seed=5)), refs, "bfloat16", "portions", BOUND)
+    assert core.executor.program is not None and core.executor.program_steps > 8
+    core.storage.manager.check_invariants()
+
+
+def test_llama3_8b_layer_sizes_decode_steps_of_24_40_and_64_requests(full_model):
+    """Steps of single tokens of 24, 40 and 64 requests of unequal contexts at these sizes, each kind once
+    launched kernel by kernel and captured, then replayed: the 17-and-more-rows products left as partial sums, the
+    rotary kernel that adds them up, the attention over the cache with the longest contexts first."""
+    from lmsf_amd.engine import StepEntry, load_engine_core
+    folder, cfg, w = full_model
+    V = cfg["vocab_size"]
+    lens = [9 + (61 * i + 3 * i * i) % 109 for i in range(64)]
+    assert len(set(lens)) > 30
+    reqs = {i: random_tokens(n, V, 500 + i) for i, n in enumerate(lens)}
+    tail = 4
+    refs = {i: plain_llama_forward(cfg, w, toks, last=tail) for i, toks in reqs.items()}
+    core = load_engine_core(folder, dtype="bfloat16", block_size=16, num_pages=sum(-(-n // 16) for n in lens) + 2,
+                            max_num_seqs=64)
+    ex = core.executor
+    for i, toks in reqs.items():
+        ex.step([StepEntry(i, toks[:-tail], [])])
+    got = {i: [] for i in reqs}
+
+    def decode(ids, k):
+        out = ex.step([StepEntry(i, [reqs[i][len(reqs[i]) - tail + k]], [0]) for i in ids]).float().cpu()
+        for row, i in zip(out, ids):
+            got[i].append(row)
+
+    first, rest = list(range(24)), list(range(24, 64))
+    decode(first, 0), decode(rest, 0)            # launched one by one, then captured
+    decode(first, 1), decode(rest, 1)            # replayed
+    decode(first + rest, 2)                      # 64: launched and captured
+    decode(rest + first, 3)                      # replayed, in another order
+    kinds = {b for (b, _bucket) in ex._static}
+    assert {24, 40, 64} <= kinds and all(sb.graph is not None for sb in ex._static.values())
+    check({i: torch.stack(rows) for i, rows in got.items()}, refs, "bfloat16", "decode steps of 24, 40 and 64", BOUND)

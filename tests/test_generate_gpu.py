@@ -91,6 +91,41 @@ def test_temperature_sampling_seeded(tmp_path):
     assert c != a
 
 
+def test_baseline_configuration_two_sampled_tokens_follow_the_plain_logits(tmp_path):
+    """Tiny B in float32, six prompts of 3 to 300 tokens cut into portions of 64 beside the requests that already
+    decode, 24 tokens each at temperature 0.7 with seeds: every sampled token is the argmax of the *plain*
+    logits of the engine's own prefix, divided by the temperature, plus the noise of (seed, number of the draw,
+    vocabulary index)."""
+    import numpy as np
+    from torch_ops import gumbel_noise
+    from lmsf_amd.engine import EngineArgs, LLMEngine
+    from lmsf_amd.sampling import SamplingParams
+    folder, cfg = make_model_folder(tmp_path, "B")
+    cfg_dict, w = read_model_folder(folder)
+    V = cfg.vocab_size
+    prompts = [random_tokens(n, V, 800 + n) for n in (3, 17, 64, 120, 211, 300)]
+    engine = LLMEngine(EngineArgs(model=folder, dtype="float32", block_size=16, num_gpu_blocks_override=128,
+                                  max_num_seqs=8, prefill_chunk_size=64, max_num_batched_tokens=96))
+    for i, p in enumerate(prompts):
+        engine.add_request(i, p, SamplingParams(temperature=0.7, max_tokens=24, ignore_eos=True, seed=900 + i))
+    done, mixed_steps = {}, 0
+    while engine.has_unfinished_requests():
+        for out in engine.step():
+            if out.finished:
+                done[out.request_id] = out.outputs[0].token_ids
+        last = engine.last_step
+        mixed_steps += 1 if last["prefill_tokens"] and last["decode_tokens"] else 0
+    assert mixed_steps >= 3, "portions of prompts were meant to run beside decoding requests"
+    inv_t = np.float32(1.0) / np.float32(0.7)
+    for i, p in enumerate(prompts):
+        gen = done[i]
+        assert len(gen) == 24
+        logits = plain_llama_forward(cfg_dict, w, p + gen[:-1])[len(p) - 1:]
+        for k, tok in enumerate(gen):
+            y = logits[k] * float(inv_t) + gumbel_noise(900 + i, k, V)
+            assert int(torch.argmax(y)) == tok or float(y.max() - y[tok]) < 1e-4, (i, k)
+
+
 def test_command_line(tmp_path):
     folder, cfg = make_model_folder(tmp_path, "A")
     cfg_dict, w = read_model_folder(folder)

@@ -17,19 +17,21 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 TRACE_RUN = os.path.join(ROOT, "bin", "trace_run")
 
 
-def tolerance(dtype, ref):
+def tolerance(dtype, ref, bf16_bound=1.5e-2):
     """float32: rounding of sums of a few hundred terms. bfloat16: activations are rounded to 8 bits of
-    mantissa between kernels, a few times per layer; the bound is relative to the largest logit."""
+    mantissa between kernels, a few times per layer; the bound is relative to the largest logit. What the
+    rounding costs grows with the spread of the attention scores (std^2 * width of the weights): with the tiny
+    configurations' N(0, 0.02) it is 0.3 % of the largest logit."""
     scale = ref.abs().max().item()
-    return 3e-5 * max(1.0, scale) if dtype == "float32" else 4e-2 * max(0.25, scale)
+    return 3e-5 * max(1.0, scale) if dtype == "float32" else bf16_bound * max(0.25, scale)
 
 
-def check(got, refs, dtype, what):
+def check(got, refs, dtype, what, bf16_bound=1.5e-2):
     for rid, ref in refs.items():
         assert rid in got, (what, rid)
         assert got[rid].shape == ref.shape, (what, rid, got[rid].shape, ref.shape)
         err = (got[rid] - ref).abs()
-        t = tolerance(dtype, ref)
+        t = tolerance(dtype, ref, bf16_bound)
         if err.max().item() > t:
             pos = int(torch.nonzero(err.max(dim=1).values > t)[0])
             raise AssertionError("%s: request %r first differs at position %d (page offset %d): max err %.3g > %.3g"
@@ -369,3 +371,27 @@ def test_recorded_program_gives_the_bits_of_the_parts(models, which, dtype):
             assert torch.equal(a[rid], b[rid]), rid
     refs = {rid: plain_llama_forward(cfg, w, toks) for rid, toks in reqs.items()}
     check(outs[0][1], refs, dtype, "recorded program, mixed")
+
+
+@pytest.mark.parametrize("which", ["A", "B", "C", "W"])
+def test_bfloat16_with_peaked_attention_in_every_layer(tmp_path, which):
+    """Weights several times larger than the usual N(0, 0.02): the scores of every layer get a spread (their
+    standard deviation is about std^2 * width, here 0.4) and every query leans on some keys more than on others.
+    Measured at these sizes: changing one far token of a prompt then moves the last position's logits by 8 to
+    30 % of the largest logit, while bfloat16 rounding costs under 1 % (it grows with the same spread: 2 to 4 %
+    at a spread of 2.5, which is why the weights are not larger still). So a key read from a wrong page or slot,
+    in any layer, is an order of magnitude beyond the bound. All four ways of cutting."""
+    import math
+    width = TINY[which][0]["hidden_size"]
+    folder, cfg_obj = make_model_folder(tmp_path, which, dtype="bfloat16", std=math.sqrt(0.4 / width))
+    cfg, w = read_model_folder(folder)
+    reqs = requests_for(cfg, which)
+    refs = {rid: plain_llama_forward(cfg, w, toks) for rid, toks in reqs.items()}
+    longest = -(-max(len(t) for t in reqs.values()) // 64) * 64
+    bs = TINY[which][2]
+    core = engine(folder, which, "bfloat16", num_pages=(longest + 128) // bs)
+    check(replay_in_process(core.executor, trace_whole(reqs)), refs, "bfloat16", "peaked, whole")
+    check(replay_in_process(core.executor, trace_bulk_then_single(reqs)), refs, "bfloat16", "peaked, bulk then single")
+    check(replay_in_process(core.executor, trace_portions(reqs, seed=3)), refs, "bfloat16", "peaked, portions")
+    check(replay_in_process(core.executor, trace_mixed(reqs, longest + 128, seed=6)), refs, "bfloat16", "peaked, mixed")
+    core.storage.manager.check_invariants()
