@@ -31,6 +31,12 @@ int lmsf_embedding(const int* ids, const void* table, int table_dtype, float* ou
 int lmsf_gated_act(const void* in, void* out, int dtype, int n_tokens, int I, long in_stride, int kind, hipStream_t
     stream);
 
+// gemm_large.hip
+int lmsf_gemm_large_plan(int M, int N, int K, int act);
+long lmsf_gemm_large_scratch_floats(int M, int N, int n_split);
+int lmsf_gemm_large(const void* x, long ldx, const void* W, long ldw, const void* bias, void* y, long ldy, int M, int
+    N, int K, int act, int plan, float* scratch, int reduce, hipStream_t stream);
+
 // gemm_mid.hip
 int lmsf_gemm_mid_splits(int M, int N, int K, int act);
 long lmsf_gemm_mid_scratch_floats(int M, int N, int n_split, int act);
@@ -79,6 +85,11 @@ int lmsf_gemv_scaled_qkv_rope_cache(const void* x, long ldx, const void* W, long
     ldy, int M, int K, const int* positions, const float* table, int max_pos, const int* slots, void* k_pages, void*
     v_pages, long num_pages, int nh, int nkv, int d, int ps, const float* sumsq, int n_partials, float eps,
     hipStream_t stream);
+
+// measure.hip
+int lmsf_measure_read(const void* src, long bytes, void* sink, hipStream_t stream);
+int lmsf_measure_copy(const void* src, void* dst, long bytes, hipStream_t stream);
+double lmsf_measure_mfma(void* sink, int iters, int blocks, hipStream_t stream);
 
 // norm.hip
 int lmsf_add_rms_norm(const void* branch, int branch_dtype, float* residual, const void* weight, int weight_dtype,

@@ -211,6 +211,41 @@ int linear_mid(Run& r, const Value& x, const void* W, long ldw, int w_rows, cons
   return 0;
 }
 
+// HipOps._linear_large
+int linear_large(Run& r, const Value& x, const void* W, long ldw, int w_rows, const void* bias, int act, bool pending_ok,
+                 void* out, Value* res) {
+  const int M = x.M, K = x.N;
+  const int N = act ? w_rows / 2 : w_rows;
+  const int plan = lmsf_gemm_large_plan(M, N, K, act);
+  const int splits = plan % 16;
+  float* scratch = nullptr;
+  if (splits > 1) {
+    TAKE(s, float*, (size_t)splits * M * N * 4);
+    scratch = s;
+    if (pending_ok) {
+      LAUNCH(lmsf_gemm_large(x.p, x.ld, W, ldw, nullptr, nullptr, 0, M, N, K, 0, plan, scratch, 0, r.stream));
+      Value v;
+      v.kind = V_PENDING;
+      v.partials = scratch;
+      v.n_split = splits;
+      v.bias = bias;
+      v.dtype = LMSF_BF16;
+      v.M = M;
+      v.N = N;
+      *res = v;
+      return 0;
+    }
+  }
+  void* y = out;
+  if (y == nullptr) {
+    TAKE(yy, void*, (size_t)M * N * 2);
+    y = yy;
+  }
+  LAUNCH(lmsf_gemm_large(x.p, x.ld, W, ldw, bias, y, N, M, N, K, act, plan, scratch, 1, r.stream));
+  *res = tensor(y, LMSF_BF16, M, N);
+  return 0;
+}
+
 // HipOps.linear
 int op_linear(Run& r, const Value& x, const void* W, int wdtype, long ldw, int N, const void* bias, int out_dtype,
               bool pending_ok, void* out, Value* res) {
@@ -225,6 +260,8 @@ int op_linear(Run& r, const Value& x, const void* W, int wdtype, long ldw, int N
   if (both_bf16 && t.skinny_max_rows < M && M <= t.mid_max_rows && m_ok &&
       (M <= 64 || N <= t.mid_wide_max_cols || out_dtype == LMSF_F32))
     return linear_mid(r, x, W, ldw, N, bias, 0, out_dtype, pending_ok && out_dtype == LMSF_BF16, out, res);
+  if (both_bf16 && out_dtype == LMSF_BF16 && t.mid_max_rows < M && M <= t.large_max_rows && m_ok)
+    return linear_large(r, x, W, ldw, N, bias, 0, pending_ok, out, res);
   if (pending_ok && both_bf16 && out_dtype == LMSF_BF16 && s_ok && M > 0) {
     if ((M <= std::min(t.fuse_stream_rows, t.gemv_max_rows) && gemv_ok(M, K)) ||
         M <= std::min(std::min(t.fuse_norm_rows, t.skinny_max_rows), 16)) {
@@ -464,6 +501,8 @@ int op_linear_gated(Run& r, const Value& x_in, const void* W, int wdtype, long l
   }
   if (both_bf16 && t.skinny_max_rows < M && M <= 64 && mid_ok(x.p, x.ld, K, W, ldw, w_rows))
     return linear_mid(r, x, W, ldw, w_rows, bias, kind, LMSF_BF16, false, nullptr, res);
+  if (both_bf16 && 64 < M && M <= t.large_max_rows && mid_ok(x.p, x.ld, K, W, ldw, w_rows))
+    return linear_large(r, x, W, ldw, w_rows, bias, kind, false, nullptr, res);
   Value gu;
   RC(op_linear(r, x, W, wdtype, ldw, w_rows, bias, x.dtype, false, nullptr, &gu));
   TAKE(y, void*, (size_t)M * I * esize(gu.dtype));

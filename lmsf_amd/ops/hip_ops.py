@@ -68,6 +68,7 @@ class HipOps:
         self.mid_wide_max_cols = 8192  # beyond 64 rows only products of up to this many columns: the library is good at the wide ones (measured)
         self.mid_max_rows = 128        # rows up to which the 17-and-more-rows kernel beats the library (64 with the gated activation)
         self.skinny_max_rows = 16      # rows up to which the few-rows kernel beats the library (measured)
+        self.large_max_rows = 256      # rows up to which the many-rows kernel beats the library (measured; 0: never)
 
     # ------------------------------------------------------------------ helpers
 
@@ -565,6 +566,10 @@ class HipOps:
         if (both_bf16 and self.skinny_max_rows < M <= self.mid_max_rows and self._mid_ok(x, weight)
                 and (M <= 64 or N <= self.mid_wide_max_cols or out_dtype == torch.float32)):
             return self._linear_mid(x, weight, bias, 0, out_dtype, pending_ok and out_dtype == torch.bfloat16, out=out)
+        if (both_bf16 and out_dtype == torch.bfloat16 and self.mid_max_rows < M <= self.large_max_rows
+                and self._mid_ok(x, weight)):
+            # 129 to 256 rows: the library is weak there (0.12 to 0.5 PFLOP/s at these widths)
+            return self._linear_large(x, weight, bias, 0, pending_ok, out=out)
         if pending_ok and both_bf16 and out_dtype == torch.bfloat16 and self._skinny_ok(x, weight) and M > 0:
             if (M <= min(self.fuse_stream_rows, self.gemv_max_rows) and self._gemv_ok(M, K)) \
                     or M <= min(self.fuse_norm_rows, self.skinny_max_rows, 16):
@@ -659,6 +664,9 @@ class HipOps:
         if (x.dim() == 2 and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
                 and self.skinny_max_rows < M <= 64 and x.shape[1] == weight.shape[1] and self._mid_ok(x, weight)):
             return self._linear_mid(x, weight, bias, kinds[kind])
+        if (x.dim() == 2 and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
+                and 64 < M <= self.large_max_rows and x.shape[1] == weight.shape[1] and self._mid_ok(x, weight)):
+            return self._linear_large(x, weight, bias, kinds[kind])
         return self.gated_act(self.linear(x, weight, bias), kind)
 
     @staticmethod
@@ -691,6 +699,30 @@ class HipOps:
         self._check(self.lib.lmsf_gemm_mid(_ptr(x), x.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(y),
                                            _code(out_dtype), y.stride(0), M, N, K, act, splits, _ptr(scratch),
                                            self._stream()))
+        return y
+
+    def _linear_large(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], act: int,
+                      pending_ok: bool = False, out: Optional[torch.Tensor] = None, plan: Optional[int] = None):
+        """The many-rows product (csrc/gemm_large.hip); operands as ``_mid_ok`` asks them."""
+        self._dev(x, weight, bias)
+        M, K = x.shape
+        N = weight.shape[0] // 2 if act else weight.shape[0]
+        if bias is not None and (bias.shape != (weight.shape[0],) or bias.dtype != weight.dtype
+                                 or not bias.is_contiguous()):
+            raise ValueError("linear: bias must be [%d] of the weight's dtype" % weight.shape[0])
+        if plan is None:
+            plan = self.lib.lmsf_gemm_large_plan(M, N, K, act)
+        splits = plan % 16
+        scratch = None
+        if splits > 1:
+            scratch = torch.empty((splits, M, N), dtype=torch.float32, device=x.device)
+            if pending_ok:
+                self._check(self.lib.lmsf_gemm_large(_ptr(x), x.stride(0), _ptr(weight), weight.stride(0), None, None, 0,
+                                                     M, N, K, 0, plan, _ptr(scratch), 0, self._stream()))
+                return PendingProduct(scratch, bias, torch.bfloat16)
+        y = out if out is not None else torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+        self._check(self.lib.lmsf_gemm_large(_ptr(x), x.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(y),
+                                             y.stride(0), M, N, K, act, plan, _ptr(scratch), 1, self._stream()))
         return y
 
     @staticmethod

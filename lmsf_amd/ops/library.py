@@ -64,6 +64,9 @@ _SIGNATURES = {
     "lmsf_gemm_mid": (c_int, [_P, c_long, _P, c_long, _P, _P, c_int, c_long, c_int, c_int, c_int, c_int, c_int, _P, _P]),
     "lmsf_gemm_mid_partial": (c_int, [_P, c_long, _P, c_long, c_int, c_int, c_int, c_int, _P, _P]),
     "lmsf_gemm_mid_reduce": (c_int, [_P, _P, _P, c_int, c_long, c_int, c_int, c_int, _P]),
+    "lmsf_gemm_large_plan": (c_int, [c_int, c_int, c_int, c_int]),
+    "lmsf_gemm_large_scratch_floats": (c_long, [c_int, c_int, c_int]),
+    "lmsf_gemm_large": (c_int, [_P, c_long, _P, c_long, _P, _P, c_long, c_int, c_int, c_int, c_int, c_int, _P, c_int, _P]),
     "lmsf_add_rms_norm_partial": (c_int, [_P, _P, c_int, c_int, _P, _P, c_int, _P, c_int, _P, c_int, c_int, c_float,
                                           c_float, _P]),
     "lmsf_rope_cache_write_partial": (c_int, [_P, _P, c_int, _P, c_long, c_int, _P, _P, c_int, c_int, c_int, _P, _P, _P,

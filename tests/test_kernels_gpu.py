@@ -396,7 +396,8 @@ def test_linear_float32_is_exact_float32(ops, M, N, K, bias):
 @pytest.mark.parametrize("M,N,K", [(1, 1000, 128), (7, 331, 80), (64, 640, 352), (65, 512, 176), (300, 1024, 512),
                                    (17, 328, 128), (33, 4096, 4096), (64, 6144, 4096), (48, 1000, 14336), (64, 4096, 1024),
                                    (65, 4096, 4096), (96, 1000, 14336), (97, 328, 128), (128, 6144, 4096), (127, 4096, 1024),
-                                   (200, 1000, 1024)])
+                                   (200, 1000, 1024), (129, 4096, 4096), (130, 328, 192), (192, 6144, 4096),
+                                   (256, 4096, 14336), (255, 1000, 128), (300, 6144, 4096), (2048, 1000, 1024)])
 @pytest.mark.parametrize("bias", [False, True])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
 def test_linear_bfloat16(ops, ref, M, N, K, bias, out_dtype):
@@ -412,7 +413,8 @@ def test_linear_bfloat16(ops, ref, M, N, K, bias, out_dtype):
 
 
 @pytest.mark.parametrize("M,I,K", [(1, 176, 64), (8, 14336, 4096), (16, 208, 80), (13, 1000, 328), (40, 352, 128),
-                                   (64, 14336, 4096), (20, 1000, 1024)])
+                                   (64, 14336, 4096), (20, 1000, 1024), (65, 14336, 4096), (100, 1000, 1024),
+                                   (129, 352, 128), (200, 14336, 4096), (256, 1000, 192), (300, 1000, 1024)])
 @pytest.mark.parametrize("kind", ["silu", "gelu"])
 @pytest.mark.parametrize("bias", [False, True])
 def test_linear_gated(ops, ref, M, I, K, kind, bias):
@@ -688,6 +690,45 @@ def test_split_heuristic_counts_the_gated_forms_extra_kernel(ops):
         assert ops.lib.lmsf_gemm_mid_splits(M, 14336, 4096, 1) == 1
         assert ops.lib.lmsf_gemm_mid_splits(M, 4096, 4096, 0) >= 4
         assert ops.lib.lmsf_gemm_mid_splits(M, 4096, 14336, 0) >= 4
+
+
+@pytest.mark.parametrize("M,N,K", [(129, 4096, 4096), (192, 4096, 14336), (256, 6144, 4096), (150, 328, 192),
+                                   (256, 136, 64), (65, 1000, 1024)])
+def test_linear_many_rows_every_tiling_and_split(ops, ref, M, N, K):
+    """The many-rows product (csrc/gemm_large.hip) with each of its tilings, in one piece and with K split into
+    parts whose float32 partial sums are added up by the reduction kernel or stay for the norm that follows: all
+    against the float32 product, and a split product against the unsplit one of the same tiling."""
+    from lmsf_amd.ops.handles import PendingProduct
+    g = torch.Generator().manual_seed(M + N + K)
+    x = dev(torch.randn(M, K, generator=g).to(torch.bfloat16))
+    w = dev((torch.randn(N, K, generator=g) * K ** -0.5).to(torch.bfloat16))
+    b = dev(torch.randn(N, generator=g).to(torch.bfloat16))
+    want = ref.linear(x, w, b, out_dtype=torch.float32)
+    scale = want.abs().max().item()
+    for tiling in (0, 1, 2):
+        whole = ops._linear_large(x, w, b, 0, plan=tiling * 16 + 1)
+        assert (whole.float() - want).abs().max().item() <= 1e-2 * scale, tiling
+        for parts in (2, 3, 8):
+            if parts > K // 64:
+                continue
+            got = ops._linear_large(x, w, b, 0, plan=tiling * 16 + parts)
+            assert (got.float() - whole.float()).abs().max().item() <= 1e-2 * scale, (tiling, parts)
+            pending = ops._linear_large(x, w, b, 0, pending_ok=True, plan=tiling * 16 + parts)
+            assert isinstance(pending, PendingProduct) and pending.partials.shape == (parts, M, N)
+            assert torch.equal(ops.materialize(pending), got)
+    plan = ops.lib.lmsf_gemm_large_plan(M, N, K, 0)
+    assert 0 <= plan // 16 <= 2 and 1 <= plan % 16 <= 8
+    # what the engine calls: the same numbers through linear, and as the branch of a norm
+    y = ops.linear(x, w, b)
+    assert (y.float() - want).abs().max().item() <= 1e-2 * scale
+    if M > ops.mid_max_rows:
+        res = dev(torch.randn(M, N, generator=g))
+        nw = dev(torch.randn(N, generator=g).to(torch.bfloat16))
+        p = ops.linear(x, w, b, pending_ok=True)
+        r1, r2 = res.clone(), res.clone()
+        a = ops.add_rms_norm(p, r1, nw, 1e-5, torch.bfloat16)
+        c = ops.add_rms_norm(y, r2, nw, 1e-5, torch.bfloat16)
+        assert torch.equal(a, c) and torch.equal(r1, r2)
 
 
 def test_linear_mixed_storage(ops, ref):
