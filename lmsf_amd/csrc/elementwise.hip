@@ -39,6 +39,26 @@ extern "C" int lmsf_embedding(const int* ids, const void* table, int table_dtype
   return 0;
 }
 
+// ---------------------------------------------------------------- token ids from the step before
+// ids[i] = prev[src[i]] where src[i] >= 0: a step that is launched before the host has read the tokens that the
+// step before it sampled takes them from where the sampler left them on the device.
+__global__ __launch_bounds__(256) void patch_tokens_kernel(int* __restrict__ ids, const int* __restrict__ src,
+                                                           const int* __restrict__ prev, int n, int n_prev) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  const int s = src[i];
+  if (s >= 0 && s < n_prev) ids[i] = prev[s];
+}
+
+extern "C" int lmsf_patch_tokens(int* ids, const int* src, const int* prev, int n, int n_prev, hipStream_t stream) {
+  LMSF_CHECK(ids && src && prev, "patch_tokens: null pointer");
+  LMSF_CHECK(n >= 0 && n_prev >= 0, "patch_tokens: bad sizes n=%d n_prev=%d", n, n_prev);
+  if (n == 0) return 0;
+  hipLaunchKernelGGL(patch_tokens_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, ids, src, prev, n, n_prev);
+  LMSF_LAUNCH_CHECK("patch_tokens");
+  return 0;
+}
+
 // ---------------------------------------------------------------- gated activation
 // out[t, i] = act(in[t, i]) * in[t, I + i], act computed in float32.
 // kind 0: silu(x) = x / (1 + exp(-x))   (vllm/kernels/activation_kernels.cu:26-42)

@@ -56,6 +56,9 @@ bool Scheduler::abort(int64_t id) {
 }
 
 void Scheduler::finish(int64_t id) {
+  // (a request may end while it waits: one that was preempted after its last token had been sampled)
+  auto w = std::find(waiting_.begin(), waiting_.end(), id);
+  if (w != waiting_.end()) waiting_.erase(w);
   remove_running(id);
   release(id);
   forget(id);

@@ -36,6 +36,7 @@ class EngineArgs:
     prefill_chunk_size: Optional[int] = None
     num_gpu_blocks_override: Optional[int] = None
     enforce_eager: bool = False                    # True: never capture decode steps as HIP graphs
+    run_ahead: bool = True                         # False: never launch a step before the tokens of the one before are read
     skip_tokenizer_init: bool = False              # True: work on token ids even if the folder has a tokenizer.json
     device: str = "cuda:0"
 
@@ -78,6 +79,8 @@ class EngineArgs:
         a("--prefill-chunk-size", type=int, default=None, help="longest portion of a prompt in one step")
         a("--num-gpu-blocks-override", type=int, default=None, help="pages of the cache instead of sizing from memory")
         a("--enforce-eager", action="store_true", help="run decode steps kernel by kernel instead of as HIP graphs")
+        a("--no-run-ahead", dest="run_ahead", action="store_false",
+          help="launch a step only after the tokens of the step before it have been read")
         a("--skip-tokenizer-init", action="store_true", help="do not load the folder's tokenizer.json")
         a("--device", default="cuda:0")
         return parser

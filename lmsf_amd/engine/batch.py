@@ -18,6 +18,9 @@ class StepEntry:
     request_id: Hashable
     tokens: Sequence[int]
     want: Sequence[int] = ()
+    # >= 0: the entry is one token that the host does not know yet, row ``prev_row`` of the tokens that the step
+    # before this one sampled (``ModelExecutor.step(..., prev_tokens=...)``); ``tokens`` then holds a placeholder
+    prev_row: int = -1
 
 
 @dataclass

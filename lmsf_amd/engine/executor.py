@@ -37,6 +37,7 @@ class ModelExecutor:
         self.vocab_size = model.spec.vocab_size
         self._pinned: Optional[torch.Tensor] = None
         self._pinned_np: Optional[np.ndarray] = None
+        self._prev_tokens: Optional[torch.Tensor] = None   # the step before's sampled tokens, while a step is built
         # steps of single tokens run at a padded batch size and are captured as HIP graphs, one per padded
         # size and context bucket, the least recently used dropped beyond max_graphs
         self.pad_decode = all(getattr(p, "graph_safe", False) for p in model.parts())
@@ -57,12 +58,17 @@ class ModelExecutor:
 
     # ------------------------------------------------------------------ the step
 
-    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def step(self, entries: Sequence[StepEntry], prev_tokens: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Run one batch. Returns float32 logits [R, V] on the device, rows in the order of the entries
         and of each entry's ``want``. Raises OutOfPages (and takes nothing) if the cache cannot hold
-        the new tokens."""
+        the new tokens. ``prev_tokens`` (int32, on the device): the tokens that the step before sampled, for
+        entries that name one of them (``StepEntry.prev_row``) instead of a token the host knows."""
         entries = [e for e in entries if len(e.tokens) > 0]
         self._validate(entries)
+        from_prev = any(e.prev_row >= 0 for e in entries)
+        if from_prev and prev_tokens is None:
+            raise StepError("an entry names a token of the step before, which was not given")
+        self._prev_tokens = prev_tokens if from_prev else None
         if not entries:
             return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.rt.device)
         mgr = self.manager
@@ -131,6 +137,8 @@ class ModelExecutor:
                 raise StepError("request %r appears twice in one step" % (e.request_id,))
             seen.add(e.request_id)
             n = len(e.tokens)
+            if e.prev_row >= 0 and n != 1:
+                raise StepError("request %r: a token of the step before stands for exactly one token" % (e.request_id,))
             if n == 1:
                 bad = not (0 <= int(e.tokens[0]) < V)
             else:
@@ -184,6 +192,10 @@ class ModelExecutor:
         single = N == S
         n_all = Np if static is not None else N
         order_at, total = total, total + (_pad4(n_all) if single else 0)
+        # where tokens come from the step before: per token the row of that step's sampled tokens, or -1
+        src_at = 0
+        if self._prev_tokens is not None or static is not None:
+            src_at, total = total, total + _pad4(n_all)
         # a step that the recorded program may run carries its attention plan behind that
         plan_at = plan_cap = 0
         if self.program is not None and static is None and N != S and (N, R) not in self.program._refused:
@@ -210,6 +222,15 @@ class ModelExecutor:
             section("token_ids")[:] = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in entries])
         if R:
             section("logit_rows")[:] = logit_rows
+        if src_at:
+            src = host_np[src_at:src_at + n_all]
+            src[:] = -1
+            if self._prev_tokens is not None:
+                at = 0
+                for e, n in zip(entries, lens):
+                    if e.prev_row >= 0:
+                        src[at] = e.prev_row
+                    at += n
         try:
             mgr.fill_step(handles, starts_a, lens, widths, raw_offsets, host_np)
         except CacheError as e:
@@ -232,6 +253,9 @@ class ModelExecutor:
         # the copy is synchronous: the staging buffer is free again when the next step fills it
         if static is not None:
             static.device_buffer.copy_(host, non_blocking=False)
+            if self._prev_tokens is not None:
+                self.rt.ops.patch_tokens(static.device_buffer[offsets["token_ids"][0]:offsets["token_ids"][0] + n_all],
+                                         static.device_buffer[src_at:src_at + n_all], self._prev_tokens)
             if static.context is not None:
                 return static.context
             dev = static.device_buffer
@@ -245,6 +269,8 @@ class ModelExecutor:
             o, n = offsets[name]
             return dev[o:o + n]
 
+        if static is None and self._prev_tokens is not None:
+            self.rt.ops.patch_tokens(view("token_ids"), dev[src_at:src_at + n_all], self._prev_tokens)
         S_all = Sp if static is not None else S
         if static is None:
             seg_starts = section("seg_starts").tolist()
@@ -297,7 +323,7 @@ class ModelExecutor:
         if sb is None:
             widths = [-(-bucket // g.page_size) for g in self.manager.groups]
             _, _, total = self.manager.step_layout(Bp, Bp, Bp, widths)
-            sb = _StaticBatch(Bp, widths, torch.zeros(total + _pad4(Bp), dtype=torch.int32, device=self.rt.device),
+            sb = _StaticBatch(Bp, widths, torch.zeros(total + 2 * _pad4(Bp), dtype=torch.int32, device=self.rt.device),
                               bucket)
             self._static[(Bp, bucket)] = sb
             while len(self._static) > self.max_graphs:

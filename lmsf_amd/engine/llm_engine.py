@@ -22,6 +22,31 @@ from .scheduler import Scheduler, SchedulerConfig, StepPlan
 from .sequence import Sequence, SequenceState
 
 
+class _SeqSet:
+    """Sequences by identity."""
+
+    def __init__(self, ids):
+        self._ids = set(ids)
+
+    def __contains__(self, seq) -> bool:
+        return id(seq) in self._ids
+
+    def __bool__(self) -> bool:
+        return bool(self._ids)
+
+
+class _InFlight:
+    """A step that has been launched: its plan, the requests it samples for and where their tokens will be."""
+
+    __slots__ = ("plan", "sampled", "tokens_dev", "t_start", "pending_of", "host_tokens", "event")
+
+    def __init__(self, plan, sampled, tokens_dev, t_start, pending_of):
+        self.plan, self.sampled, self.tokens_dev, self.t_start = plan, sampled, tokens_dev, t_start
+        self.pending_of = pending_of      # requests whose token of the step before this step took from the device
+        self.host_tokens = None
+        self.event = None
+
+
 class LLMEngine:
     def __init__(self, args: EngineArgs, ops: Any = None):
         args.verify()
@@ -46,6 +71,11 @@ class LLMEngine:
         self.logger = init_logging(args.log_dir, args.alsologtostderr) if (args.log_dir or args.alsologtostderr) else None
         self.metrics = Metrics(logger=self.logger)
         self.last_step: Dict[str, Any] = {}
+        # one step may be in flight on the GPU while the host prepares the next (see ``step``)
+        self.run_ahead = bool(getattr(args, "run_ahead", True))
+        self._inflight: Optional[_InFlight] = None
+        self._token_slots = [[None, None], [None, None]]     # pinned buffer and event, two steps in turn
+        self._token_turn = 0
 
     @classmethod
     def from_engine_args(cls, args: EngineArgs) -> "LLMEngine":
@@ -115,10 +145,49 @@ class LLMEngine:
 
     def step(self) -> List[RequestOutput]:
         """Schedule, run the model once, sample, apply the stop rules
-        (core/src/engine/llm_engine.rs:536-582)."""
+        (core/src/engine/llm_engine.rs:536-582); returns the outputs of the step that has finished.
+
+        The host runs one step ahead of the GPU where it can: once a step and its sampler are launched, the
+        next step is scheduled and launched before the first one's tokens are read. Its single tokens come from
+        where the sampler left them on the device (``StepEntry.prev_row``), everything else a step needs
+        (positions, pages, block tables) does not depend on their values. The host's work between two steps
+        then passes while the GPU computes. What cannot be known without the values: a request that ends with
+        an end-of-sequence token or a stop string has one more token computed for nothing, which is dropped.
+        A step is not launched ahead when a request of the step before reaches its length limit with the token
+        being sampled, or uses penalties (which count the tokens on the host)."""
+        outputs: List[RequestOutput] = []
+        if self._inflight is None:
+            self._inflight = self._launch(outputs, None)
+            if self._inflight is None:
+                return outputs
+        cur = self._inflight
+        ahead = None
+        if self.run_ahead and self._may_run_ahead(cur):
+            for seq in cur.sampled:
+                seq.pending = 1           # counts as a token from here on; its value comes when ``cur`` is finished
+            try:
+                ahead = self._launch(outputs, cur)
+            except BaseException:
+                for seq in cur.sampled:
+                    seq.pending = 0
+                raise
+        self._finish(cur, outputs)
+        self._inflight = ahead if self.scheduler.has_unfinished() else None
+        return outputs
+
+    def _may_run_ahead(self, cur: "_InFlight") -> bool:
+        limit = self.core.max_model_len
+        for seq in cur.sampled:
+            if seq.params.has_penalties or len(seq.output_token_ids) + 1 >= seq.params.max_tokens \
+                    or seq.length + 1 >= limit:
+                return False
+        return True
+
+    def _launch(self, outputs: List[RequestOutput], prev: Optional["_InFlight"]) -> Optional["_InFlight"]:
+        """Schedule a step, launch it and its sampler; nothing here waits for the GPU. ``prev``: the step in
+        flight, whose sampled tokens this one may take from the device."""
         t_start = time.monotonic()
         plan: StepPlan = self.scheduler.schedule()
-        outputs: List[RequestOutput] = []
         now = time.monotonic()
         for seq in plan.ignored + plan.capped:
             seq.metrics.finished_time = now
@@ -126,21 +195,62 @@ class LLMEngine:
             outputs.append(RequestOutput.from_sequence(seq, None))
         self.stats["preemptions"] += len(plan.preempted)
         if plan.empty:
-            return outputs
-        entries = [StepEntry(s.seq.request_id, s.seq.tokens(s.start, s.n_tokens),
-                             [s.n_tokens - 1] if s.samples else []) for s in plan.scheduled]
-        logits = self.core.executor.step(entries)
+            return None
+        prev_row = {}
+        if prev is not None:
+            prev_row = {id(seq): i for i, seq in enumerate(prev.sampled) if seq.pending}
+        entries = []
+        pending_of = set()
+        for s in plan.scheduled:
+            row = prev_row.get(id(s.seq), -1)
+            if row >= 0 and s.start + s.n_tokens == s.seq.length:
+                pending_of.add(id(s.seq))
+            else:
+                row = -1
+            entries.append(StepEntry(s.seq.request_id, s.seq.tokens(s.start, s.n_tokens),
+                                     [s.n_tokens - 1] if s.samples else [], prev_row=row))
+        logits = self.core.executor.step(entries, prev_tokens=prev.tokens_dev if pending_of else None)
         self.stats["steps"] += 1
         sampled = []
         for s in plan.scheduled:
             s.seq.num_computed += s.n_tokens
             if s.samples:
                 sampled.append(s.seq)
-        rows = [SamplingRow(seq.params, seq.seed, len(seq.output_token_ids), seq.prompt_token_ids,
+        rows = [SamplingRow(seq.params, seq.seed, len(seq.output_token_ids) + seq.pending, seq.prompt_token_ids,
                             seq.output_token_ids) for seq in sampled]
-        tokens = self.sampler.sample(logits, rows)
+        tokens_dev = self.sampler.sample_on_device(logits, rows)
+        rec = _InFlight(plan, sampled, tokens_dev, t_start, _SeqSet(pending_of))
+        if tokens_dev is not None and tokens_dev.is_cuda:
+            # the tokens travel to pinned memory behind the sampler, ahead of whatever is launched next; the
+            # event says when they are there
+            n = tokens_dev.numel()
+            slot = self._token_slots[self._token_turn]
+            self._token_turn ^= 1
+            if slot[0] is None or slot[0].numel() < n:
+                slot[0] = torch.empty(max(n, 256), dtype=torch.int32, pin_memory=True)
+                slot[1] = torch.cuda.Event()
+            slot[0][:n].copy_(tokens_dev, non_blocking=True)
+            slot[1].record()
+            rec.host_tokens, rec.event = slot[0], slot[1]
+        return rec
+
+    def _finish(self, rec: "_InFlight", outputs: List[RequestOutput]) -> None:
+        """Read the step's tokens, append them, apply the stop rules."""
+        n = len(rec.sampled)
+        if n == 0:
+            tokens: List[int] = []
+        elif rec.event is not None:
+            rec.event.synchronize()
+            tokens = rec.host_tokens[:n].tolist()
+        else:
+            tokens = [int(t) for t in rec.tokens_dev.tolist()]
         now = time.monotonic()
-        for seq, tok in zip(sampled, tokens):
+        n_sampled = 0
+        for seq, tok in zip(rec.sampled, tokens):
+            seq.pending = 0
+            if seq.state.finished or self._requests.get(seq.request_id) is not seq:
+                continue          # it ended with the step before (or was aborted): this token was one too many
+            n_sampled += 1
             seq.output_token_ids.append(tok)
             if seq.metrics.first_token_time is None:
                 seq.metrics.first_token_time = now
@@ -157,11 +267,10 @@ class LLMEngine:
                 self.scheduler.finish(seq)
                 self._requests.pop(seq.request_id, None)
             outputs.append(RequestOutput.from_sequence(seq, tok, piece))
-        n_tokens = plan.num_tokens
-        self.stats["generated_tokens"] += len(sampled)
+        n_tokens = rec.plan.num_tokens
+        self.stats["generated_tokens"] += n_sampled
         self.stats["tokens"] += n_tokens
-        self._record_step(plan, n_tokens, len(sampled), outputs, t_start)
-        return outputs
+        self._record_step(rec.plan, n_tokens, n_sampled, outputs, rec.t_start)
 
     def _record_step(self, plan: StepPlan, n_tokens: int, n_sampled: int, outputs: List[RequestOutput],
                      t_start: float) -> None:

@@ -59,10 +59,11 @@ class Sequence:
     prompt: Optional[str] = None           # the prompt's text, if the request came as text
     output_text: str = ""                  # text of the generated tokens (engines with a tokenizer)
     detokenizer: Any = None                # engine.detokenizer.IncrementalDetokenizer
+    pending: int = 0                       # 1 while a sampled token is still on the device, unread by the host
 
     @property
     def length(self) -> int:
-        return len(self.prompt_token_ids) + len(self.output_token_ids)
+        return len(self.prompt_token_ids) + len(self.output_token_ids) + self.pending
 
     @property
     def remaining(self) -> int:
@@ -70,6 +71,12 @@ class Sequence:
         return self.length - self.num_computed
 
     def tokens(self, start: int, n: int) -> List[int]:
+        """Token ids of positions start .. start + n - 1 (a pending token's place holds 0)."""
+        if self.pending and start + n == self.length:
+            return self.tokens_known(start, n - 1) + [0]
+        return self.tokens_known(start, n)
+
+    def tokens_known(self, start: int, n: int) -> List[int]:
         p = len(self.prompt_token_ids)
         if start + n <= p:
             return self.prompt_token_ids[start:start + n]

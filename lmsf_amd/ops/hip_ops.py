@@ -112,6 +112,16 @@ class HipOps:
                                             float(scale), _ptr(self._bad_flag), self._stream()))
         return out
 
+    def patch_tokens(self, ids: torch.Tensor, src: torch.Tensor, prev: torch.Tensor) -> None:
+        """ids[i] = prev[src[i]] where src[i] >= 0 (all int32, on the device): a step launched ahead takes the
+        tokens that the step before it sampled from where the sampler left them."""
+        self._dev(ids, src, prev)
+        self._i32(ids, "ids")
+        self._i32(src, "src", ids.numel())
+        self._i32(prev, "prev")
+        self._check(self.lib.lmsf_patch_tokens(_ptr(ids), _ptr(src), _ptr(prev), ids.numel(), prev.numel(),
+                                               self._stream()))
+
     def bad_token_seen(self) -> bool:
         """True if an embedding call since the last query met an id outside the vocabulary."""
         if self._bad_flag is None:

@@ -9,7 +9,7 @@ from typing import Optional
 
 from ..csrc import build as _build
 
-ABI_VERSION = 20
+ABI_VERSION = 21
 
 _lib: Optional[ctypes.CDLL] = None
 _lib_path: Optional[str] = None
@@ -25,6 +25,7 @@ _SIGNATURES = {
     "lmsf_abi_version": (c_int, []),
     "lmsf_device_arch": (c_int, [c_char_p, c_int]),
     "lmsf_embedding": (c_int, [_P, _P, c_int, _P, c_int, c_int, c_int, c_float, _P, _P]),
+    "lmsf_patch_tokens": (c_int, [_P, _P, _P, c_int, c_int, _P]),
     "lmsf_add_rms_norm": (c_int, [_P, c_int, _P, _P, c_int, _P, c_int, _P, c_int, c_int, c_float, c_float, _P]),
     "lmsf_rope_cache_write": (c_int, [_P, _P, _P, c_int, c_int, c_long, _P, _P, c_int, c_int, c_int, _P, _P, _P,
                                       c_long, c_int, c_int, c_int, c_int, _P]),

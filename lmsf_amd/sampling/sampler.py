@@ -39,11 +39,16 @@ class Sampler:
 
     def sample(self, logits: torch.Tensor, rows: Sequence[SamplingRow]) -> List[int]:
         """One token id per row of float32 ``logits`` [R, V]."""
+        out = self.sample_on_device(logits, rows)
+        return [] if out is None else [int(t) for t in out.tolist()]
+
+    def sample_on_device(self, logits: torch.Tensor, rows: Sequence[SamplingRow]) -> Optional[torch.Tensor]:
+        """The same, left on the device (int32 [R]; None for no rows): nothing here waits for the GPU."""
         R = len(rows)
         if logits.shape[0] != R:
             raise ValueError("%d rows of logits for %d requests" % (logits.shape[0], R))
         if R == 0:
-            return []
+            return None
         if any(r.params.has_penalties for r in rows):
             logits = logits.clone()
             tokens: List[int] = []
@@ -92,7 +97,7 @@ class Sampler:
                 out = self.ops.sample(logits, temperature, None, None, None, seeds, draws)
             else:
                 out = self.ops.sample(logits, temperature, d[5 * R:6 * R], fd[R:2 * R], fd[2 * R:3 * R], seeds, draws)
-        return [int(t) for t in out.tolist()]
+        return out
 
 
 def _to_i64(seed: int) -> int:

@@ -99,6 +99,8 @@ class Scheduler:
         """The engine decided that ``seq`` is done: drop it and give back what it holds."""
         if seq in self.running:
             self.running.remove(seq)
+        if seq in self.waiting:           # preempted after its last token had been sampled
+            self.waiting.remove(seq)
         self._release(seq)
 
     def _release(self, seq: Sequence) -> None:
@@ -234,6 +236,8 @@ class Scheduler:
         goes back, and it returns to the front of the waiting queue."""
         if seq in self.running:
             self.running.remove(seq)
+        if seq in self.waiting:           # preempted after its last token had been sampled
+            self.waiting.remove(seq)
         self._release(seq)
         seq.num_computed = 0
         seq.num_preemptions += 1

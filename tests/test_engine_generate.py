@@ -127,3 +127,41 @@ def test_sampling_params_follow_the_reference():
     assert p.greedy and (p.top_k, p.top_p, p.min_p) == (-1, 1.0, 0.0)
     d = SamplingParams()
     assert (d.temperature, d.top_p, d.top_k, d.max_tokens, d.repetition_penalty) == (1.0, 1.0, -1, 128, 1.0)
+
+
+@pytest.mark.parametrize("pages", [64, 8])
+def test_running_a_step_ahead_changes_no_token(tmp_path, pages):
+    """The host launches the next step before it has read the tokens of the one in flight. Requests that end
+    on a stop token (found out one step late), by their length limit (known in advance), with penalties (never
+    run ahead), requests that arrive under way, an abort, and so few pages that requests are preempted: the
+    outputs are those of an engine that reads every step's tokens before it schedules the next."""
+    results = []
+    for ahead in (False, True):
+        engine, folder, cfg = make_engine(tmp_path, "A", pages=pages, prefill_chunk_size=16, run_ahead=ahead)
+        V = cfg.vocab_size
+        stop_ids = list(range(0, V, 16))          # one token id in sixteen stops a request: they end early
+        def add(i, n, **kw):
+            engine.add_request(i, random_tokens(n, V, 90 + i), SamplingParams(seed=77 + i, **kw))
+        add(0, 20, temperature=0.9, max_tokens=30, stop_token_ids=stop_ids)
+        add(1, 17, temperature=0.0, max_tokens=30, ignore_eos=True)
+        add(2, 9, temperature=0.7, max_tokens=4, ignore_eos=True, presence_penalty=0.5)
+        done, launched_ahead, steps = {}, 0, 0
+        while engine.has_unfinished_requests():
+            for out in engine.step():
+                if out.finished:
+                    done[out.request_id] = (out.outputs[0].token_ids, out.outputs[0].finish_reason)
+            launched_ahead += engine._inflight is not None
+            steps += 1
+            if steps == 3:
+                add(3, 5, temperature=1.0, max_tokens=18, stop_token_ids=stop_ids)
+                add(4, 30, temperature=0.0, max_tokens=20, ignore_eos=True)
+            if steps == 9:
+                engine.abort_request(4)
+        assert (launched_ahead > 5) == ahead
+        assert (engine.stats["preemptions"] > 0) == (pages == 8)
+        assert set(done) == {0, 1, 2, 3}
+        results.append(done)
+        engine.core.storage.manager.check_invariants()
+        assert engine.core.storage.manager.num_free_pages(0) == pages
+    assert results[0] == results[1]
+    assert results[0][1][1] == "length" and "stop" in {r[1] for r in results[0].values()}

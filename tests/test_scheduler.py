@@ -239,3 +239,23 @@ def test_random_load_keeps_invariants(seed):
     assert len(done) == 30 and not sched.has_unfinished()
     cache.check_invariants()
     assert cache.num_free_pages() == 24 and cache.num_free_state_slots() == 5
+
+
+def test_a_request_may_finish_while_it_waits():
+    """A request preempted after its last token was sampled ends in the waiting queue: the engine finishes it
+    there, and the queue must not keep it."""
+    sched, cache = make(num_pages=4, page_size=4, budget=16, max_len=64)
+    old, new = seq("old", 12, 0), seq("new", 4, 1)
+    sched.add(old)
+    sched.add(new)
+    run_plan(sched, cache, sched.schedule())
+    plan = sched.schedule()                                   # no page for both: "new" goes back to waiting
+    assert [x.request_id for x in plan.preempted] == ["new"]
+    run_plan(sched, cache, plan)
+    sched.finish(new)                                         # ... and turns out to have ended with its last token
+    assert [s.request_id for s in sched.waiting] == [] and sched.has_unfinished()
+    for _ in range(3):
+        plan = sched.schedule()
+        assert [(s.seq.request_id, s.n_tokens) for s in plan.scheduled] == [("old", 1)]
+        run_plan(sched, cache, plan)
+    cache.check_invariants()

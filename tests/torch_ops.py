@@ -64,6 +64,10 @@ class TorchOps:
     def bad_token_seen(self):
         return False
 
+    def patch_tokens(self, ids, src, prev):
+        take = src[:ids.numel()] >= 0
+        ids[take] = prev[src[:ids.numel()][take].long()].to(ids.dtype)
+
     def add_rms_norm(self, branch, residual, weight, eps, out_dtype, rows=None, weight_offset=0.0, defer_ok=False):
         x = None
         if branch is not None:
