@@ -272,6 +272,7 @@ def main():
     max_seqs = max([64, args.batch] + point_batches)
     engine = make_engine(cfg, args, max_num_seqs=max_seqs, dtype=args.dtype)
     wbytes = weight_bytes(engine)
+    cache_pages = engine.core.storage.groups[0].num_pages if engine.core.storage.groups else 0
     kv_per_token = 2 * cfg["num_key_value_heads"] * cfg["head_dim"] * cfg["num_hidden_layers"] * \
         (2 if args.dtype == "bfloat16" else 4)
 
@@ -332,6 +333,7 @@ def main():
             "intermediate_size": cfg["intermediate_size"], "vocab_size": cfg["vocab_size"],
             "max_context": cfg["max_position_embeddings"], "block_size": 16, "prompt_len": args.prompt_len,
             "mean_decode_context": round(mean_ctx, 1), "prefill_tokens": args.prefill_tokens,
+            "cache_pages": cache_pages, "gpu_memory_utilization": args.gpu_memory_utilization,
         },
         "prefill": {"value": round(args.prefill_tokens / pt, 1), "tokens": args.prefill_tokens,
                     "ms": round(pt * 1e3, 3), "frac": round(pflops / pt / peak, 4)},

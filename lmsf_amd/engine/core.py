@@ -62,7 +62,8 @@ def build_model(arch: Architecture, config: ArchConfig, rt: Runtime, model_dir: 
         std = 0.02
         store = torch.float32 if rt.dtype == torch.float32 else torch.bfloat16
         load_weights_from_generator(model.parts(),
-                                    lambda name, decl: random_tensor(name, decl, seed, std, store, rt.device))
+                                    lambda name, decl: random_tensor(name, decl, seed, std, store, rt.device),
+                                    device=rt.device)
     elif load_format == "auto":
         if model_dir is None:
             raise ValueError("a model folder is needed unless load_format is 'random'")

@@ -50,14 +50,17 @@ class FusedLinear(Part):
         sources differ in element type the buffer takes the widest."""
         if len(self.sources) == 1:
             return fetch(self._name(self.sources[0][0], what)).contiguous()
-        out: Optional[torch.Tensor] = None
+        # the buffer is made before the first source is read: made after it, torch would cut it out of the block
+        # that the source's conversion has just freed and leave a hole of the difference for good
+        tail = (self.in_features,) if what == "weight" else ()
+        out = torch.empty((self.out_features,) + tail, dtype=self.rt.dtype, device=self.rt.device)
         row = 0
         for sub, rows in self.sources:
             t = fetch(self._name(sub, what))
-            if out is None:
-                out = torch.empty((self.out_features,) + tuple(t.shape[1:]), dtype=t.dtype, device=t.device)
-            elif t.dtype != out.dtype and t.dtype == torch.float32:
-                out = out.to(torch.float32)
+            if t.dtype != out.dtype and t.dtype == torch.float32:
+                out = out.to(torch.float32)           # a source stored in 32 bits: the buffer takes the widest type
+            if t.device != out.device:
+                out = out.to(t.device)
             out[row:row + rows].copy_(t)
             row += rows
             del t
