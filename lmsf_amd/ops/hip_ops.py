@@ -517,12 +517,31 @@ class HipOps:
         if len(single) == len(lens):
             plan = _AttentionPlan(None, 0, None, len(single), max_context)
         else:
-            both = torch.tensor(tiles + single, dtype=torch.int32).to(dev)
+            both = self._upload_ints(tiles + single, dev)
             plan = _AttentionPlan(both[:len(tiles)], len(tiles) // 2,
                                   both[len(tiles):] if single else None, len(single), max_context)
         if aux is not None:
             aux[key] = plan
         return plan
+
+    def _upload_ints(self, values, dev: torch.device) -> torch.Tensor:
+        """int32 values to the device through pinned memory, without waiting for the copy. Four buffers take
+        turns; before a buffer is written again its last copy's event is waited for (long past, as a rule)."""
+        n = len(values)
+        turn = self._pinned_turn = (getattr(self, "_pinned_turn", -1) + 1) % 4
+        bufs = self.__dict__.setdefault("_pinned_ints", [None] * 4)
+        events = self.__dict__.setdefault("_pinned_events", [None] * 4)
+        if events[turn] is not None:
+            events[turn].synchronize()
+        if bufs[turn] is None or bufs[turn].numel() < n:
+            bufs[turn] = torch.empty(max(n, 4096), dtype=torch.int32, pin_memory=True)
+        host = bufs[turn][:n]
+        host.numpy()[:] = values
+        out = host.to(dev, non_blocking=True)
+        if events[turn] is None:
+            events[turn] = torch.cuda.Event()
+        events[turn].record()
+        return out
 
     # ------------------------------------------------------------------ feed-forward
 

@@ -56,13 +56,14 @@ class PagedAttention(Mixer):
     @property
     def accepts_normed(self) -> bool:
         # the fused projection takes the norm into itself; an encoding that acts on the projections needs h
-        return self.position is None or hasattr(self.position, "rotary_table")
+        return self.position is None or self.position.rotary_table() is not None
 
     def forward(self, h: torch.Tensor, ctx, binding: CacheBinding, pending_ok: bool = False):
         ops = self.rt.ops
         group = ctx.groups[binding.group]
         slots = group.slots if binding.writes_cache else None
-        if self.position is not None and not hasattr(self.position, "rotary_table"):
+        rotary = self.position.rotary_table() if self.position is not None else None
+        if self.position is not None and rotary is None:
             # an encoding that acts on the projections itself
             qkv = self.qkv.forward(h)
             self.position.apply(qkv, self.nh, self.nkv, self.d, ctx.positions)
@@ -70,7 +71,7 @@ class PagedAttention(Mixer):
                 ops.rope_cache_write(qkv, self.nh, self.nkv, self.d, ctx.positions, None, 0, True, slots,
                                      binding.k_pages, binding.v_pages)
         else:
-            table, rot, neox = self.position.rotary_table() if self.position is not None else (None, 0, True)
+            table, rot, neox = rotary if rotary is not None else (None, 0, True)
             qkv = ops.qkv_rope_cache(h, self.qkv.weight, self.qkv.bias, self.nh, self.nkv, self.d, ctx.positions,
                                      table, rot, neox, slots, binding.k_pages, binding.v_pages)
         a = ops.paged_attention(qkv, binding.k_pages, binding.v_pages, group.block_tables, ctx.seg_of_token,

@@ -190,6 +190,11 @@ class PositionEncoding(Part):
     """Encodes positions into queries and keys. A mixer that owns one asks it for what its fused
     kernel needs (``rotary_table``) or lets it act on the tensors (``apply``)."""
 
+    def rotary_table(self):
+        """(float32 table [max_positions, rot] = [cos | sin], rot, neox pairing) if the encoding is a rotation
+        that the fused rotate-and-store kernel can apply; None (the default) if it acts through ``apply``."""
+        return None
+
     def apply(self, qkv: torch.Tensor, nh: int, nkv: int, d: int, positions: torch.Tensor) -> None:
         raise NotImplementedError
 
