@@ -17,7 +17,9 @@
 // at 2,048 rows where the library's 256 x 256 tiles (wave tiles of 128 x 128) reach 1.2. Tried and measured, not
 // kept: steps of 32 k with rows of 64 bytes and the next step's operands read under the multiplications (0.56);
 // the same prefetch within steps of 64 k with the barrier in the middle of a step (0.74); tiles of 256 x 256 with two
-// stages, which is all LDS holds of them (0.6, the compiler spills around 256 accumulators).
+// stages, which is all LDS holds of them (0.6, the compiler spills around 256 accumulators); the same tiles with the
+// 32 x 32 x 16 instruction, wave tiles of 128 x 128 and no spills (0.85 to 1.0: two stages do not cover the way from
+// memory).
 //
 // Workgroups that share rows of W run on the same XCD, one after the other in launch order, so that a panel of W
 // comes from memory once and from that XCD's L2 afterwards: with 8 XCDs taking workgroups in turn, workgroup b
