@@ -55,6 +55,7 @@ class ModelExecutor:
             from ..ops.program import record_program
             self.program = record_program(model, rt.ops)
         self.program_steps = 0          # steps that the program ran
+        self.program_workspace_bytes = 32 << 20    # the workspace's first size; it doubles when a step finds no room
 
     # ------------------------------------------------------------------ the step
 
@@ -105,7 +106,7 @@ class ModelExecutor:
             if ctx.all_single or plan_ptr is not None:
                 stream = _raw_stream(_current_device())
                 capturing = torch.cuda.is_current_stream_capturing()
-                nbytes = max(prog.workspace.numel() if prog.workspace is not None else 0, 32 << 20)
+                nbytes = max(prog.workspace.numel() if prog.workspace is not None else 0, self.program_workspace_bytes)
                 while True:
                     if not capturing:
                         prog.ensure_workspace(nbytes)

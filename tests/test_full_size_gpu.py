@@ -144,3 +144,26 @@ def test_loading_leaves_no_holes_in_device_memory():
     slack = torch.cuda.memory_reserved() - torch.cuda.memory_allocated() - base
     weights = sum(t.numel() * t.element_size() for p in core.model.parts() for t in p.tensors())
     assert weights > 5e9 and slack < (200 << 20), (slack, weights)
+
+
+def test_recorded_program_at_these_sizes_with_the_smallest_workspace(full_model):
+    """The step program against the parts at Llama-3-8B widths, bit for bit, with a workspace that starts at
+    1 MB and doubles until a step fits: the ring of temporaries then wraps as often as it can, and a buffer
+    handed out while its last reader is still to come would show."""
+    from lmsf_amd.engine import load_engine_core
+    folder, cfg, w = full_model
+    V = cfg["vocab_size"]
+    reqs = {"a": random_tokens(150, V, 31), "b": random_tokens(60, V, 32), "c": random_tokens(23, V, 33)}
+    steps = trace_mixed(reqs, 24 * 16, seed=9) + trace_portions({"d": random_tokens(200, V, 34)}, seed=2)
+    outs = []
+    for use_program in (True, False):
+        core = load_engine_core(folder, dtype="bfloat16", block_size=16, num_pages=24, max_num_seqs=8,
+                                use_program=use_program, enforce_eager=True)
+        core.executor.program_workspace_bytes = 1 << 20
+        outs.append(replay_in_process(core.executor, steps))
+        if use_program:
+            assert core.executor.program_steps > 30
+            grown = core.executor.program.workspace.numel()
+            assert (1 << 20) < grown <= (64 << 20), grown
+    for rid in outs[0]:
+        assert torch.equal(outs[0][rid], outs[1][rid]), rid
