@@ -224,6 +224,71 @@ def serve_run(args, emit=True):
     return line
 
 
+def products_run(args):
+    """The four matrix products of a layer at the headline shape, for some numbers of rows: the BLAS library's
+    (through torch) against this package's choice (``HipOps.linear`` / ``linear_gated``), microseconds by HIP
+    events around a HIP graph of eight calls, the weight read from memory every time. One JSON line per product and number of rows."""
+    import torch
+    from lmsf_amd.ops import get_ops
+    ops = get_ops()
+    cfg = SHAPES[args.shape][1]
+    H, I = cfg["hidden_size"], cfg["intermediate_size"]
+    d, nh, nkv = cfg["head_dim"], cfg["num_attention_heads"], cfg["num_key_value_heads"]
+    shapes = {"qkv": ((nh + 2 * nkv) * d, H, False), "o": (H, nh * d, False), "gate_up": (2 * I, H, True),
+              "down": (H, I, False)}
+    g = torch.Generator(device="cuda:0").manual_seed(1)
+
+    def timed(f, reps=8):
+        """Microseconds a call: ``reps`` calls recorded into a HIP graph once (no host time between the kernels),
+        replayed six times between events; the median."""
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                f()
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for _ in range(reps):
+                f()
+        times = []
+        for _ in range(6):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            graph.replay()
+            b.record()
+            b.synchronize()
+            times.append(a.elapsed_time(b) / reps)
+        del graph
+        return sorted(times)[len(times) // 2] * 1e3
+    for name, (N, K, gated) in shapes.items():
+        W = (torch.randn(N, K, device="cuda:0", generator=g) * 0.02).to(torch.bfloat16)
+        # as in a model, every call streams its weight from memory: the copies in turn are larger together than
+        # the 256 MB of the memory-side cache
+        copies = [W] + [W.clone() for _ in range(int(1.5e9 // (N * K * 2)))]
+        turn = [0]
+
+        def weight():
+            turn[0] = (turn[0] + 1) % len(copies)
+            return copies[turn[0]]
+        for M in [int(m) for m in args.rows.split(",")]:
+            x = torch.randn(M, K, device="cuda:0", generator=g).to(torch.bfloat16)
+            if gated:
+                lib = lambda w: ops.gated_act(torch.nn.functional.linear(x, w), "silu")    # noqa: E731
+                own = lambda w: ops.linear_gated(x, w, None, "silu")                          # noqa: E731
+            else:
+                lib = lambda w: torch.nn.functional.linear(x, w)                              # noqa: E731
+                own = lambda w: ops.linear(x, w)                                              # noqa: E731
+            a, b = own(W).float(), lib(W).float()
+            err = (a - b).abs().max().item() / b.abs().max().item()
+            t_lib, t_own = timed(lambda: lib(weight())), timed(lambda: own(weight()))
+            flops = 2.0 * M * N * K
+            print(json.dumps({"product": name, "rows": M, "N": N, "K": K, "library_us": round(t_lib, 1),
+                              "library_PFLOPs": round(flops / t_lib / 1e9, 3), "engine_us": round(t_own, 1),
+                              "engine_PFLOPs": round(flops / t_own / 1e9, 3), "max_diff_of_largest": err}))
+            del a, b
+
+
 def prefill_flops(cfg, T):
     """Multiply-adds times two of a causal prefill of T tokens: the linear layers on every token, the
     attention scores and values over the causal half, the LM head on one row."""
@@ -247,9 +312,11 @@ def main():
     ap.add_argument("--max-num-batched-tokens", type=int, default=8192)
     ap.add_argument("--gpu-memory-utilization", type=float, default=0.85)
     ap.add_argument("--skip-points", action="store_true", help="leave out the batch 1 and batch 64 runs")
-    ap.add_argument("--workload", default="decode", choices=["decode", "serve"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "serve", "products"],
                     help="decode: the default line (Llama-3-8B shape); serve: continuous batching of 64 requests at "
-                         "Llama-2-7B shape, a line of its own")
+                         "Llama-2-7B shape, a line of its own; products: a layer's matrix products alone, the "
+                         "library's against the engine's choice, at --rows")
+    ap.add_argument("--rows", default="17,64,100,128,129,192,256,512,2048", help="products: numbers of rows")
     ap.add_argument("--prefill-chunk-size", type=int, default=1024, help="serve: longest portion of a prompt in a step")
     ap.add_argument("--shape", default="llama3-8b", choices=sorted(SHAPES),
                     help="decode: the model whose layer sizes are measured (default: the headline configuration)")
@@ -261,6 +328,9 @@ def main():
 
     if args.workload == "serve":
         serve_run(args)
+        return
+    if args.workload == "products":
+        products_run(args)
         return
     import torch
     shape_name, shape_cfg = SHAPES[args.shape]
