@@ -919,3 +919,11 @@ def test_apply_penalties(ops, ref):
     ref.apply_penalties(b, *args)
     assert torch.allclose(a, b, atol=1e-6)
     assert not torch.equal(a, dev(logits))
+
+
+def test_measured_rates_are_plausible(ops):
+    """The yardstick kernels of bench.py run (a buffer whose size is no multiple of the grid: the last workgroup
+    takes the rest) and report rates of the order of this hardware's."""
+    rates = ops.measure(nbytes=(1 << 28) + 4096 * 7 + 16, reps=1)
+    assert 500 < rates["read_GBps"] < 20000 and 500 < rates["copy_GBps"] < 20000
+    assert 100 < rates["mfma_bf16_TFLOPs"] < 5000
