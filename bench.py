@@ -320,12 +320,22 @@ def main():
     ap.add_argument("--prefill-chunk-size", type=int, default=1024, help="serve: longest portion of a prompt in a step")
     ap.add_argument("--shape", default="llama3-8b", choices=sorted(SHAPES),
                     help="decode: the model whose layer sizes are measured (default: the headline configuration)")
+    ap.add_argument("--tunable", action="append", default=[], metavar="NAME=INT",
+                    help="set an attribute of ops.HipOps (a number of rows at which kernels change, a variant) first")
     ap.add_argument("--points", default="1,64,128", help="decode: further batch sizes, comma separated")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this engine runs on one GPU; --gpus %d is not supported" % args.gpus)
         sys.exit(2)
 
+    if args.tunable:
+        from lmsf_amd.ops import get_ops
+        ops = get_ops()
+        for item in args.tunable:
+            name, _, value = item.partition("=")
+            if not hasattr(ops, name) or not isinstance(getattr(ops, name), int):
+                raise SystemExit("bench.py: HipOps has no integer attribute %r" % name)
+            setattr(ops, name, int(value))
     if args.workload == "serve":
         serve_run(args)
         return

@@ -69,6 +69,7 @@ class HipOps:
         self.mid_max_rows = 128        # rows up to which the 17-and-more-rows kernel beats the library (64 with the gated activation)
         self.skinny_max_rows = 16      # rows up to which the few-rows kernel beats the library (measured)
         self.large_max_rows = 256      # rows up to which the many-rows kernel beats the library (measured; 0: never)
+        self.large_deep_max_rows = 512  # the same for products whose K is at least three times N (down: 65 against 74 us at 320 rows, 87 against 95 at 512)
 
     # ------------------------------------------------------------------ helpers
 
@@ -595,8 +596,9 @@ class HipOps:
         if (both_bf16 and self.skinny_max_rows < M <= self.mid_max_rows and self._mid_ok(x, weight)
                 and (M <= 64 or N <= self.mid_wide_max_cols or out_dtype == torch.float32)):
             return self._linear_mid(x, weight, bias, 0, out_dtype, pending_ok and out_dtype == torch.bfloat16, out=out)
-        if (both_bf16 and out_dtype == torch.bfloat16 and self.mid_max_rows < M <= self.large_max_rows
-                and self._mid_ok(x, weight)):
+        if (both_bf16 and out_dtype == torch.bfloat16 and self._mid_ok(x, weight)
+                and (self.mid_max_rows < M <= self.large_max_rows
+                     or (self.large_max_rows < M <= self.large_deep_max_rows and K >= 3 * N))):
             # 129 to 256 rows: the library is weak there (0.12 to 0.5 PFLOP/s at these widths)
             return self._linear_large(x, weight, bias, 0, pending_ok, out=out)
         if pending_ok and both_bf16 and out_dtype == torch.bfloat16 and self._skinny_ok(x, weight) and M > 0:
