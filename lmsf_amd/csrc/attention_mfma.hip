@@ -288,9 +288,20 @@ __device__ __forceinline__ unsigned lds_address(const void* p) {
 // only rescaled when a row's maximum has moved.
 // How far (in powers of two) a row's scores may rise above the reference of its exponentials before the
 // accumulators are rescaled: 2^24 times a few thousand keys times the values stays far inside float32.
+//
+// What bounds it (measured with timestamps inside the kernel and with parts of the step taken out): a wave that
+// is alone on its SIMD takes 970 ns for a step whose 32 matrix instructions need 250: the vector instructions
+// around them (scale, exponential, sum, conversion: 250 ns even with everything else removed), the waits for
+// LDS, the transfers and the barrier each add their own share, because one wave issues one instruction at a
+// time and a v_exp_f32 never runs beside a matrix instruction (a fused multiply-add does: measured apart). Two
+// waves on a SIMD hide most of that from each other (600 ns for the two), and more do not fit the registers.
+// At 2,048 tokens the longest tile's workgroup is alone on its compute unit for most of its 64 steps, and the
+// kernel takes as long as that workgroup: 5 us of set-up and 64 x 970 ns; at 8,192 tokens the tiles are many
+// and the kernel reaches 0.85 PFLOP/s. Tried, measured, not kept: the next step's scores multiplied beside the
+// current step's exponentials, in the order fixed with scheduling groups (the same times within 3 percent).
 #define PREFILL_LAZY_LOG2 24.0f
-template <int DPAD, int NQB, int STAGES>
-__global__ __launch_bounds__(256) void attn_prefill_dma_kernel(
+template <int DPAD, int NQB, int STAGES, int NW>
+__global__ __launch_bounds__(NW * 64, (NW == 8 ? 4 : 1)) void attn_prefill_dma_kernel(
     const bf16_t* __restrict__ q, long q_stride, bf16_t* __restrict__ out, long out_stride,
     const bf16_t* __restrict__ k_pages, const bf16_t* __restrict__ v_pages, const int* __restrict__ block_tables,
     int btw, const int* __restrict__ tiles, const int* __restrict__ seg, const int* __restrict__ pos, int nh, int nkv,
@@ -300,7 +311,8 @@ __global__ __launch_bounds__(256) void attn_prefill_dma_kernel(
   constexpr bool PR_POW2 = (PR & (PR - 1)) == 0;
   constexpr int KTILE = 32 * DPAD * 2;           // bytes; the V^T tile has the same size
   constexpr int STAGE = 2 * KTILE;
-  constexpr int LPW = DPAD / 32;                 // transfers per wave and stage (DPAD / 8 in all)
+  constexpr int LPW = DPAD / (8 * NW);           // transfers per wave and stage (DPAD / 8 in all)
+  static_assert(LPW * 8 * NW == DPAD && NW * NQB == 8, "the waves share the transfers evenly and hold 128 rows");
   extern __shared__ __align__(16) unsigned char lds_raw[];   // [STAGES][STAGE], then the block table
   int* lds_bt = reinterpret_cast<int*>(lds_raw + STAGES * STAGE);
   // Which (tile, kv head, block of heads) this workgroup takes. The caller lists the tiles with the most keys
@@ -327,7 +339,7 @@ __global__ __launch_bounds__(256) void attn_prefill_dma_kernel(
   const int n_steps = (p_last - k_begin) / 32 + 1;
   const int blk0 = k_begin >> ps_log2;                                   // first block of the table that is needed
   const int n_blk = min(min(btw, (p_last >> ps_log2) + 1) - blk0, bt_cap);   // the host made sure bt_cap suffices
-  for (int i = tid; i < n_blk; i += 256) lds_bt[i] = bt[blk0 + i];
+  for (int i = tid; i < n_blk; i += NW * 64) lds_bt[i] = bt[blk0 + i];
 
   int rpos[NQB], rlo[NQB];
   long qoff[NQB], ooff[NQB];
@@ -379,7 +391,7 @@ __global__ __launch_bounds__(256) void attn_prefill_dma_kernel(
   }
 
   // what this lane moves in every step: transfer i of the wave covers pieces j * 64 .. j * 64 + 63 of a stage,
-  // j = w + 4 i; the first DPAD / 16 transfers are the K tile, the others the V^T tile. A step starts at a
+  // j = w + NW i; the first DPAD / 16 transfers are the K tile, the others the V^T tile. A step starts at a
   // multiple of 32 keys and pages are powers of two, so a key's block and its place in the page are each a
   // part that is the same for the whole wave (from the step) plus a part that never changes (from the lane).
   const unsigned page_stride = (unsigned)(nkv * d) << ps_log2;   // elements per page, K and V alike
@@ -388,7 +400,7 @@ __global__ __launch_bounds__(256) void attn_prefill_dma_kernel(
   const bf16_t* t_base[LPW];   // the pages plus everything of the offset that never changes
 #pragma unroll
   for (int i = 0; i < LPW; ++i) {
-    const int j = w + 4 * i;
+    const int j = w + NW * i;
     if (j < DPAD / 16) {
       const int P = j * 64 + l;
       const int row = P / PR, slot = P - row * PR;
@@ -442,22 +454,34 @@ __global__ __launch_bounds__(256) void attn_prefill_dma_kernel(
     for (int s = 0; s < DS; ++s) asm volatile("" : "+v"(qf[j][s].v));
   __syncthreads();   // the block table is in LDS
 
+  // The pages of this lane's transfers are looked up one step before the transfers are issued, so that the
+  // way to LDS and back is over by then (looked up where they are needed, the four lookups of a step cost a
+  // wave that runs alone on its SIMD a tenth of the step).
+  int page_of[LPW];
+  auto lookup = [&](int kb) {
+    const int blk_step = (kb >> ps_log2) - blk0;              // the step's part, the same for the wave
+#pragma unroll
+    for (int i = 0; i < LPW; ++i)
+      page_of[i] = lds_bt[max(0, min(blk_step + t_blk[i], n_blk - 1))];   // keys beyond the last block are masked: any valid page
+  };
   // this wave's transfers of the step that starts at key kb, into the stage at byte ``stage_byte``
   auto issue = [&](int kb, int stage_byte) {
-    const int blk_step = (kb >> ps_log2) - blk0, in_page = kb & pm;   // the step's parts, the same for the wave
+    const int in_page = kb & pm;
 #pragma unroll
     for (int i = 0; i < LPW; ++i) {
-      const int blk = min(blk_step + t_blk[i], n_blk - 1);   // keys beyond the last block are masked: any valid page
-      const unsigned long long off =
-          (unsigned long long)(unsigned)lds_bt[blk] * page_stride + (unsigned)(in_page * t_mul[i]);
+      const unsigned long long off = (unsigned long long)(unsigned)page_of[i] * page_stride + (unsigned)(in_page * t_mul[i]);
       global_to_lds_16(t_base[i] + off, __builtin_amdgcn_readfirstlane(lds_address(lds_raw) + stage_byte +
-                                                                       (w + 4 * i) * 1024));
+                                                                       (w + NW * i) * 1024));
     }
   };
 
 #pragma unroll
   for (int s = 0; s < STAGES - 1; ++s)
-    if (s < n_steps) issue(k_begin + s * 32, s * STAGE);
+    if (s < n_steps) {
+      lookup(k_begin + s * 32);
+      issue(k_begin + s * 32, s * STAGE);
+    }
+  lookup(k_begin + (STAGES - 1) * 32);
 
   int consume = 0, produce = (STAGES - 1) * STAGE;   // byte offsets of the stage read now and of the one filled now
   for (int it = 0; it < n_steps; ++it) {
@@ -468,24 +492,32 @@ __global__ __launch_bounds__(256) void attn_prefill_dma_kernel(
     else
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();   // everybody's part of step ``it`` is there, and everybody is done with step ``it - 1``
-    if (it + STAGES - 1 < n_steps) issue(kbase + (STAGES - 1) * 32, produce);
+    if (it + STAGES - 1 < n_steps) {
+      issue(kbase + (STAGES - 1) * 32, produce);
+      lookup(kbase + STAGES * 32);
+    }
     produce = produce + STAGE == STAGES * STAGE ? 0 : produce + STAGE;
     if (kbase <= wmax && kbase + 31 >= wlo) {
       const unsigned char* st_base = lds_raw + consume;
+      // 2 * NQB sums that do not depend on each other, one matrix instruction of each in turn: none waits for
+      // the one before it
       f32x4_t st[2][NQB];
+      Frag8 kf[2][DS];
 #pragma unroll
-      for (int b = 0; b < 2; ++b) {
-        Frag8 kf[DS];
+      for (int b = 0; b < 2; ++b)
 #pragma unroll
-        for (int s = 0; s < DS; ++s) kf[s].q = *reinterpret_cast<const uint4*>(st_base + koff[b][s]);
+        for (int s = 0; s < DS; ++s) kf[b][s].q = *reinterpret_cast<const uint4*>(st_base + koff[b][s]);
 #pragma unroll
-        for (int j = 0; j < NQB; ++j) {
-          f32x4_t a = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+      for (int b = 0; b < 2; ++b)
 #pragma unroll
-          for (int s = 0; s < DS; ++s) a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[s].v, qf[j][s].v, a, 0, 0, 0);
-          st[b][j] = a;
-        }
-      }
+        for (int j = 0; j < NQB; ++j) st[b][j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < DS; ++s)
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+          for (int j = 0; j < NQB; ++j)
+            st[b][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[b][s].v, qf[j][s].v, st[b][j], 0, 0, 0);
       // the V^T fragments are asked for now and used after the softmax, which covers their way from LDS
       Frag8 vf[DV];
 #pragma unroll
@@ -579,8 +611,12 @@ static int launch_prefill_dma(dim3 grid, hipStream_t stream, const bf16_t* q, lo
   // four stages of a head size of 128 and the table are 72 KB: two workgroups share a compute unit's LDS,
   // and one's softmax runs beside the other's matrix products
   constexpr int STAGES = DPAD <= 128 ? 4 : 3;
+  // Eight waves of 16 rows each where the transfers divide evenly among them (head sizes of 64 and 128), else
+  // four waves of 32 rows: the workgroup of a long tile that is alone on its compute unit then still has two
+  // waves on every SIMD, which hide each other's waits.
+  constexpr int NW = (DPAD == 64 || DPAD == 128) ? 8 : 4;
   const size_t smem = (size_t)STAGES * 4 * 32 * DPAD + PREFILL_BT_CAP * sizeof(int);
-  auto kernel = attn_prefill_dma_kernel<DPAD, 2, STAGES>;
+  auto kernel = attn_prefill_dma_kernel<DPAD, 8 / NW, STAGES, NW>;
   static bool configured = false;   // per instantiation
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -591,8 +627,8 @@ static int launch_prefill_dma(dim3 grid, hipStream_t stream, const bf16_t* q, lo
     }
     configured = true;
   }
-  hipLaunchKernelGGL(kernel, dim3(grid.x * grid.y), dim3(256), smem, stream, q, q_stride, out, out_stride, k_pages, v_pages,
-                     block_tables, btw, tiles, seg, pos, nh, nkv, d, ps_log2, scale_log2, window, HB, n_hb,
+  hipLaunchKernelGGL(kernel, dim3(grid.x * grid.y), dim3(NW * 64), smem, stream, q, q_stride, out, out_stride, k_pages,
+                     v_pages, block_tables, btw, tiles, seg, pos, nh, nkv, d, ps_log2, scale_log2, window, HB, n_hb,
                      PREFILL_BT_CAP, lmsf_compute_units());
   return 0;
 }
