@@ -244,7 +244,8 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
   }
 }
 
-// The same with the keys and values staged in LDS by the workgroup and read from there by its four waves;
+// The same with the keys and values staged in LDS by the workgroup and read from there by its waves (NW: eight
+// of 16 rows where the transfers divide evenly among them, else four of 32 rows);
 // the kernel above has every wave fetch them from global memory for itself and spends its time waiting.
 // Here tiles of 32 keys travel from global memory straight into LDS (global_load_lds_dwordx4: lane i of a
 // wave writes its 16 bytes at the wave's LDS base + 16 i, whatever global address it reads), STAGES - 1
@@ -289,16 +290,18 @@ __device__ __forceinline__ unsigned lds_address(const void* p) {
 // How far (in powers of two) a row's scores may rise above the reference of its exponentials before the
 // accumulators are rescaled: 2^24 times a few thousand keys times the values stays far inside float32.
 //
-// What bounds it (measured with timestamps inside the kernel and with parts of the step taken out): a wave that
-// is alone on its SIMD takes 970 ns for a step whose 32 matrix instructions need 250: the vector instructions
-// around them (scale, exponential, sum, conversion: 250 ns even with everything else removed), the waits for
-// LDS, the transfers and the barrier each add their own share, because one wave issues one instruction at a
-// time and a v_exp_f32 never runs beside a matrix instruction (a fused multiply-add does: measured apart). Two
-// waves on a SIMD hide most of that from each other (600 ns for the two), and more do not fit the registers.
-// At 2,048 tokens the longest tile's workgroup is alone on its compute unit for most of its 64 steps, and the
-// kernel takes as long as that workgroup: 5 us of set-up and 64 x 970 ns; at 8,192 tokens the tiles are many
-// and the kernel reaches 0.85 PFLOP/s. Tried, measured, not kept: the next step's scores multiplied beside the
-// current step's exponentials, in the order fixed with scheduling groups (the same times within 3 percent).
+// What bounds it (measured with timestamps inside the kernel, with parts of the step taken out, and with
+// counters): the matrix pipe is busy 35 percent of the time, the vector issue port 60 percent, both at once 13
+// percent; a step's 32 matrix instructions a SIMD need 250 ns, the step takes 520 ns where two workgroups share a
+// compute unit (8,192 tokens: 0.88 PFLOP/s) and 860 ns where one is alone. Around the matrix instructions stand,
+// per 16 rows and 32 keys, 84 vector instructions (scale, exponential, sum, conversion, largest score, the
+// transfers' addresses), the waits for LDS and the barrier; a v_exp_f32 never runs beside a matrix instruction (a
+// fused multiply-add does: measured apart), and a wave issues one instruction at a time, so what hides these is
+// other waves: eight waves of 16 rows (four on a SIMD, two of them the workgroup's own) against four waves of 32
+// rows (two on a SIMD) took 13 percent off at 2,048 tokens, where the longest tile's workgroup is alone on its
+// compute unit for most of its 64 steps and the kernel takes as long as that workgroup (4.4 us of set-up, 64 x
+// 860 ns). Tried, measured, not kept: the next step's scores multiplied beside the current step's exponentials,
+// in the order fixed with scheduling groups (four waves of 32 rows: the same times within 3 percent).
 #define PREFILL_LAZY_LOG2 24.0f
 template <int DPAD, int NQB, int STAGES, int NW>
 __global__ __launch_bounds__(NW * 64, (NW == 8 ? 4 : 1)) void attn_prefill_dma_kernel(
@@ -462,7 +465,7 @@ __global__ __launch_bounds__(NW * 64, (NW == 8 ? 4 : 1)) void attn_prefill_dma_k
     const int blk_step = (kb >> ps_log2) - blk0;              // the step's part, the same for the wave
 #pragma unroll
     for (int i = 0; i < LPW; ++i)
-      page_of[i] = lds_bt[max(0, min(blk_step + t_blk[i], n_blk - 1))];   // keys beyond the last block are masked: any valid page
+      page_of[i] = lds_bt[min(blk_step + t_blk[i], n_blk - 1)];   // keys beyond the last block are masked: any valid page
   };
   // this wave's transfers of the step that starts at key kb, into the stage at byte ``stage_byte``
   auto issue = [&](int kb, int stage_byte) {
