@@ -29,6 +29,8 @@
 #include <limits.h>
 #include <math.h>
 
+#include <type_traits>
+
 union Frag8 {
   bf16x8_t v;
   uint4 q;
@@ -302,7 +304,14 @@ __device__ __forceinline__ unsigned lds_address(const void* p) {
 // compute unit for most of its 64 steps and the kernel takes as long as that workgroup (4.4 us of set-up, 64 x
 // 860 ns). Tried, measured, not kept: the next step's scores multiplied beside the current step's exponentials,
 // in the order fixed with scheduling groups (four waves of 32 rows: the same times within 3 percent).
+// Also not kept: two groups of eight waves in a workgroup of 16, each with half of a tile's keys, put together
+// through LDS at the end (the longest tile would take half the steps): 66.6 against 63.9 us at 2,048 tokens,
+// 727 against 626 at 8,192; a barrier over 16 waves and one workgroup a compute unit cost more than the balance gives.
 #define PREFILL_LAZY_LOG2 24.0f
+// Entries of a block table that the LDS-staged kernel can keep beside its stages, and how many copies of the
+// last entry follow it there.
+#define PREFILL_BT_CAP 2048
+#define PREFILL_BT_PAD 8
 template <int DPAD, int NQB, int STAGES, int NW>
 __global__ __launch_bounds__(NW * 64, (NW == 8 ? 4 : 1)) void attn_prefill_dma_kernel(
     const bf16_t* __restrict__ q, long q_stride, bf16_t* __restrict__ out, long out_stride,
@@ -342,7 +351,8 @@ __global__ __launch_bounds__(NW * 64, (NW == 8 ? 4 : 1)) void attn_prefill_dma_k
   const int n_steps = (p_last - k_begin) / 32 + 1;
   const int blk0 = k_begin >> ps_log2;                                   // first block of the table that is needed
   const int n_blk = min(min(btw, (p_last >> ps_log2) + 1) - blk0, bt_cap);   // the host made sure bt_cap suffices
-  for (int i = tid; i < n_blk; i += NW * 64) lds_bt[i] = bt[blk0 + i];
+  // (PREFILL_BT_PAD entries after the last one repeat it: the lookups of the steps ahead need no bound then)
+  for (int i = tid; i < n_blk + PREFILL_BT_PAD; i += NW * 64) lds_bt[i] = bt[blk0 + min(i, n_blk - 1)];
 
   int rpos[NQB], rlo[NQB];
   long qoff[NQB], ooff[NQB];
@@ -366,10 +376,10 @@ __global__ __launch_bounds__(NW * 64, (NW == 8 ? 4 : 1)) void attn_prefill_dma_k
       wmaxlo = max(wmaxlo, rlo[j]);
     }
   }
-  wmax = wave_max_i(wmax);
-  wlo = wave_min_i(wlo);
-  wminpos = wave_min_i(wminpos);   // a step whose keys all lie in [wmaxlo, wminpos] needs no mask
-  wmaxlo = wave_max_i(wmaxlo);
+  wmax = __builtin_amdgcn_readfirstlane(wave_max_i(wmax));
+  wlo = __builtin_amdgcn_readfirstlane(wave_min_i(wlo));
+  wminpos = __builtin_amdgcn_readfirstlane(wave_min_i(wminpos));   // a step whose keys all lie in [wmaxlo, wminpos] needs no mask
+  wmaxlo = __builtin_amdgcn_readfirstlane(wave_max_i(wmaxlo));
 
   Frag8 qf[NQB][DS];
 #pragma unroll
@@ -384,10 +394,13 @@ __global__ __launch_bounds__(NW * 64, (NW == 8 ? 4 : 1)) void attn_prefill_dma_k
     }
 
   f32x4_t acc[DV][NQB];
-  float m[NQB], lsum[NQB];
+  // (neg_m: what is added to a scaled score before the exponential; a row that has seen nothing yet has only
+  // masked keys: exp2(-inf) = 0 whatever is added)
+  float m[NQB], neg_m[NQB], lsum[NQB];
 #pragma unroll
   for (int j = 0; j < NQB; ++j) {
     m[j] = -INFINITY;
+    neg_m[j] = 0.f;
     lsum[j] = 0.f;
 #pragma unroll
     for (int v = 0; v < DV; ++v) acc[v][j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
@@ -465,7 +478,7 @@ __global__ __launch_bounds__(NW * 64, (NW == 8 ? 4 : 1)) void attn_prefill_dma_k
     const int blk_step = (kb >> ps_log2) - blk0;              // the step's part, the same for the wave
 #pragma unroll
     for (int i = 0; i < LPW; ++i)
-      page_of[i] = lds_bt[min(blk_step + t_blk[i], n_blk - 1)];   // keys beyond the last block are masked: any valid page
+      page_of[i] = lds_bt[min(blk_step, n_blk) + t_blk[i]];   // keys beyond the last block are masked: any valid page
   };
   // this wave's transfers of the step that starts at key kb, into the stage at byte ``stage_byte``
   auto issue = [&](int kb, int stage_byte) {
@@ -486,8 +499,11 @@ __global__ __launch_bounds__(NW * 64, (NW == 8 ? 4 : 1)) void attn_prefill_dma_k
     }
   lookup(k_begin + (STAGES - 1) * 32);
 
-  int consume = 0, produce = (STAGES - 1) * STAGE;   // byte offsets of the stage read now and of the one filled now
-  for (int it = 0; it < n_steps; ++it) {
+  // One step; SI: which stage holds it (a constant, so that the places of the operands in LDS are constants in
+  // the instructions and cost no additions).
+  auto step = [&](auto SI, int it) {
+    constexpr int consume = decltype(SI)::value * STAGE;                                  // the stage read now
+    constexpr int produce = ((decltype(SI)::value + STAGES - 1) % STAGES) * STAGE;       // the stage filled now
     const int kbase = k_begin + it * 32;
     // step ``it`` has arrived when at most the transfers of the later steps are outstanding
     if (it + STAGES - 2 < n_steps)
@@ -499,7 +515,6 @@ __global__ __launch_bounds__(NW * 64, (NW == 8 ? 4 : 1)) void attn_prefill_dma_k
       issue(kbase + (STAGES - 1) * 32, produce);
       lookup(kbase + STAGES * 32);
     }
-    produce = produce + STAGE == STAGES * STAGE ? 0 : produce + STAGE;
     if (kbase <= wmax && kbase + 31 >= wlo) {
       const unsigned char* st_base = lds_raw + consume;
       // 2 * NQB sums that do not depend on each other, one matrix instruction of each in turn: none waits for
@@ -543,28 +558,28 @@ __global__ __launch_bounds__(NW * 64, (NW == 8 ? 4 : 1)) void attn_prefill_dma_k
             if (key > rpos[j] || key < rlo[j]) r[e] = -INFINITY;
           }
         }
-        float mx = fmaxf(fmaxf(fmaxf(r[0], r[1]), fmaxf(r[2], r[3])), fmaxf(fmaxf(r[4], r[5]), fmaxf(r[6], r[7])));
-        mx = max_over_lane_groups(mx);
+        const float mx = fmaxf(fmaxf(fmaxf(r[0], r[1]), fmaxf(r[2], r[3])), fmaxf(fmaxf(r[4], r[5]), fmaxf(r[6], r[7])));
         // m is the reference the exponentials are taken against, not the running maximum: any reference gives
         // the same softmax as long as nothing overflows, and bfloat16 probabilities and float32 sums have room
         // for 2^LAZY above it. So the accumulators (which the matrix cores hold where other instructions cannot
         // reach them without copies) are rescaled only when a row's scores rise that far above its reference,
-        // which after a row's first step happens almost never.
-        const float cand = mx * scale_log2;                    // the scale is positive
-        if (__builtin_expect(__any(cand > m[j] + PREFILL_LAZY_LOG2), 0)) {
+        // which after a row's first step happens almost never. The four lanes that hold a row's scores need
+        // the same reference, so the row's largest score is taken over them, but only where one of them has
+        // found a score that far up.
+        if (__builtin_expect(__any(mx * scale_log2 > m[j] + PREFILL_LAZY_LOG2), 0)) {   // the scale is positive
+          const float cand = max_over_lane_groups(mx) * scale_log2;
           const float m_new = cand > m[j] + PREFILL_LAZY_LOG2 ? cand : m[j];
           const float corr = (m[j] == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m[j] - m_new);   // nothing summed yet: keep
           lsum[j] *= corr;
 #pragma unroll
           for (int v = 0; v < DV; ++v) acc[v][j] *= corr;
           m[j] = m_new;
+          neg_m[j] = (m_new == -INFINITY) ? 0.f : -m_new;
         }
-        // a row that has seen nothing yet has only masked keys here: exp2(-inf) = 0 whatever is subtracted
-        const float neg_m = (m[j] == -INFINITY) ? 0.f : -m[j];
         float pv[8], ps_ = 0.f;
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-          pv[e] = __builtin_amdgcn_exp2f(fmaf(r[e], scale_log2, neg_m));
+          pv[e] = __builtin_amdgcn_exp2f(fmaf(r[e], scale_log2, neg_m[j]));
           ps_ += pv[e];
         }
         lsum[j] += ps_;
@@ -578,7 +593,13 @@ __global__ __launch_bounds__(NW * 64, (NW == 8 ? 4 : 1)) void attn_prefill_dma_k
 #pragma unroll
         for (int j = 0; j < NQB; ++j) acc[v][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[v].v, pf[j].v, acc[v][j], 0, 0, 0);
     }
-    consume = consume + STAGE == STAGES * STAGE ? 0 : consume + STAGE;
+  };
+  for (int it = 0; it < n_steps; it += STAGES) {
+    step(std::integral_constant<int, 0>(), it);
+    if (it + 1 < n_steps) step(std::integral_constant<int, 1>(), it + 1);
+    if (it + 2 < n_steps) step(std::integral_constant<int, 2>(), it + 2);
+    if constexpr (STAGES == 4)
+      if (it + 3 < n_steps) step(std::integral_constant<int, 3>(), it + 3);
   }
 
 #pragma unroll
@@ -601,8 +622,6 @@ __global__ __launch_bounds__(NW * 64, (NW == 8 ? 4 : 1)) void attn_prefill_dma_k
   }
 }
 
-// Entries of a block table that the LDS-staged kernel can keep beside its stages.
-#define PREFILL_BT_CAP 2048
 
 template <int DPAD>
 static int launch_prefill_dma(dim3 grid, hipStream_t stream, const bf16_t* q, long q_stride, bf16_t* out,
@@ -618,7 +637,7 @@ static int launch_prefill_dma(dim3 grid, hipStream_t stream, const bf16_t* q, lo
   // four waves of 32 rows: the workgroup of a long tile that is alone on its compute unit then still has two
   // waves on every SIMD, which hide each other's waits.
   constexpr int NW = (DPAD == 64 || DPAD == 128) ? 8 : 4;
-  const size_t smem = (size_t)STAGES * 4 * 32 * DPAD + PREFILL_BT_CAP * sizeof(int);
+  const size_t smem = (size_t)STAGES * 4 * 32 * DPAD + (PREFILL_BT_CAP + PREFILL_BT_PAD) * sizeof(int);
   auto kernel = attn_prefill_dma_kernel<DPAD, 8 / NW, STAGES, NW>;
   static bool configured = false;   // per instantiation
   if (!configured) {
