@@ -293,16 +293,16 @@ __device__ __forceinline__ unsigned lds_address(const void* p) {
 // accumulators are rescaled: 2^24 times a few thousand keys times the values stays far inside float32.
 //
 // What bounds it (measured with timestamps inside the kernel, with parts of the step taken out, and with
-// counters): the matrix pipe is busy 35 percent of the time, the vector issue port 60 percent, both at once 13
-// percent; a step's 32 matrix instructions a SIMD need 250 ns, the step takes 520 ns where two workgroups share a
-// compute unit (8,192 tokens: 0.88 PFLOP/s) and 860 ns where one is alone. Around the matrix instructions stand,
-// per 16 rows and 32 keys, 84 vector instructions (scale, exponential, sum, conversion, largest score, the
+// counters): the matrix pipe is busy 39 percent of the time, the vector issue port 56 percent, both at once 15
+// percent; a step's 32 matrix instructions a SIMD need 250 ns, the step takes 490 ns where two workgroups share a
+// compute unit (8,192 tokens: 0.94 PFLOP/s) and 800 ns where one is alone. Around the matrix instructions stand,
+// per 16 rows and 32 keys, 67 vector instructions (scale, exponential, sum, conversion, largest score, the
 // transfers' addresses), the waits for LDS and the barrier; a v_exp_f32 never runs beside a matrix instruction (a
 // fused multiply-add does: measured apart), and a wave issues one instruction at a time, so what hides these is
 // other waves: eight waves of 16 rows (four on a SIMD, two of them the workgroup's own) against four waves of 32
 // rows (two on a SIMD) took 13 percent off at 2,048 tokens, where the longest tile's workgroup is alone on its
-// compute unit for most of its 64 steps and the kernel takes as long as that workgroup (4.4 us of set-up, 64 x
-// 860 ns). Tried, measured, not kept: the next step's scores multiplied beside the current step's exponentials,
+// compute unit for most of its 64 steps and the kernel takes as long as that workgroup (4.4 us of set-up, 64
+// steps). Tried, measured, not kept: the next step's scores multiplied beside the current step's exponentials,
 // in the order fixed with scheduling groups (four waves of 32 rows: the same times within 3 percent).
 // Also not kept: two groups of eight waves in a workgroup of 16, each with half of a tile's keys, put together
 // through LDS at the end (the longest tile would take half the steps): 66.6 against 63.9 us at 2,048 tokens,
