@@ -229,6 +229,31 @@ def test_matrix_core_attention_other_ways_of_cutting_the_work(ops, ref, shape, v
     assert torch.allclose(a.float(), b.float(), **tol(torch.bfloat16)), (a.float() - b.float()).abs().max()
 
 
+@pytest.mark.parametrize("d,ps", [(64, 16), (96, 8), (128, 16), (128, 32), (160, 16)])
+def test_prefill_attention_every_number_of_steps(ops, ref, d, ps):
+    """The LDS-staged prefill kernel walks the keys in steps of 32 through a ring of three or four stages, its
+    loop unrolled by the stages, with the pages of the steps ahead looked up in a padded copy of the block table:
+    prompts of 1 to 12 steps (every remainder of the ring, a last page that is full, one that holds a single
+    token), alone and after a context, in head sizes that run with eight waves of 16 rows (64, 128), four of 32
+    (96) and three stages (160)."""
+    nh, nkv = 4, 2
+    scale = 1.0 / math.sqrt(d)
+    for seg_lens, ctx_lens in (([1, 31, 32, 33], [1, 31, 32, 33]), ([64, 65, 95], [64, 65, 95]),
+                               ([128, 129, 97], [128, 129, 97]), ([160, 200, 256], [160, 200, 256]),
+                               ([290, 383], [290, 383]), ([3, 40, 17], [99, 232, 385]), ([33], [321])):
+        q, kp, vp, bt, seg, pos = _paged_case(torch.bfloat16, nh, nkv, d, ps, seg_lens, ctx_lens,
+                                              seed=d + ps + sum(ctx_lens), spike=True)
+        want = ref.paged_attention(q, kp, vp, bt, seg, pos, nh, nkv, d, scale, 0)
+        got = ops.paged_attention(q, kp, vp, bt, seg, pos, nh, nkv, d, scale, 0, kernel="mfma")
+        assert torch.allclose(got.float(), want.float(), **tol(torch.bfloat16)), \
+            (seg_lens, ctx_lens, (got.float() - want.float()).abs().max())
+        for window in (33, 100):
+            want = ref.paged_attention(q, kp, vp, bt, seg, pos, nh, nkv, d, scale, window)
+            got = ops.paged_attention(q, kp, vp, bt, seg, pos, nh, nkv, d, scale, window, kernel="mfma")
+            assert torch.allclose(got.float(), want.float(), **tol(torch.bfloat16)), \
+                (seg_lens, ctx_lens, window, (got.float() - want.float()).abs().max())
+
+
 @pytest.mark.parametrize("order", [1, 2])
 def test_decode_attention_in_a_given_order_of_tokens(ops, ref, order):
     """A step of single tokens whose contexts differ, with the tokens listed longest context first and either
