@@ -226,8 +226,9 @@ def serve_run(args, emit=True):
 
 def products_run(args):
     """The four matrix products of a layer at the headline shape, for some numbers of rows: the BLAS library's
-    (through torch) against this package's choice (``HipOps.linear`` / ``linear_gated``), microseconds by HIP
-    events around a HIP graph of eight calls, the weight read from memory every time. One JSON line per product and number of rows."""
+    (through torch) against this package's choice (``HipOps.linear`` / ``linear_gated``). Microseconds by HIP
+    events around a HIP graph of eight calls (no host time between the kernels), the weight read from memory
+    every time. One JSON line per product and number of rows."""
     import torch
     from lmsf_amd.ops import get_ops
     ops = get_ops()
