@@ -254,6 +254,37 @@ def test_prefill_attention_every_number_of_steps(ops, ref, d, ps):
                 (seg_lens, ctx_lens, window, (got.float() - want.float()).abs().max())
 
 
+def test_matrix_core_attention_random_geometries(ops):
+    """Sixty random geometries (heads, groups, head sizes in steps of 16, page sizes, windows, mixes of single
+    tokens and portions of prompts after contexts of any length): the matrix-core kernels against the general
+    kernel, which the other tests hold against the plain implementation."""
+    g = torch.Generator().manual_seed(2024)
+
+    def pick(options):
+        return options[int(torch.randint(0, len(options), (1,), generator=g))]
+
+    for case in range(60):
+        nkv = pick([1, 2, 3, 8])
+        nh = nkv * pick([1, 2, 4, 5])
+        d = pick([16, 32, 48, 64, 80, 96, 112, 128, 160, 256])
+        ps = pick([4, 8, 16, 32, 64])
+        window = pick([0, 0, 7, 64, 300])
+        n_seg = pick([1, 2, 3, 5])
+        seg_lens, ctx_lens = [], []
+        for _ in range(n_seg):
+            new = pick([1, 1, 2, 17, 33, 70, 130])
+            before = pick([0, 0, 1, 15, 31, 32, 100, 257, 600])
+            seg_lens.append(new)
+            ctx_lens.append(new + before)
+        q, kp, vp, bt, seg, pos = _paged_case(torch.bfloat16, nh, nkv, d, ps, seg_lens, ctx_lens, seed=case, spike=True)
+        scale = 1.0 / math.sqrt(d)
+        a = ops.paged_attention(q, kp, vp, bt, seg, pos, nh, nkv, d, scale, window, kernel="mfma")
+        b = ops.paged_attention(q, kp, vp, bt, seg, pos, nh, nkv, d, scale, window, kernel="generic")
+        err = (a.float() - b.float()).abs().max().item()
+        assert torch.allclose(a.float(), b.float(), **tol(torch.bfloat16)), \
+            (case, nh, nkv, d, ps, window, seg_lens, ctx_lens, err)
+
+
 @pytest.mark.parametrize("order", [1, 2])
 def test_decode_attention_in_a_given_order_of_tokens(ops, ref, order):
     """A step of single tokens whose contexts differ, with the tokens listed longest context first and either
