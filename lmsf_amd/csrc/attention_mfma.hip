@@ -670,7 +670,10 @@ static int launch_prefill_dma(dim3 grid, hipStream_t stream, const bf16_t* q, lo
 // longer: each fence writes back or drops what the die's L2 holds. With stores and loads at device scope and a
 // wait for the stores' acknowledgement instead of the fences, the three trips to memory in a row (results,
 // counter, results) cost what the second kernel's start costs: 10.8 against 9.9 us at 8 tokens of 585 keys, 12.5
-// against 13.8 at 1,024 keys, 18 against 23 at one token of 8,000 keys in 16 splits. Not kept.)
+// against 13.8 at 1,024 keys, 18 against 23 at one token of 8,000 keys in 16 splits. Not kept. Nor were
+// workgroups of 16 waves that take a context's keys unsplit and need no second kernel: 26.8 against 12.6 us at 8
+// tokens of 585 keys, with keys and values that come from memory; one compute unit pulls a context's 300 KB far
+// slower than eight do.)
 template <int DPAD>
 __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
     const bf16_t* __restrict__ q, long q_stride, const bf16_t* __restrict__ k_pages,
