@@ -54,8 +54,8 @@ __device__ __forceinline__ float large_activation(float g, float u, int act) {
 // BM: rows of x per workgroup (128 or 256). BN: rows of W per workgroup (128 or 256; with ACT half of them gate rows
 // and half the up rows of the same outputs). ACT: 0 none, 1 SiLU-gated, 2 GELU-gated. PARTIAL: float32 partial sums
 // of this workgroup's part of K instead of the result (not with ACT).
-template <int BM, int BN, int STAGES, int ACT, bool PARTIAL>
-__global__ __launch_bounds__(256) void gemm_large_kernel(const bf16_t* __restrict__ x, long ldx,
+template <int BM, int BN, int STAGES, int ACT, bool PARTIAL, int KG>
+__global__ __launch_bounds__(256 * KG) void gemm_large_kernel(const bf16_t* __restrict__ x, long ldx,
                                                          const bf16_t* __restrict__ W, long ldw,
                                                          const bf16_t* __restrict__ bias, bf16_t* __restrict__ y,
                                                          long ldy, float* __restrict__ part, int M, int N, int K,
@@ -64,10 +64,15 @@ __global__ __launch_bounds__(256) void gemm_large_kernel(const bf16_t* __restric
   constexpr int MT = BM / 32;                      // accumulator tiles along x per wave
   constexpr int NT = BN / 32;                      // along W
   constexpr int W_BYTES = BN * LARGE_ROW, X_BYTES = BM * LARGE_ROW, STAGE = W_BYTES + X_BYTES;
-  constexpr int W_LOADS = BN / 8 / 4, X_LOADS = BM / 8 / 4;   // transfers of 8 rows per wave and step
+  // KG groups of four waves: with two, both hold the same tile of outputs and each multiplies one 32-wide half of
+  // every step, so that a SIMD has two waves and one's matrix instructions run while the other waits for its
+  // operands; the groups' sums are added through LDS at the end.
+  constexpr int W_LOADS = BN / 8 / (4 * KG), X_LOADS = BM / 8 / (4 * KG);   // transfers of 8 rows per wave and step
+  static_assert(W_LOADS * 8 * 4 * KG == BN && X_LOADS * 8 * 4 * KG == BM, "the waves share the transfers evenly");
   constexpr int LPW = W_LOADS + X_LOADS;
   extern __shared__ __align__(16) unsigned char lds[];
-  const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
+  const int tid = threadIdx.x, wave = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
+  const int kg = KG == 1 ? 0 : wave >> 2, w = wave & 3;
   const int wm = w & 1, wn = w >> 1;
 
   // which tile: all row tiles of one panel of W on one XCD, next to each other in time
@@ -107,22 +112,23 @@ __global__ __launch_bounds__(256) void gemm_large_kernel(const bf16_t* __restric
   unsigned dst[LPW];                               // byte offset inside a stage; the same for all lanes of the wave
 #pragma unroll
   for (int i = 0; i < W_LOADS; ++i) {
-    const int j = (w * W_LOADS + i) * 8 + trow, piece = (tslot - j) & 7;
+    const int j = (wave * W_LOADS + i) * 8 + trow, piece = (tslot - j) & 7;
     src[i] = W + (long)w_row(j) * ldw + piece * 8 + (long)c_begin * 64;
-    dst[i] = (w * W_LOADS + i) * 8 * LARGE_ROW;
+    dst[i] = (wave * W_LOADS + i) * 8 * LARGE_ROW;
   }
 #pragma unroll
   for (int i = 0; i < X_LOADS; ++i) {
-    const int j = (w * X_LOADS + i) * 8 + trow, piece = (tslot - j) & 7;
+    const int j = (wave * X_LOADS + i) * 8 + trow, piece = (tslot - j) & 7;
     int m = m0 + j;
     if (m > M - 1) m = M - 1;
     src[W_LOADS + i] = x + (long)m * ldx + piece * 8 + (long)c_begin * 64;
-    dst[W_LOADS + i] = W_BYTES + (w * X_LOADS + i) * 8 * LARGE_ROW;
+    dst[W_LOADS + i] = W_BYTES + (wave * X_LOADS + i) * 8 * LARGE_ROW;
   }
   // where this lane reads its operands in a 16-row tile: row r, pieces 4 s + g of the two 32-wide halves of a step
   int foff[2];
 #pragma unroll
   for (int s = 0; s < 2; ++s) foff[s] = r * LARGE_ROW + (((s * 4 + g) + r) & 7) * 16;
+  const int foff_mine = foff[kg];                  // with two groups: the half of a step that this group multiplies
 
   f32x4_t acc[NT][MT];
 #pragma unroll
@@ -153,14 +159,15 @@ __global__ __launch_bounds__(256) void gemm_large_kernel(const bf16_t* __restric
     produce = produce + STAGE == STAGES * STAGE ? 0 : produce + STAGE;
     const unsigned char* st = lds + consume;
 #pragma unroll
-    for (int s = 0; s < 2; ++s) {
+    for (int s = 0; s < 2 / KG; ++s) {
+      const int fo = KG == 2 ? foff_mine : foff[s];
       bf16x8_t a[NT], bb[MT];
 #pragma unroll
       for (int t = 0; t < NT; ++t)
-        a[t] = *reinterpret_cast<const bf16x8_t*>(st + a_base + t * 16 * LARGE_ROW + foff[s]);
+        a[t] = *reinterpret_cast<const bf16x8_t*>(st + a_base + t * 16 * LARGE_ROW + fo);
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
-        bb[mt] = *reinterpret_cast<const bf16x8_t*>(st + b_base + mt * 16 * LARGE_ROW + foff[s]);
+        bb[mt] = *reinterpret_cast<const bf16x8_t*>(st + b_base + mt * 16 * LARGE_ROW + fo);
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -169,6 +176,24 @@ __global__ __launch_bounds__(256) void gemm_large_kernel(const bf16_t* __restric
     consume = consume + STAGE == STAGES * STAGE ? 0 : consume + STAGE;
   }
 
+  if constexpr (KG == 2) {
+    // the second group's sums go to the first through LDS (the stages are done with), lane to lane
+    static_assert((size_t)4 * NT * MT * 1024 <= (size_t)STAGES * STAGE, "the exchange fits the stages");
+    __syncthreads();
+    f32x4_t* xch = reinterpret_cast<f32x4_t*>(lds) + (size_t)w * NT * MT * 64 + l;
+    if (kg == 1) {
+#pragma unroll
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) xch[(t * MT + mt) * 64] = acc[t][mt];
+    }
+    __syncthreads();
+    if (kg == 1) return;
+#pragma unroll
+    for (int t = 0; t < NT; ++t)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) acc[t][mt] += xch[(t * MT + mt) * 64];
+  }
   // this lane holds, for row m = m0 + BM / 2 wm + 16 mt + r of x, four neighbouring outputs per tile t
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
@@ -212,11 +237,11 @@ __global__ __launch_bounds__(256) void gemm_large_kernel(const bf16_t* __restric
   }
 }
 
-template <int BM, int BN, int STAGES, int ACT, bool PARTIAL>
+template <int BM, int BN, int STAGES, int ACT, bool PARTIAL, int KG = 1>
 static int launch_large(hipStream_t stream, const bf16_t* x, long ldx, const bf16_t* W, long ldw, const bf16_t* bias,
                         bf16_t* y, long ldy, float* part, int M, int N, int K, int n_split) {
   const size_t smem = (size_t)STAGES * (BN + BM) * LARGE_ROW;
-  auto kernel = gemm_large_kernel<BM, BN, STAGES, ACT, PARTIAL>;
+  auto kernel = gemm_large_kernel<BM, BN, STAGES, ACT, PARTIAL, KG>;
   static bool configured = false;   // per instantiation
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -230,13 +255,15 @@ static int launch_large(hipStream_t stream, const bf16_t* x, long ldx, const bf1
   constexpr int n_out = ACT ? BN / 2 : BN;
   const int tiles_m = (M + BM - 1) / BM, tiles_n = (N + n_out - 1) / n_out;
   const int groups = (tiles_n + 7) / 8;
-  hipLaunchKernelGGL(kernel, dim3(groups * tiles_m * 8, n_split), dim3(256), smem, stream, x, ldx, W, ldw, bias, y, ldy,
+  hipLaunchKernelGGL(kernel, dim3(groups * tiles_m * 8, n_split), dim3(256 * KG), smem, stream, x, ldx, W, ldw, bias, y, ldy,
                      part, M, N, K, n_split, tiles_m, tiles_n);
   return 0;
 }
 
-// The tilings: rows of x, rows of W per workgroup.
-static const int kLargeTiles[3][2] = {{128, 128}, {256, 128}, {192, 128}};
+// The tilings: rows of x, rows of W per workgroup; 3 to 5 are 0 to 2 with two groups of four waves (at 129 to 256
+// rows 2 to 6 percent faster where K is long, the same elsewhere; at 2,048 rows 6 to 14 percent, which is still
+// 0.75 to 1.0 PFLOP/s against the library's 1.05 to 1.2).
+static const int kLargeTiles[6][2] = {{128, 128}, {256, 128}, {192, 128}, {128, 128}, {256, 128}, {192, 128}};
 
 template <int ACT, bool PARTIAL>
 static int launch_tiling(int tiling, hipStream_t stream, const bf16_t* x, long ldx, const bf16_t* W, long ldw,
@@ -244,7 +271,11 @@ static int launch_tiling(int tiling, hipStream_t stream, const bf16_t* x, long l
   switch (tiling) {
     case 0: return launch_large<128, 128, 4, ACT, PARTIAL>(stream, x, ldx, W, ldw, bias, y, ldy, part, M, N, K, n_split);
     case 1: return launch_large<256, 128, 3, ACT, PARTIAL>(stream, x, ldx, W, ldw, bias, y, ldy, part, M, N, K, n_split);
-    default: return launch_large<192, 128, 4, ACT, PARTIAL>(stream, x, ldx, W, ldw, bias, y, ldy, part, M, N, K, n_split);
+    case 2: return launch_large<192, 128, 4, ACT, PARTIAL>(stream, x, ldx, W, ldw, bias, y, ldy, part, M, N, K, n_split);
+    // the same tiles with two groups of four waves
+    case 3: return launch_large<128, 128, 4, ACT, PARTIAL, 2>(stream, x, ldx, W, ldw, bias, y, ldy, part, M, N, K, n_split);
+    case 4: return launch_large<256, 128, 3, ACT, PARTIAL, 2>(stream, x, ldx, W, ldw, bias, y, ldy, part, M, N, K, n_split);
+    default: return launch_large<192, 128, 4, ACT, PARTIAL, 2>(stream, x, ldx, W, ldw, bias, y, ldy, part, M, N, K, n_split);
   }
 }
 
@@ -272,7 +303,7 @@ extern "C" int lmsf_gemm_large_plan(int M, int N, int K, int act) {
       const double traffic = s > 1 ? (double)M * N * 8.0 * s / 4.0e12 + 4.0e-6 : 0.0;
       if (product + traffic < best_cost - 1e-9) {
         best_cost = product + traffic;
-        best = tiling * 16 + s;
+        best = (tiling + 3) * 16 + s;             // (the tilings with two groups of waves)
       }
     }
   }
@@ -298,7 +329,7 @@ extern "C" int lmsf_gemm_large(const void* x, long ldx, const void* W, long ldw,
                                int M, int N, int K, int act, int plan, float* scratch, int reduce,
                                hipStream_t stream) {
   const int tiling = plan / 16, n_split = plan % 16;
-  LMSF_CHECK(tiling >= 0 && tiling < 3, "gemm_large: unknown tiling %d", tiling);
+  LMSF_CHECK(tiling >= 0 && tiling < 6, "gemm_large: unknown tiling %d", tiling);
   LMSF_CHECK(x && W && (y || (n_split > 1 && !reduce)), "gemm_large: null pointer");
   LMSF_CHECK(M > 0 && N > 0 && K > 0, "gemm_large: bad sizes M=%d N=%d K=%d", M, N, K);
   LMSF_CHECK(K % 64 == 0 && N % 8 == 0, "gemm_large: K must be a multiple of 64 and N of 8, got K=%d N=%d", K, N);
