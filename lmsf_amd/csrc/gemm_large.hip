@@ -21,6 +21,12 @@
 // 32 x 32 x 16 instruction, wave tiles of 128 x 128 and no spills (0.85 to 1.0: two stages do not cover the way from
 // memory).
 //
+// Counters of this kernel and of the library's on the same product (2,048 x 14,336 x 4,096, the weight in cache):
+// the same 1.47e7 matrix instructions; beside each of them 0.71 other vector instructions here and 0.06 there; the
+// matrix pipe busy 42 percent of the time here, with 1.6 waves a SIMD that wait 39 percent of their time, and 62
+// percent there, with one wave a SIMD. The library's loop is scheduled by hand around every wait; here two groups
+// of waves cover some of each other's (they share the step's barrier, so they wait at the same moments).
+//
 // Workgroups that share rows of W run on the same XCD, one after the other in launch order, so that a panel of W
 // comes from memory once and from that XCD's L2 afterwards: with 8 XCDs taking workgroups in turn, workgroup b
 // runs on XCD b mod 8, and the tiles are numbered so that all row tiles of one panel of W differ by multiples of 8.
