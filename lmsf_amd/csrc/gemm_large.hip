@@ -36,6 +36,8 @@
 // four outputs n = (l / 16) * 4 .. + 3.
 #include "common.h"
 
+#include <type_traits>
+
 #pragma clang diagnostic push
 #pragma clang diagnostic ignored "-Winline-asm"   // m0 is named as clobbered on purpose
 __device__ __forceinline__ void large_global_to_lds_16(const void* src, unsigned lds_base_uniform) {
@@ -152,9 +154,12 @@ __global__ __launch_bounds__(256 * KG) void gemm_large_kernel(const bf16_t* __re
   for (int s = 0; s < STAGES - 1; ++s)
     if (s < n_steps) issue(s, s * STAGE);
 
-  int consume = 0, produce = (STAGES - 1) * STAGE;
   const int a_base = (BN / 2 * wn) * LARGE_ROW, b_base = W_BYTES + (BM / 2 * wm) * LARGE_ROW;
-  for (int it = 0; it < n_steps; ++it) {
+  // One step; SI: which stage holds it (a constant, so that the operands' places in LDS are constants in the
+  // instructions and cost no additions).
+  auto step = [&](auto SI, int it) {
+    constexpr int consume = decltype(SI)::value * STAGE;
+    constexpr int produce = ((decltype(SI)::value + STAGES - 1) % STAGES) * STAGE;
     // step ``it`` has arrived when at most the transfers of the later steps are outstanding
     if (it + STAGES - 2 < n_steps)
       asm volatile("s_waitcnt vmcnt(%0)" ::"n"((STAGES - 2) * LPW) : "memory");
@@ -162,7 +167,6 @@ __global__ __launch_bounds__(256 * KG) void gemm_large_kernel(const bf16_t* __re
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();   // everybody's part of step ``it`` is there, and everybody is done with step ``it - 1``
     if (it + STAGES - 1 < n_steps) issue(it + STAGES - 1, produce);
-    produce = produce + STAGE == STAGES * STAGE ? 0 : produce + STAGE;
     const unsigned char* st = lds + consume;
 #pragma unroll
     for (int s = 0; s < 2 / KG; ++s) {
@@ -179,7 +183,14 @@ __global__ __launch_bounds__(256 * KG) void gemm_large_kernel(const bf16_t* __re
 #pragma unroll
         for (int t = 0; t < NT; ++t) acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t], bb[mt], acc[t][mt], 0, 0, 0);
     }
-    consume = consume + STAGE == STAGES * STAGE ? 0 : consume + STAGE;
+  };
+  static_assert(STAGES == 3 || STAGES == 4, "the loop is unrolled by three or four stages");
+  for (int it = 0; it < n_steps; it += STAGES) {
+    step(std::integral_constant<int, 0>(), it);
+    if (it + 1 < n_steps) step(std::integral_constant<int, 1>(), it + 1);
+    if (it + 2 < n_steps) step(std::integral_constant<int, 2>(), it + 2);
+    if constexpr (STAGES == 4)
+      if (it + 3 < n_steps) step(std::integral_constant<int, 3>(), it + 3);
   }
 
   if constexpr (KG == 2) {
