@@ -69,7 +69,7 @@ class HipOps:
         self.mid_max_rows = 128        # rows up to which the 17-and-more-rows kernel beats the library (64 with the gated activation)
         self.skinny_max_rows = 16      # rows up to which the few-rows kernel beats the library (measured)
         self.large_max_rows = 256      # rows up to which the many-rows kernel beats the library (measured; 0: never)
-        self.large_deep_max_rows = 512  # the same for products whose K is at least three times N (down: 65 against 74 us at 320 rows, 87 against 95 at 512)
+        self.large_deep_max_rows = 1024  # the same for products whose K is at least three times N (down: 57 against 76 us at 320 rows, 74 against 94 at 512, 102 against 108 at 768, level at 1,024)
 
     # ------------------------------------------------------------------ helpers
 

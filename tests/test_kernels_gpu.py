@@ -749,7 +749,7 @@ def test_split_heuristic_counts_the_gated_forms_extra_kernel(ops):
 
 
 @pytest.mark.parametrize("M,N,K", [(129, 4096, 4096), (192, 4096, 14336), (256, 6144, 4096), (150, 328, 192),
-                                   (256, 136, 64), (65, 1000, 1024), (300, 128, 448), (512, 1024, 3072)])
+                                   (256, 136, 64), (65, 1000, 1024), (300, 128, 448), (512, 1024, 3072), (1000, 256, 768)])
 def test_linear_many_rows_every_tiling_and_split(ops, ref, M, N, K):
     """The many-rows product (csrc/gemm_large.hip) with each of its tilings, in one piece and with K split into
     parts whose float32 partial sums are added up by the reduction kernel or stay for the norm that follows: all
