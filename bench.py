@@ -390,6 +390,11 @@ def main():
         p512 = prefill_run(engine, 512, reps=5, seed=4)
         points["prefill_512_tok_s"] = round(512 / p512, 1)
         points["prefill_512_frac"] = round(prefill_flops(cfg, 512) / p512 / peak, 4)
+        long_prompt = min(8192, args.max_num_batched_tokens, cfg["max_position_embeddings"])
+        if long_prompt > args.prefill_tokens:
+            pl = prefill_run(engine, long_prompt, reps=3, seed=6)
+            points["prefill_%d_tok_s" % long_prompt] = round(long_prompt / pl, 1)
+            points["prefill_%d_frac" % long_prompt] = round(prefill_flops(cfg, long_prompt) / pl / peak, 4)
         if args.shape == "llama3-8b" and args.dtype == "bfloat16":
             # continuous batching at Llama-2-7B shape needs the memory: the first engine goes
             del engine
