@@ -718,11 +718,32 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
   for (int v = 0; v < DV; ++v) acc[v] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, lsum = 0.f;
 
+  // The pages of a step's keys are looked up one step ahead (four entries of the block table a lane: the two
+  // blocks of 16 keys whose rows it fetches, the two groups of four keys whose values it fetches), so that the
+  // keys' addresses do not wait for a trip to the table.
+  auto page_of = [&](int key) {
+    int blk = key / G.ps;
+    if (blk > G.btw - 1) blk = G.btw - 1;   // keys beyond the table are masked below; stay inside it
+    return G.bt[blk];
+  };
+  auto k_at = [&](int page, int key) { return ((long)(page * G.nkv + G.kvh) * G.ps + (key - (key / G.ps) * G.ps)) * G.d; };
+  auto v_at = [&](int page, int key) { return (long)(page * G.nkv + G.kvh) * G.d * G.ps + (key - (key / G.ps) * G.ps); };
+  int pg[4];
+  {
+    const int kb = c0 + w * 32;
+    pg[0] = page_of(kb + c); pg[1] = page_of(kb + 16 + c); pg[2] = page_of(kb + 4 * g); pg[3] = page_of(kb + 16 + 4 * g);
+  }
   for (int kbase = c0 + w * 32; kbase < c1; kbase += 128) {
+    int pg_next[4] = {pg[0], pg[1], pg[2], pg[3]};
+    if (kbase + 128 < c1) {
+      const int kb = kbase + 128;
+      pg_next[0] = page_of(kb + c); pg_next[1] = page_of(kb + 16 + c);
+      pg_next[2] = page_of(kb + 4 * g); pg_next[3] = page_of(kb + 16 + 4 * g);
+    }
     Frag8 kf[2][DS];
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
-      const long kr = k_row_offset(G, kbase + b * 16 + c);
+      const long kr = k_at(pg[b], kbase + b * 16 + c);
 #pragma unroll
       for (int s = 0; s < DS; ++s) {
         const int d0 = s * 32 + g * 8;
@@ -732,7 +753,7 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
           kf[b][s].q = make_uint4(0, 0, 0, 0);
       }
     }
-    const long vo0 = v_col_offset(G, kbase + 4 * g), vo1 = v_col_offset(G, kbase + 16 + 4 * g);
+    const long vo0 = v_at(pg[2], kbase + 4 * g), vo1 = v_at(pg[3], kbase + 16 + 4 * g);
     Frag8 vf[DV];
 #pragma unroll
     for (int v = 0; v < DV; ++v) {
@@ -782,6 +803,8 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
         acc[v] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[v].v, pf.v, acc[v], 0, 0, 0);
       }
     }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) pg[i] = pg_next[i];
   }
   lsum += __shfl_xor(lsum, 16, 64);
   lsum += __shfl_xor(lsum, 32, 64);
