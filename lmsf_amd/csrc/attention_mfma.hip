@@ -673,7 +673,10 @@ static int launch_prefill_dma(dim3 grid, hipStream_t stream, const bf16_t* q, lo
 // against 13.8 at 1,024 keys, 18 against 23 at one token of 8,000 keys in 16 splits. Not kept. Nor were
 // workgroups of 16 waves that take a context's keys unsplit and need no second kernel: 26.8 against 12.6 us at 8
 // tokens of 585 keys, with keys and values that come from memory; one compute unit pulls a context's 300 KB far
-// slower than eight do.)
+// slower than eight do. Nor a dealing of a step's 32 keys that makes a lane's eight scores eight keys in a row, as
+// the prefill kernel has it, so that their values are one 16-byte load from one page instead of two of 8 bytes
+// from two: 35.5 against 37 us at 64 tokens of 585 keys, but 68 against 63.7 at 128 and 222 against 217 at 64
+// tokens of 1,150 keys with 32 kv heads.)
 template <int DPAD>
 __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
     const bf16_t* __restrict__ q, long q_stride, const bf16_t* __restrict__ k_pages,
