@@ -263,10 +263,17 @@ def products_run(args):
         del graph
         return sorted(times)[len(times) // 2] * 1e3
     for name, (N, K, gated) in shapes.items():
-        W = (torch.randn(N, K, device="cuda:0", generator=g) * 0.02).to(torch.bfloat16)
+        # rows as far apart as the engine lays a weight's rows out
+        pad = ops.weight_row_pad(K, torch.bfloat16)
+
+        def laid_out(t):
+            buf = torch.empty(N, K + pad, dtype=torch.bfloat16, device="cuda:0")
+            buf[:, :K].copy_(t)
+            return buf[:, :K]
+        W = laid_out(torch.randn(N, K, device="cuda:0", generator=g) * 0.02)
         # as in a model, every call streams its weight from memory: the copies in turn are larger together than
         # the 256 MB of the memory-side cache
-        copies = [W] + [W.clone() for _ in range(int(1.5e9 // (N * K * 2)))]
+        copies = [W] + [laid_out(W) for _ in range(int(1.5e9 // (N * K * 2)))]
         turn = [0]
 
         def weight():

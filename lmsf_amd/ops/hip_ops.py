@@ -69,6 +69,7 @@ class HipOps:
         self.mid_max_rows = 128        # rows up to which the 17-and-more-rows kernel beats the library (64 with the gated activation)
         self.skinny_max_rows = 16      # rows up to which the few-rows kernel beats the library (measured)
         self.large_max_rows = 256      # rows up to which the many-rows kernel beats the library (measured; 0: never)
+        self.weight_row_pad_bytes = 128
         self.large_deep_max_rows = 1024  # the same for products whose K is at least three times N (down: 57 against 76 us at 320 rows, 74 against 94 at 512, 102 against 108 at 768, level at 1,024)
 
     # ------------------------------------------------------------------ helpers
@@ -561,6 +562,15 @@ class HipOps:
         return out
 
     # ------------------------------------------------------------------ matrix products
+
+    def weight_row_pad(self, in_features: int, dtype: torch.dtype) -> int:
+        """Elements to leave between the end of one row of a linear layer's weight and the start of the next.
+        With rows of 8 KB (or any multiple of 4 KB) lying back to back, the 128 rows that a workgroup of the
+        many-rows products reads side by side begin on the same memory channel: a kernel that only reads a
+        28,672 x 4,096 matrix that way gets 4.9 TB/s, and 5.8 with 128 bytes between the rows (64 rows: 5.3 and
+        6.05; the few-rows products' 16 rows: 5.9 and 6.1). Every product takes the distance between rows as an
+        argument."""
+        return self.weight_row_pad_bytes // torch.empty((), dtype=dtype).element_size()
 
     def linear(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
                out_dtype: Optional[torch.dtype] = None, pending_ok: bool = False,

@@ -43,24 +43,33 @@ class FusedLinear(Part):
                 out[self._name(sub, "bias")] = TensorDecl((rows,))
         return out
 
+    def _buffer(self, what: str, dtype: torch.dtype, device) -> torch.Tensor:
+        """The fused tensor's memory. A weight's rows are laid out with the distance between two rows that the
+        kernels ask for (``ops.weight_row_pad``: a few elements more than a row holds, so that rows do not all
+        begin on the same memory channel); what is returned is the [out, in] view of it."""
+        if what != "weight":
+            return torch.empty((self.out_features,), dtype=dtype, device=device)
+        pad_of = getattr(self.rt.ops, "weight_row_pad", None)
+        pad = int(pad_of(self.in_features, dtype)) if pad_of is not None else 0
+        buf = torch.empty((self.out_features, self.in_features + pad), dtype=dtype, device=device)
+        return buf[:, :self.in_features]
+
     def _gather(self, fetch: Callable[[str], torch.Tensor], what: str) -> torch.Tensor:
         """The sources' tensors as the row slices of one buffer, allocated once; every source is copied in
         as it is read and dropped at once, so that beside the fused tensor only one source is alive at a time
         (core/src/model_executor/layers/linear.rs:573-583, :603-622 copy into a zeroed buffer likewise). If
         sources differ in element type the buffer takes the widest."""
-        if len(self.sources) == 1:
-            return fetch(self._name(self.sources[0][0], what)).contiguous()
         # the buffer is made before the first source is read: made after it, torch would cut it out of the block
         # that the source's conversion has just freed and leave a hole of the difference for good
-        tail = (self.in_features,) if what == "weight" else ()
-        out = torch.empty((self.out_features,) + tail, dtype=self.rt.dtype, device=self.rt.device)
+        out = self._buffer(what, self.rt.dtype, self.rt.device)
         row = 0
         for sub, rows in self.sources:
             t = fetch(self._name(sub, what))
-            if t.dtype != out.dtype and t.dtype == torch.float32:
-                out = out.to(torch.float32)           # a source stored in 32 bits: the buffer takes the widest type
-            if t.device != out.device:
-                out = out.to(t.device)
+            if (t.dtype != out.dtype and t.dtype == torch.float32) or t.device != out.device:
+                # a source stored in 32 bits: the buffer takes the widest type (and lies where the sources lie)
+                wider = self._buffer(what, torch.float32 if t.dtype == torch.float32 else out.dtype, t.device)
+                wider[:row].copy_(out[:row])
+                out = wider
             out[row:row + rows].copy_(t)
             row += rows
             del t

@@ -222,6 +222,32 @@ def test_loading_keeps_one_source_tensor_alive_beside_the_weights(tmp_path):
     assert torch.equal(wide.blocks[0].mixer.qkv.weight[256:288], raw["model.layers.0.self_attn.k_proj.weight"])
 
 
+def test_weight_rows_lie_as_far_apart_as_the_kernels_ask(tmp_path):
+    """The kernel object says how many elements to leave between two rows of a linear layer's weight; fused and
+    single matrices, and buffers that widen to 32 bits on the way, are laid out so, and hold the checkpoint's
+    values."""
+    from types import SimpleNamespace
+    from lmsf_amd.weights.loader import load_weights_from_generator
+    folder, cfg = make_model_folder(tmp_path, "B")
+    raw = load_file(os.path.join(folder, "model.safetensors"))
+    ops = SimpleNamespace(weight_row_pad=lambda in_features, dtype: 24 if dtype == torch.bfloat16 else 12)
+    rt = Runtime(ops=ops, device=torch.device("cpu"), dtype=torch.bfloat16, max_positions=cfg.max_position_embeddings)
+    model = DecoderModel(get_architecture(cfg.architecture).build_spec(cfg), rt)
+    load_weights_from_generator(model.parts(), lambda n, d: raw[n].clone() if n.endswith("layers.1.self_attn.v_proj.weight")
+                                else raw[n].to(torch.bfloat16))
+    p = "model.layers.0."
+    qkv, down = model.blocks[0].mixer.qkv.weight, model.blocks[0].feed_forward.down.weight
+    assert qkv.stride() == (qkv.shape[1] + 24, 1) and down.stride() == (down.shape[1] + 24, 1)
+    assert torch.equal(qkv, torch.cat([raw[p + "self_attn.%s_proj.weight" % n] for n in "qkv"]).to(torch.bfloat16))
+    assert torch.equal(down, raw[p + "mlp.down_proj.weight"].to(torch.bfloat16))
+    assert model.blocks[0].mixer.qkv.bias.is_contiguous()
+    wide = model.blocks[1].mixer.qkv.weight       # its last source is stored in 32 bits
+    assert wide.dtype == torch.float32 and wide.stride() == (wide.shape[1] + 12, 1)
+    p = "model.layers.1.self_attn."
+    assert torch.equal(wide, torch.cat([raw[p + "q_proj.weight"].to(torch.bfloat16).float(),
+                                        raw[p + "k_proj.weight"].to(torch.bfloat16).float(), raw[p + "v_proj.weight"]]))
+
+
 def _is_model_tensor(model, t):
     return any(getattr(p, a, None) is not None and getattr(p, a).data_ptr() == t.data_ptr()
                for p in model.parts() for a in ("weight", "bias"))
