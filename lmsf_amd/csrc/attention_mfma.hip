@@ -676,8 +676,13 @@ static int launch_prefill_dma(dim3 grid, hipStream_t stream, const bf16_t* q, lo
 // slower than eight do. Nor a dealing of a step's 32 keys that makes a lane's eight scores eight keys in a row, as
 // the prefill kernel has it, so that their values are one 16-byte load from one page instead of two of 8 bytes
 // from two: 35.5 against 37 us at 64 tokens of 585 keys, but 68 against 63.7 at 128 and 222 against 217 at 64
-// tokens of 1,150 keys with 32 kv heads.)
-template <int DPAD>
+// tokens of 1,150 keys with 32 kv heads. Nor two sets of fragments a wave, the next step's keys and values asked for
+// before this step is multiplied (the table's entries for the step after asked for first, since loads come back in
+// the order they were asked for): the same times at 64 and 128 tokens and at 8,000 keys, so it is not a wave's
+// waiting for its own loads that bounds the kernel at 4.4 to 4.9 TB/s there.)
+// FULL: the head size is DPAD itself (a multiple of 32); the loads and products of a step then run without a test
+// each for the part of DPAD beyond the head size (8 tokens of 585 keys: 12.3 -> 11.6 us with the reduction).
+template <int DPAD, bool FULL>
 __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
     const bf16_t* __restrict__ q, long q_stride, const bf16_t* __restrict__ k_pages,
     const bf16_t* __restrict__ v_pages, const int* __restrict__ block_tables, int btw,
@@ -724,48 +729,41 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
   // The pages of a step's keys are looked up one step ahead (four entries of the block table a lane: the two
   // blocks of 16 keys whose rows it fetches, the two groups of four keys whose values it fetches), so that the
   // keys' addresses do not wait for a trip to the table.
+  const int klast = c1 - 1;
   auto page_of = [&](int key) {
-    int blk = key / G.ps;
-    if (blk > G.btw - 1) blk = G.btw - 1;   // keys beyond the table are masked below; stay inside it
-    return G.bt[blk];
+    // keys beyond the range are masked below; their addresses stay inside the pages that the range has
+    return G.bt[min(key, klast) / G.ps];
   };
   auto k_at = [&](int page, int key) { return ((long)(page * G.nkv + G.kvh) * G.ps + (key - (key / G.ps) * G.ps)) * G.d; };
   auto v_at = [&](int page, int key) { return (long)(page * G.nkv + G.kvh) * G.d * G.ps + (key - (key / G.ps) * G.ps); };
-  int pg[4];
-  {
-    const int kb = c0 + w * 32;
-    pg[0] = page_of(kb + c); pg[1] = page_of(kb + 16 + c); pg[2] = page_of(kb + 4 * g); pg[3] = page_of(kb + 16 + 4 * g);
-  }
-  for (int kbase = c0 + w * 32; kbase < c1; kbase += 128) {
-    int pg_next[4] = {pg[0], pg[1], pg[2], pg[3]};
-    if (kbase + 128 < c1) {
-      const int kb = kbase + 128;
-      pg_next[0] = page_of(kb + c); pg_next[1] = page_of(kb + 16 + c);
-      pg_next[2] = page_of(kb + 4 * g); pg_next[3] = page_of(kb + 16 + 4 * g);
-    }
-    Frag8 kf[2][DS];
+  auto lookup = [&](int kb, int* out) {
+    out[0] = page_of(kb + c); out[1] = page_of(kb + 16 + c); out[2] = page_of(kb + 4 * g); out[3] = page_of(kb + 16 + 4 * g);
+  };
+  // the keys and values of one step of 32 keys, as the matrix instructions take them
+  auto fetch = [&](Frag8 (&kf)[2][DS], Frag8 (&vf)[DV], const int* pg, int kbase) {
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
       const long kr = k_at(pg[b], kbase + b * 16 + c);
 #pragma unroll
       for (int s = 0; s < DS; ++s) {
         const int d0 = s * 32 + g * 8;
-        if (d0 < d)
+        if (FULL || d0 < d)
           kf[b][s].q = *reinterpret_cast<const uint4*>(k_pages + kr + d0);
         else
           kf[b][s].q = make_uint4(0, 0, 0, 0);
       }
     }
     const long vo0 = v_at(pg[2], kbase + 4 * g), vo1 = v_at(pg[3], kbase + 16 + 4 * g);
-    Frag8 vf[DV];
 #pragma unroll
     for (int v = 0; v < DV; ++v) {
-      if (v * 16 < d) {
+      if (FULL || v * 16 < d) {
         const long dvo = (long)(v * 16 + c) * ps;
         vf[v].h[0] = *reinterpret_cast<const uint2*>(v_pages + vo0 + dvo);
         vf[v].h[1] = *reinterpret_cast<const uint2*>(v_pages + vo1 + dvo);
       }
     }
+  };
+  auto compute = [&](Frag8 (&kf)[2][DS], Frag8 (&vf)[DV], int kbase) {
     float sv[8];
     float mx = -INFINITY;
 #pragma unroll
@@ -801,11 +799,20 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
     pf.w[3] = pack2_bf16(pv[6], pv[7]);
 #pragma unroll
     for (int v = 0; v < DV; ++v) {
-      if (v * 16 < d) {
+      if (FULL || v * 16 < d) {
         acc[v] *= corr;
         acc[v] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[v].v, pf.v, acc[v], 0, 0, 0);
       }
     }
+  };
+  int pg[4];
+  lookup(c0 + w * 32, pg);
+  for (int kbase = c0 + w * 32; kbase < c1; kbase += 128) {
+    int pg_next[4] = {pg[0], pg[1], pg[2], pg[3]};
+    if (kbase + 128 < c1) lookup(kbase + 128, pg_next);
+    Frag8 kf[2][DS], vf[DV];
+    fetch(kf, vf, pg, kbase);
+    compute(kf, vf, kbase);
 #pragma unroll
     for (int i = 0; i < 4; ++i) pg[i] = pg_next[i];
   }
@@ -1021,14 +1028,14 @@ extern "C" int lmsf_paged_attention_prefill_mfma(const void* q, long q_stride, v
   return 0;
 }
 
-template <int DPAD>
+template <int DPAD, bool FULL>
 static int launch_decode(dim3 grid, hipStream_t stream, const bf16_t* q, long q_stride, const bf16_t* k_pages,
                          const bf16_t* v_pages, const int* block_tables, int btw, const int* tok_idx, const int* seg,
                          const int* pos, int nh, int nkv, int d, int ps, float scale_log2, int window, int HB, int n_hb,
                          int chunk, int n_splits, float* part_o, float* part_ml, bf16_t* out, long out_stride,
                          int heads_first) {
   const size_t smem = (size_t)(4 * 16 * (DPAD + 4) + 128) * sizeof(float);
-  auto kernel = attn_decode_mfma_kernel<DPAD>;
+  auto kernel = attn_decode_mfma_kernel<DPAD, FULL>;
   static bool configured = false;   // per instantiation
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -1083,10 +1090,11 @@ extern "C" int lmsf_paged_attention_decode_mfma(const void* q, long q_stride, vo
   float* part_ml = scratch + (long)n * nh * n_splits * d;
   dim3 grid(heads_first ? nkv * n_hb : n, heads_first ? n : nkv * n_hb, n_splits);
   int rc = 0;
-#define LAUNCH(DP)                                                                                              \
-  rc = launch_decode<DP>(grid, stream, (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, \
-                         block_tables, btw, tok_idx, seg, pos, nh, nkv, d, ps, scale_log2, window, HB, n_hb, chunk, \
-                         n_splits, part_o, part_ml, (bf16_t*)out, out_stride, heads_first)
+#define DECODE_ARGS                                                                                                 \
+  grid, stream, (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_tables, btw, tok_idx, \
+      seg, pos, nh, nkv, d, ps, scale_log2, window, HB, n_hb, chunk, n_splits, part_o, part_ml, (bf16_t*)out,       \
+      out_stride, heads_first
+#define LAUNCH(DP) rc = d == DP ? launch_decode<DP, true>(DECODE_ARGS) : launch_decode<DP, false>(DECODE_ARGS)
   switch (dpad) {
     case 32: LAUNCH(32); break;
     case 64: LAUNCH(64); break;
@@ -1098,6 +1106,7 @@ extern "C" int lmsf_paged_attention_decode_mfma(const void* q, long q_stride, vo
     default: LAUNCH(256); break;
   }
 #undef LAUNCH
+#undef DECODE_ARGS
   if (rc) return rc;
   LMSF_LAUNCH_CHECK("paged_attention_decode");
   if (n_splits == 1) return 0;
