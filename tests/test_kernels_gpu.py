@@ -468,6 +468,32 @@ def test_linear_bfloat16(ops, ref, M, N, K, bias, out_dtype):
     assert torch.allclose(y.float(), want, **t), (y.float() - want).abs().max()
 
 
+@pytest.mark.parametrize("M", [1, 2, 8, 16, 24, 64, 100, 128, 200, 256, 300, 600, 2048])
+def test_products_over_a_weight_whose_rows_lie_apart(ops, M):
+    """The engine lays a weight's rows out further apart than they are long (`weight_row_pad`) and fills what is
+    between with nothing: every product, for every number of rows, plain and gated, bfloat16 and float32, gives over
+    such a weight the bits that it gives over the same rows lying back to back, whatever lies between them."""
+    g = torch.Generator().manual_seed(M)
+    for (N, K, gated) in ((384, 512, False), (4096, 1024, False), (1024, 3072, False), (704, 256, True),
+                          (2048, 1024, True)):
+        for dtype in (torch.bfloat16, torch.float32):
+            if dtype == torch.float32 and (M > 64 or N * K > 1 << 20):
+                continue
+            pad = ops.weight_row_pad(K, dtype)
+            assert pad * torch.empty((), dtype=dtype).element_size() == 128
+            x = dev(torch.randn(M, K, generator=g).to(dtype))
+            w = dev((torch.randn(N, K, generator=g) * K ** -0.5).to(dtype))
+            buf = torch.full((N, K + pad), float("nan"), dtype=dtype, device=w.device)
+            apart = buf[:, :K]
+            apart.copy_(w)
+            f = (lambda t: ops.linear_gated(x, t, None, "silu")) if gated else (lambda t: ops.linear(x, t))
+            a, b = f(w), f(apart)
+            assert torch.equal(a, b) and not torch.isnan(b.float()).any(), (M, N, K, gated, dtype)
+            if not gated:
+                a32, b32 = ops.linear(x, w, out_dtype=torch.float32), ops.linear(x, apart, out_dtype=torch.float32)
+                assert torch.equal(a32, b32), (M, N, K, dtype)
+
+
 @pytest.mark.parametrize("M,I,K", [(1, 176, 64), (8, 14336, 4096), (16, 208, 80), (13, 1000, 328), (40, 352, 128),
                                    (64, 14336, 4096), (20, 1000, 1024), (65, 14336, 4096), (100, 1000, 1024),
                                    (129, 352, 128), (200, 14336, 4096), (256, 1000, 192), (300, 1000, 1024)])
