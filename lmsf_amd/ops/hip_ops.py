@@ -69,7 +69,7 @@ class HipOps:
         self.mid_max_rows = 128        # rows up to which the 17-and-more-rows kernel beats the library (64 with the gated activation)
         self.skinny_max_rows = 16      # rows up to which the few-rows kernel beats the library (measured)
         self.large_max_rows = 256      # rows up to which the many-rows kernel beats the library (measured; 0: never)
-        self.weight_row_pad_bytes = 128
+        self.weight_row_pad_bytes = 512
         self.large_deep_max_rows = 1024  # the same for products whose K is at least three times N (down: 57 against 76 us at 320 rows, 74 against 94 at 512, 102 against 108 at 768, level at 1,024)
 
     # ------------------------------------------------------------------ helpers
@@ -565,10 +565,13 @@ class HipOps:
 
     def weight_row_pad(self, in_features: int, dtype: torch.dtype) -> int:
         """Elements to leave between the end of one row of a linear layer's weight and the start of the next.
-        With rows of 8 KB (or any multiple of 4 KB) lying back to back, the 128 rows that a workgroup of the
-        many-rows products reads side by side begin on the same memory channel: a kernel that only reads a
-        28,672 x 4,096 matrix that way gets 4.9 TB/s, and 5.8 with 128 bytes between the rows (64 rows: 5.3 and
-        6.05; the few-rows products' 16 rows: 5.9 and 6.1). Every product takes the distance between rows as an
+        With rows of 8 KB (or any multiple of 4 KB) lying back to back, the rows that a workgroup reads side by
+        side begin on the same memory channels: a kernel that only reads a 28,672 x 4,096 matrix 64 rows at a
+        time, 128 bytes of each, gets 4.8 TB/s, and 5.6 to 5.75 with 128 to 2,048 bytes between the rows; 16 rows
+        at a time, 1 KB of each: 5.0 and 5.9 to 6.0. Which distances help depends on the row's length (rows of
+        16 KB: 128 bytes hurt, 256 and more help; rows of 28 KB: 256 hurts); 512 bytes help or do no harm at 4,096,
+        8,192, 14,336 and 28,672 columns, for the few-rows, the many-rows and the library's products alike (gate_up
+        of 57,344 x 8,192 at 64 rows: 207 -> 181 us). Every product takes the distance between rows as an
         argument."""
         return self.weight_row_pad_bytes // torch.empty((), dtype=dtype).element_size()
 

@@ -473,6 +473,7 @@ def test_products_over_a_weight_whose_rows_lie_apart(ops, M):
     """The engine lays a weight's rows out further apart than they are long (`weight_row_pad`) and fills what is
     between with nothing: every product, for every number of rows, plain and gated, bfloat16 and float32, gives over
     such a weight the bits that it gives over the same rows lying back to back, whatever lies between them."""
+    assert ops.weight_row_pad_bytes % 16 == 0
     g = torch.Generator().manual_seed(M)
     for (N, K, gated) in ((384, 512, False), (4096, 1024, False), (1024, 3072, False), (704, 256, True),
                           (2048, 1024, True)):
@@ -480,7 +481,7 @@ def test_products_over_a_weight_whose_rows_lie_apart(ops, M):
             if dtype == torch.float32 and (M > 64 or N * K > 1 << 20):
                 continue
             pad = ops.weight_row_pad(K, dtype)
-            assert pad * torch.empty((), dtype=dtype).element_size() == 128
+            assert pad > 0 and pad * torch.empty((), dtype=dtype).element_size() == ops.weight_row_pad_bytes
             x = dev(torch.randn(M, K, generator=g).to(dtype))
             w = dev((torch.randn(N, K, generator=g) * K ** -0.5).to(dtype))
             buf = torch.full((N, K + pad), float("nan"), dtype=dtype, device=w.device)
