@@ -10,7 +10,7 @@ import dataclasses
 import json
 import os
 from dataclasses import dataclass
-from typing import Any, Dict, List, Optional, Tuple
+from typing import Any, Dict, Optional, Tuple
 
 
 class ConfigError(ValueError):

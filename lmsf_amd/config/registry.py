@@ -7,7 +7,7 @@ holds both; an architecture is added by one ``register_architecture`` call and n
 in the package names it.
 """
 from dataclasses import dataclass
-from typing import Any, Callable, Dict, Optional, Tuple
+from typing import Any, Callable, Dict, Tuple
 
 from .model_config import ArchConfig, ConfigError, read_config_json
 

@@ -4,7 +4,6 @@ This is the common base of the engine (scheduler + sampler on top) and of trace 
 on top). Reference: Worker::from + Worker::init_cache (core/src/worker/model_worker.rs:34-126) and
 the sizing of the cache from free device memory (:128-162).
 """
-import os
 import warnings
 from dataclasses import dataclass
 from typing import Any, Optional, Sequence

@@ -8,7 +8,7 @@ exactly the tokens it was given, and commits them to the cache. Sampling is a se
 trace replay can take the logits.
 """
 from collections import OrderedDict
-from typing import Dict, Hashable, List, Optional, Sequence, Tuple
+from typing import Hashable, Optional, Sequence, Tuple
 
 import numpy as np
 import torch

@@ -1,7 +1,7 @@
 """What the engine hands back per request and step
 (core/src/common/output.rs:5-132: RequestOutput with its CompletionOutputs). The text fields are
 filled by engines that have the model's tokenizer and are empty otherwise."""
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 from typing import Hashable, List, Optional
 
 from .sequence import RequestMetrics, Sequence

@@ -80,8 +80,7 @@ def main(argv=None) -> int:
     os.makedirs(args.out, exist_ok=True)
     t0 = time.time()
     _say("starting (first import of torch can take a minute or two)")
-    import numpy as np
-    import torch  # noqa: F401
+    import torch  # noqa: F401  (the long first import, announced above)
 
     from lmsf_amd.engine import StepEntry, load_engine_core
 

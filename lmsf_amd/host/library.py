@@ -2,7 +2,7 @@
 (``lmsf_amd/csrc/host``). It has no GPU code and is built with the system's C++ compiler at its first
 use, so the host side of the engine runs wherever the package does."""
 import ctypes
-from ctypes import POINTER, c_char_p, c_double, c_int, c_int64, c_ubyte, c_void_p
+from ctypes import POINTER, c_char_p, c_double, c_int, c_int64, c_void_p
 from typing import Optional
 
 from ..csrc import build as _build

@@ -5,7 +5,7 @@ Embedding, the layers in the order of the schedule, final norm on the wanted row
 loop). The model holds no sizes of its own: everything comes from the spec.
 """
 import inspect
-from typing import Dict, List, Optional, Sequence, Tuple
+from typing import List, Optional, Sequence, Tuple
 
 import torch
 

@@ -11,7 +11,7 @@ the same steps, but attends to the step's own k and v for prompts
 prompts beside single decoded tokens. Query head h uses kv head h / (nh / nkv) (attention.rs:91-103).
 """
 import math
-from typing import Any, Callable, Dict, Mapping, Optional
+from typing import Optional
 
 import torch
 

@@ -11,7 +11,7 @@ and repeats it per architecture (gemma.rs, chatglm.rs); its only plug point is t
 of the linear layers (core/src/model_executor/layers/linear.rs:28-42).
 """
 from dataclasses import dataclass, field
-from typing import Any, Callable, Dict, List, Mapping, Optional, Sequence, Tuple
+from typing import Any, Callable, Dict, Mapping, Optional, Sequence, Tuple
 
 import torch
 

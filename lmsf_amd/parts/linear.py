@@ -5,7 +5,7 @@ y = x W^T (+ b), W stored [out, in]. The reference fuses q, k, v into one weight
 gate, up into one of 2 I rows (:325-497, offsets :364-366) by copying the checkpoint tensors into
 row slices of a zeroed buffer at load time; the same is done here, for weights and biases alike.
 """
-from typing import Callable, Dict, List, Optional, Sequence, Tuple
+from typing import Callable, Dict, Optional, Sequence, Tuple
 
 import torch
 

@@ -3,8 +3,6 @@
 core/src/model_executor/models/llama/llama.rs:223-274: gate and up are one fused product of 2 I
 rows (gate first), then silu_and_mul (vllm/kernels/activation_kernels.cu:26-42), then down.
 """
-from typing import Optional
-
 import torch
 
 from .base import FeedForward, Runtime, register_part

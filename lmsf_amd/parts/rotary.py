@@ -11,7 +11,7 @@ original context length o: L < o / high_freq_factor keeps f, L > o / low_freq_fa
 f / factor, in between (1 - s) f / factor + s f with s = (o / L - low) / (high - low).
 """
 import math
-from typing import Any, Callable, Dict, Mapping, Optional
+from typing import Any, Callable, Mapping, Optional
 
 import torch
 

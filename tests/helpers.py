@@ -5,7 +5,7 @@ import random
 
 import torch
 
-from lmsf_amd.config import LlamaConfig, RopeScaling
+from lmsf_amd.config import LlamaConfig
 from lmsf_amd.weights import write_random_model
 
 # Two configurations that differ in every size and option.

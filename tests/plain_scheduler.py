@@ -19,7 +19,7 @@ What happens when pages run out is written out once, at the top of lmsf_amd/csrc
 import time
 from collections import deque
 from dataclasses import dataclass, field
-from typing import Deque, Dict, Hashable, List, Optional
+from typing import Deque, Hashable, List, Optional
 
 from plain_cache_manager import CacheManager
 from lmsf_amd.engine.sequence import Sequence, SequenceState

@@ -2,7 +2,6 @@
 plain implementation's, preemption by recompute changes nothing, seeded sampling does not depend
 on the batch, and the stop rules."""
 import pytest
-import torch
 
 from helpers import TINY, make_model_folder, random_tokens
 from plain_llama import plain_greedy_generate, read_model_folder

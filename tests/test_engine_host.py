@@ -1,7 +1,6 @@
 """The host side of the step function (cache manager, batch building, model assembly) run on the
 CPU with torch stand-ins for the kernels, against the plain implementation. The kernels
 themselves are tested on the GPU."""
-import os
 
 import pytest
 import torch

@@ -2,7 +2,6 @@
 command line, in float32 and bfloat16, against the plain implementation."""
 import os
 import subprocess
-import sys
 
 import pytest
 import torch

@@ -2,8 +2,6 @@
 together differently from the same parts (a layer twice, a layer reading another layer's cache, a
 window); and toy parts defined here (a mixer with state of its own, a feed-forward with routing,
 another position encoding) registered, built and stepped without touching the package."""
-import math
-import os
 
 import pytest
 import torch

@@ -14,7 +14,7 @@ import torch
 import torch.nn.functional as F
 
 import plain_llama as P
-from helpers import TINY, make_model_folder, random_tokens
+from helpers import make_model_folder, random_tokens
 
 
 def rnd(*shape, seed=0, scale=1.0):

@@ -11,7 +11,7 @@ from torch_ops import TorchOps
 
 from lmsf_amd.engine import EngineArgs, LLMEngine
 from lmsf_amd.engine.detokenizer import IncrementalDetokenizer, Tokenizer, load_tokenizer
-from lmsf_amd.engine.llm_engine import LLM, check_stop
+from lmsf_amd.engine.llm_engine import check_stop
 from lmsf_amd.engine.sequence import Sequence, SequenceState
 from lmsf_amd.sampling import SamplingParams
 

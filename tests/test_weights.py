@@ -7,7 +7,7 @@ import pytest
 import torch
 from safetensors.torch import load_file, save_file
 
-from helpers import TINY, TINY_A, TINY_B, make_model_folder
+from helpers import TINY_A, TINY_B, make_model_folder
 
 from lmsf_amd.config import LlamaConfig, get_architecture
 from lmsf_amd.models import DecoderModel
