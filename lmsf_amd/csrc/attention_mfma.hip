@@ -707,7 +707,7 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
   if (c0 >= c1) return;
   KvView G;
   G.k = k_pages; G.v = v_pages; G.btw = btw; G.nkv = nkv; G.d = d; G.ps = ps; G.kvh = kvh;
-  G.bt = block_tables + (long)seg[tok] * btw;
+  G.bt = block_tables + (long)(seg ? seg[tok] : tok) * btw;   // (no seg: token i is request i, one trip to memory fewer)
 
   const int hin = hb * HB + c;
   const bool valid = c < HB && hin < n_rep;
@@ -869,22 +869,39 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
 __global__ __launch_bounds__(256) void attn_decode_reduce_serial_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml, bf16_t* __restrict__ out, long out_stride,
     const int* __restrict__ tok_idx, const int* __restrict__ pos, int nh, int d, int window, int chunk, int n_splits) {
-  const int i_tok = blockIdx.x, head = blockIdx.y;
+  // One thread per output element (the block has at least d threads). Everything a thread needs is asked for at
+  // once, the position beside the partial results of all splits (those of splits without keys hold whatever the
+  // memory held and are dropped unread): one trip to memory before the sums instead of three in a row.
+  const int i_tok = blockIdx.x, head = blockIdx.y, dv = threadIdx.x;
   const int tok = tok_idx ? tok_idx[i_tok] : i_tok;
   const int p = pos[tok];
-  const int lo = window > 0 ? max(0, p - window + 1) : 0;
-  const int s0 = ((lo / 32) * 32) / chunk, s1 = min(n_splits - 1, p / chunk);
   const long base = ((long)i_tok * nh + head) * n_splits;
-  float M = -INFINITY;
-  for (int s = s0; s <= s1; ++s) M = fmaxf(M, part_ml[(base + s) * 2]);
-  float ls = 0.f;
-  for (int s = s0; s <= s1; ++s) ls += exp2f(part_ml[(base + s) * 2] - M) * part_ml[(base + s) * 2 + 1];
-  const float inv = 1.0f / ls;
-  for (int dv = threadIdx.x; dv < d; dv += blockDim.x) {
-    float o = 0.f;
-    for (int s = s0; s <= s1; ++s) o += exp2f(part_ml[(base + s) * 2] - M) * part_o[(base + s) * d + dv];
-    out[(long)tok * out_stride + (long)head * d + dv] = f32_to_bf16(o * inv);
+  float pm[REDUCE_SERIAL_SPLITS], pl[REDUCE_SERIAL_SPLITS], po[REDUCE_SERIAL_SPLITS];
+#pragma unroll
+  for (int s = 0; s < REDUCE_SERIAL_SPLITS; ++s) {
+    if (s < n_splits) {
+      const float2 ml = *reinterpret_cast<const float2*>(part_ml + (base + s) * 2);
+      pm[s] = ml.x;
+      pl[s] = ml.y;
+      po[s] = dv < d ? part_o[(base + s) * d + dv] : 0.f;
+    }
   }
+  const int lo = window > 0 ? max(0, p - window + 1) : 0;
+  const int s0 = ((lo / 32) * 32) / chunk, s1 = min(n_splits - 1, p / chunk);   // splits s0 .. s1 have keys
+  float M = -INFINITY;
+#pragma unroll
+  for (int s = 0; s < REDUCE_SERIAL_SPLITS; ++s)
+    if (s >= s0 && s <= s1) M = fmaxf(M, pm[s]);
+  float ls = 0.f, o = 0.f;
+#pragma unroll
+  for (int s = 0; s < REDUCE_SERIAL_SPLITS; ++s) {
+    if (s >= s0 && s <= s1) {
+      const float f = exp2f(pm[s] - M);
+      ls += f * pl[s];
+      o += f * po[s];
+    }
+  }
+  if (dv < d) out[(long)tok * out_stride + (long)head * d + dv] = f32_to_bf16(o * (1.0f / ls));
 }
 
 __global__ __launch_bounds__(REDUCE_THREADS) void attn_decode_reduce_kernel(
@@ -1061,15 +1078,16 @@ extern "C" long lmsf_attention_decode_scratch_floats(int n, int nh, int d, int n
 // in this order from 16 tokens on (order 0; 1 and 2 force one of the two arrangements), so the longest contexts
 // should come first where they differ. chunk: keys per split, a multiple of 128;
 // n_splits * chunk must cover the longest context. scratch: lmsf_attention_decode_scratch_floats floats
-// (not touched with n_splits == 1).
+// (not touched with n_splits == 1). seg null: token i is the only token of request i (row i of the block tables),
+// as in a step of single tokens.
 extern "C" int lmsf_paged_attention_decode_mfma(const void* q, long q_stride, void* out, long out_stride,
                                                 const void* k_pages, const void* v_pages, long num_pages,
                                                 const int* block_tables, int btw, const int* tok_idx, int n,
                                                 const int* seg, const int* pos, int nh, int nkv, int d, int ps,
                                                 float scale, int window, int chunk, int n_splits, float* scratch,
                                                 int order, hipStream_t stream) {
-  if (int rc = check_common("paged_attention_decode", q, out, k_pages, v_pages, block_tables, seg, pos, q_stride,
-                            out_stride, num_pages, btw, nh, nkv, d, ps, window))
+  if (int rc = check_common("paged_attention_decode", q, out, k_pages, v_pages, block_tables, seg ? seg : pos, pos,
+                            q_stride, out_stride, num_pages, btw, nh, nkv, d, ps, window))
     return rc;
   LMSF_CHECK(n >= 0 && scratch != nullptr && lmsf_aligned16(scratch), "paged_attention_decode: bad arguments (scratch must be 16-byte aligned)");
   LMSF_CHECK(chunk > 0 && chunk % 128 == 0 && n_splits > 0 && n_splits <= 65535,

@@ -639,7 +639,9 @@ int op_attention(Run& r, const Value& q, const LmsfOpDesc& op, const int* tables
   int n_tiles = 0, n_single = 0;
   const int max_context = st.max_context;
   if (st.all_single) {
-    single = st.longest_first;
+    // the order matters from 16 tokens on (the kernel starts the longest contexts first); below that the tokens
+    // are taken as they come, which saves the kernel the trip to the list
+    single = N >= 16 ? st.longest_first : nullptr;
     n_single = N;
   } else {
     const int tq = lmsf_attention_tile_tokens(nh, nkv);
@@ -670,8 +672,9 @@ int op_attention(Run& r, const Value& q, const LmsfOpDesc& op, const int* tables
     const long floats = n_splits > 1 ? lmsf_attention_decode_scratch_floats(n_single, nh, d, n_splits) : 1;
     TAKE(scratch, float*, (size_t)floats * 4);
     LAUNCH(lmsf_paged_attention_decode_mfma(q.p, q.ld, out, (long)nh * d, op.k_pages, op.v_pages, op.num_pages, tables,
-                                            width, single, n_single, st.seg_of, st.positions, nh, nkv, d, ps, op.scale,
-                                            op.window, chunk, n_splits, scratch, t.decode_attention_order, r.stream));
+                                            width, single, n_single, st.all_single ? nullptr : st.seg_of, st.positions, nh, nkv,
+                                            d, ps, op.scale, op.window, chunk, n_splits, scratch, t.decode_attention_order,
+                                            r.stream));
   }
   return 0;
 }

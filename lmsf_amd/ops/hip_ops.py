@@ -69,7 +69,7 @@ class HipOps:
         self.mid_max_rows = 128        # rows up to which the 17-and-more-rows kernel beats the library (64 with the gated activation)
         self.skinny_max_rows = 16      # rows up to which the few-rows kernel beats the library (measured)
         self.large_max_rows = 256      # rows up to which the many-rows kernel beats the library (measured; 0: never)
-        self.weight_row_pad_bytes = 512
+        self.weight_row_pad_bytes = 512  # bytes left between two rows of a linear layer's weight (see weight_row_pad)
         self.large_deep_max_rows = 1024  # the same for products whose K is at least three times N (down: 57 against 76 us at 320 rows, 74 against 94 at 512, 102 against 108 at 768, level at 1,024)
 
     # ------------------------------------------------------------------ helpers
@@ -471,8 +471,8 @@ class HipOps:
             scratch = torch.empty(floats if n_splits > 1 else 1, dtype=torch.float32, device=q.device)
             self._check(self.lib.lmsf_paged_attention_decode_mfma(
                 _ptr(q), q.stride(0), _ptr(out), out.stride(0), *common, _ptr(plan.single_tokens), plan.n_single,
-                _ptr(seg), _ptr(pos), nh, nkv, d, ps, float(scale), int(window or 0), chunk, n_splits,
-                _ptr(scratch), self.decode_attention_order, self._stream()))
+                None if plan.token_is_request else _ptr(seg), _ptr(pos), nh, nkv, d, ps, float(scale),
+                int(window or 0), chunk, n_splits, _ptr(scratch), self.decode_attention_order, self._stream()))
         return out
 
     def _attention_plan(self, batch, seg: torch.Tensor, pos: torch.Tensor, nh: int, nkv: int) -> "_AttentionPlan":
@@ -488,7 +488,10 @@ class HipOps:
             lens, starts, max_context = batch.host_seg_lens, batch.host_seg_starts, batch.max_context
             first_pos = batch.host_seg_first_pos
             if batch.replayed or batch.all_single:
-                plan = _AttentionPlan(None, 0, getattr(batch, "longest_first", None), batch.n_tokens, max_context)
+                # the order matters from 16 tokens on (the kernel starts the longest contexts first); below that
+                # the tokens are taken as they come, which saves the kernel the trip to the list
+                order = getattr(batch, "longest_first", None) if batch.n_tokens >= 16 else None
+                plan = _AttentionPlan(None, 0, order, batch.n_tokens, max_context, token_is_request=True)
                 aux[key] = plan
                 return plan
         else:
@@ -869,14 +872,15 @@ class HipOps:
 
 
 class _AttentionPlan:
-    __slots__ = ("tiles", "n_tiles", "single_tokens", "n_single", "max_context")
+    __slots__ = ("tiles", "n_tiles", "single_tokens", "n_single", "max_context", "token_is_request")
 
-    def __init__(self, tiles, n_tiles, single_tokens, n_single, max_context):
+    def __init__(self, tiles, n_tiles, single_tokens, n_single, max_context, token_is_request=False):
         self.tiles = tiles                    # int32 [n_tiles, 2] on the device, or None
         self.n_tiles = n_tiles
         self.single_tokens = single_tokens    # int32 flat indices of the one-token requests; None: every token
         self.n_single = n_single
         self.max_context = max_context
+        self.token_is_request = token_is_request   # a step of single tokens: token i is request i of the tables
 
 
 _default_ops: Optional[HipOps] = None
