@@ -29,6 +29,12 @@ __device__ __forceinline__ void mid_global_to_lds_16(const void* src, unsigned l
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(lds_base_uniform)
                : "memory", "m0");
 }
+// The same for data that is read once (the weights): marked non-temporal, it does not push out of the caches what
+// is read again and again (x).
+__device__ __forceinline__ void mid_global_to_lds_16_once(const void* src, unsigned lds_base_uniform) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off nt" ::"v"(src), "s"(lds_base_uniform)
+               : "memory", "m0");
+}
 #pragma clang diagnostic pop
 __device__ __forceinline__ unsigned mid_lds_address(const void* p) {
   return (unsigned)(size_t)(__attribute__((address_space(3))) const unsigned char*)p;
@@ -117,8 +123,13 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const bf16_t* __restrict_
   const unsigned lds0 = mid_lds_address(lds);
   auto issue = [&](int step, int stage_byte) {
 #pragma unroll
-    for (int i = 0; i < LPW; ++i)
-      mid_global_to_lds_16(src[i] + (long)step * 64, __builtin_amdgcn_readfirstlane(lds0 + stage_byte + dst[i]));
+    for (int i = 0; i < LPW; ++i) {
+      const unsigned to = __builtin_amdgcn_readfirstlane(lds0 + stage_byte + dst[i]);
+      if (i < 2 * WT)
+        mid_global_to_lds_16_once(src[i] + (long)step * 64, to);
+      else
+        mid_global_to_lds_16(src[i] + (long)step * 64, to);
+    }
   };
 #pragma unroll
   for (int s = 0; s < MID_STAGES - 1; ++s)
