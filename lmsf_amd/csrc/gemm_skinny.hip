@@ -126,15 +126,20 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __re
 
   // K is a multiple of 8, so a 16-byte piece is inside or outside the row as a whole; a piece outside
   // is read from the start of the row instead and multiplied by nothing (its x piece is zeroed)
-#define SKINNY_FETCH(buf, chunk)                                                                \
+  // The weights are read once: their loads are marked non-temporal, so that they do not push out of the caches what is
+  // read again and again (x). A fetch that is only made to keep the loop in one shape (live == false: the wave has
+  // no further chunk) asks for a piece of x instead, which the caches hold, and its result is never used.
+#define SKINNY_FETCH(buf, chunk, live)                                                          \
   {                                                                                             \
     const int k_ = (chunk) * KC;                                                                \
     const bool ok_ = (k_ + lcol) < K;                                                           \
     const int kk_ = ok_ ? k_ : -lcol;                                                           \
     const unsigned keep_ = ok_ ? 0xffffffffu : 0u;                                              \
+    const bool live_ = (live);                                                                  \
     _Pragma("unroll") for (int i = 0; i < T::LOADS; ++i) {                                      \
       _Pragma("unroll") for (int wt = 0; wt < WT; ++wt) {                                       \
-        wreg[buf][wt][i] = *reinterpret_cast<const u32x4_t*>(W + woff[wt][i] + kk_);            \
+        const bf16_t* from_ = live_ ? W + woff[wt][i] : x + xoff[0][i];                         \
+        wreg[buf][wt][i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(from_ + kk_)); \
       }                                                                                         \
       _Pragma("unroll") for (int mt = 0; mt < MT; ++mt) {                                       \
         xreg[buf][mt][i] = *reinterpret_cast<const u32x4_t*>(x + xoff[mt][i] + kk_) & keep_;    \
@@ -142,8 +147,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __re
     }                                                                                           \
   }
 
-  // Every fetch is unconditional (a wave without a further chunk fetches its current one again, from
-  // cache), which keeps the staged pieces in registers across the loop.
+  // Every fetch is unconditional, which keeps the staged pieces in registers across the loop.
   // SCALED: this thread's share of the sums of squares (row tid % 16). Loads come back in the order they were
   // asked for: these go first and are added up once the first weights have been asked for, so that waiting
   // for them does not wait for the weights.
@@ -173,7 +177,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __re
   }
   int c = wave;
 #pragma unroll
-  for (int b = 0; b < DEPTH; ++b) SKINNY_FETCH(b, c + b * NW < nchunks ? c + b * NW : 0);
+  for (int b = 0; b < DEPTH; ++b) SKINNY_FETCH(b, c + b * NW < nchunks ? c + b * NW : 0, c + b * NW < nchunks);
   float ssq = 0.f;
   if (SCALED) {
 #pragma unroll
@@ -196,7 +200,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __re
         for (int mt = 0; mt < MT; ++mt) *reinterpret_cast<u32x4_t*>(my + (WT + mt) * T::TILE_BYTES + off) = xreg[b][mt][i];
       }
       const int ahead = c + DEPTH * NW;
-      SKINNY_FETCH(b, ahead < nchunks ? ahead : c);
+      SKINNY_FETCH(b, ahead < nchunks ? ahead : c, ahead < nchunks);
       // LDS -> operands (MFMA layout), multiply
 #pragma unroll
       for (int s = 0; s < T::STEPS; ++s) {
