@@ -23,6 +23,7 @@
 #include "common.h"
 
 typedef __bf16 gemv_bf16x2_t __attribute__((ext_vector_type(2)));
+typedef unsigned int gemv_u32x4_t __attribute__((ext_vector_type(4)));
 
 #define GEMV_WAVES 8
 #define GEMV_UNROLL 8   // 16-byte pieces per lane in flight per row: 8 x 512 = 4,096 elements of K
@@ -76,7 +77,13 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_kernel(const bf16_t* __r
 #pragma unroll
     for (int j = 0; j < GEMV_UNROLL; ++j) {
       const int k = c.kb + j * 512 + lane * 8;
-      wv[j] = k < K ? *reinterpret_cast<const uint4*>(w_row + k) : make_uint4(0u, 0u, 0u, 0u);
+      // (read once: marked non-temporal, so that the weights do not push x and the stream out of the caches)
+      if (k < K) {
+        const gemv_u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const gemv_u32x4_t*>(w_row + k));
+        wv[j] = make_uint4(v.x, v.y, v.z, v.w);
+      } else {
+        wv[j] = make_uint4(0u, 0u, 0u, 0u);
+      }
     }
   };
   auto advance = [&](GemvCursor& c) {
