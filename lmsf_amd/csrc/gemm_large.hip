@@ -44,6 +44,12 @@ __device__ __forceinline__ void large_global_to_lds_16(const void* src, unsigned
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(lds_base_uniform)
                : "memory", "m0");
 }
+// The same for data that this launch reads once: marked non-temporal, it does not push out of the caches what is
+// read again and again.
+__device__ __forceinline__ void large_global_to_lds_16_once(const void* src, unsigned lds_base_uniform) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off nt" ::"v"(src), "s"(lds_base_uniform)
+               : "memory", "m0");
+}
 #pragma clang diagnostic pop
 __device__ __forceinline__ unsigned large_lds_address(const void* p) {
   return (unsigned)(size_t)(__attribute__((address_space(3))) const unsigned char*)p;
@@ -145,10 +151,18 @@ __global__ __launch_bounds__(256 * KG) void gemm_large_kernel(const bf16_t* __re
     for (int mt = 0; mt < MT; ++mt) acc[t][mt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 
   const unsigned lds0 = large_lds_address(lds);
+  // (with one tile of rows every row of W is read once by the whole launch; with several, the later tiles find W in
+  // the die's L2, where it should stay)
+  const bool w_once = tiles_m == 1;
   auto issue = [&](int step, int stage_byte) {
 #pragma unroll
-    for (int i = 0; i < LPW; ++i)
-      large_global_to_lds_16(src[i] + (long)step * 64, __builtin_amdgcn_readfirstlane(lds0 + stage_byte + dst[i]));
+    for (int i = 0; i < LPW; ++i) {
+      const unsigned to = __builtin_amdgcn_readfirstlane(lds0 + stage_byte + dst[i]);
+      if (i < W_LOADS && w_once)
+        large_global_to_lds_16_once(src[i] + (long)step * 64, to);
+      else
+        large_global_to_lds_16(src[i] + (long)step * 64, to);
+    }
   };
 #pragma unroll
   for (int s = 0; s < STAGES - 1; ++s)
