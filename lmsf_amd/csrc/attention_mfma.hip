@@ -31,6 +31,7 @@
 
 #include <type_traits>
 
+typedef unsigned int attn_u32x2_t __attribute__((ext_vector_type(2)));
 union Frag8 {
   bf16x8_t v;
   uint4 q;
@@ -748,7 +749,7 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
       for (int s = 0; s < DS; ++s) {
         const int d0 = s * 32 + g * 8;
         if (FULL || d0 < d)
-          kf[b][s].q = *reinterpret_cast<const uint4*>(k_pages + kr + d0);
+          kf[b][s].v = __builtin_nontemporal_load(reinterpret_cast<const bf16x8_t*>(k_pages + kr + d0));
         else
           kf[b][s].q = make_uint4(0, 0, 0, 0);
       }
@@ -758,8 +759,10 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
     for (int v = 0; v < DV; ++v) {
       if (FULL || v * 16 < d) {
         const long dvo = (long)(v * 16 + c) * ps;
-        vf[v].h[0] = *reinterpret_cast<const uint2*>(v_pages + vo0 + dvo);
-        vf[v].h[1] = *reinterpret_cast<const uint2*>(v_pages + vo1 + dvo);
+        // (a step's keys and values are read once by the launch: marked non-temporal)
+        const attn_u32x2_t lo2 = __builtin_nontemporal_load(reinterpret_cast<const attn_u32x2_t*>(v_pages + vo0 + dvo));
+        const attn_u32x2_t hi2 = __builtin_nontemporal_load(reinterpret_cast<const attn_u32x2_t*>(v_pages + vo1 + dvo));
+        vf[v].w[0] = lo2.x; vf[v].w[1] = lo2.y; vf[v].w[2] = hi2.x; vf[v].w[3] = hi2.y;
       }
     }
   };
