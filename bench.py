@@ -412,6 +412,7 @@ def main():
             points["serve_tok_s"] = serve["value"]
             points["serve_total_tok_s"] = serve["config"]["total_tok_per_s"]
             points["serve_ms_per_step"] = serve["ms_per_step"]
+            points["serve_preemptions"] = serve["config"]["preemptions"]
 
     line = {
         "metric": "decode tok/s at batch %d (%s %s)" % (args.batch, shape_name, "bf16" if args.dtype == "bfloat16" else "fp32"),
