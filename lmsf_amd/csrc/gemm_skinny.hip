@@ -73,7 +73,9 @@ struct NormAroundArgs {
 
 // ACT: 0 none (plain linear layer), 1 silu-gated, 2 gelu-gated, 3 rotary embedding and cache write,
 // 4 add to the stream and prepare the norm that follows (y receives bf16(stream * w))
-template <int MT, int KC, int NW, typename TOut, int ACT, int DEPTH, bool SCALED>
+// XROWS: rows of a tile of x that are fetched and staged, 16 or (one row tile of up to 8 rows) 8; the columns of the
+// result that belong to the others are never stored.
+template <int MT, int KC, int NW, typename TOut, int ACT, int DEPTH, bool SCALED, int XROWS>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ x, long ldx,
                                                               const bf16_t* __restrict__ W, long ldw,
                                                               const bf16_t* __restrict__ bias, TOut* __restrict__ y,
@@ -81,6 +83,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __re
                                                               NormAroundArgs na) {
   using T = SkinnyTile<KC>;
   constexpr int WT = (ACT >= 1 && ACT <= 3) ? 2 : 1;   // W tiles per chunk: gate and up, the two halves of a head, or one
+  constexpr int XLOADS = (XROWS + T::ROWS_PER_LOAD - 1) / T::ROWS_PER_LOAD;   // load instructions per tile of x
+  static_assert(XROWS == 16 || (XROWS == 8 && MT == 1 && XLOADS < T::LOADS), "8 rows of x: one row tile, and a whole load fewer");
   static_assert(!(SCALED || ACT == 4) || MT == 1, "the forms around a norm take up to 16 rows");
   static_assert(ACT != 4 || NW >= 4, "the epilogue of the product before a norm has a thread for each of the tile's 256 elements");
   extern __shared__ __align__(16) unsigned char lds[];
@@ -142,7 +146,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __re
         wreg[buf][wt][i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(from_ + kk_)); \
       }                                                                                         \
       _Pragma("unroll") for (int mt = 0; mt < MT; ++mt) {                                       \
-        xreg[buf][mt][i] = *reinterpret_cast<const u32x4_t*>(x + xoff[mt][i] + kk_) & keep_;    \
+        if (i < XLOADS)                                                                         \
+          xreg[buf][mt][i] = *reinterpret_cast<const u32x4_t*>(x + xoff[mt][i] + kk_) & keep_;  \
       }                                                                                         \
     }                                                                                           \
   }
@@ -197,7 +202,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __re
 #pragma unroll
         for (int wt = 0; wt < WT; ++wt) *reinterpret_cast<u32x4_t*>(my + wt * T::TILE_BYTES + off) = wreg[b][wt][i];
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) *reinterpret_cast<u32x4_t*>(my + (WT + mt) * T::TILE_BYTES + off) = xreg[b][mt][i];
+        for (int mt = 0; mt < MT; ++mt)
+          if (i < XLOADS) *reinterpret_cast<u32x4_t*>(my + (WT + mt) * T::TILE_BYTES + off) = xreg[b][mt][i];
       }
       const int ahead = c + DEPTH * NW;
       SKINNY_FETCH(b, ahead < nchunks ? ahead : c, ahead < nchunks);
@@ -339,16 +345,15 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __re
   }
 }
 
-template <int MT, int KC, int NW, typename TOut, int ACT, int DEPTH = 1, bool SCALED = false>
-static int launch_skinny(const void* x, long ldx, const void* W, long ldw, const void* bias, void* y, long ldy, int M,
-                         int N, int K, hipStream_t stream, RopeCacheArgs rc = RopeCacheArgs(),
-                         NormAroundArgs na = NormAroundArgs()) {
+template <int MT, int KC, int NW, typename TOut, int ACT, int DEPTH, bool SCALED, int XROWS>
+static int launch_skinny_x(const void* x, long ldx, const void* W, long ldw, const void* bias, void* y, long ldy, int M,
+                           int N, int K, hipStream_t stream, RopeCacheArgs rc, NormAroundArgs na) {
   using T = SkinnyTile<KC>;
   constexpr int WT = (ACT >= 1 && ACT <= 3) ? 2 : 1;
   const size_t stage = (size_t)NW * (WT + MT) * T::TILE_BYTES;
   const size_t red = (size_t)NW * WT * MT * 64 * 4 * sizeof(float) + ((SCALED || ACT == 4) ? 256 * sizeof(float) : 0);
   const size_t smem = stage > red ? stage : red;
-  auto kernel = gemm_skinny_kernel<MT, KC, NW, TOut, ACT, DEPTH, SCALED>;
+  auto kernel = gemm_skinny_kernel<MT, KC, NW, TOut, ACT, DEPTH, SCALED, XROWS>;
   static bool configured = false;   // per instantiation
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -364,6 +369,18 @@ static int launch_skinny(const void* x, long ldx, const void* W, long ldw, const
   hipLaunchKernelGGL(kernel, dim3(blocks), dim3(NW * 64), smem, stream, (const bf16_t*)x, ldx, (const bf16_t*)W, ldw,
                      (const bf16_t*)bias, (TOut*)y, ldy, M, N, K, rc, na);
   return 0;
+}
+
+template <int MT, int KC, int NW, typename TOut, int ACT, int DEPTH = 1, bool SCALED = false>
+static int launch_skinny(const void* x, long ldx, const void* W, long ldw, const void* bias, void* y, long ldy, int M,
+                         int N, int K, hipStream_t stream, RopeCacheArgs rc = RopeCacheArgs(),
+                         NormAroundArgs na = NormAroundArgs()) {
+  // up to 8 rows (and tiles whose loads cover 8 rows each): half of x's tile is neither fetched nor staged
+  if constexpr (MT == 1 && SkinnyTile<KC>::ROWS_PER_LOAD <= 8) {
+    if (M <= 8)
+      return launch_skinny_x<MT, KC, NW, TOut, ACT, DEPTH, SCALED, 8>(x, ldx, W, ldw, bias, y, ldy, M, N, K, stream, rc, na);
+  }
+  return launch_skinny_x<MT, KC, NW, TOut, ACT, DEPTH, SCALED, 16>(x, ldx, W, ldw, bias, y, ldy, M, N, K, stream, rc, na);
 }
 
 // x [M, K] bfloat16 (row stride ldx), W [N, K] bfloat16 (row stride ldw), bias [N] bfloat16 or null,
