@@ -257,10 +257,15 @@ int op_linear(Run& r, const Value& x, const void* W, int wdtype, long ldw, int N
   const int M = x.M, K = x.N;
   const bool both_bf16 = x.dtype == LMSF_BF16 && wdtype == LMSF_BF16;
   const bool m_ok = mid_ok(x.p, x.ld, K, W, ldw, N), s_ok = skinny_ok(x.p, x.ld, K, W, ldw);
+  // (deep: K at least three times N; such products go to the many-rows kernel from fewer rows on, and stay with it
+  // beyond large_max_rows, which is then not this program's business)
+  const bool deep = (long)K >= 3L * N && out_dtype == LMSF_BF16;
   if (both_bf16 && t.skinny_max_rows < M && M <= t.mid_max_rows && m_ok &&
-      (M <= 64 || N <= t.mid_wide_max_cols || out_dtype == LMSF_F32))
+      (M <= 64 || N <= t.mid_wide_max_cols || out_dtype == LMSF_F32) && !(deep && M > t.large_deep_min_rows))
     return linear_mid(r, x, W, ldw, N, bias, 0, out_dtype, pending_ok && out_dtype == LMSF_BF16, out, res);
-  if (both_bf16 && out_dtype == LMSF_BF16 && t.mid_max_rows < M && M <= t.large_max_rows && m_ok)
+  if (both_bf16 && out_dtype == LMSF_BF16 && m_ok &&
+      ((t.mid_max_rows < M && M <= t.large_max_rows) ||
+       (deep && t.large_deep_min_rows < M && M <= t.large_max_rows)))
     return linear_large(r, x, W, ldw, N, bias, 0, pending_ok, out, res);
   if (pending_ok && both_bf16 && out_dtype == LMSF_BF16 && s_ok && M > 0) {
     if ((M <= std::min(t.fuse_stream_rows, t.gemv_max_rows) && gemv_ok(M, K)) ||

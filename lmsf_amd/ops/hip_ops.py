@@ -70,6 +70,7 @@ class HipOps:
         self.skinny_max_rows = 16      # rows up to which the few-rows kernel beats the library (measured)
         self.large_max_rows = 256      # rows up to which the many-rows kernel beats the library (measured; 0: never)
         self.weight_row_pad_bytes = 512  # bytes left between two rows of a linear layer's weight (see weight_row_pad)
+        self.large_deep_min_rows = 64    # products whose K is at least three times N go to the many-rows kernel from beyond this many rows already (down at 128 rows: 42.8 -> 38.0 us; decode at batch 128: 6.63 -> 6.53 ms a step, at 96: 5.83 -> 5.74)
         self.large_deep_max_rows = 1024  # the same for products whose K is at least three times N (down: 57 against 76 us at 320 rows, 74 against 94 at 512, 102 against 108 at 768, level at 1,024)
 
     # ------------------------------------------------------------------ helpers
@@ -609,12 +610,14 @@ class HipOps:
             return out if out is not None else torch.empty((M, N), dtype=out_dtype, device=x.device)
 
         both_bf16 = x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
+        deep = K >= 3 * N and out_dtype == torch.bfloat16
         if (both_bf16 and self.skinny_max_rows < M <= self.mid_max_rows and self._mid_ok(x, weight)
-                and (M <= 64 or N <= self.mid_wide_max_cols or out_dtype == torch.float32)):
+                and (M <= 64 or N <= self.mid_wide_max_cols or out_dtype == torch.float32)
+                and not (deep and M > self.large_deep_min_rows)):
             return self._linear_mid(x, weight, bias, 0, out_dtype, pending_ok and out_dtype == torch.bfloat16, out=out)
         if (both_bf16 and out_dtype == torch.bfloat16 and self._mid_ok(x, weight)
                 and (self.mid_max_rows < M <= self.large_max_rows
-                     or (self.large_max_rows < M <= self.large_deep_max_rows and K >= 3 * N))):
+                     or (deep and self.large_deep_min_rows < M <= self.large_deep_max_rows))):
             # 129 to 256 rows: the library is weak there (0.12 to 0.5 PFLOP/s at these widths)
             return self._linear_large(x, weight, bias, 0, pending_ok, out=out)
         if pending_ok and both_bf16 and out_dtype == torch.bfloat16 and self._skinny_ok(x, weight) and M > 0:
