@@ -279,9 +279,11 @@ extern "C" int lmsf_gemm_mid_splits(int M, int N, int K, int act) {
     if (s > 1 && chunks / s < 8) break;       // at least 8 steps per workgroup
     const long wg = blocks * s, rounds = (wg + 255) / 256;
     const double fill = (double)wg / (256.0 * rounds);
-    // partial sums are written and read again; the gated form also needs a kernel of its own to add them up
-    // (about 5 us, the time of 40 MB), the plain form's are added up by the kernel that takes the product
-    const double cost = w_bytes / fill + (s > 1 ? 2.0 * s * wt * (double)M * N * 4 + (act ? 40e6 : 0.0) : 0.0);
+    // partial sums are written and read again, and a byte of them costs about three of the weights' (measured: QKV of
+    // 6,144 x 4,096 at 64 rows 18.5 us in 2 parts against 20.8 in 5, of 12,288 x 4,096 26.3 in one piece against 31.8
+    // in 4; o and down of 4,096 columns stay at 4 parts); the gated form also needs a kernel of its own to add them
+    // up (about 5 us, the time of 40 MB), the plain form's are added up by the kernel that takes the product
+    const double cost = w_bytes / fill + (s > 1 ? 6.0 * s * wt * (double)M * N * 4 + (act ? 40e6 : 0.0) : 0.0);
     if (s == 1 || cost < best_cost) {
       best = s;
       best_cost = cost;
