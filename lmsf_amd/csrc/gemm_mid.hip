@@ -64,23 +64,24 @@ __device__ __forceinline__ void mid_store4(float* p, const float* o) {
 
 // MT: tiles of 16 rows of x (2, 4, 6 or 8). ACT: 0 none, 1 silu-gated, 2 gelu-gated (W = [gate rows; up rows], N
 // outputs). PARTIAL: write float32 partial sums of this workgroup's part of K instead of the result.
-// PAIR (with ACT, without PARTIAL): a workgroup owns 32 outputs instead of 64; waves 0 and 1 multiply their gate
-// rows, waves 2 and 3 the up rows of the same outputs, and the two meet in LDS for the activation. Twice as many
-// workgroups, two to a compute unit: the weights stream faster that way (4.7 -> 5.0 TB/s at 17 to 32 rows).
-template <int MT, int ACT, bool PARTIAL, typename TOut, bool PAIR = false>
+// (A form of the gated product with 32 outputs a workgroup, waves 0 and 1 on the gate rows and 2 and 3 on the up rows
+// of the same outputs, twice as many workgroups, two to a compute unit, was ahead at 17 to 48 rows while the
+// weights' rows lay back to back and were loaded like anything else: 4.7 -> 5.0 TB/s. With the rows apart and the
+// transfers non-temporal it is behind at every number of rows, 42.3 against 40.5 us at 17 rows and 50.1 against 42.7
+// at 48, and is gone.)
+template <int MT, int ACT, bool PARTIAL, typename TOut>
 __global__ __launch_bounds__(256) void gemm_mid_kernel(const bf16_t* __restrict__ x, long ldx,
                                                        const bf16_t* __restrict__ W, long ldw,
                                                        const bf16_t* __restrict__ bias, TOut* __restrict__ y,
                                                        long ldy, float* __restrict__ part, int M, int N, int K,
                                                        int n_split) {
-  static_assert(!PAIR || (ACT != 0 && !PARTIAL), "the paired form is the gated product in one piece");
-  constexpr int WT = (ACT && !PAIR) ? 2 : 1;
+  constexpr int WT = ACT ? 2 : 1;
   constexpr int STAGE = (4 * WT + MT) * MID_TILE;
   constexpr int XL = MT / 2;           // halves of x tiles this wave moves per step (2 MT halves over 4 waves)
   constexpr int LPW = 2 * WT + XL;     // transfers per wave and step
   extern __shared__ __align__(16) unsigned char lds[];
   const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
-  const int n0 = blockIdx.x * (PAIR ? 32 : 64), split = blockIdx.y;
+  const int n0 = blockIdx.x * 64, split = blockIdx.y;
   const int chunks = K / 64;
   const int c_begin = (int)((long)split * chunks / n_split), c_end = (int)((long)(split + 1) * chunks / n_split);
   const int n_steps = c_end - c_begin;
@@ -94,10 +95,10 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const bf16_t* __restrict_
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       const int row = 8 * h + trow, piece = (tslot - row) & 7;
-      int n = n0 + (PAIR ? 16 * (w & 1) : 16 * w) + row;
+      int n = n0 + 16 * w + row;
       if (n > N - 1) n = N - 1;        // rows beyond the matrix repeat the last row and are not stored
-      const int half = PAIR ? (w >> 1) : t;   // 0: the gate's rows (or the only ones), 1: the up projection's
-      src[t * 2 + h] = W + (long)(n + half * N) * ldw + piece * 8 + (long)c_begin * 64;
+      // t: 0 the gate's rows (or the only ones), 1: the up projection's
+      src[t * 2 + h] = W + (long)(n + t * N) * ldw + piece * 8 + (long)c_begin * 64;
       dst[t * 2 + h] = (w * WT + t) * MID_TILE + h * 1024;
     }
 #pragma unroll
@@ -161,33 +162,6 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const bf16_t* __restrict_
     consume = consume + STAGE == MID_STAGES * STAGE ? 0 : consume + STAGE;
   }
 
-  if (PAIR) {
-    // the up rows' sums go through LDS to the waves that hold the gate rows' sums of the same outputs
-    __syncthreads();                   // everybody is done with the last stage
-    float* ex = reinterpret_cast<float*>(lds);   // [2 waves][MT][64 lanes][4]
-    if (w >= 2) {
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) *reinterpret_cast<f32x4_t*>(ex + (((w - 2) * MT + mt) * 64 + l) * 4) = acc[0][mt];
-    }
-    __syncthreads();
-    const int n = n0 + 16 * w + 4 * g;
-    if (w >= 2 || n >= N) return;
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const int m = mt * 16 + r;
-      if (m >= M) continue;
-      const f32x4_t up = *reinterpret_cast<const f32x4_t*>(ex + ((w * MT + mt) * 64 + l) * 4);
-      float o[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const float gg = acc[0][mt][i] + (bias ? bf16_to_f32(bias[n + i]) : 0.f);
-        const float uu = up[i] + (bias ? bf16_to_f32(bias[N + n + i]) : 0.f);
-        o[i] = mid_activation(gg, uu, ACT);
-      }
-      mid_store4(y + (long)m * ldy + n, o);
-    }
-    return;
-  }
   // this lane holds, for token m = mt * 16 + r, the outputs n = n0 + 16 w + 4 g .. + 3
   const int n = n0 + 16 * w + 4 * g;
   if (n >= N) return;                  // N is a multiple of 4 where it is not a multiple of 64 (checked by the host)
@@ -245,12 +219,12 @@ __global__ __launch_bounds__(256) void gemm_mid_reduce_kernel(const float* __res
   mid_store4(y + (long)m * ldy + n, o);
 }
 
-template <int MT, int ACT, bool PARTIAL, typename TOut, bool PAIR = false>
+template <int MT, int ACT, bool PARTIAL, typename TOut>
 static int launch_mid(dim3 grid, hipStream_t stream, const bf16_t* x, long ldx, const bf16_t* W, long ldw,
                       const bf16_t* bias, TOut* y, long ldy, float* part, int M, int N, int K, int n_split) {
-  constexpr int WT = (ACT && !PAIR) ? 2 : 1;
+  constexpr int WT = ACT ? 2 : 1;
   const size_t smem = (size_t)MID_STAGES * (4 * WT + MT) * MID_TILE;
-  auto kernel = gemm_mid_kernel<MT, ACT, PARTIAL, TOut, PAIR>;
+  auto kernel = gemm_mid_kernel<MT, ACT, PARTIAL, TOut>;
   static bool configured = false;   // per instantiation
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -319,20 +293,6 @@ static int mid_product(const bf16_t* xb, long ldx, const bf16_t* Wb, long ldw, c
                        long ldy, int M, int N, int K, int act, int n_split, float* scratch, hipStream_t stream) {
   dim3 grid((N + 63) / 64, n_split);
   int rc = 0;
-  if (act != 0 && n_split == 1 && out_dtype != LMSF_F32 && M <= 48) {
-    // the gated product in one piece, up to 48 rows: 32 outputs a workgroup (gate_up of 28,672 x 4,096 at 17 / 32 /
-    // 48 / 64 rows: 46.8 / 47.4 / 50.1 / 52.6 us against 50.4 / 49.8 / 50.6 / 51.4 with 64 outputs a workgroup; every
-    // workgroup reads all of x, and with more rows that outweighs the faster stream of the weights)
-    dim3 pgrid((N + 31) / 32, 1);
-#define MIDP(MT_, ACT_) \
-  rc = launch_mid<MT_, ACT_, false, bf16_t, true>(pgrid, stream, xb, ldx, Wb, ldw, bb, (bf16_t*)y, ldy, scratch, M, N, K, 1)
-    if (M <= 32) { if (act == 1) MIDP(2, 1); else MIDP(2, 2); }
-    else { if (act == 1) MIDP(4, 1); else MIDP(4, 2); }
-#undef MIDP
-    if (rc) return rc;
-    LMSF_LAUNCH_CHECK("gemm_mid (gated)");
-    return 0;
-  }
 #define MID(MT_, ACT_, T_)                                                                                          \
   rc = n_split > 1                                                                                                  \
            ? launch_mid<MT_, ACT_, true, T_>(grid, stream, xb, ldx, Wb, ldw, bb, (T_*)y, ldy, scratch, M, N, K, n_split) \
