@@ -42,6 +42,9 @@ int lmsf_gemm_mid_splits(int M, int N, int K, int act);
 long lmsf_gemm_mid_scratch_floats(int M, int N, int n_split, int act);
 int lmsf_gemm_mid(const void* x, long ldx, const void* W, long ldw, const void* bias, void* y, int out_dtype, long
     ldy, int M, int N, int K, int act, int n_split, float* scratch, hipStream_t stream);
+int lmsf_gemm_mid_scaled_fits(int M, int N, int K, int in_tiles);
+int lmsf_gemm_mid_scaled(const void* x, long ldx, const void* W, long ldw, const void* bias, void* y, long ldy, int M,
+    int N, int K, int act, const float* sumsq, int in_tiles, float eps, hipStream_t stream);
 int lmsf_gemm_mid_partial(const void* x, long ldx, const void* W, long ldw, int M, int N, int K, int n_split, float*
     scratch, hipStream_t stream);
 int lmsf_gemm_mid_reduce(const float* scratch, const void* bias, void* y, int out_dtype, long ldy, int M, int N, int

@@ -69,12 +69,24 @@ __device__ __forceinline__ void mid_store4(float* p, const float* o) {
 // weights' rows lay back to back and were loaded like anything else: 4.7 -> 5.0 TB/s. With the rows apart and the
 // transfers non-temporal it is behind at every number of rows, 42.3 against 40.5 us at 17 rows and 50.1 against 42.7
 // at 48, and is gone.)
+// What the gated product takes when it stands after a norm whose row factor it applies itself (up to 16 rows): x is
+// then bf16(stream * w), sumsq [tiles][16] the sums of stream^2 over 16 columns per row (rows >= M: 0), and the rows
+// of both products are multiplied by rsqrt(sum / H + eps) before bias and activation, as the few-rows product does
+// (gemm_skinny.hip). sumsq null: no factor.
+struct MidRowScale {
+  const float* sumsq;
+  int tiles;
+  float eps;
+  int H;
+};
+#define MID_SCALE_HELD 16   // sums a thread holds: thread t has row t % 16 of the tiles t / 16, t / 16 + 16, ...
+
 template <int MT, int ACT, bool PARTIAL, typename TOut>
 __global__ __launch_bounds__(256) void gemm_mid_kernel(const bf16_t* __restrict__ x, long ldx,
                                                        const bf16_t* __restrict__ W, long ldw,
                                                        const bf16_t* __restrict__ bias, TOut* __restrict__ y,
                                                        long ldy, float* __restrict__ part, int M, int N, int K,
-                                                       int n_split) {
+                                                       int n_split, MidRowScale rs) {
   constexpr int WT = ACT ? 2 : 1;
   constexpr int STAGE = (4 * WT + MT) * MID_TILE;
   constexpr int XL = MT / 2;           // halves of x tiles this wave moves per step (2 MT halves over 4 waves)
@@ -121,6 +133,17 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const bf16_t* __restrict_
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[t][mt] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
 
+  // The row factor's sums are asked for before the first weights (loads come back in the order they were asked for)
+  // and added up after the last step, when nothing waits for them any more.
+  constexpr bool MAY_SCALE = ACT != 0 && !PARTIAL;
+  float held[MID_SCALE_HELD];
+  if (MAY_SCALE && rs.sumsq) {
+#pragma unroll
+    for (int k = 0; k < MID_SCALE_HELD; ++k) {
+      const int t = (tid >> 4) + 16 * k;
+      held[k] = t < rs.tiles ? rs.sumsq[t * 16 + (tid & 15)] : 0.f;
+    }
+  }
   const unsigned lds0 = mid_lds_address(lds);
   auto issue = [&](int step, int stage_byte) {
 #pragma unroll
@@ -162,6 +185,20 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const bf16_t* __restrict_
     consume = consume + STAGE == MID_STAGES * STAGE ? 0 : consume + STAGE;
   }
 
+  float inv = 1.f;                     // the factor of row r (rows of the first tile only: up to 16 rows)
+  if (MAY_SCALE && rs.sumsq) {
+    float sum = 0.f;
+#pragma unroll
+    for (int k = 0; k < MID_SCALE_HELD; ++k) sum += held[k];
+    __syncthreads();                   // everybody is done with the last stage
+    float* red = reinterpret_cast<float*>(lds);
+    red[tid] = sum;
+    __syncthreads();
+    float total = 0.f;
+#pragma unroll
+    for (int k = 0; k < 16; ++k) total += red[k * 16 + r];   // in a fixed order
+    inv = rsqrtf(total / (float)rs.H + rs.eps);
+  }
   // this lane holds, for token m = mt * 16 + r, the outputs n = n0 + 16 w + 4 g .. + 3
   const int n = n0 + 16 * w + 4 * g;
   if (n >= N) return;                  // N is a multiple of 4 where it is not a multiple of 64 (checked by the host)
@@ -181,8 +218,8 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const bf16_t* __restrict_
         if (ACT == 0) {
           o[i] = acc[0][mt][i] + (bias ? bf16_to_f32(bias[n + i]) : 0.f);
         } else {
-          const float gg = acc[0][mt][i] + (bias ? bf16_to_f32(bias[n + i]) : 0.f);
-          const float uu = acc[WT - 1][mt][i] + (bias ? bf16_to_f32(bias[N + n + i]) : 0.f);
+          const float gg = acc[0][mt][i] * inv + (bias ? bf16_to_f32(bias[n + i]) : 0.f);
+          const float uu = acc[WT - 1][mt][i] * inv + (bias ? bf16_to_f32(bias[N + n + i]) : 0.f);
           o[i] = mid_activation(gg, uu, ACT);
         }
       }
@@ -221,7 +258,8 @@ __global__ __launch_bounds__(256) void gemm_mid_reduce_kernel(const float* __res
 
 template <int MT, int ACT, bool PARTIAL, typename TOut>
 static int launch_mid(dim3 grid, hipStream_t stream, const bf16_t* x, long ldx, const bf16_t* W, long ldw,
-                      const bf16_t* bias, TOut* y, long ldy, float* part, int M, int N, int K, int n_split) {
+                      const bf16_t* bias, TOut* y, long ldy, float* part, int M, int N, int K, int n_split,
+                      MidRowScale rs) {
   constexpr int WT = ACT ? 2 : 1;
   const size_t smem = (size_t)MID_STAGES * (4 * WT + MT) * MID_TILE;
   auto kernel = gemm_mid_kernel<MT, ACT, PARTIAL, TOut>;
@@ -235,7 +273,7 @@ static int launch_mid(dim3 grid, hipStream_t stream, const bf16_t* x, long ldx, 
     }
     configured = true;
   }
-  hipLaunchKernelGGL(kernel, grid, dim3(256), smem, stream, x, ldx, W, ldw, bias, y, ldy, part, M, N, K, n_split);
+  hipLaunchKernelGGL(kernel, grid, dim3(256), smem, stream, x, ldx, W, ldw, bias, y, ldy, part, M, N, K, n_split, rs);
   return 0;
 }
 
@@ -290,13 +328,14 @@ static int mid_check(const void* x, long ldx, const void* W, long ldw, int M, in
 
 // The product's kernel: the result into y (n_split == 1) or partial sums into scratch.
 static int mid_product(const bf16_t* xb, long ldx, const bf16_t* Wb, long ldw, const bf16_t* bb, void* y, int out_dtype,
-                       long ldy, int M, int N, int K, int act, int n_split, float* scratch, hipStream_t stream) {
+                       long ldy, int M, int N, int K, int act, int n_split, float* scratch, hipStream_t stream,
+                       MidRowScale rs = MidRowScale{nullptr, 0, 0.f, 0}) {
   dim3 grid((N + 63) / 64, n_split);
   int rc = 0;
 #define MID(MT_, ACT_, T_)                                                                                          \
   rc = n_split > 1                                                                                                  \
-           ? launch_mid<MT_, ACT_, true, T_>(grid, stream, xb, ldx, Wb, ldw, bb, (T_*)y, ldy, scratch, M, N, K, n_split) \
-           : launch_mid<MT_, ACT_, false, T_>(grid, stream, xb, ldx, Wb, ldw, bb, (T_*)y, ldy, scratch, M, N, K, n_split)
+           ? launch_mid<MT_, ACT_, true, T_>(grid, stream, xb, ldx, Wb, ldw, bb, (T_*)y, ldy, scratch, M, N, K, n_split, rs) \
+           : launch_mid<MT_, ACT_, false, T_>(grid, stream, xb, ldx, Wb, ldw, bb, (T_*)y, ldy, scratch, M, N, K, n_split, rs)
   if (out_dtype == LMSF_F32) {
     if (M <= 32) MID(2, 0, float); else if (M <= 64) MID(4, 0, float); else if (M <= 96) MID(6, 0, float); else MID(8, 0, float);
   } else if (M <= 32) {
@@ -347,6 +386,35 @@ extern "C" int lmsf_gemm_mid(const void* x, long ldx, const void* W, long ldw, c
 // The two halves of a product without activation whose K is split (n_split >= 2): the partial sums alone,
 // scratch[(s * M + m) * N + n], for a kernel that reduces them while it loads its operand (LmsfPartialSum);
 // and the reduction alone, y = sum over s + bias, for a caller that turns out to need the plain result.
+// Whether the gated product after a norm should run here rather than in the few-rows kernel: when its workgroups (64
+// outputs each) fit on the chip at once, so that every compute unit streams one share of the weights from the first
+// step to the last (gate_up of 28,672 x 4,096 at 8 rows: 39.5 us against 43.9, at 16 rows 39.4 against 47.3; of
+// 57,344 x 8,192, 448 workgroups: 158.7 against 144.8, which stays with the few-rows kernel).
+extern "C" int lmsf_gemm_mid_scaled_fits(int M, int N, int K, int in_tiles) {
+  return M >= 1 && M <= 16 && N > 0 && N % 4 == 0 && K > 0 && K % 64 == 0 && in_tiles == (K + 15) / 16 &&
+         in_tiles <= 16 * MID_SCALE_HELD && (N + 63) / 64 <= lmsf_compute_units();
+}
+
+// The gated product (act 1 silu, 2 gelu) after a norm, with up to 16 rows: x [M, K] is bf16(stream * w) and sumsq
+// [in_tiles][16] its sums of squares, as the few-rows product before the norm writes them (lmsf_gemm_skinny_add_norm);
+// the rows of both products are multiplied by rsqrt(sum / K + eps) before bias and activation. K = 16 in_tiles at
+// most 4,096 (each thread holds 16 of the sums). In one piece, no split of K.
+extern "C" int lmsf_gemm_mid_scaled(const void* x, long ldx, const void* W, long ldw, const void* bias, void* y, long ldy,
+                                    int M, int N, int K, int act, const float* sumsq, int in_tiles, float eps,
+                                    hipStream_t stream) {
+  LMSF_CHECK(act == 1 || act == 2, "gemm_mid_scaled: activation %d (1 silu, 2 gelu)", act);
+  LMSF_CHECK(M >= 0 && M <= 16, "gemm_mid_scaled: M=%d outside [0, 16]", M);
+  if (int rc = mid_check(x, ldx, W, ldw, M, N, K, 1, nullptr, act)) return rc;
+  LMSF_CHECK(y != nullptr && lmsf_aligned16(y) && ldy >= N && ldy % 4 == 0,
+             "gemm_mid_scaled: y must be 16-byte aligned with a row stride that covers N and is a multiple of 4");
+  LMSF_CHECK(sumsq != nullptr && in_tiles > 0 && in_tiles == (K + 15) / 16 && in_tiles <= 16 * MID_SCALE_HELD,
+             "gemm_mid_scaled: %d sums of squares must cover %d columns (at most %d)", in_tiles, K, 16 * 16 * MID_SCALE_HELD);
+  if (M == 0) return 0;
+  const MidRowScale rs = {sumsq, in_tiles, eps, K};
+  return mid_product((const bf16_t*)x, ldx, (const bf16_t*)W, ldw, (const bf16_t*)bias, y, LMSF_BF16, ldy, M, N, K, act, 1,
+                     nullptr, stream, rs);
+}
+
 extern "C" int lmsf_gemm_mid_partial(const void* x, long ldx, const void* W, long ldw, int M, int N, int K,
                                      int n_split, float* scratch, hipStream_t stream) {
   if (int rc = mid_check(x, ldx, W, ldw, M, N, K, n_split, scratch)) return rc;

@@ -40,7 +40,7 @@ enum {
 typedef struct {
   int fuse_norm_rows, fuse_stream_rows, gemv_max_rows, skinny_variant, mid_wide_max_cols, mid_max_rows,
       skinny_max_rows, prefill_attention_variant, decode_attention_order, decode_attention_splits, use_library_gemm,
-      large_max_rows, large_deep_min_rows;
+      large_max_rows, large_deep_min_rows, mid_scaled_rows;
 } LmsfTunables;
 
 // One operation. Registers (in0, in1, out) are numbered in the order they are first written; -1: none.

@@ -479,7 +479,10 @@ int op_linear_gated(Run& r, const Value& x_in, const void* W, int wdtype, long l
     const int M = x.M, K = x.N;
     if (wdtype == LMSF_BF16 && skinny_ok(x.p, x.ld, K, W, ldw) && (x.rows_per_tile == 16 || gemv_ok(M, K))) {
       TAKE(y, void*, (size_t)M * I * 2);
-      if (x.rows_per_tile != 16)
+      if (x.rows_per_tile == 16 && M <= t.mid_scaled_rows && mid_ok(x.p, x.ld, K, W, ldw, w_rows) &&
+          lmsf_gemm_mid_scaled_fits(M, I, K, x.tiles))
+        LAUNCH(lmsf_gemm_mid_scaled(x.p, x.ld, W, ldw, bias, y, I, M, I, K, kind, x.sumsq, x.tiles, x.eps, r.stream));
+      else if (x.rows_per_tile != 16)
         LAUNCH(lmsf_gemv_scaled(x.p, x.ld, W, ldw, bias, y, I, M, I, K, kind, x.sumsq, x.tiles, x.eps, r.stream));
       else
         LAUNCH(lmsf_gemm_skinny_scaled(x.p, x.ld, W, ldw, bias, y, I, M, I, K, kind, x.sumsq, x.tiles, x.eps,

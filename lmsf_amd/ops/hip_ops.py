@@ -71,6 +71,7 @@ class HipOps:
         self.large_max_rows = 256      # rows up to which the many-rows kernel beats the library (measured; 0: never)
         self.weight_row_pad_bytes = 512  # bytes left between two rows of a linear layer's weight (see weight_row_pad)
         self.large_deep_min_rows = 64    # products whose K is at least three times N go to the many-rows kernel from beyond this many rows already (down at 128 rows: 42.8 -> 38.0 us; decode at batch 128: 6.63 -> 6.53 ms a step, at 96: 5.83 -> 5.74)
+        self.mid_scaled_rows = 16        # rows up to which the gated product after a norm runs in the 17-and-more-rows kernel where that kernel's workgroups fit on the chip at once (0: never)
         self.large_deep_max_rows = 1024  # the same for products whose K is at least three times N (down: 57 against 76 us at 320 rows, 74 against 94 at 512, 102 against 108 at 768, level at 1,024)
 
     # ------------------------------------------------------------------ helpers
@@ -687,6 +688,12 @@ class HipOps:
             if bias is not None and (bias.shape != (2 * I,) or bias.dtype != weight.dtype or not bias.is_contiguous()):
                 raise ValueError("linear_gated: bias must be [%d] of the weight's dtype" % (2 * I))
             y = torch.empty((M, I), dtype=torch.bfloat16, device=x.device)
+            if (x.rows_per_tile == 16 and M <= self.mid_scaled_rows and self._mid_ok(x.xw, weight)
+                    and self.lib.lmsf_gemm_mid_scaled_fits(M, I, K, x.tiles)):
+                self._check(self.lib.lmsf_gemm_mid_scaled(
+                    _ptr(x.xw), x.xw.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(y), y.stride(0), M, I, K,
+                    kinds[kind], _ptr(x.sumsq), x.tiles, x.eps, self._stream()))
+                return y
             if x.rows_per_tile != 16:
                 self._check(self.lib.lmsf_gemv_scaled(
                     _ptr(x.xw), x.xw.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(y), y.stride(0), M, I, K,

@@ -63,6 +63,8 @@ _SIGNATURES = {
     "lmsf_gemm_mid_splits": (c_int, [c_int, c_int, c_int, c_int]),
     "lmsf_gemm_mid_scratch_floats": (c_long, [c_int, c_int, c_int, c_int]),
     "lmsf_gemm_mid": (c_int, [_P, c_long, _P, c_long, _P, _P, c_int, c_long, c_int, c_int, c_int, c_int, c_int, _P, _P]),
+    "lmsf_gemm_mid_scaled_fits": (c_int, [c_int, c_int, c_int, c_int]),
+    "lmsf_gemm_mid_scaled": (c_int, [_P, c_long, _P, c_long, _P, _P, c_long, c_int, c_int, c_int, c_int, _P, c_int, c_float, _P]),
     "lmsf_gemm_mid_partial": (c_int, [_P, c_long, _P, c_long, c_int, c_int, c_int, c_int, _P, _P]),
     "lmsf_gemm_mid_reduce": (c_int, [_P, _P, _P, c_int, c_long, c_int, c_int, c_int, _P]),
     "lmsf_gemm_large_plan": (c_int, [c_int, c_int, c_int, c_int]),

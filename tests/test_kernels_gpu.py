@@ -678,6 +678,43 @@ def test_products_of_one_or_two_rows(ops, ref, M, N, K, bias):
         ops.gemv_max_rows = 2
 
 
+@pytest.mark.parametrize("M", [3, 8, 16])
+@pytest.mark.parametrize("H,I", [(1024, 1004), (4096, 2048), (256, 16384)])
+@pytest.mark.parametrize("bias", [False, True])
+def test_gated_product_after_a_norm_in_either_kernel(ops, ref, M, H, I, bias):
+    """The gated product that applies the norm's row factor itself runs in the 17-and-more-rows kernel where that
+    kernel's workgroups fit on the chip at once, else in the few-rows kernel: the two agree with each other and with
+    the plain formula, with outputs that are no multiple of 64 and with a bias."""
+    from lmsf_amd.ops.handles import ScaledRows
+    g = torch.Generator().manual_seed(M * H + I)
+    x = dev(torch.randn(M, H, generator=g).bfloat16())
+    w = dev((torch.randn(H, H, generator=g) * H ** -0.5).bfloat16())
+    nw = dev(torch.randn(H, generator=g).bfloat16())
+    res = dev(torch.randn(M, H, generator=g) * 3.0)
+    p = ops.linear(x, w, None, pending_ok=True)
+    h = ops.add_rms_norm(p, res.clone(), nw, 1e-5, torch.bfloat16, defer_ok=True)
+    assert isinstance(h, ScaledRows) and h.rows_per_tile == 16
+    wg = dev((torch.randn(2 * I, H, generator=g) * H ** -0.5).bfloat16())
+    bg = dev(torch.randn(2 * I, generator=g).bfloat16()) if bias else None
+    assert ops.lib.lmsf_gemm_mid_scaled_fits(M, I, H, h.tiles) == 1
+    want_h = ref.add_rms_norm(ops.linear(x, w), res.clone(), nw, 1e-5, torch.bfloat16)
+    for kind in ("silu", "gelu"):
+        here = ops.linear_gated(h, wg, bg, kind)
+        before = ops.mid_scaled_rows
+        ops.mid_scaled_rows = 0
+        try:
+            there = ops.linear_gated(h, wg, bg, kind)
+        finally:
+            ops.mid_scaled_rows = before
+        want = ref.linear_gated(want_h, wg, bg, kind).float()
+        t = 2e-2 * max(1.0, want.abs().max().item())
+        assert here.shape == (M, I) and (here.float() - want).abs().max().item() <= t
+        assert (here.float() - there.float()).abs().max().item() <= t and not torch.isnan(here.float()).any()
+    # too many workgroups for the chip, or sums of squares that a thread cannot hold: the few-rows kernel
+    assert ops.lib.lmsf_gemm_mid_scaled_fits(M, 64 * 257, H, h.tiles) == 0
+    assert ops.lib.lmsf_gemm_mid_scaled_fits(M, I, 8192, 512) == 0 and ops.lib.lmsf_gemm_mid_scaled_fits(17, I, H, h.tiles) == 0
+
+
 @pytest.mark.parametrize("M,stream_rows", [(1, 1), (2, 2), (2, 1), (8, 1), (16, 1)])
 @pytest.mark.parametrize("H,K,nh,nkv,d,I", [(4096, 4096, 32, 8, 128, 1024), (1000, 14336, 5, 5, 64, 331), (80, 128, 3, 1, 32, 77),
                                             (8200, 256, 2, 2, 64, 96)])
