@@ -389,10 +389,13 @@ extern "C" int lmsf_gemm_mid(const void* x, long ldx, const void* W, long ldw, c
 // Whether the gated product after a norm should run here rather than in the few-rows kernel: when its workgroups (64
 // outputs each) fit on the chip at once, so that every compute unit streams one share of the weights from the first
 // step to the last (gate_up of 28,672 x 4,096 at 8 rows: 39.5 us against 43.9, at 16 rows 39.4 against 47.3; of
-// 57,344 x 8,192, 448 workgroups: 158.7 against 144.8, which stays with the few-rows kernel).
+// 57,344 x 8,192, 448 workgroups: 158.7 against 144.8, which stays with the few-rows kernel), and when they do not
+// leave too many compute units without one (22,016 x 4,096, 172 workgroups on 256 units: 39.0 against 33.7 us at 8
+// rows, 35.2 against 38.5 at 16): from 0.8 of the units on with up to 8 rows, from 0.58 on beyond.
 extern "C" int lmsf_gemm_mid_scaled_fits(int M, int N, int K, int in_tiles) {
+  const long blocks = (N + 63) / 64, cus = lmsf_compute_units();
   return M >= 1 && M <= 16 && N > 0 && N % 4 == 0 && K > 0 && K % 64 == 0 && in_tiles == (K + 15) / 16 &&
-         in_tiles <= 16 * MID_SCALE_HELD && (N + 63) / 64 <= lmsf_compute_units();
+         in_tiles <= 16 * MID_SCALE_HELD && blocks <= cus && blocks * 100 >= cus * (M <= 8 ? 80 : 58);
 }
 
 // The gated product (act 1 silu, 2 gelu) after a norm, with up to 16 rows: x [M, K] is bf16(stream * w) and sumsq

@@ -679,7 +679,7 @@ def test_products_of_one_or_two_rows(ops, ref, M, N, K, bias):
 
 
 @pytest.mark.parametrize("M", [3, 8, 16])
-@pytest.mark.parametrize("H,I", [(1024, 1004), (4096, 2048), (256, 16384)])
+@pytest.mark.parametrize("H,I", [(1024, 14300), (4096, 14336), (256, 16384)])
 @pytest.mark.parametrize("bias", [False, True])
 def test_gated_product_after_a_norm_in_either_kernel(ops, ref, M, H, I, bias):
     """The gated product that applies the norm's row factor itself runs in the 17-and-more-rows kernel where that
@@ -710,7 +710,10 @@ def test_gated_product_after_a_norm_in_either_kernel(ops, ref, M, H, I, bias):
         t = 2e-2 * max(1.0, want.abs().max().item())
         assert here.shape == (M, I) and (here.float() - want).abs().max().item() <= t
         assert (here.float() - there.float()).abs().max().item() <= t and not torch.isnan(here.float()).any()
-    # too many workgroups for the chip, or sums of squares that a thread cannot hold: the few-rows kernel
+    # too many workgroups for the chip, too few to keep most of it busy, or sums of squares that a thread cannot hold:
+    # the few-rows kernel
+    assert ops.lib.lmsf_gemm_mid_scaled_fits(8, 11008, H, h.tiles) == 0 and ops.lib.lmsf_gemm_mid_scaled_fits(16, 11008, H, h.tiles) == 1
+    assert ops.lib.lmsf_gemm_mid_scaled_fits(16, 2048, H, h.tiles) == 0
     assert ops.lib.lmsf_gemm_mid_scaled_fits(M, 64 * 257, H, h.tiles) == 0
     assert ops.lib.lmsf_gemm_mid_scaled_fits(M, I, 8192, 512) == 0 and ops.lib.lmsf_gemm_mid_scaled_fits(17, I, H, h.tiles) == 0
 
