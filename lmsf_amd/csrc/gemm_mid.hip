@@ -59,7 +59,7 @@ __device__ __forceinline__ void mid_store4(float* p, const float* o) {
   *reinterpret_cast<float4*>(p) = make_float4(o[0], o[1], o[2], o[3]);
 }
 
-#define MID_STAGES 5
+#define MID_STAGES_OF(TW) ((TW) == 2 ? 4 : 5)   // stages of the ring: what fits into the 160 KB of LDS
 #define MID_TILE 2048
 
 // MT: tiles of 16 rows of x (2, 4, 6 or 8). ACT: 0 none, 1 silu-gated, 2 gelu-gated (W = [gate rows; up rows], N
@@ -79,21 +79,23 @@ struct MidRowScale {
   float eps;
   int H;
 };
-#define MID_SCALE_HELD 16   // sums a thread holds: thread t has row t % 16 of the tiles t / 16, t / 16 + 16, ...
+#define MID_SCALE_HELD 32   // sums a thread holds: thread t has row t % 16 of the tiles t / 16, t / 16 + 16, ...
 
-template <int MT, int ACT, bool PARTIAL, typename TOut>
+template <int MT, int ACT, bool PARTIAL, typename TOut, int TW>
 __global__ __launch_bounds__(256) void gemm_mid_kernel(const bf16_t* __restrict__ x, long ldx,
                                                        const bf16_t* __restrict__ W, long ldw,
                                                        const bf16_t* __restrict__ bias, TOut* __restrict__ y,
                                                        long ldy, float* __restrict__ part, int M, int N, int K,
                                                        int n_split, MidRowScale rs) {
-  constexpr int WT = ACT ? 2 : 1;
+  constexpr int WP = ACT ? 2 : 1;      // projections: gate and up, or the only one
+  constexpr int WT = WP * TW;          // tiles of 16 rows of W per wave: TW of each projection
+  constexpr int STAGES = MID_STAGES_OF(TW);
   constexpr int STAGE = (4 * WT + MT) * MID_TILE;
   constexpr int XL = MT / 2;           // halves of x tiles this wave moves per step (2 MT halves over 4 waves)
   constexpr int LPW = 2 * WT + XL;     // transfers per wave and step
   extern __shared__ __align__(16) unsigned char lds[];
   const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, r = l & 15, g = l >> 4;
-  const int n0 = blockIdx.x * 64, split = blockIdx.y;
+  const int n0 = blockIdx.x * (64 * TW), split = blockIdx.y;
   const int chunks = K / 64;
   const int c_begin = (int)((long)split * chunks / n_split), c_end = (int)((long)(split + 1) * chunks / n_split);
   const int n_steps = c_end - c_begin;
@@ -107,10 +109,11 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const bf16_t* __restrict_
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       const int row = 8 * h + trow, piece = (tslot - row) & 7;
-      int n = n0 + 16 * w + row;
+      // tile t of this wave: projection t / TW (0 the gate's rows or the only ones, 1 the up projection's), the
+      // wave's 16 outputs number t % TW
+      int n = n0 + 16 * (w * TW + t % TW) + row;
       if (n > N - 1) n = N - 1;        // rows beyond the matrix repeat the last row and are not stored
-      // t: 0 the gate's rows (or the only ones), 1: the up projection's
-      src[t * 2 + h] = W + (long)(n + t * N) * ldw + piece * 8 + (long)c_begin * 64;
+      src[t * 2 + h] = W + (long)(n + (t / TW) * N) * ldw + piece * 8 + (long)c_begin * 64;
       dst[t * 2 + h] = (w * WT + t) * MID_TILE + h * 1024;
     }
 #pragma unroll
@@ -156,19 +159,19 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const bf16_t* __restrict_
     }
   };
 #pragma unroll
-  for (int s = 0; s < MID_STAGES - 1; ++s)
+  for (int s = 0; s < STAGES - 1; ++s)
     if (s < n_steps) issue(s, s * STAGE);
 
-  int consume = 0, produce = (MID_STAGES - 1) * STAGE;
+  int consume = 0, produce = (STAGES - 1) * STAGE;
   for (int it = 0; it < n_steps; ++it) {
     // step ``it`` has arrived when at most the transfers of the later steps are outstanding
-    if (it + MID_STAGES - 2 < n_steps)
-      asm volatile("s_waitcnt vmcnt(%0)" ::"n"((MID_STAGES - 2) * LPW) : "memory");
+    if (it + STAGES - 2 < n_steps)
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"((STAGES - 2) * LPW) : "memory");
     else
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();   // everybody's part of step ``it`` is there, and everybody is done with step ``it - 1``
-    if (it + MID_STAGES - 1 < n_steps) issue(it + MID_STAGES - 1, produce);
-    produce = produce + STAGE == MID_STAGES * STAGE ? 0 : produce + STAGE;
+    if (it + STAGES - 1 < n_steps) issue(it + STAGES - 1, produce);
+    produce = produce + STAGE == STAGES * STAGE ? 0 : produce + STAGE;
     const unsigned char* st = lds + consume;
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
@@ -182,7 +185,7 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const bf16_t* __restrict_
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t], b[mt], acc[t][mt], 0, 0, 0);
     }
-    consume = consume + STAGE == MID_STAGES * STAGE ? 0 : consume + STAGE;
+    consume = consume + STAGE == STAGES * STAGE ? 0 : consume + STAGE;
   }
 
   float inv = 1.f;                     // the factor of row r (rows of the first tile only: up to 16 rows)
@@ -199,31 +202,34 @@ __global__ __launch_bounds__(256) void gemm_mid_kernel(const bf16_t* __restrict_
     for (int k = 0; k < 16; ++k) total += red[k * 16 + r];   // in a fixed order
     inv = rsqrtf(total / (float)rs.H + rs.eps);
   }
-  // this lane holds, for token m = mt * 16 + r, the outputs n = n0 + 16 w + 4 g .. + 3
-  const int n = n0 + 16 * w + 4 * g;
-  if (n >= N) return;                  // N is a multiple of 4 where it is not a multiple of 64 (checked by the host)
+  // this lane holds, for token m = mt * 16 + r, the outputs n = n0 + 16 (w TW + tw) + 4 g .. + 3
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    const int m = mt * 16 + r;
-    if (m >= M) continue;
-    if (PARTIAL) {
-      // partial sums: [split][tile of W rows (gate, up)][M][N]
+  for (int tw = 0; tw < TW; ++tw) {
+    const int n = n0 + 16 * (w * TW + tw) + 4 * g;
+    if (n >= N) continue;              // N is a multiple of 4 where it is not a multiple of 64 (checked by the host)
 #pragma unroll
-      for (int t = 0; t < WT; ++t)
-        *reinterpret_cast<f32x4_t*>(part + (((long)split * WT + t) * M + m) * N + n) = acc[t][mt];
-    } else {
-      float o[4];
+    for (int mt = 0; mt < MT; ++mt) {
+      const int m = mt * 16 + r;
+      if (m >= M) continue;
+      if (PARTIAL) {
+        // partial sums: [split][projection (gate, up)][M][N]
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        if (ACT == 0) {
-          o[i] = acc[0][mt][i] + (bias ? bf16_to_f32(bias[n + i]) : 0.f);
-        } else {
-          const float gg = acc[0][mt][i] * inv + (bias ? bf16_to_f32(bias[n + i]) : 0.f);
-          const float uu = acc[WT - 1][mt][i] * inv + (bias ? bf16_to_f32(bias[N + n + i]) : 0.f);
-          o[i] = mid_activation(gg, uu, ACT);
+        for (int p = 0; p < WP; ++p)
+          *reinterpret_cast<f32x4_t*>(part + (((long)split * WP + p) * M + m) * N + n) = acc[p * TW + tw][mt];
+      } else {
+        float o[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if (ACT == 0) {
+            o[i] = acc[tw][mt][i] + (bias ? bf16_to_f32(bias[n + i]) : 0.f);
+          } else {
+            const float gg = acc[tw][mt][i] * inv + (bias ? bf16_to_f32(bias[n + i]) : 0.f);
+            const float uu = acc[(WP - 1) * TW + tw][mt][i] * inv + (bias ? bf16_to_f32(bias[N + n + i]) : 0.f);
+            o[i] = mid_activation(gg, uu, ACT);
+          }
         }
+        mid_store4(y + (long)m * ldy + n, o);
       }
-      mid_store4(y + (long)m * ldy + n, o);
     }
   }
 }
@@ -256,13 +262,14 @@ __global__ __launch_bounds__(256) void gemm_mid_reduce_kernel(const float* __res
   mid_store4(y + (long)m * ldy + n, o);
 }
 
-template <int MT, int ACT, bool PARTIAL, typename TOut>
+template <int MT, int ACT, bool PARTIAL, typename TOut, int TW = 1>
 static int launch_mid(dim3 grid, hipStream_t stream, const bf16_t* x, long ldx, const bf16_t* W, long ldw,
                       const bf16_t* bias, TOut* y, long ldy, float* part, int M, int N, int K, int n_split,
                       MidRowScale rs) {
-  constexpr int WT = ACT ? 2 : 1;
-  const size_t smem = (size_t)MID_STAGES * (4 * WT + MT) * MID_TILE;
-  auto kernel = gemm_mid_kernel<MT, ACT, PARTIAL, TOut>;
+  static_assert(TW == 1 || TW == 2, "one or two tiles of each projection per wave");
+  constexpr int WT = (ACT ? 2 : 1) * TW;
+  const size_t smem = (size_t)MID_STAGES_OF(TW) * (4 * WT + MT) * MID_TILE;
+  auto kernel = gemm_mid_kernel<MT, ACT, PARTIAL, TOut, TW>;
   static bool configured = false;   // per instantiation
   if (!configured) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
@@ -389,19 +396,26 @@ extern "C" int lmsf_gemm_mid(const void* x, long ldx, const void* W, long ldw, c
 // Whether the gated product after a norm should run here rather than in the few-rows kernel: when its workgroups (64
 // outputs each) fit on the chip at once, so that every compute unit streams one share of the weights from the first
 // step to the last (gate_up of 28,672 x 4,096 at 8 rows: 39.5 us against 43.9, at 16 rows 39.4 against 47.3; of
-// 57,344 x 8,192, 448 workgroups: 158.7 against 144.8, which stays with the few-rows kernel), and when they do not
-// leave too many compute units without one (22,016 x 4,096, 172 workgroups on 256 units: 39.0 against 33.7 us at 8
-// rows, 35.2 against 38.5 at 16): from 0.8 of the units on with up to 8 rows, from 0.58 on beyond.
+// 57,344 x 8,192, 448 workgroups: 158.7 against 144.8), and when they do not leave too many compute units without
+// one (22,016 x 4,096, 172 workgroups on 256 units: 39.0 against 33.7 us at 8 rows, 35.2 against 38.5 at 16): from
+// 0.8 of the units on with up to 8 rows, from 0.58 on beyond. Where workgroups of 64 outputs are too many, those of
+// 128 take over beyond 8 rows (57,344 x 8,192 in 224 workgroups: a decode step of 80 such layers at 16 rows 25.6 ms
+// against 26.7, about 14 us a layer; at 4 and 8 rows 23.7 against 23.6 and 24.0 against 24.0, left to the few-rows
+// kernel).
+// Outputs a workgroup of the gated product after a norm takes: 64, or 128 (each wave two tiles of either projection,
+// a ring of 4 stages) where workgroups of 64 would be more than the chip holds at once.
+static int mid_scaled_outputs(int N) { return (N + 63) / 64 <= lmsf_compute_units() ? 64 : 128; }
 extern "C" int lmsf_gemm_mid_scaled_fits(int M, int N, int K, int in_tiles) {
-  const long blocks = (N + 63) / 64, cus = lmsf_compute_units();
+  const long per = mid_scaled_outputs(N), blocks = (N + per - 1) / per, cus = lmsf_compute_units();
   return M >= 1 && M <= 16 && N > 0 && N % 4 == 0 && K > 0 && K % 64 == 0 && in_tiles == (K + 15) / 16 &&
-         in_tiles <= 16 * MID_SCALE_HELD && blocks <= cus && blocks * 100 >= cus * (M <= 8 ? 80 : 58);
+         in_tiles <= 16 * MID_SCALE_HELD && blocks <= cus && blocks * 100 >= cus * (M <= 8 ? 80 : 58) &&
+         (per == 64 || M > 8);
 }
 
 // The gated product (act 1 silu, 2 gelu) after a norm, with up to 16 rows: x [M, K] is bf16(stream * w) and sumsq
 // [in_tiles][16] its sums of squares, as the few-rows product before the norm writes them (lmsf_gemm_skinny_add_norm);
 // the rows of both products are multiplied by rsqrt(sum / K + eps) before bias and activation. K = 16 in_tiles at
-// most 4,096 (each thread holds 16 of the sums). In one piece, no split of K.
+// most 8,192 (each thread holds 32 of the sums). In one piece, no split of K.
 extern "C" int lmsf_gemm_mid_scaled(const void* x, long ldx, const void* W, long ldw, const void* bias, void* y, long ldy,
                                     int M, int N, int K, int act, const float* sumsq, int in_tiles, float eps,
                                     hipStream_t stream) {
@@ -414,6 +428,16 @@ extern "C" int lmsf_gemm_mid_scaled(const void* x, long ldx, const void* W, long
              "gemm_mid_scaled: %d sums of squares must cover %d columns (at most %d)", in_tiles, K, 16 * 16 * MID_SCALE_HELD);
   if (M == 0) return 0;
   const MidRowScale rs = {sumsq, in_tiles, eps, K};
+  if (mid_scaled_outputs(N) == 128) {
+    const dim3 grid((N + 127) / 128, 1);
+    const int rc = act == 1 ? launch_mid<2, 1, false, bf16_t, 2>(grid, stream, (const bf16_t*)x, ldx, (const bf16_t*)W, ldw,
+                                                                 (const bf16_t*)bias, (bf16_t*)y, ldy, nullptr, M, N, K, 1, rs)
+                            : launch_mid<2, 2, false, bf16_t, 2>(grid, stream, (const bf16_t*)x, ldx, (const bf16_t*)W, ldw,
+                                                                 (const bf16_t*)bias, (bf16_t*)y, ldy, nullptr, M, N, K, 1, rs);
+    if (rc) return rc;
+    LMSF_LAUNCH_CHECK("gemm_mid_scaled");
+    return 0;
+  }
   return mid_product((const bf16_t*)x, ldx, (const bf16_t*)W, ldw, (const bf16_t*)bias, y, LMSF_BF16, ldy, M, N, K, act, 1,
                      nullptr, stream, rs);
 }

@@ -679,12 +679,13 @@ def test_products_of_one_or_two_rows(ops, ref, M, N, K, bias):
 
 
 @pytest.mark.parametrize("M", [3, 8, 16])
-@pytest.mark.parametrize("H,I", [(1024, 14300), (4096, 14336), (256, 16384)])
+@pytest.mark.parametrize("H,I", [(1024, 14300), (4096, 14336), (256, 16384), (512, 28600), (8192, 14336)])
 @pytest.mark.parametrize("bias", [False, True])
 def test_gated_product_after_a_norm_in_either_kernel(ops, ref, M, H, I, bias):
     """The gated product that applies the norm's row factor itself runs in the 17-and-more-rows kernel where that
     kernel's workgroups fit on the chip at once, else in the few-rows kernel: the two agree with each other and with
-    the plain formula, with outputs that are no multiple of 64 and with a bias."""
+    the plain formula, with outputs that are no multiple of 64 and with a bias; so does the form with 128 outputs a
+    workgroup, which takes over where workgroups of 64 outputs would be more than the chip holds at once."""
     from lmsf_amd.ops.handles import ScaledRows
     g = torch.Generator().manual_seed(M * H + I)
     x = dev(torch.randn(M, H, generator=g).bfloat16())
@@ -696,10 +697,19 @@ def test_gated_product_after_a_norm_in_either_kernel(ops, ref, M, H, I, bias):
     assert isinstance(h, ScaledRows) and h.rows_per_tile == 16
     wg = dev((torch.randn(2 * I, H, generator=g) * H ** -0.5).bfloat16())
     bg = dev(torch.randn(2 * I, generator=g).bfloat16()) if bias else None
-    assert ops.lib.lmsf_gemm_mid_scaled_fits(M, I, H, h.tiles) == 1
+    # the form with 128 outputs a workgroup is chosen beyond 8 rows only; asked for directly it takes any number
+    assert ops.lib.lmsf_gemm_mid_scaled_fits(M, I, H, h.tiles) == (1 if I <= 16384 or M > 8 else 0)
+    assert ops.lib.lmsf_gemm_mid_scaled_fits(16, I, H, h.tiles) == 1
     want_h = ref.add_rms_norm(ops.linear(x, w), res.clone(), nw, 1e-5, torch.bfloat16)
     for kind in ("silu", "gelu"):
-        here = ops.linear_gated(h, wg, bg, kind)
+        if ops.lib.lmsf_gemm_mid_scaled_fits(M, I, H, h.tiles):
+            here = ops.linear_gated(h, wg, bg, kind)
+        else:
+            from lmsf_amd.ops.hip_ops import _ptr
+            here = torch.empty((M, I), dtype=torch.bfloat16, device=h.xw.device)
+            ops._check(ops.lib.lmsf_gemm_mid_scaled(
+                _ptr(h.xw), h.xw.stride(0), _ptr(wg), wg.stride(0), _ptr(bg), _ptr(here), here.stride(0), M, I, H,
+                {"silu": 1, "gelu": 2}[kind], _ptr(h.sumsq), h.tiles, h.eps, ops._stream()))
         before = ops.mid_scaled_rows
         ops.mid_scaled_rows = 0
         try:
@@ -715,7 +725,8 @@ def test_gated_product_after_a_norm_in_either_kernel(ops, ref, M, H, I, bias):
     assert ops.lib.lmsf_gemm_mid_scaled_fits(8, 11008, H, h.tiles) == 0 and ops.lib.lmsf_gemm_mid_scaled_fits(16, 11008, H, h.tiles) == 1
     assert ops.lib.lmsf_gemm_mid_scaled_fits(16, 2048, H, h.tiles) == 0
     assert ops.lib.lmsf_gemm_mid_scaled_fits(M, 64 * 257, H, h.tiles) == 0
-    assert ops.lib.lmsf_gemm_mid_scaled_fits(M, I, 8192, 512) == 0 and ops.lib.lmsf_gemm_mid_scaled_fits(17, I, H, h.tiles) == 0
+    assert ops.lib.lmsf_gemm_mid_scaled_fits(M, 128 * 257, H, h.tiles) == 0
+    assert ops.lib.lmsf_gemm_mid_scaled_fits(M, I, 16384, 1024) == 0 and ops.lib.lmsf_gemm_mid_scaled_fits(17, I, H, h.tiles) == 0
 
 
 @pytest.mark.parametrize("M,stream_rows", [(1, 1), (2, 2), (2, 1), (8, 1), (16, 1)])
