@@ -11,8 +11,8 @@
 // (tops/src/cublas.rs:29-114).
 //
 // Tiles of 64 k travel from global memory straight into LDS (global_load_lds_dwordx4: lane i of a wave
-// writes its 16 bytes at the wave's LDS base + 16 i), four steps ahead of the one being multiplied; each
-// wave moves its own rows of W and a quarter of x. A tile is 16 rows of 128 bytes; the 16-byte piece c of
+// writes its 16 bytes at the wave's LDS base + 16 i), four steps ahead of the one being multiplied (three in the
+// form whose waves own two tiles of each projection); each wave moves its own rows of W and a quarter of x. A tile is 16 rows of 128 bytes; the 16-byte piece c of
 // row r lies in slot (c + r) mod 8 of its row, which keeps the operand reads of a wave on distinct
 // banks without padding (the transfer cannot pad). One barrier per step.
 //
@@ -63,7 +63,8 @@ __device__ __forceinline__ void mid_store4(float* p, const float* o) {
 #define MID_TILE 2048
 
 // MT: tiles of 16 rows of x (2, 4, 6 or 8). ACT: 0 none, 1 silu-gated, 2 gelu-gated (W = [gate rows; up rows], N
-// outputs). PARTIAL: write float32 partial sums of this workgroup's part of K instead of the result.
+// outputs). PARTIAL: write float32 partial sums of this workgroup's part of K instead of the result. TW: tiles of 16
+// outputs a wave owns (of each projection), so 64 TW outputs a workgroup.
 // (A form of the gated product with 32 outputs a workgroup, waves 0 and 1 on the gate rows and 2 and 3 on the up rows
 // of the same outputs, twice as many workgroups, two to a compute unit, was ahead at 17 to 48 rows while the
 // weights' rows lay back to back and were loaded like anything else: 4.7 -> 5.0 TB/s. With the rows apart and the
