@@ -331,6 +331,9 @@ def main():
     ap.add_argument("--tunable", action="append", default=[], metavar="NAME=INT",
                     help="set an attribute of ops.HipOps (a number of rows at which kernels change, a variant) first")
     ap.add_argument("--points", default="1,64,128", help="decode: further batch sizes, comma separated")
+    ap.add_argument("--max-context", type=int, default=None,
+                    help="decode: positions the model allows, for --prompt-len beyond the shape's own "
+                         "(--batch 1 --prompt-len 120000 --max-context 131072 --skip-points)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this engine runs on one GPU; --gpus %d is not supported" % args.gpus)
@@ -356,6 +359,8 @@ def main():
     full_layers = cfg["num_hidden_layers"]
     if args.layers:
         cfg["num_hidden_layers"] = args.layers
+    if args.max_context:
+        cfg["max_position_embeddings"] = args.max_context
     point_batches = [] if args.skip_points else [int(x) for x in args.points.split(",") if x]
     max_seqs = max([64, args.batch] + point_batches)
     engine = make_engine(cfg, args, max_num_seqs=max_seqs, dtype=args.dtype)

@@ -309,9 +309,10 @@ __device__ __forceinline__ unsigned lds_address(const void* p) {
 // through LDS at the end (the longest tile would take half the steps): 66.6 against 63.9 us at 2,048 tokens,
 // 727 against 626 at 8,192; a barrier over 16 waves and one workgroup a compute unit cost more than the balance gives.
 #define PREFILL_LAZY_LOG2 24.0f
-// Entries of a block table that the LDS-staged kernel can keep beside its stages, and how many copies of the
-// last entry follow it there.
+// Entries of a block table that the LDS-staged kernel keeps beside its stages at a time, and how many copies of the
+// table's last entry follow them there. PREFILL_BT_CAP_SMALL: a window for tests, which moves at short contexts.
 #define PREFILL_BT_CAP 2048
+#define PREFILL_BT_CAP_SMALL 64
 #define PREFILL_BT_PAD 8
 template <int DPAD, int NQB, int STAGES, int NW>
 __global__ __launch_bounds__(NW * 64, (NW == 8 ? 4 : 1)) void attn_prefill_dma_kernel(
@@ -351,9 +352,12 @@ __global__ __launch_bounds__(NW * 64, (NW == 8 ? 4 : 1)) void attn_prefill_dma_k
   const int k_begin = window > 0 ? (max(0, p_first - window + 1) / 32) * 32 : 0;
   const int n_steps = (p_last - k_begin) / 32 + 1;
   const int blk0 = k_begin >> ps_log2;                                   // first block of the table that is needed
-  const int n_blk = min(min(btw, (p_last >> ps_log2) + 1) - blk0, bt_cap);   // the host made sure bt_cap suffices
-  // (PREFILL_BT_PAD entries after the last one repeat it: the lookups of the steps ahead need no bound then)
-  for (int i = tid; i < n_blk + PREFILL_BT_PAD; i += NW * 64) lds_bt[i] = bt[blk0 + min(i, n_blk - 1)];
+  const int n_blk = min(btw, (p_last >> ps_log2) + 1) - blk0;             // blocks of the table that are needed
+  // LDS holds bt_cap of them at a time, from block wbase on (counted from blk0), and PREFILL_BT_PAD more: entries
+  // after the table's last one repeat it, so the lookups of the steps ahead need no bound. A tile with more blocks
+  // than that (a prompt's portion after tens of thousands of tokens) moves the window on as it walks the keys.
+  int wbase = 0;
+  for (int i = tid; i < min(n_blk, bt_cap) + PREFILL_BT_PAD; i += NW * 64) lds_bt[i] = bt[blk0 + min(i, n_blk - 1)];
 
   int rpos[NQB], rlo[NQB];
   long qoff[NQB], ooff[NQB];
@@ -476,10 +480,10 @@ __global__ __launch_bounds__(NW * 64, (NW == 8 ? 4 : 1)) void attn_prefill_dma_k
   // wave that runs alone on its SIMD a tenth of the step).
   int page_of[LPW];
   auto lookup = [&](int kb) {
-    const int blk_step = (kb >> ps_log2) - blk0;              // the step's part, the same for the wave
+    const int blk_step = min((kb >> ps_log2) - blk0, n_blk) - wbase;   // the step's part, the same for the wave
 #pragma unroll
     for (int i = 0; i < LPW; ++i)
-      page_of[i] = lds_bt[min(blk_step, n_blk) + t_blk[i]];   // keys beyond the last block are masked: any valid page
+      page_of[i] = lds_bt[blk_step + t_blk[i]];               // keys beyond the last block are masked: any valid page
   };
   // this wave's transfers of the step that starts at key kb, into the stage at byte ``stage_byte``
   auto issue = [&](int kb, int stage_byte) {
@@ -514,6 +518,15 @@ __global__ __launch_bounds__(NW * 64, (NW == 8 ? 4 : 1)) void attn_prefill_dma_k
     __syncthreads();   // everybody's part of step ``it`` is there, and everybody is done with step ``it - 1``
     if (it + STAGES - 1 < n_steps) {
       issue(kbase + (STAGES - 1) * 32, produce);
+      // The window of the table moves on when the next lookup would leave it (the same for the whole workgroup).
+      // Nobody reads the table between this step's barrier and the one below: the lookups of the step before
+      // are done, this step's follow.
+      const int next_blk = min(((kbase + STAGES * 32) >> ps_log2) - blk0, n_blk);
+      if (next_blk - wbase >= bt_cap) {
+        wbase = next_blk;
+        for (int i = tid; i < bt_cap + PREFILL_BT_PAD; i += NW * 64) lds_bt[i] = bt[blk0 + min(wbase + i, n_blk - 1)];
+        __syncthreads();
+      }
       lookup(kbase + STAGES * 32);
     }
     if (kbase <= wmax && kbase + 31 >= wlo) {
@@ -628,7 +641,7 @@ template <int DPAD>
 static int launch_prefill_dma(dim3 grid, hipStream_t stream, const bf16_t* q, long q_stride, bf16_t* out,
                               long out_stride, const bf16_t* k_pages, const bf16_t* v_pages, const int* block_tables,
                               int btw, const int* tiles, const int* seg, const int* pos, int nh, int nkv, int d, int ps,
-                              float scale_log2, int window, int HB, int n_hb) {
+                              float scale_log2, int window, int HB, int n_hb, int bt_cap) {
   int ps_log2 = 0;
   while ((1 << ps_log2) < ps) ++ps_log2;
   // four stages of a head size of 128 and the table are 72 KB: two workgroups share a compute unit's LDS,
@@ -652,7 +665,7 @@ static int launch_prefill_dma(dim3 grid, hipStream_t stream, const bf16_t* q, lo
   }
   hipLaunchKernelGGL(kernel, dim3(grid.x * grid.y), dim3(NW * 64), smem, stream, q, q_stride, out, out_stride, k_pages,
                      v_pages, block_tables, btw, tiles, seg, pos, nh, nkv, d, ps_log2, scale_log2, window, HB, n_hb,
-                     PREFILL_BT_CAP, lmsf_compute_units());
+                     bt_cap, lmsf_compute_units());
   return 0;
 }
 
@@ -990,7 +1003,8 @@ extern "C" int lmsf_attention_tile_tokens(int nh, int nkv) {
 
 // tiles: int32 [n_tiles, 2] = (first flat token, number of tokens <= lmsf_attention_tile_tokens); all tokens
 // of a tile belong to one request and stand at consecutive positions. variant 0: keys and values staged in
-// LDS where the page size and the table's width allow it (the default); 1: every wave fetches them itself.
+// LDS where the page size allows it (the default); 1: every wave fetches them itself; 2: as 0 with a window of 64
+// entries of the block table in LDS instead of 2,048, so that it moves at contexts that a test can afford.
 extern "C" int lmsf_paged_attention_prefill_mfma(const void* q, long q_stride, void* out, long out_stride,
                                                  const void* k_pages, const void* v_pages, long num_pages,
                                                  const int* block_tables, int btw, const int* tiles, int n_tiles,
@@ -1007,13 +1021,14 @@ extern "C" int lmsf_paged_attention_prefill_mfma(const void* q, long q_stride, v
   const float scale_log2 = scale * 1.44269504088896340736f;
   dim3 grid(n_tiles, nkv * n_hb), block(256);
   const int dpad = (d + 31) / 32 * 32;
-  if (variant == 0 && ps >= 8 && (ps & (ps - 1)) == 0 && btw <= PREFILL_BT_CAP) {
+  if ((variant == 0 || variant == 2) && ps >= 8 && (ps & (ps - 1)) == 0) {
     // tiles staged in LDS
+    const int bt_cap = variant == 2 ? PREFILL_BT_CAP_SMALL : PREFILL_BT_CAP;
     int rc = 0;
 #define LAUNCH_LDS(DP)                                                                                           \
   rc = launch_prefill_dma<DP>(grid, stream, (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride,                \
                               (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_tables, btw, tiles, seg, pos, \
-                              nh, nkv, d, ps, scale_log2, window, HB, n_hb)
+                              nh, nkv, d, ps, scale_log2, window, HB, n_hb, bt_cap)
     switch (dpad) {
       case 32: LAUNCH_LDS(32); break;
       case 64: LAUNCH_LDS(64); break;

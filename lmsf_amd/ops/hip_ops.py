@@ -58,7 +58,7 @@ class HipOps:
                 "the kernels are built for gfx950 only; this device reports %r" % self.device_arch)
         self._bad_flag = None
         self.use_library_gemm = True   # bfloat16 matrix products of many rows go to the BLAS library
-        self.prefill_attention_variant = 0   # 0: keys and values staged in LDS; 1: fetched by every wave for itself
+        self.prefill_attention_variant = 0   # 0: keys and values staged in LDS; 1: fetched by every wave for itself; 2: as 0 with a short window of the block table in LDS (for tests)
         self.decode_attention_order = 0      # 0: chosen from the number of workgroups; 1: the tokens of a head start together; 2: the heads of a token
         self.decode_attention_splits = 0     # 0: chosen from the batch and the context; n: at most n splits of the keys
         self.fuse_norm_rows = 16             # with up to this many rows (beyond fuse_stream_rows) the products around a norm do its work (0: never)

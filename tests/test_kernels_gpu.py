@@ -212,8 +212,34 @@ def test_paged_attention_matrix_core_kernels(ops, ref, shape, window):
     assert torch.allclose(c.float(), b.float(), **tol(torch.bfloat16)), (c.float() - b.float()).abs().max()
 
 
+@pytest.mark.parametrize("ps,first,window", [(8, 16400, 0), (16, 16380, 0), (32, 16385, 0), (8, 16400, 5000)])
+def test_prefill_attention_beyond_the_block_tables_window(ops, ref, ps, first, window):
+    """The LDS-staged prefill kernel keeps 2,048 entries of a request's block table in LDS at a time (64 in the form
+    for tests) and moves that window on as it walks the keys: portions of a prompt that stand after so many tokens
+    that the table is longer than the window (more than 2,048 pages of 8 tokens; with 64 entries, pages of 16 and 32
+    too), beside a short request, and with a sliding window that starts deep inside the table. One far key per kv
+    head stands out, so a page looked up in the wrong window would show."""
+    nh, nkv, d = 4, 2, 32
+    scale = 1.0 / math.sqrt(d)
+    seg_lens, ctx_lens = [70, 33, 5], [first + 70, 100, first // 2]
+    q, kp, vp, bt, seg, pos = _paged_case(torch.bfloat16, nh, nkv, d, ps, seg_lens, ctx_lens, seed=ps + first, spike=True)
+    # a key far from the start stands out too: in the third window of 64 entries, and beyond 2,048 pages of 8 tokens
+    far = first - 7
+    kp[int(bt[0, far // ps]), :, far % ps, :] *= 5.0
+    assert ps > 8 or bt.shape[1] > 2048
+    want = ref.paged_attention(q, kp, vp, bt, seg, pos, nh, nkv, d, scale, window)
+    for variant in (0, 2):
+        ops.prefill_attention_variant = variant
+        try:
+            got = ops.paged_attention(q, kp, vp, bt, seg, pos, nh, nkv, d, scale, window, kernel="mfma")
+        finally:
+            ops.prefill_attention_variant = 0
+        assert torch.allclose(got.float(), want.float(), **tol(torch.bfloat16)), \
+            (variant, (got.float() - want.float()).abs().max())
+
+
 @pytest.mark.parametrize("shape", MFMA_SHAPES)
-@pytest.mark.parametrize("variant,splits", [(1, 1), (0, 3), (1, 64)])
+@pytest.mark.parametrize("variant,splits", [(1, 1), (0, 3), (1, 64), (2, 1)])
 def test_matrix_core_attention_other_ways_of_cutting_the_work(ops, ref, shape, variant, splits):
     """The forms that the planner picks only for other workloads: every wave fetching keys and values for itself
     (prefill), the keys of a single token in one part, in three, in as many as there are 128-key chunks."""
