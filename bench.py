@@ -175,8 +175,18 @@ LLAMA31_70B = dict(
     max_position_embeddings=16384, tie_word_embeddings=False, attention_bias=False, hidden_act="silu",
     torch_dtype="bfloat16", bos_token_id=128000, eos_token_id=128001)
 
+# a small model of the same architecture: head size 64, tied embeddings, few and narrow layers (launches count)
+LLAMA32_1B = dict(
+    architectures=["LlamaForCausalLM"], model_type="llama", vocab_size=128256, hidden_size=2048,
+    intermediate_size=8192, num_hidden_layers=16, num_attention_heads=32, num_key_value_heads=8, head_dim=64,
+    rms_norm_eps=1e-5, rope_theta=500000.0,
+    rope_scaling=dict(rope_type="llama3", factor=32.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                      original_max_position_embeddings=8192),
+    max_position_embeddings=16384, tie_word_embeddings=True, attention_bias=False, hidden_act="silu",
+    torch_dtype="bfloat16", bos_token_id=128000, eos_token_id=128001)
+
 SHAPES = {"llama3-8b": ("Llama-3-8B", LLAMA3_8B), "llama2-7b": ("Llama-2-7B", LLAMA2_7B),
-          "llama3.1-70b": ("Llama-3.1-70B", LLAMA31_70B)}
+          "llama3.1-70b": ("Llama-3.1-70B", LLAMA31_70B), "llama3.2-1b": ("Llama-3.2-1B", LLAMA32_1B)}
 
 
 def serve_run(args, emit=True):
