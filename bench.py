@@ -41,7 +41,7 @@ def make_engine(cfg, args, max_num_seqs, dtype, prefill_chunk_size=None):
     folder = tempfile.mkdtemp(prefix="lmsf_bench_")
     with open(os.path.join(folder, "config.json"), "w") as f:
         json.dump(cfg, f)
-    return LLMEngine(EngineArgs(model=folder, dtype=dtype, block_size=16, load_format="random", seed=0,
+    return LLMEngine(EngineArgs(model=folder, dtype=dtype, block_size=getattr(args, "block_size", 16), load_format="random", seed=0,
                                 max_num_seqs=max_num_seqs, max_num_batched_tokens=args.max_num_batched_tokens,
                                 gpu_memory_utilization=args.gpu_memory_utilization,
                                 prefill_chunk_size=prefill_chunk_size))
@@ -341,6 +341,7 @@ def main():
     ap.add_argument("--tunable", action="append", default=[], metavar="NAME=INT",
                     help="set an attribute of ops.HipOps (a number of rows at which kernels change, a variant) first")
     ap.add_argument("--points", default="1,64,128", help="decode: further batch sizes, comma separated")
+    ap.add_argument("--block-size", type=int, default=16, help="tokens a page of the cache")
     ap.add_argument("--max-context", type=int, default=None,
                     help="decode: positions the model allows, for --prompt-len beyond the shape's own "
                          "(--batch 1 --prompt-len 120000 --max-context 131072 --skip-points)")
@@ -445,7 +446,7 @@ def main():
             "hidden_size": cfg["hidden_size"], "heads": cfg["num_attention_heads"],
             "kv_heads": cfg["num_key_value_heads"], "head_dim": cfg["head_dim"],
             "intermediate_size": cfg["intermediate_size"], "vocab_size": cfg["vocab_size"],
-            "max_context": cfg["max_position_embeddings"], "block_size": 16, "prompt_len": args.prompt_len,
+            "max_context": cfg["max_position_embeddings"], "block_size": args.block_size, "prompt_len": args.prompt_len,
             "mean_decode_context": round(mean_ctx, 1), "prefill_tokens": args.prefill_tokens,
             "cache_pages": cache_pages, "gpu_memory_utilization": args.gpu_memory_utilization,
         },

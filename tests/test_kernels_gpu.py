@@ -312,14 +312,14 @@ def test_matrix_core_attention_random_geometries(ops):
 
 
 @pytest.mark.parametrize("order", [1, 2])
-@pytest.mark.parametrize("B", [19, 7])
-def test_decode_attention_in_a_given_order_of_tokens(ops, ref, order, B):
+@pytest.mark.parametrize("B,ps", [(19, 8), (7, 8), (19, 32), (7, 64)])
+def test_decode_attention_in_a_given_order_of_tokens(ops, ref, order, B, ps):
     """A step of single tokens whose contexts differ, with the tokens listed longest context first and either
     arrangement of the workgroups: the same result as in the order they come in. (In such a step the kernel takes
     token i as request i without looking the request up, and below 16 tokens it does not go through the list.)"""
     from types import SimpleNamespace
     g = torch.Generator().manual_seed(21 + B)
-    nh, nkv, d, ps = 6, 3, 48, 8
+    nh, nkv, d = 6, 3, 48
     lens = [int(x) for x in torch.randint(1, 300, (B,), generator=g)]
     per = [-(-n // ps) for n in lens]
     pages = sum(per) + 3
@@ -348,12 +348,14 @@ def test_decode_attention_in_a_given_order_of_tokens(ops, ref, order, B):
     assert torch.equal(got, plain)
 
 
-@pytest.mark.parametrize("nh,nkv,d,ps", [(4, 2, 16, 8), (5, 5, 48, 16), (6, 3, 80, 4), (8, 2, 128, 16), (2, 1, 256, 32), (3, 1, 112, 16)])
+@pytest.mark.parametrize("nh,nkv,d,ps", [(4, 2, 16, 8), (5, 5, 48, 16), (6, 3, 80, 4), (8, 2, 128, 16), (2, 1, 256, 32), (3, 1, 112, 16),
+                                         (8, 2, 128, 32), (5, 5, 48, 64), (6, 3, 80, 128), (4, 2, 64, 24)])
 @pytest.mark.parametrize("window", [0, 700])
 def test_decode_attention_reduction_over_many_splits(ops, ref, nh, nkv, d, ps, window):
     """More than 16 splits of a long context are added up by groups of lanes that take every G-th split (up to
     16: one loop per output element); requests of other lengths in the same call use fewer of the splits, and a
-    window leaves the first ones without keys."""
+    window leaves the first ones without keys. Pages of 32 tokens and more run in the form of the kernel that deals
+    a step's keys so that a lane's eight are eight in a row."""
     ctx_lens = [2500, 1, 2300, 130]
     q, kp, vp, bt, seg, pos = _paged_case(torch.bfloat16, nh, nkv, d, ps, [1, 1, 1, 1], ctx_lens, seed=nh + d, spike=True)
     scale = 1.0 / math.sqrt(d)
