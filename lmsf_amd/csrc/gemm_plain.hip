@@ -68,6 +68,81 @@ __global__ __launch_bounds__(256) void gemm_plain_kernel(const TA* __restrict__ 
   }
 }
 
+// The same product for up to 16 rows of bfloat16 operands that the weight-streaming kernels refuse (a K that is no
+// multiple of 8, rows that do not start on 16-byte boundaries): with so few rows the tiles above leave most of the
+// chip idle (N / 64 workgroups, each walking all of K: 4,160 x 11,100 at 8 rows 1,290 us). Here a wave owns one output
+// column; lane l takes k = l, l + 64, ... with 2-byte loads, which need no alignment, and the lanes' sums are added
+// up in a fixed order. float32 products and sums.
+#define GP_FEW_ROWS 16
+// MT: rows the kernel walks (M rounded up to 1, 2, 4, 8 or 16; the rows beyond M repeat row M - 1 and are not written),
+// so that the loop has no tests and the loads of several steps are in flight together. VEC: elements a load (2 where K
+// and the row strides are even and the operands start on 4-byte boundaries, else 1).
+template <typename TO, int MT, int VEC>
+__global__ __launch_bounds__(256) void gemm_plain_few_kernel(const bf16_t* __restrict__ A, long lda,
+                                                             const bf16_t* __restrict__ W, long ldw,
+                                                             const bf16_t* __restrict__ bias, TO* __restrict__ C,
+                                                             long ldc, int M, int N, int K) {
+  const int lane = threadIdx.x & 63;
+  const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (n >= N) return;
+  float acc[MT];
+  const bf16_t* a[MT];
+#pragma unroll
+  for (int m = 0; m < MT; ++m) {
+    acc[m] = 0.f;
+    a[m] = A + (long)min(m, M - 1) * lda;
+  }
+  const bf16_t* w = W + (long)n * ldw;
+  if (VEC == 2) {
+#pragma unroll 4
+    for (int k = 2 * lane; k < K; k += 128) {   // K is even: a pair never straddles the end
+      const unsigned wp = *reinterpret_cast<const unsigned*>(w + k);
+      const float w0 = __uint_as_float(wp << 16), w1 = __uint_as_float(wp & 0xffff0000u);
+#pragma unroll
+      for (int m = 0; m < MT; ++m) {
+        const unsigned xp = *reinterpret_cast<const unsigned*>(a[m] + k);
+        acc[m] = fmaf(__uint_as_float(xp << 16), w0, acc[m]);
+        acc[m] = fmaf(__uint_as_float(xp & 0xffff0000u), w1, acc[m]);
+      }
+    }
+  } else {
+#pragma unroll 4
+    for (int k = lane; k < K; k += 64) {
+      const float wv = bf16_to_f32(w[k]);
+#pragma unroll
+      for (int m = 0; m < MT; ++m) acc[m] = fmaf(bf16_to_f32(a[m][k]), wv, acc[m]);
+    }
+  }
+#pragma unroll
+  for (int m = 0; m < MT; ++m) {
+    float r = acc[m];
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) r += __shfl_xor(r, off, 64);
+    if (lane == 0 && m < M) {
+      if (bias) r += bf16_to_f32(bias[n]);
+      C[(long)m * ldc + n] = from_f32<TO>(r);
+    }
+  }
+}
+
+template <typename TO>
+static void launch_gemm_plain_few(const void* A, long lda, const void* W, long ldw, const void* bias, void* C, long ldc,
+                                  int M, int N, int K, hipStream_t stream) {
+  const dim3 grid((N + 3) / 4), block(256);
+  const bool pairs = K % 2 == 0 && lda % 2 == 0 && ldw % 2 == 0 && (size_t)A % 4 == 0 && (size_t)W % 4 == 0;
+#define FEW(MT_)                                                                                                       \
+  do {                                                                                                                 \
+    if (pairs)                                                                                                         \
+      hipLaunchKernelGGL((gemm_plain_few_kernel<TO, MT_, 2>), grid, block, 0, stream, (const bf16_t*)A, lda,           \
+                         (const bf16_t*)W, ldw, (const bf16_t*)bias, (TO*)C, ldc, M, N, K);                            \
+    else                                                                                                               \
+      hipLaunchKernelGGL((gemm_plain_few_kernel<TO, MT_, 1>), grid, block, 0, stream, (const bf16_t*)A, lda,           \
+                         (const bf16_t*)W, ldw, (const bf16_t*)bias, (TO*)C, ldc, M, N, K);                            \
+  } while (0)
+  if (M <= 1) FEW(1); else if (M <= 2) FEW(2); else if (M <= 4) FEW(4); else if (M <= 8) FEW(8); else FEW(16);
+#undef FEW
+}
+
 template <typename TA, typename TW, typename TO>
 static void launch_gemm_plain(const void* A, long lda, const void* W, long ldw, const void* bias, void* C, long ldc,
                               int M, int N, int K, hipStream_t stream) {
@@ -86,6 +161,14 @@ extern "C" int lmsf_gemm_plain(const void* A, int a_dtype, long lda, const void*
   LMSF_CHECK(lda >= K && ldw >= K && ldc >= N, "gemm_plain: leading dimensions too small");
   LMSF_CHECK((M + GP_TILE - 1) / GP_TILE <= 65535, "gemm_plain: M=%d too large", M);
   if (M == 0) return 0;
+  if (M <= GP_FEW_ROWS && a_dtype == LMSF_BF16 && w_dtype == LMSF_BF16) {
+    if (c_dtype == LMSF_BF16)
+      launch_gemm_plain_few<bf16_t>(A, lda, W, ldw, bias, C, ldc, M, N, K, stream);
+    else
+      launch_gemm_plain_few<float>(A, lda, W, ldw, bias, C, ldc, M, N, K, stream);
+    LMSF_LAUNCH_CHECK("gemm_plain");
+    return 0;
+  }
   const int key = a_dtype * 100 + w_dtype * 10 + c_dtype;
   switch (key) {
     case 0: launch_gemm_plain<float, float, float>(A, lda, W, ldw, bias, C, ldc, M, N, K, stream); break;

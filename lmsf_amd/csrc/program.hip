@@ -331,7 +331,7 @@ int op_linear(Run& r, const Value& x, const void* W, int wdtype, long ldw, int N
       return 0;
     }
   }
-  if (t.use_library_gemm && both_bf16 && M > t.skinny_max_rows) {
+  if (t.use_library_gemm && both_bf16 && M > t.skinny_max_rows && out_dtype == LMSF_BF16) {
     lmsf_set_error("program: a bfloat16 product of %d rows, %d columns over %d goes to the BLAS library", M, N, K);
     return LMSF_PROGRAM_NOT_NATIVE;
   }
@@ -509,8 +509,8 @@ int op_linear_gated(Run& r, const Value& x_in, const void* W, int wdtype, long l
   }
   if (both_bf16 && t.skinny_max_rows < M && M <= 64 && mid_ok(x.p, x.ld, K, W, ldw, w_rows))
     return linear_mid(r, x, W, ldw, w_rows, bias, kind, LMSF_BF16, false, nullptr, res);
-  if (both_bf16 && 64 < M && M <= t.large_max_rows && mid_ok(x.p, x.ld, K, W, ldw, w_rows))
-    return linear_large(r, x, W, ldw, w_rows, bias, kind, false, nullptr, res);
+  if (both_bf16 && 64 < M && M <= t.large_max_rows && mid_ok(x.p, x.ld, K, W, ldw, w_rows) && I % 8 == 0)
+    return linear_large(r, x, W, ldw, w_rows, bias, kind, false, nullptr, res);   // (it writes eight outputs at a time)
   Value gu;
   RC(op_linear(r, x, W, wdtype, ldw, w_rows, bias, x.dtype, false, nullptr, &gu));
   TAKE(y, void*, (size_t)M * I * esize(gu.dtype));

@@ -654,11 +654,13 @@ class HipOps:
                         _ptr(xs), xs.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(ys),
                         _code(out_dtype), ys.stride(0), rows, N, K, self.skinny_variant, 0, self._stream()))
                 return y
-        if self.use_library_gemm and both_bf16 and M > self.skinny_max_rows:
+        if self.use_library_gemm and both_bf16 and M > self.skinny_max_rows and out_dtype == torch.bfloat16:
+            # (float32 output that no kernel above takes, a K that is no multiple of 8, goes to the plain kernel below:
+            # the library would round it to bfloat16 first)
             y = torch.nn.functional.linear(x, weight, bias)
             if out is not None:
                 return out.copy_(y)
-            return y if out_dtype == torch.bfloat16 else y.to(out_dtype)
+            return y
         y = new()
         self._check(self.lib.lmsf_gemm_plain(_ptr(x), _code(x.dtype), x.stride(0), _ptr(weight), _code(weight.dtype),
                                              weight.stride(0), _ptr(bias), _ptr(y), _code(out_dtype), y.stride(0),
@@ -722,7 +724,8 @@ class HipOps:
                 and self.skinny_max_rows < M <= 64 and x.shape[1] == weight.shape[1] and self._mid_ok(x, weight)):
             return self._linear_mid(x, weight, bias, kinds[kind])
         if (x.dim() == 2 and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
-                and 64 < M <= self.large_max_rows and x.shape[1] == weight.shape[1] and self._mid_ok(x, weight)):
+                and 64 < M <= self.large_max_rows and x.shape[1] == weight.shape[1] and self._mid_ok(x, weight)
+                and I % 8 == 0):    # (that kernel writes its outputs eight at a time)
             return self._linear_large(x, weight, bias, kinds[kind])
         return self.gated_act(self.linear(x, weight, bias), kind)
 

@@ -483,7 +483,10 @@ def test_linear_float32_is_exact_float32(ops, M, N, K, bias):
                                    (17, 328, 128), (33, 4096, 4096), (64, 6144, 4096), (48, 1000, 14336), (64, 4096, 1024),
                                    (65, 4096, 4096), (96, 1000, 14336), (97, 328, 128), (128, 6144, 4096), (127, 4096, 1024),
                                    (200, 1000, 1024), (129, 4096, 4096), (130, 328, 192), (192, 6144, 4096),
-                                   (256, 4096, 14336), (255, 1000, 128), (300, 6144, 4096), (2048, 1000, 1024)])
+                                   (256, 4096, 14336), (255, 1000, 128), (300, 6144, 4096), (2048, 1000, 1024),
+                                   # a K that is no multiple of 8 (even and odd): no streaming kernel takes it
+                                   (1, 333, 11100), (3, 130, 331), (8, 4160, 1004), (13, 77, 2001), (16, 520, 250),
+                                   (17, 130, 331), (100, 77, 1004)])
 @pytest.mark.parametrize("bias", [False, True])
 @pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
 def test_linear_bfloat16(ops, ref, M, N, K, bias, out_dtype):
@@ -527,7 +530,10 @@ def test_products_over_a_weight_whose_rows_lie_apart(ops, M):
 
 @pytest.mark.parametrize("M,I,K", [(1, 176, 64), (8, 14336, 4096), (16, 208, 80), (13, 1000, 328), (40, 352, 128),
                                    (64, 14336, 4096), (20, 1000, 1024), (65, 14336, 4096), (100, 1000, 1024),
-                                   (129, 352, 128), (200, 14336, 4096), (256, 1000, 192), (300, 1000, 1024)])
+                                   (129, 352, 128), (200, 14336, 4096), (256, 1000, 192), (300, 1000, 1024),
+                                   # outputs that are 4 modulo 8, 2 modulo 4 and odd, at every kernel's numbers of rows
+                                   (8, 1004, 192), (40, 1004, 192), (100, 1004, 192), (200, 11100, 4160), (100, 250, 64),
+                                   (40, 331, 128), (130, 331, 128)])
 @pytest.mark.parametrize("kind", ["silu", "gelu"])
 @pytest.mark.parametrize("bias", [False, True])
 def test_linear_gated(ops, ref, M, I, K, kind, bias):

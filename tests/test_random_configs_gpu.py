@@ -40,10 +40,28 @@ def draw_config(seed):
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("seed", [3, 15, 35, 65, 72, 74, 127, 157])
 def test_a_configuration_drawn_at_random(tmp_path, seed, dtype):
+    cfg_dict, page, lens = draw_config(seed)
+    replay_every_way(tmp_path, cfg_dict, page, lens, seed, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("H,I,V", [(72, 172, 331), (64, 250, 1000), (136, 331, 97), (192, 1004, 2050)])
+def test_widths_that_no_kernel_tiles_evenly(tmp_path, H, I, V, dtype):
+    """Feed-forward widths that are 4 modulo 8, 2 modulo 4 and odd, with prompts of 17 to 64, 65 to 256 and more rows in
+    a step: each number of rows has matrix kernels of its own that ask for multiples of 4 or 8 outputs, and a product
+    that none of them takes goes to the library."""
+    cfg_dict = dict(architectures=["LlamaForCausalLM"], model_type="llama", vocab_size=V, hidden_size=H,
+                    intermediate_size=I, num_hidden_layers=2, num_attention_heads=4, num_key_value_heads=2, head_dim=16,
+                    rms_norm_eps=1e-5, rope_theta=10000.0, rope_scaling=None, max_position_embeddings=512,
+                    tie_word_embeddings=False, attention_bias=False, mlp_bias=I % 2 == 0, hidden_act="silu",
+                    bos_token_id=1, eos_token_id=2)
+    replay_every_way(tmp_path, cfg_dict, 16, [40, 100, 3, 300, 180], H + I, dtype)
+
+
+def replay_every_way(tmp_path, cfg_dict, page, lens, seed, dtype):
     from lmsf_amd.config import LlamaConfig
     from lmsf_amd.engine import load_engine_core
     from lmsf_amd.weights import write_random_model
-    cfg_dict, page, lens = draw_config(seed)
     folder = os.path.join(str(tmp_path), "m")
     write_random_model(folder, LlamaConfig.from_dict(dict(cfg_dict, torch_dtype=dtype)), seed=seed, dtype=dtype)
     cfg, w = read_model_folder(folder)
