@@ -76,70 +76,90 @@ __global__ __launch_bounds__(256) void gemm_plain_kernel(const TA* __restrict__ 
 #define GP_FEW_ROWS 16
 // MT: rows the kernel walks (M rounded up to 1, 2, 4, 8 or 16; the rows beyond M repeat row M - 1 and are not written),
 // so that the loop has no tests and the loads of several steps are in flight together. VEC: elements a load (2 where K
-// and the row strides are even and the operands start on 4-byte boundaries, else 1).
-template <typename TO, int MT, int VEC>
+// and the row strides are even and the operands start on 4-byte boundaries, else 1). COLS: output columns a wave owns,
+// more with more rows: every column's wave reads all of x from the caches, and with 16 rows and one column a wave that
+// is 16 loads of x for each of W (4,160 x 11,100 at 16 rows: 1.5 GB through the caches).
+template <typename TO, int MT, int VEC, int COLS>
 __global__ __launch_bounds__(256) void gemm_plain_few_kernel(const bf16_t* __restrict__ A, long lda,
                                                              const bf16_t* __restrict__ W, long ldw,
                                                              const bf16_t* __restrict__ bias, TO* __restrict__ C,
                                                              long ldc, int M, int N, int K) {
   const int lane = threadIdx.x & 63;
-  const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (n >= N) return;
-  float acc[MT];
+  const int n0 = (blockIdx.x * 4 + (threadIdx.x >> 6)) * COLS;
+  if (n0 >= N) return;
+  float acc[MT][COLS];
   const bf16_t* a[MT];
+  const bf16_t* w[COLS];
 #pragma unroll
   for (int m = 0; m < MT; ++m) {
-    acc[m] = 0.f;
     a[m] = A + (long)min(m, M - 1) * lda;
+#pragma unroll
+    for (int c = 0; c < COLS; ++c) acc[m][c] = 0.f;
   }
-  const bf16_t* w = W + (long)n * ldw;
+#pragma unroll
+  for (int c = 0; c < COLS; ++c) w[c] = W + (long)min(n0 + c, N - 1) * ldw;   // columns beyond N repeat the last one
   if (VEC == 2) {
-#pragma unroll 4
+#pragma unroll 2
     for (int k = 2 * lane; k < K; k += 128) {   // K is even: a pair never straddles the end
-      const unsigned wp = *reinterpret_cast<const unsigned*>(w + k);
-      const float w0 = __uint_as_float(wp << 16), w1 = __uint_as_float(wp & 0xffff0000u);
+      float w0[COLS], w1[COLS];
+#pragma unroll
+      for (int c = 0; c < COLS; ++c) {
+        const unsigned wp = *reinterpret_cast<const unsigned*>(w[c] + k);
+        w0[c] = __uint_as_float(wp << 16);
+        w1[c] = __uint_as_float(wp & 0xffff0000u);
+      }
 #pragma unroll
       for (int m = 0; m < MT; ++m) {
         const unsigned xp = *reinterpret_cast<const unsigned*>(a[m] + k);
-        acc[m] = fmaf(__uint_as_float(xp << 16), w0, acc[m]);
-        acc[m] = fmaf(__uint_as_float(xp & 0xffff0000u), w1, acc[m]);
+        const float x0 = __uint_as_float(xp << 16), x1 = __uint_as_float(xp & 0xffff0000u);
+#pragma unroll
+        for (int c = 0; c < COLS; ++c) acc[m][c] = fmaf(x1, w1[c], fmaf(x0, w0[c], acc[m][c]));
       }
     }
   } else {
-#pragma unroll 4
+#pragma unroll 2
     for (int k = lane; k < K; k += 64) {
-      const float wv = bf16_to_f32(w[k]);
+      float wv[COLS];
 #pragma unroll
-      for (int m = 0; m < MT; ++m) acc[m] = fmaf(bf16_to_f32(a[m][k]), wv, acc[m]);
+      for (int c = 0; c < COLS; ++c) wv[c] = bf16_to_f32(w[c][k]);
+#pragma unroll
+      for (int m = 0; m < MT; ++m) {
+        const float xv = bf16_to_f32(a[m][k]);
+#pragma unroll
+        for (int c = 0; c < COLS; ++c) acc[m][c] = fmaf(xv, wv[c], acc[m][c]);
+      }
     }
   }
 #pragma unroll
-  for (int m = 0; m < MT; ++m) {
-    float r = acc[m];
+  for (int m = 0; m < MT; ++m)
 #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) r += __shfl_xor(r, off, 64);
-    if (lane == 0 && m < M) {
-      if (bias) r += bf16_to_f32(bias[n]);
-      C[(long)m * ldc + n] = from_f32<TO>(r);
+    for (int c = 0; c < COLS; ++c) {
+      float r = acc[m][c];
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) r += __shfl_xor(r, off, 64);
+      if (lane == 0 && m < M && n0 + c < N) {
+        if (bias) r += bf16_to_f32(bias[n0 + c]);
+        C[(long)m * ldc + n0 + c] = from_f32<TO>(r);
+      }
     }
-  }
 }
 
 template <typename TO>
 static void launch_gemm_plain_few(const void* A, long lda, const void* W, long ldw, const void* bias, void* C, long ldc,
                                   int M, int N, int K, hipStream_t stream) {
-  const dim3 grid((N + 3) / 4), block(256);
+  const dim3 block(256);
   const bool pairs = K % 2 == 0 && lda % 2 == 0 && ldw % 2 == 0 && (size_t)A % 4 == 0 && (size_t)W % 4 == 0;
-#define FEW(MT_)                                                                                                       \
+#define FEW(MT_, COLS_)                                                                                                \
   do {                                                                                                                 \
+    const dim3 grid((N + 4 * COLS_ - 1) / (4 * COLS_));                                                                \
     if (pairs)                                                                                                         \
-      hipLaunchKernelGGL((gemm_plain_few_kernel<TO, MT_, 2>), grid, block, 0, stream, (const bf16_t*)A, lda,           \
+      hipLaunchKernelGGL((gemm_plain_few_kernel<TO, MT_, 2, COLS_>), grid, block, 0, stream, (const bf16_t*)A, lda,    \
                          (const bf16_t*)W, ldw, (const bf16_t*)bias, (TO*)C, ldc, M, N, K);                            \
     else                                                                                                               \
-      hipLaunchKernelGGL((gemm_plain_few_kernel<TO, MT_, 1>), grid, block, 0, stream, (const bf16_t*)A, lda,           \
+      hipLaunchKernelGGL((gemm_plain_few_kernel<TO, MT_, 1, COLS_>), grid, block, 0, stream, (const bf16_t*)A, lda,    \
                          (const bf16_t*)W, ldw, (const bf16_t*)bias, (TO*)C, ldc, M, N, K);                            \
   } while (0)
-  if (M <= 1) FEW(1); else if (M <= 2) FEW(2); else if (M <= 4) FEW(4); else if (M <= 8) FEW(8); else FEW(16);
+  if (M <= 1) FEW(1, 1); else if (M <= 2) FEW(2, 1); else if (M <= 4) FEW(4, 2); else if (M <= 8) FEW(8, 4); else FEW(16, 4);
 #undef FEW
 }
 
