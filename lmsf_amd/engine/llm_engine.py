@@ -5,6 +5,7 @@ LLMEngine mirrors the reference's (core/src/engine/llm_engine.rs:74-582): ``add_
 samples and applies the stop rules. ``LLM.generate`` is the convenience loop around it.
 """
 import hashlib
+import sys
 import time
 from typing import Any, Dict, Hashable, List, Optional, Sequence as Seq, Set, Union
 
@@ -189,6 +190,14 @@ class LLMEngine:
         t_start = time.monotonic()
         plan: StepPlan = self.scheduler.schedule()
         now = time.monotonic()
+        for seq in plan.ignored:
+            # as the reference's scheduler warns (core/src/sched/scheduler.rs:368-388)
+            msg = ("Input prompt of request %r (%d tokens) is too long: it exceeds the limit of the engine or the capacity "
+                   "of the cache; ignored" % (seq.request_id, len(seq.prompt_token_ids)))
+            if self.logger is not None:
+                self.logger.warning(msg)
+            else:
+                print("warning: " + msg, file=sys.stderr)
         for seq in plan.ignored + plan.capped:
             seq.metrics.finished_time = now
             self._requests.pop(seq.request_id, None)

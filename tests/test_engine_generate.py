@@ -164,3 +164,16 @@ def test_running_a_step_ahead_changes_no_token(tmp_path, pages):
         assert engine.core.storage.manager.num_free_pages(0) == pages
     assert results[0] == results[1]
     assert results[0][1][1] == "length" and "stop" in {r[1] for r in results[0].values()}
+
+
+def test_a_prompt_that_is_too_long_is_ignored_with_a_warning(tmp_path, capsys):
+    """A prompt beyond the engine's length limit finishes at once without a token, as in the reference's scheduler
+    (core/src/sched/scheduler.rs:368-381), and the engine says so; the request beside it runs as usual."""
+    engine, folder, cfg = make_engine(tmp_path, "A", max_model_len=16)
+    engine.add_request("long", random_tokens(40, cfg.vocab_size, 1), SamplingParams(temperature=0.0, max_tokens=4))
+    engine.add_request("fits", random_tokens(5, cfg.vocab_size, 2), SamplingParams(temperature=0.0, max_tokens=4, ignore_eos=True))
+    done = run(engine)
+    assert done["long"].outputs[0].token_ids == [] and done["long"].outputs[0].finish_reason == "length"
+    assert len(done["fits"].outputs[0].token_ids) == 4
+    err = capsys.readouterr().err
+    assert "'long'" in err and "40 tokens" in err and "too long" in err and "'fits'" not in err
