@@ -672,8 +672,9 @@ int op_attention(Run& r, const Value& q, const LmsfOpDesc& op, const int* tables
   if (n_single) {
     const int n_hb = ((nh / nkv) + 15) / 16;
     const int most = (max_context + 127) / 128;
-    const int fill = max_context >= 32768 && n_single * nkv * n_hb >= 32 ? 1024 : 512;   // (as HipOps.paged_attention chooses)
-    int want = std::max(1, std::min(most, fill / (n_single * nkv * n_hb)));
+    const int pairs = n_single * nkv * n_hb;   // (as HipOps.paged_attention chooses)
+    const int fill = max_context >= 49152 && pairs >= 16 ? 2048 : max_context >= 32768 && pairs >= 32 ? 1024 : 512;
+    int want = std::max(1, std::min(most, fill / pairs));
     if (want == 2 && max_context <= 512) want = 1;
     if (t.decode_attention_splits) want = std::min(most, t.decode_attention_splits);
     const int chunk = (((max_context + want - 1) / want) + 127) / 128 * 128;

@@ -465,7 +465,11 @@ class HipOps:
             # With contexts of tens of thousands of keys twice as many do better (8 tokens of 100,000 keys: a step of
             # 21.2 -> 19.2 ms, 16 of 50,000: 21.6 -> 18.9, 4 of 100,000: 12.3 -> 11.8; 8 and 32 of 32,000: the same),
             # unless a single token's heads would be cut into more than 64 parts (one token of 120,000: 5.54 -> 5.64).
-            fill = 1024 if plan.max_context >= 32768 and plan.n_single * nkv * n_hb >= 32 else 512
+            # From 49,152 keys on, four times as many, from 16 pairs of token and kv head on (2 tokens of 100,000 keys:
+            # 8.28 -> 7.33 ms; 4: 12.3 -> 11.9; 16 of 50,000: 18.9 either way).
+            pairs = plan.n_single * nkv * n_hb
+            fill = 2048 if plan.max_context >= 49152 and pairs >= 16 else \
+                1024 if plan.max_context >= 32768 and pairs >= 32 else 512
             want = max(1, min(most, fill // (plan.n_single * nkv * n_hb)))
             if want == 2 and plan.max_context <= 512:
                 want = 1
