@@ -25,6 +25,15 @@ int lmsf_paged_attention_decode_mfma(const void* q, long q_stride, void* out, lo
     const int* pos, int nh, int nkv, int d, int ps, float scale, int window, int chunk, int n_splits, float* scratch,
     int order, hipStream_t stream);
 
+// blas.hip
+int lmsf_blas_init(long workspace_bytes);
+int lmsf_blas_ready();
+int lmsf_blas_linear(const void* x, long ldx, const void* W, long ldw, const void* bias, void* y, long ldy, int M, int
+    N, int K, hipStream_t stream);
+int lmsf_blas_tune(const void* x, long ldx, const void* const* Ws, int n_weights, long ldw, const void* bias, void* y,
+    long ldy, int M, int N, int K, int n_candidates, int reps, float* times_us, hipStream_t stream);
+long lmsf_blas_plans();
+
 // elementwise.hip
 int lmsf_embedding(const int* ids, const void* table, int table_dtype, float* out, int n_tokens, int H, int V, float
     scale, int* bad_flag, hipStream_t stream);

@@ -4,14 +4,16 @@
 
 #include <hip/hip_runtime.h>
 
+#include "dispatch.h"
+
 #ifdef __cplusplus
 extern "C" {
 #endif
 
 #define LMSF_MAX_GROUPS 8
+#define LMSF_MAX_PLANS 4
 
-// return values of lmsf_program_run beside 0 and errors
-#define LMSF_PROGRAM_NOT_NATIVE 3   // the step needs a product that only the BLAS library has; nothing was launched
+// return value of lmsf_program_run beside 0 and errors
 #define LMSF_PROGRAM_NO_ROOM 4      // the workspace is too small for the step; nothing was launched
 
 enum {
@@ -22,6 +24,9 @@ enum {
   LMSF_OP_LINEAR,
   LMSF_OP_LINEAR_GATED,
   LMSF_OP_MATERIALIZE,
+  LMSF_OP_ROPE_CACHE_WRITE,
+  LMSF_OP_GATED_ACT,
+  LMSF_OP_CALLBACK,
   LMSF_OP_COUNT
 };
 
@@ -36,24 +41,23 @@ enum {
   LMSF_CTX_TABLES = 32    // + cache group
 };
 
-// The numbers of rows at which the products change kernels (the attributes of the same names of ops.HipOps).
-typedef struct {
-  int fuse_norm_rows, fuse_stream_rows, gemv_max_rows, skinny_variant, mid_wide_max_cols, mid_max_rows,
-      skinny_max_rows, prefill_attention_variant, decode_attention_order, decode_attention_splits, use_library_gemm,
-      large_max_rows, large_deep_min_rows, mid_scaled_rows;
-} LmsfTunables;
-
 // One operation. Registers (in0, in1, out) are numbered in the order they are first written; -1: none.
-//   embedding:       out = rows of w [vocab, N] (wdtype) at the ids ctx0, times scale, float32
-//   add_rms_norm:    out = norm(in0 + in1) * (w + weight_offset); in1 is the float32 stream [*, N], updated in
-//                    place; rows_ctx: only these rows; defer_ok: the reader of out takes rows whose factor is missing
-//   qkv_rope_cache:  out = in0 w^T + bias, w [N, K]; q and k heads rotated by table [max_pos, rot] at the positions
-//                    ctx0; k and v stored in the pages at the slots ctx1 (none: not stored)
-//   attention:       out = attention of the first nh * d columns of in0 over the pages, block tables ctx0
-//   linear:          out = in0 w^T + bias in out_dtype; pending_ok: the reader of out takes an unfinished product;
-//                    is_head: the result goes to the step's logits buffer
-//   linear_gated:    out = act(in0 wg^T) * (in0 wu^T), w = [wg; wu] of N = 2 I rows; act 1: SiLU, 2: GELU
-//   materialize:     out = in0 as a finished tensor
+//   embedding:        out = rows of w [vocab, N] (wdtype) at the ids ctx0, times scale, float32
+//   add_rms_norm:     out = norm(in0 + in1) * (w + weight_offset); in1 is the float32 stream [*, N], updated in
+//                     place; rows_ctx: only these rows; defer_ok: the reader of out takes rows whose factor is missing
+//   qkv_rope_cache:   out = in0 w^T + bias, w [N, K]; q and k heads rotated by table [max_pos, rot] at the positions
+//                     ctx0; k and v stored in the pages at the slots ctx1 (none: not stored)
+//   attention:        out = attention of the first nh * d columns of in0 over the pages, block tables ctx0
+//   linear:           out = in0 w^T + bias in out_dtype; pending_ok: the reader of out takes an unfinished product;
+//                     is_head: the result goes to the step's logits buffer
+//   linear_gated:     out = act(in0 wg^T) * (in0 wu^T), w = [wg; wu] of N = 2 I rows; act 1: SiLU, 2: GELU
+//   materialize:      out = in0 as a finished tensor
+//   rope_cache_write: in0 [*, (nh + 2 nkv) d] rotated in place and stored, as the second half of qkv_rope_cache
+//   gated_act:        out = act(in0[:, :I]) * in0[:, I:], N = 2 I; act as above
+//   callback:         the caller's function (lmsf_program_set_callback) is called with ``callback_id`` and where
+//                     in0, in1 and out lie; out has N columns of out_dtype and as many rows as in0 (as the step has
+//                     wanted rows with rows_ctx, as the step has tokens without in0); out -1: the callback works on
+//                     in0 in place; is_head: out is the step's logits buffer
 typedef struct {
   int kind, in0, in1, out;
   int ctx0, ctx1, rows_ctx;
@@ -68,7 +72,17 @@ typedef struct {
   int nh, nkv, d, rot, neox, ps, window, max_pos, act, defer_ok, pending_ok, is_head, vocab;
   long num_pages;
   float eps, weight_offset, scale;
+  int callback_id;
 } LmsfOpDesc;
+
+// Where the attention plan of a step that is not all single tokens lies (lmsf_program_plan fills it): per tile
+// size of the program's attention operations, the pairs (first flat index, tokens) of the tiles and the flat
+// indices of the single tokens, as offsets in ints into the plan's array.
+typedef struct {
+  int n_plans;
+  int tq[LMSF_MAX_PLANS], n_tiles[LMSF_MAX_PLANS], n_single[LMSF_MAX_PLANS];
+  long tiles_at[LMSF_MAX_PLANS], single_at[LMSF_MAX_PLANS];
+} LmsfPlanInfo;
 
 // One step: its sizes, its device arrays (engine.batch.StepContext), the workspace and where the logits go.
 typedef struct {
@@ -82,17 +96,33 @@ typedef struct {
   const int* tables[LMSF_MAX_GROUPS];
   int widths[LMSF_MAX_GROUPS];
   const int* plan;                    // device copy of what lmsf_program_plan wrote (null for single tokens)
+  LmsfPlanInfo plan_info;             // and where its parts lie
   void* workspace;
   long workspace_bytes;
   float* logits;                      // [n_logit_rows, vocabulary]
   int* bad_flag;                      // set by the embedding when an id lies outside the vocabulary
 } LmsfStepDesc;
 
+// A tensor handed to a callback: bytes from the workspace's start (-1: none, -2: the logits buffer).
+typedef struct {
+  long offset;
+  int rows, cols, dtype;
+} LmsfTensorRef;
+typedef struct {
+  int callback_id;
+  LmsfTensorRef in0, in1, out;
+} LmsfCallbackArgs;
+// Returns 0, or non-zero to stop the step with an error. Called on the thread that runs the step, between the
+// launches before it and after it; whatever it launches belongs on the step's stream.
+typedef int (*LmsfCallbackFn)(const LmsfCallbackArgs* args);
+
 void* lmsf_program_create(const LmsfTunables* tunables);
 void lmsf_program_destroy(void* program);
 int lmsf_program_add(void* program, const LmsfOpDesc* op);
 int lmsf_program_seal(void* program);
-long lmsf_program_plan(void* program, int S, const int* seg_lens, const int* seg_first_pos, int* out, long capacity);
+void lmsf_program_set_callback(void* program, LmsfCallbackFn fn);
+long lmsf_program_plan(void* program, int S, const int* seg_lens, const int* seg_first_pos, int* out, long capacity,
+                       LmsfPlanInfo* info);
 long lmsf_program_plan_capacity(void* program, int N);
 int lmsf_program_run(void* program, const LmsfStepDesc* step, int check_only, hipStream_t stream);
 

@@ -13,7 +13,11 @@
 // to come. Temporaries live in a ring: a register's memory is free again after the last operation that reads
 // it; the few registers that live long (the residual stream) are taken from the other end of the workspace.
 // Before anything is launched the whole step is walked once without launching, so a step that does not fit
-// the workspace, or needs a product this library does not have, is refused with nothing done.
+// the workspace is refused with nothing done. Which kernel an operation runs in is not decided here: the
+// functions of dispatch.h say, as they do for the Python face of the kernels. Products that go to the BLAS
+// library are called through blas.hip, so a step of any number of tokens is one call. A part that the
+// recorder could not follow (it computes on its activations itself) is a callback operation: the program
+// hands the caller's function the places of its operands in the workspace and goes on after it returns.
 #include "program.h"
 
 #include "common.h"
@@ -58,12 +62,6 @@ struct Block {
   size_t begin, end;
 };
 
-struct PlanOfTile {
-  int tq = 0;
-  long tiles_at = 0, single_at = 0;   // in ints from the plan's start
-  int n_tiles = 0, n_single = 0;
-};
-
 struct Program {
   std::vector<LmsfOpDesc> ops;
   std::vector<int> last_use;        // per register: index of the last operation that reads it
@@ -72,8 +70,8 @@ struct Program {
   int n_regs = 0;
   bool sealed = false;
   LmsfTunables tun;
-  std::vector<PlanOfTile> plans;    // one per distinct tile size of the attention operations
-  int plan_max_context = 0;
+  std::vector<int> tile_sizes;      // the distinct tile sizes of the attention operations
+  LmsfCallbackFn callback = nullptr;
 };
 
 const int kLongLife = 12;   // a register read this many operations after it was written lives at the far end
@@ -154,13 +152,23 @@ struct Run {
   if (var == nullptr) return LMSF_PROGRAM_NO_ROOM
 
 inline int esize(int dtype) { return dtype == LMSF_F32 ? 4 : 2; }
-inline bool skinny_ok(const void* x, long ldx, int K, const void* W, long ldw) {
-  return K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0 && lmsf_aligned16(x) && lmsf_aligned16(W);
+
+// what the functions of dispatch.h want to know of a product x W^T, W of ``w_rows`` rows
+LmsfProductShape shape_of(const void* x, int x_dtype, long ldx, int M, int K, const void* W, int wdtype, long ldw,
+                          int w_rows, int out_dtype) {
+  LmsfProductShape s;
+  s.M = M;
+  s.N = w_rows;
+  s.K = K;
+  s.x_dtype = x_dtype;
+  s.w_dtype = wdtype;
+  s.out_dtype = out_dtype;
+  s.ldx = ldx;
+  s.ldw = ldw;
+  s.x_ok16 = lmsf_aligned16(x);
+  s.w_ok16 = lmsf_aligned16(W);
+  return s;
 }
-inline bool mid_ok(const void* x, long ldx, int K, const void* W, long ldw, int w_rows) {
-  return K % 64 == 0 && w_rows % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0 && lmsf_aligned16(x) && lmsf_aligned16(W);
-}
-inline bool gemv_ok(int M, int K) { return (long)M * K * 2 <= 128 * 1024; }
 
 Value tensor(void* p, int dtype, int M, int N) {
   Value v;
@@ -176,26 +184,30 @@ Value tensor(void* p, int dtype, int M, int N) {
 int op_linear(Run& r, const Value& x, const void* W, int wdtype, long ldw, int N, const void* bias, int out_dtype,
               bool pending_ok, void* out, Value* res);
 
+Value pending(float* partials, int splits, const void* bias, int dtype, int M, int N) {
+  Value v;
+  v.kind = V_PENDING;
+  v.partials = partials;
+  v.n_split = splits;
+  v.bias = bias;
+  v.dtype = dtype;
+  v.M = M;
+  v.N = N;
+  return v;
+}
+
+// the 17-and-more-rows kernel; act 0: plain, else the gated activation over W's two halves
 int linear_mid(Run& r, const Value& x, const void* W, long ldw, int w_rows, const void* bias, int act, int out_dtype,
-               bool pending_ok, void* out, Value* res) {
+               const LmsfRoute& rt, void* out, Value* res) {
   const int M = x.M, K = x.N;
   const int N = act ? w_rows / 2 : w_rows;
-  const int splits = lmsf_gemm_mid_splits(M, N, K, act);
-  if (pending_ok && act == 0 && splits > 1) {
-    TAKE(partials, float*, (size_t)splits * M * N * 4);
-    LAUNCH(lmsf_gemm_mid_partial(x.p, x.ld, W, ldw, M, N, K, splits, partials, r.stream));
-    Value v;
-    v.kind = V_PENDING;
-    v.partials = partials;
-    v.n_split = splits;
-    v.bias = bias;
-    v.dtype = out_dtype;
-    v.M = M;
-    v.N = N;
-    *res = v;
+  if (rt.pending) {
+    TAKE(partials, float*, (size_t)rt.splits * M * N * 4);
+    LAUNCH(lmsf_gemm_mid_partial(x.p, x.ld, W, ldw, M, N, K, rt.splits, partials, r.stream));
+    *res = pending(partials, rt.splits, bias, out_dtype, M, N);
     return 0;
   }
-  const long floats = lmsf_gemm_mid_scratch_floats(M, N, splits, act);
+  const long floats = lmsf_gemm_mid_scratch_floats(M, N, rt.splits, act);
   float* scratch = nullptr;
   if (floats > 0) {
     TAKE(s, float*, (size_t)floats * 4);
@@ -206,33 +218,23 @@ int linear_mid(Run& r, const Value& x, const void* W, long ldw, int w_rows, cons
     TAKE(yy, void*, (size_t)M * N * esize(out_dtype));
     y = yy;
   }
-  LAUNCH(lmsf_gemm_mid(x.p, x.ld, W, ldw, bias, y, out_dtype, N, M, N, K, act, splits, scratch, r.stream));
+  LAUNCH(lmsf_gemm_mid(x.p, x.ld, W, ldw, bias, y, out_dtype, N, M, N, K, act, rt.splits, scratch, r.stream));
   *res = tensor(y, out_dtype, M, N);
   return 0;
 }
 
-// HipOps._linear_large
-int linear_large(Run& r, const Value& x, const void* W, long ldw, int w_rows, const void* bias, int act, bool pending_ok,
-                 void* out, Value* res) {
+// the many-rows kernel
+int linear_large(Run& r, const Value& x, const void* W, long ldw, int w_rows, const void* bias, int act,
+                 const LmsfRoute& rt, void* out, Value* res) {
   const int M = x.M, K = x.N;
   const int N = act ? w_rows / 2 : w_rows;
-  const int plan = lmsf_gemm_large_plan(M, N, K, act);
-  const int splits = plan % 16;
   float* scratch = nullptr;
-  if (splits > 1) {
-    TAKE(s, float*, (size_t)splits * M * N * 4);
+  if (rt.splits > 1) {
+    TAKE(s, float*, (size_t)rt.splits * M * N * 4);
     scratch = s;
-    if (pending_ok) {
-      LAUNCH(lmsf_gemm_large(x.p, x.ld, W, ldw, nullptr, nullptr, 0, M, N, K, 0, plan, scratch, 0, r.stream));
-      Value v;
-      v.kind = V_PENDING;
-      v.partials = scratch;
-      v.n_split = splits;
-      v.bias = bias;
-      v.dtype = LMSF_BF16;
-      v.M = M;
-      v.N = N;
-      *res = v;
+    if (rt.pending) {
+      LAUNCH(lmsf_gemm_large(x.p, x.ld, W, ldw, nullptr, nullptr, 0, M, N, K, 0, rt.plan, scratch, 0, r.stream));
+      *res = pending(scratch, rt.splits, bias, LMSF_BF16, M, N);
       return 0;
     }
   }
@@ -241,12 +243,12 @@ int linear_large(Run& r, const Value& x, const void* W, long ldw, int w_rows, co
     TAKE(yy, void*, (size_t)M * N * 2);
     y = yy;
   }
-  LAUNCH(lmsf_gemm_large(x.p, x.ld, W, ldw, bias, y, N, M, N, K, act, plan, scratch, 1, r.stream));
+  LAUNCH(lmsf_gemm_large(x.p, x.ld, W, ldw, bias, y, N, M, N, K, act, rt.plan, scratch, 1, r.stream));
   *res = tensor(y, LMSF_BF16, M, N);
   return 0;
 }
 
-// HipOps.linear
+// y = x W^T + bias (HipOps.linear launches the same kernels for the same routes)
 int op_linear(Run& r, const Value& x, const void* W, int wdtype, long ldw, int N, const void* bias, int out_dtype,
               bool pending_ok, void* out, Value* res) {
   const LmsfTunables& t = r.prog->tun;
@@ -255,94 +257,59 @@ int op_linear(Run& r, const Value& x, const void* W, int wdtype, long ldw, int N
     return 1;
   }
   const int M = x.M, K = x.N;
-  const bool both_bf16 = x.dtype == LMSF_BF16 && wdtype == LMSF_BF16;
-  const bool m_ok = mid_ok(x.p, x.ld, K, W, ldw, N), s_ok = skinny_ok(x.p, x.ld, K, W, ldw);
-  // (deep: K at least three times N; such products go to the many-rows kernel from fewer rows on, and stay with it
-  // beyond large_max_rows, which is then not this program's business)
-  const bool deep = (long)K >= 3L * N && out_dtype == LMSF_BF16;
-  if (both_bf16 && t.skinny_max_rows < M && M <= t.mid_max_rows && m_ok &&
-      (M <= 64 || N <= t.mid_wide_max_cols || out_dtype == LMSF_F32) && !(deep && M > t.large_deep_min_rows))
-    return linear_mid(r, x, W, ldw, N, bias, 0, out_dtype, pending_ok && out_dtype == LMSF_BF16, out, res);
-  if (both_bf16 && out_dtype == LMSF_BF16 && m_ok &&
-      ((t.mid_max_rows < M && M <= t.large_max_rows) ||
-       (deep && t.large_deep_min_rows < M && M <= t.large_max_rows)))
-    return linear_large(r, x, W, ldw, N, bias, 0, pending_ok, out, res);
-  if (pending_ok && both_bf16 && out_dtype == LMSF_BF16 && s_ok && M > 0) {
-    if ((M <= std::min(t.fuse_stream_rows, t.gemv_max_rows) && gemv_ok(M, K)) ||
-        M <= std::min(std::min(t.fuse_norm_rows, t.skinny_max_rows), 16)) {
-      Value v;
-      v.kind = V_DEFERRED;
-      v.x = x.p;
-      v.ldx = x.ld;
-      v.K = K;
-      v.W = W;
-      v.ldw = ldw;
-      v.bias = bias;
-      v.dtype = out_dtype;
-      v.M = M;
-      v.N = N;
-      *res = v;
-      return 0;
-    }
-  }
-  if (both_bf16 && 0 < M && M <= std::min(1, t.gemv_max_rows) && s_ok && gemv_ok(M, K) && (long)N * K <= (1L << 28)) {
-    void* y = out;
-    if (y == nullptr) {
-      TAKE(yy, void*, (size_t)M * N * esize(out_dtype));
-      y = yy;
-    }
-    LAUNCH(lmsf_gemv(x.p, x.ld, W, ldw, bias, y, out_dtype, N, M, N, K, 0, r.stream));
-    *res = tensor(y, out_dtype, M, N);
+  const LmsfProductShape shape = shape_of(x.p, x.dtype, x.ld, M, K, W, wdtype, ldw, N, out_dtype);
+  LmsfRoute rt;
+  lmsf_route_linear(&t, &shape, pending_ok ? 1 : 0, &rt);
+  if (rt.route == LMSF_ROUTE_MID) return linear_mid(r, x, W, ldw, N, bias, 0, out_dtype, rt, out, res);
+  if (rt.route == LMSF_ROUTE_LARGE) return linear_large(r, x, W, ldw, N, bias, 0, rt, out, res);
+  if (rt.route == LMSF_ROUTE_DEFERRED) {
+    Value v;
+    v.kind = V_DEFERRED;
+    v.x = x.p;
+    v.ldx = x.ld;
+    v.K = K;
+    v.W = W;
+    v.ldw = ldw;
+    v.bias = bias;
+    v.dtype = out_dtype;
+    v.M = M;
+    v.N = N;
+    *res = v;
     return 0;
-  }
-  if (both_bf16 && out_dtype == LMSF_F32 && M > t.mid_max_rows && m_ok) {
-    // float32 output for many rows: as many rows at a time as the kernel for 17 and more rows takes
-    void* y = out;
-    if (y == nullptr) {
-      TAKE(yy, void*, (size_t)M * N * 4);
-      y = yy;
-    }
-    for (int r0 = 0; r0 < M; r0 += t.mid_max_rows) {
-      const int rows = std::min(t.mid_max_rows, M - r0);
-      Value xs = x;
-      xs.p = (char*)x.p + (size_t)r0 * x.ld * 2;
-      xs.M = rows;
-      Value part;
-      RC(op_linear(r, xs, W, wdtype, ldw, N, bias, out_dtype, false, (char*)y + (size_t)r0 * N * 4, &part));
-    }
-    *res = tensor(y, out_dtype, M, N);
-    return 0;
-  }
-  if (both_bf16 && s_ok) {
-    const int limit = out_dtype == LMSF_BF16 ? t.skinny_max_rows : 64;
-    if (M <= limit || out_dtype == LMSF_F32) {
-      void* y = out;
-      if (y == nullptr) {
-        TAKE(yy, void*, (size_t)M * N * esize(out_dtype));
-        y = yy;
-      }
-      for (int r0 = 0; r0 < M; r0 += 64) {
-        const int rows = std::min(64, M - r0);
-        LAUNCH(lmsf_gemm_skinny((const char*)x.p + (size_t)r0 * x.ld * 2, x.ld, W, ldw, bias,
-                                (char*)y + (size_t)r0 * N * esize(out_dtype), out_dtype, N, rows, N, K,
-                                t.skinny_variant, 0, r.stream));
-      }
-      *res = tensor(y, out_dtype, M, N);
-      return 0;
-    }
-  }
-  if (t.use_library_gemm && both_bf16 && M > t.skinny_max_rows && out_dtype == LMSF_BF16) {
-    lmsf_set_error("program: a bfloat16 product of %d rows, %d columns over %d goes to the BLAS library", M, N, K);
-    return LMSF_PROGRAM_NOT_NATIVE;
   }
   void* y = out;
   if (y == nullptr) {
     TAKE(yy, void*, (size_t)M * N * esize(out_dtype));
     y = yy;
   }
-  LAUNCH(lmsf_gemm_plain(x.p, x.dtype, x.ld, W, wdtype, ldw, bias, y, out_dtype, N, M, N, K, r.stream));
   *res = tensor(y, out_dtype, M, N);
-  return 0;
+  switch (rt.route) {
+    case LMSF_ROUTE_GEMV:
+      LAUNCH(lmsf_gemv(x.p, x.ld, W, ldw, bias, y, out_dtype, N, M, N, K, 0, r.stream));
+      return 0;
+    case LMSF_ROUTE_CHUNKS:
+      for (int r0 = 0; r0 < M; r0 += rt.chunk_rows) {
+        Value xs = x;
+        xs.p = (char*)x.p + (size_t)r0 * x.ld * esize(x.dtype);
+        xs.M = std::min(rt.chunk_rows, M - r0);
+        Value part;
+        RC(op_linear(r, xs, W, wdtype, ldw, N, bias, out_dtype, false, (char*)y + (size_t)r0 * N * esize(out_dtype),
+                     &part));
+      }
+      return 0;
+    case LMSF_ROUTE_SKINNY:
+      for (int r0 = 0; r0 < M; r0 += 64)
+        LAUNCH(lmsf_gemm_skinny((const char*)x.p + (size_t)r0 * x.ld * 2, x.ld, W, ldw, bias,
+                                (char*)y + (size_t)r0 * N * esize(out_dtype), out_dtype, N, std::min(64, M - r0), N, K,
+                                t.skinny_variant, 0, r.stream));
+      return 0;
+    case LMSF_ROUTE_BLAS:
+      LAUNCH(lmsf_blas_linear(x.p, x.ld, W, ldw, bias, y, N, M, N, K, r.stream));
+      return 0;
+    default:
+      LAUNCH(lmsf_gemm_plain(x.p, x.dtype, x.ld, W, wdtype, ldw, bias, y, out_dtype, N, M, N, K, r.stream));
+      return 0;
+  }
 }
 
 int op_add_rms_norm(Run& r, const Value& branch, float* residual, int M, int H, const void* weight, int wdtype,
@@ -401,37 +368,25 @@ int op_add_rms_norm(Run& r, const Value& branch_in, float* residual, int M, int 
     const int Mb = branch.M, N = branch.N, K = branch.K;
     const bool fits = rows == nullptr && residual != nullptr && Mb == M && N == H;
     const bool prepares = fits && defer_ok && out_dtype == LMSF_BF16 && wdtype == LMSF_BF16;
-    const bool one_or_two = fits && Mb <= std::min(t.fuse_stream_rows, t.gemv_max_rows) && gemv_ok(Mb, K);
-    if (prepares && one_or_two && gemv_ok(Mb, N)) {
-      const int parts = lmsf_gemv_partials(N);
-      TAKE(xw, void*, (size_t)Mb * N * 2 + 256 + (size_t)parts * Mb * 4);
+    LmsfRoute rt;
+    lmsf_route_deferred_norm(&t, Mb, N, K, fits ? 1 : 0, prepares ? 1 : 0, &rt);
+    if (rt.route == LMSF_ROUTE_GEMV_ADD_NORM || rt.route == LMSF_ROUTE_SKINNY_ADD_NORM) {
+      const bool one_or_two = rt.route == LMSF_ROUTE_GEMV_ADD_NORM;
+      const int tiles = one_or_two ? lmsf_gemv_partials(N) : (N + 15) / 16;
+      const int rows_per_tile = one_or_two ? Mb : 16;
+      TAKE(xw, void*, (size_t)Mb * N * 2 + 256 + (size_t)tiles * rows_per_tile * 4);
       float* sumsq = (float*)((char*)xw + (((size_t)Mb * N * 2 + 255) & ~(size_t)255));
-      LAUNCH(lmsf_gemv_add_norm(branch.x, branch.ldx, branch.W, branch.ldw, branch.bias, residual, H, weight,
-                                weight_offset, xw, N, sumsq, Mb, N, K, r.stream));
-      Value v = tensor(xw, LMSF_BF16, Mb, N);
-      v.kind = V_SCALED;
-      v.sumsq = sumsq;
-      v.tiles = parts;
-      v.rows_per_tile = Mb;
-      v.eps = eps;
-      v.weight_offset = weight_offset;
-      v.norm_weight = weight;
-      v.norm_wdtype = wdtype;
-      v.stream = residual;
-      *res = v;
-      return 0;
-    }
-    if (prepares && Mb <= std::min(std::min(t.fuse_norm_rows, t.skinny_max_rows), 16) && !one_or_two) {
-      const int tiles = (N + 15) / 16;
-      TAKE(xw, void*, (size_t)Mb * N * 2 + 256 + (size_t)tiles * 16 * 4);
-      float* sumsq = (float*)((char*)xw + (((size_t)Mb * N * 2 + 255) & ~(size_t)255));
-      LAUNCH(lmsf_gemm_skinny_add_norm(branch.x, branch.ldx, branch.W, branch.ldw, branch.bias, residual, H, weight,
-                                       weight_offset, xw, N, sumsq, Mb, N, K, t.skinny_variant, r.stream));
+      if (one_or_two)
+        LAUNCH(lmsf_gemv_add_norm(branch.x, branch.ldx, branch.W, branch.ldw, branch.bias, residual, H, weight,
+                                  weight_offset, xw, N, sumsq, Mb, N, K, r.stream));
+      else
+        LAUNCH(lmsf_gemm_skinny_add_norm(branch.x, branch.ldx, branch.W, branch.ldw, branch.bias, residual, H, weight,
+                                         weight_offset, xw, N, sumsq, Mb, N, K, t.skinny_variant, r.stream));
       Value v = tensor(xw, LMSF_BF16, Mb, N);
       v.kind = V_SCALED;
       v.sumsq = sumsq;
       v.tiles = tiles;
-      v.rows_per_tile = 16;
+      v.rows_per_tile = rows_per_tile;
       v.eps = eps;
       v.weight_offset = weight_offset;
       v.norm_weight = weight;
@@ -440,7 +395,7 @@ int op_add_rms_norm(Run& r, const Value& branch_in, float* residual, int M, int 
       *res = v;
       return 0;
     }
-    if (one_or_two) {
+    if (rt.route == LMSF_ROUTE_GEMV_ADD) {
       LAUNCH(lmsf_gemv_add(branch.x, branch.ldx, branch.W, branch.ldw, branch.bias, residual, H, Mb, N, K, r.stream));
       branch = Value();
     } else {
@@ -469,20 +424,22 @@ int op_add_rms_norm(Run& r, const Value& branch_in, float* residual, int M, int 
   return 0;
 }
 
-// HipOps.linear_gated; kind 1: SiLU, 2: GELU
+// act(x Wg^T) * (x Wu^T); kind 1: SiLU, 2: GELU (HipOps.linear_gated launches the same kernels for the same routes)
 int op_linear_gated(Run& r, const Value& x_in, const void* W, int wdtype, long ldw, int w_rows, const void* bias,
                     int kind, Value* res) {
   const LmsfTunables& t = r.prog->tun;
   Value x = x_in;
   const int I = w_rows / 2;
+  LmsfRoute rt;
   if (x.kind == V_SCALED) {
-    const int M = x.M, K = x.N;
-    if (wdtype == LMSF_BF16 && skinny_ok(x.p, x.ld, K, W, ldw) && (x.rows_per_tile == 16 || gemv_ok(M, K))) {
+    const LmsfProductShape shape = shape_of(x.p, x.dtype, x.ld, x.M, x.N, W, wdtype, ldw, w_rows, LMSF_BF16);
+    lmsf_route_linear_gated(&t, &shape, x.rows_per_tile, x.tiles, &rt);
+    if (rt.route != LMSF_ROUTE_MATERIALIZE) {
+      const int M = x.M, K = x.N;
       TAKE(y, void*, (size_t)M * I * 2);
-      if (x.rows_per_tile == 16 && M <= t.mid_scaled_rows && mid_ok(x.p, x.ld, K, W, ldw, w_rows) &&
-          lmsf_gemm_mid_scaled_fits(M, I, K, x.tiles))
+      if (rt.route == LMSF_ROUTE_MID_SCALED)
         LAUNCH(lmsf_gemm_mid_scaled(x.p, x.ld, W, ldw, bias, y, I, M, I, K, kind, x.sumsq, x.tiles, x.eps, r.stream));
-      else if (x.rows_per_tile != 16)
+      else if (rt.route == LMSF_ROUTE_GEMV_SCALED)
         LAUNCH(lmsf_gemv_scaled(x.p, x.ld, W, ldw, bias, y, I, M, I, K, kind, x.sumsq, x.tiles, x.eps, r.stream));
       else
         LAUNCH(lmsf_gemm_skinny_scaled(x.p, x.ld, W, ldw, bias, y, I, M, I, K, kind, x.sumsq, x.tiles, x.eps,
@@ -497,20 +454,19 @@ int op_linear_gated(Run& r, const Value& x_in, const void* W, int wdtype, long l
     x = m;
   }
   const int M = x.M, K = x.N;
-  const bool both_bf16 = x.dtype == LMSF_BF16 && wdtype == LMSF_BF16;
-  if (both_bf16 && 0 < M && M <= t.skinny_max_rows && skinny_ok(x.p, x.ld, K, W, ldw)) {
+  const LmsfProductShape shape = shape_of(x.p, x.dtype, x.ld, M, K, W, wdtype, ldw, w_rows, x.dtype);
+  lmsf_route_linear_gated(&t, &shape, 0, 0, &rt);
+  if (rt.route == LMSF_ROUTE_GEMV || rt.route == LMSF_ROUTE_SKINNY) {
     TAKE(y, void*, (size_t)M * I * 2);
-    if (M <= t.gemv_max_rows && gemv_ok(M, K))
+    if (rt.route == LMSF_ROUTE_GEMV)
       LAUNCH(lmsf_gemv(x.p, x.ld, W, ldw, bias, y, LMSF_BF16, I, M, I, K, kind, r.stream));
     else
       LAUNCH(lmsf_gemm_skinny(x.p, x.ld, W, ldw, bias, y, LMSF_BF16, I, M, I, K, t.skinny_variant, kind, r.stream));
     *res = tensor(y, LMSF_BF16, M, I);
     return 0;
   }
-  if (both_bf16 && t.skinny_max_rows < M && M <= 64 && mid_ok(x.p, x.ld, K, W, ldw, w_rows))
-    return linear_mid(r, x, W, ldw, w_rows, bias, kind, LMSF_BF16, false, nullptr, res);
-  if (both_bf16 && 64 < M && M <= t.large_max_rows && mid_ok(x.p, x.ld, K, W, ldw, w_rows) && I % 8 == 0)
-    return linear_large(r, x, W, ldw, w_rows, bias, kind, false, nullptr, res);   // (it writes eight outputs at a time)
+  if (rt.route == LMSF_ROUTE_MID) return linear_mid(r, x, W, ldw, w_rows, bias, kind, LMSF_BF16, rt, nullptr, res);
+  if (rt.route == LMSF_ROUTE_LARGE) return linear_large(r, x, W, ldw, w_rows, bias, kind, rt, nullptr, res);
   Value gu;
   RC(op_linear(r, x, W, wdtype, ldw, w_rows, bias, x.dtype, false, nullptr, &gu));
   TAKE(y, void*, (size_t)M * I * esize(gu.dtype));
@@ -531,20 +487,25 @@ int rope_cache_write(Run& r, const Value& qkv, const LmsfOpDesc& op, const int* 
   return 0;
 }
 
-// HipOps.qkv_rope_cache
+// The QKV product with rotation and cache write (HipOps.qkv_rope_cache launches the same kernels for the same routes)
 int op_qkv_rope_cache(Run& r, const Value& x_in, const LmsfOpDesc& op, const int* positions, const int* slots,
                       Value* res) {
   const LmsfTunables& t = r.prog->tun;
   Value x = x_in;
   const int N = (op.nh + 2 * op.nkv) * op.d;
   const float* table = (const float*)op.table;
-  const bool fused_shape = table != nullptr && slots != nullptr && op.neox && op.rot == op.d && op.d % 32 == 0 &&
-                           op.wdtype == LMSF_BF16 && op.N == N && op.k_pages != nullptr && op.cache_dtype == LMSF_BF16;
+  const auto fused_shape = [&](int K) {
+    return table != nullptr && slots != nullptr && op.neox && op.rot == op.d && op.d % 32 == 0 &&
+           op.wdtype == LMSF_BF16 && op.N == N && op.K == K && op.k_pages != nullptr && op.cache_dtype == LMSF_BF16;
+  };
+  LmsfRoute rt;
   if (x.kind == V_SCALED) {
     const int M = x.M, K = x.N;
-    if (fused_shape && op.K == K && skinny_ok(x.p, x.ld, K, op.w, op.ldw) && (x.rows_per_tile == 16 || gemv_ok(M, K))) {
+    const LmsfProductShape shape = shape_of(x.p, x.dtype, x.ld, M, K, op.w, op.wdtype, op.ldw, op.N, LMSF_BF16);
+    lmsf_route_qkv(&t, &shape, fused_shape(K) ? 1 : 0, x.rows_per_tile, &rt);
+    if (rt.route != LMSF_ROUTE_MATERIALIZE) {
       TAKE(y, void*, (size_t)M * N * 2);
-      if (x.rows_per_tile != 16)
+      if (rt.route == LMSF_ROUTE_GEMV_SCALED)
         LAUNCH(lmsf_gemv_scaled_qkv_rope_cache(x.p, x.ld, op.w, op.ldw, op.bias, y, N, M, K, positions, table,
                                                op.max_pos, slots, op.k_pages, op.v_pages, op.num_pages, op.nh, op.nkv,
                                                op.d, op.ps, x.sumsq, x.tiles, x.eps, r.stream));
@@ -562,10 +523,11 @@ int op_qkv_rope_cache(Run& r, const Value& x_in, const LmsfOpDesc& op, const int
     x = m;
   }
   const int M = x.M, K = x.N;
-  if (fused_shape && x.dtype == LMSF_BF16 && 0 < M && M <= t.skinny_max_rows && op.K == K &&
-      skinny_ok(x.p, x.ld, K, op.w, op.ldw)) {
+  const LmsfProductShape shape = shape_of(x.p, x.dtype, x.ld, M, K, op.w, op.wdtype, op.ldw, op.N, x.dtype);
+  lmsf_route_qkv(&t, &shape, fused_shape(K) ? 1 : 0, 0, &rt);
+  if (rt.route == LMSF_ROUTE_GEMV || rt.route == LMSF_ROUTE_SKINNY) {
     TAKE(y, void*, (size_t)M * N * 2);
-    if (M <= t.gemv_max_rows && gemv_ok(M, K))
+    if (rt.route == LMSF_ROUTE_GEMV)
       LAUNCH(lmsf_gemv_qkv_rope_cache(x.p, x.ld, op.w, op.ldw, op.bias, y, N, M, K, positions, table, op.max_pos, slots,
                                       op.k_pages, op.v_pages, op.num_pages, op.nh, op.nkv, op.d, op.ps, r.stream));
     else
@@ -576,8 +538,7 @@ int op_qkv_rope_cache(Run& r, const Value& x_in, const LmsfOpDesc& op, const int
     return 0;
   }
   Value y;
-  RC(op_linear(r, x, op.w, op.wdtype, op.ldw, op.N, op.bias, x.dtype,
-               M > std::max(std::max(t.fuse_stream_rows, t.fuse_norm_rows), t.skinny_max_rows), nullptr, &y));
+  RC(op_linear(r, x, op.w, op.wdtype, op.ldw, op.N, op.bias, x.dtype, rt.pending != 0, nullptr, &y));
   if (y.kind == V_PENDING) {
     if ((table == nullptr && slots == nullptr) || op.N != N) {
       Value m;
@@ -618,7 +579,7 @@ int op_qkv_rope_cache(Run& r, const Value& x_in, const LmsfOpDesc& op, const int
   return 0;
 }
 
-// HipOps.paged_attention
+// Attention over the pages (HipOps.paged_attention launches the same kernels)
 int op_attention(Run& r, const Value& q, const LmsfOpDesc& op, const int* tables, int width, Value* res) {
   const LmsfStepDesc& st = *r.st;
   const LmsfTunables& t = r.prog->tun;
@@ -653,32 +614,26 @@ int op_attention(Run& r, const Value& q, const LmsfOpDesc& op, const int* tables
     n_single = N;
   } else {
     const int tq = lmsf_attention_tile_tokens(nh, nkv);
-    const PlanOfTile* plan = nullptr;
-    for (const PlanOfTile& p : r.prog->plans)
-      if (p.tq == tq) plan = &p;
-    if (plan == nullptr || st.plan == nullptr) {
+    const LmsfPlanInfo& info = st.plan_info;
+    int at = -1;
+    for (int i = 0; i < info.n_plans && i < LMSF_MAX_PLANS; ++i)
+      if (info.tq[i] == tq) at = i;
+    if (at < 0 || st.plan == nullptr || info.n_tiles[at] + info.n_single[at] <= 0) {
       lmsf_set_error("program: the step carries no attention plan for tiles of %d tokens", tq);
       return 1;
     }
-    n_tiles = plan->n_tiles;
-    n_single = plan->n_single;
-    tiles = n_tiles ? st.plan + plan->tiles_at : nullptr;
-    single = n_single ? st.plan + plan->single_at : nullptr;
+    n_tiles = info.n_tiles[at];
+    n_single = info.n_single[at];
+    tiles = n_tiles ? st.plan + info.tiles_at[at] : nullptr;
+    single = n_single ? st.plan + info.single_at[at] : nullptr;
   }
   if (n_tiles)
     LAUNCH(lmsf_paged_attention_prefill_mfma(q.p, q.ld, out, (long)nh * d, op.k_pages, op.v_pages, op.num_pages, tables,
                                              width, tiles, n_tiles, st.seg_of, st.positions, nh, nkv, d, ps, op.scale,
                                              op.window, t.prefill_attention_variant, r.stream));
   if (n_single) {
-    const int n_hb = ((nh / nkv) + 15) / 16;
-    const int most = (max_context + 127) / 128;
-    const int pairs = n_single * nkv * n_hb;   // (as HipOps.paged_attention chooses)
-    const int fill = max_context >= 49152 && pairs >= 16 ? 2048 : max_context >= 32768 && pairs >= 32 ? 1024 : 512;
-    int want = std::max(1, std::min(most, fill / pairs));
-    if (want == 2 && max_context <= 512) want = 1;
-    if (t.decode_attention_splits) want = std::min(most, t.decode_attention_splits);
-    const int chunk = (((max_context + want - 1) / want) + 127) / 128 * 128;
-    const int n_splits = (max_context + chunk - 1) / chunk;
+    int chunk = 0, n_splits = 0;
+    lmsf_route_decode_attention(&t, n_single, nh, nkv, max_context, &chunk, &n_splits);
     const long floats = n_splits > 1 ? lmsf_attention_decode_scratch_floats(n_single, nh, d, n_splits) : 1;
     TAKE(scratch, float*, (size_t)floats * 4);
     LAUNCH(lmsf_paged_attention_decode_mfma(q.p, q.ld, out, (long)nh * d, op.k_pages, op.v_pages, op.num_pages, tables,
@@ -786,6 +741,74 @@ int run_pass(const Program& prog, const LmsfStepDesc& st, hipStream_t stream, bo
       case LMSF_OP_MATERIALIZE:
         RC(materialize(r, in0, &res));
         break;
+      case LMSF_OP_ROPE_CACHE_WRITE: {
+        if (in0.kind != V_TENSOR || in0.N != (op.nh + 2 * op.nkv) * op.d) {
+          lmsf_set_error("program: rotation and cache write need a tensor of %d columns", (op.nh + 2 * op.nkv) * op.d);
+          return 1;
+        }
+        const int* slots = op.ctx1 != LMSF_CTX_NONE ? step_array(st, op.ctx1, nullptr) : nullptr;
+        if (slots != nullptr && op.cache_dtype != in0.dtype) {
+          lmsf_set_error("program: the projection and its cache differ in type");
+          return 1;
+        }
+        RC(rope_cache_write(r, in0, op, op.ctx0 != LMSF_CTX_NONE ? step_array(st, op.ctx0, nullptr) : nullptr, slots));
+        break;
+      }
+      case LMSF_OP_GATED_ACT: {
+        if (in0.kind != V_TENSOR || in0.N != op.N || op.N % 2 != 0) {
+          lmsf_set_error("program: a gated activation needs a tensor of %d columns", op.N);
+          return 1;
+        }
+        TAKE(y, void*, (size_t)in0.M * (op.N / 2) * esize(in0.dtype));
+        LAUNCH(lmsf_gated_act(in0.p, y, in0.dtype, in0.M, op.N / 2, in0.ld, op.act - 1, stream));
+        res = tensor(y, in0.dtype, in0.M, op.N / 2);
+        break;
+      }
+      case LMSF_OP_CALLBACK: {
+        const Value& in1 = op.in1 >= 0 ? r.regs[op.in1] : none;
+        for (const Value* v : {&in0, &in1})
+          if (v->kind != V_NONE && (v->kind != V_TENSOR || v->ld != v->N)) {
+            lmsf_set_error("program: a callback's operand is not a finished tensor");
+            return 1;
+          }
+        if (prog.callback == nullptr) {
+          lmsf_set_error("program: a callback operation, and no function to call");
+          return 1;
+        }
+        const auto ref = [&](const Value& v) {
+          LmsfTensorRef t;
+          t.offset = v.kind == V_NONE ? -1 : v.p == (void*)st.logits ? -2 : (long)((char*)v.p - r.base());
+          t.rows = v.M;
+          t.cols = v.N;
+          t.dtype = v.dtype;
+          return t;
+        };
+        LmsfCallbackArgs args;
+        args.callback_id = op.callback_id;
+        args.in0 = ref(in0);
+        args.in1 = ref(in1);
+        if (op.out >= 0) {
+          const int rows = op.rows_ctx != LMSF_CTX_NONE ? R : in0.kind != V_NONE ? in0.M : N;
+          void* y = nullptr;
+          if (op.is_head) {
+            if (st.logits == nullptr) {
+              lmsf_set_error("program: the step has no buffer for its logits");
+              return 1;
+            }
+            y = st.logits;
+          } else {
+            TAKE(yy, void*, (size_t)rows * op.N * esize(op.out_dtype));
+            y = yy;
+          }
+          res = tensor(y, op.out_dtype, rows, op.N);
+        }
+        args.out = ref(res);
+        if (!r.dry && prog.callback(&args) != 0) {
+          lmsf_set_error("program: callback %d failed", op.callback_id);
+          return 1;
+        }
+        break;
+      }
       default:
         lmsf_set_error("program: unknown operation %d", op.kind);
         return 1;
@@ -823,7 +846,7 @@ extern "C" int lmsf_program_seal(void* program) {
   p->last_use.assign(p->n_regs, -1);
   p->first_def.assign(p->n_regs, -1);
   p->long_lived.assign(p->n_regs, 0);
-  p->plans.clear();
+  p->tile_sizes.clear();
   for (size_t i = 0; i < p->ops.size(); ++i) {
     const LmsfOpDesc& op = p->ops[i];
     if (op.out >= 0 && p->first_def[op.out] < 0) p->first_def[op.out] = (int)i;
@@ -831,15 +854,10 @@ extern "C" int lmsf_program_seal(void* program) {
       if (reg >= 0) p->last_use[reg] = (int)i;
     if (op.kind == LMSF_OP_ATTENTION) {
       const int tq = lmsf_attention_tile_tokens(op.nh, op.nkv);
-      bool have = false;
-      for (const PlanOfTile& pl : p->plans) have = have || pl.tq == tq;
-      if (!have) {
-        PlanOfTile pl;
-        pl.tq = tq;
-        p->plans.push_back(pl);
-      }
+      if (std::find(p->tile_sizes.begin(), p->tile_sizes.end(), tq) == p->tile_sizes.end()) p->tile_sizes.push_back(tq);
     }
   }
+  LMSF_CHECK(p->tile_sizes.size() <= LMSF_MAX_PLANS, "program_seal: attention with more than %d tile sizes", LMSF_MAX_PLANS);
   // an unfinished value points into the memory of the register it was made from (a product not yet started reads
   // its operand when the norm runs it; scaled rows are finished from the stream): the operand lives as long
   for (int pass = 0; pass < 2; ++pass)
@@ -855,32 +873,36 @@ extern "C" int lmsf_program_seal(void* program) {
   return 0;
 }
 
+extern "C" void lmsf_program_set_callback(void* program, LmsfCallbackFn fn) {
+  if (program) static_cast<Program*>(program)->callback = fn;
+}
+
 // Host side of a step that is not all single tokens: the attention plan, for every tile size the program's
 // attention operations use, written to ``out`` (host memory that the caller copies to the device with the step's
-// other arrays; LmsfStepDesc.plan is its device address). Per tile size: pairs (first flat index, tokens) of
+// other arrays; LmsfStepDesc.plan is its device address) and described in ``info``, which travels with the step
+// (LmsfStepDesc.plan_info): nothing of a plan is kept here. Per tile size: pairs (first flat index, tokens) of
 // the tiles of requests with several tokens, those with the most keys first, then the flat indices of the
 // requests with one token, the longest context first. Returns the number of ints written, or -1.
 extern "C" long lmsf_program_plan(void* program, int S, const int* seg_lens, const int* seg_first_pos, int* out,
-                                  long capacity) {
-  Program* p = static_cast<Program*>(program);
-  if (!p || !p->sealed || S < 0 || (S > 0 && (!seg_lens || !seg_first_pos))) {
+                                  long capacity, LmsfPlanInfo* info) {
+  const Program* p = static_cast<const Program*>(program);
+  if (!p || !p->sealed || !info || S < 0 || (S > 0 && (!seg_lens || !seg_first_pos))) {
     lmsf_set_error("program_plan: bad arguments");
     return -1;
   }
   long at = 0;
-  int max_context = 0;
-  for (PlanOfTile& pl : p->plans) {
+  info->n_plans = 0;
+  for (const int tq : p->tile_sizes) {
     std::vector<std::pair<int, std::pair<int, int>>> tiles;   // keys, (start, n)
     std::vector<std::pair<int, int>> single;                  // first position, flat index
     int flat = 0;
     for (int s = 0; s < S; ++s) {
       const int n = seg_lens[s], p0 = seg_first_pos[s];
-      max_context = std::max(max_context, p0 + n);
       if (n == 1) {
         single.push_back({p0, flat});
       } else {
-        for (int t = 0; t < n; t += pl.tq) {
-          const int m = std::min(pl.tq, n - t);
+        for (int t = 0; t < n; t += tq) {
+          const int m = std::min(tq, n - t);
           tiles.push_back({p0 + t + m, {flat + t, m}});
         }
       }
@@ -893,19 +915,20 @@ extern "C" long lmsf_program_plan(void* program, int S, const int* seg_lens, con
       lmsf_set_error("program_plan: %ld ints do not fit the %ld given", at + need, capacity);
       return -1;
     }
-    pl.tiles_at = at;
-    pl.n_tiles = (int)tiles.size();
+    const int i = info->n_plans++;
+    info->tq[i] = tq;
+    info->tiles_at[i] = at;
+    info->n_tiles[i] = (int)tiles.size();
     for (const auto& t : tiles) {
       out[at++] = t.second.first;
       out[at++] = t.second.second;
     }
     at = (at + 3) / 4 * 4;
-    pl.single_at = at;
-    pl.n_single = (int)single.size();
+    info->single_at[i] = at;
+    info->n_single[i] = (int)single.size();
     for (const auto& s : single) out[at++] = s.second;
     at = (at + 3) / 4 * 4;
   }
-  p->plan_max_context = max_context;
   return at;
 }
 
@@ -913,12 +936,12 @@ extern "C" long lmsf_program_plan(void* program, int S, const int* seg_lens, con
 extern "C" long lmsf_program_plan_capacity(void* program, int N) {
   Program* p = static_cast<Program*>(program);
   if (!p) return 0;
-  return (long)std::max<size_t>(1, p->plans.size()) * (2L * N + N + 16);
+  return (long)std::max<size_t>(1, p->tile_sizes.size()) * (2L * N + N + 16);
 }
 
-// Runs the step. 0: done. LMSF_PROGRAM_NOT_NATIVE: the step needs a product that only the BLAS library has;
-// LMSF_PROGRAM_NO_ROOM: the workspace is too small; in both cases nothing was launched. Other values: an error
-// (lmsf_last_error), possibly after some kernels were launched. ``check_only``: walk the step, launch nothing.
+// Runs the step. 0: done. LMSF_PROGRAM_NO_ROOM: the workspace is too small, nothing was launched. Other values:
+// an error (lmsf_last_error), possibly after some kernels were launched. ``check_only``: walk the step, launch
+// nothing (the workspace's address is then never used, only its size).
 extern "C" int lmsf_program_run(void* program, const LmsfStepDesc* step, int check_only, hipStream_t stream) {
   Program* p = static_cast<Program*>(program);
   LMSF_CHECK(p && step, "program_run: null pointer");

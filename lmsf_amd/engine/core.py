@@ -165,5 +165,6 @@ def load_engine_core(model_dir: Optional[str], dtype: Optional[str] = None, bloc
         counts = [int(num_pages)] * len(groups)
     storage = CacheStorage(model, rt, block_size, counts, num_state_slots=max_num_seqs)
     executor = ModelExecutor(model, storage, rt, max_model_len, use_graphs=not enforce_eager,
-                             use_program=use_program)
+                             use_program=use_program, max_step_tokens=max_num_batched_tokens,
+                             max_step_seqs=max_num_seqs)
     return EngineCore(arch, config, rt, model, storage, executor, max_model_len, block_size)

@@ -25,7 +25,8 @@ class StepError(ValueError):
 
 class ModelExecutor:
     def __init__(self, model, storage: CacheStorage, rt: Runtime, max_model_len: int, use_graphs: bool = True,
-                 max_graph_batch: int = 256, max_graphs: int = 48, use_program: bool = True):
+                 max_graph_batch: int = 256, max_graphs: int = 48, use_program: bool = True,
+                 max_step_tokens: Optional[int] = None, max_step_seqs: Optional[int] = None):
         self.model = model
         self.storage = storage
         self.manager: CacheManager = storage.manager
@@ -51,11 +52,44 @@ class ModelExecutor:
         # do more with their activations than hand them to the kernels (then the parts run one by one)
         self.program = None
         self.use_program = bool(use_program) and rt.device.type == "cuda"
-        if self.use_program:
-            from ..ops.program import record_program
-            self.program = record_program(model, rt.ops)
+        self.max_step_tokens = int(max_step_tokens) if max_step_tokens else None
+        self.max_step_seqs = int(max_step_seqs) if max_step_seqs else None
         self.program_steps = 0          # steps that the program ran
-        self.program_workspace_bytes = 32 << 20    # the workspace's first size; it doubles when a step finds no room
+        self.program_workspace_bytes = 32 << 20    # the workspace's size; it doubles if a step finds no room all the same
+        if self.use_program:
+            self._record_program()
+
+    def _record_program(self) -> None:
+        """Records the model's kernel calls and gives the program its workspace: once, at the size that the largest
+        step the engine will build needs (found by walking such steps without launching), so that no step in
+        the middle of serving has to allocate."""
+        from ..ops.program import record_program
+        self.program = record_program(self.model, self.rt.ops)
+        self._static.clear()            # captured steps belong to the program that launched them
+        if self.program is None:
+            return
+        if self.max_step_tokens:
+            self.program_workspace_bytes = max(self.program_workspace_bytes, self.workspace_for(
+                self.max_step_tokens, self.max_step_seqs or self.max_graph_batch))
+        self.program.ensure_workspace(self.program_workspace_bytes)
+
+    def workspace_for(self, max_tokens: int, max_seqs: int) -> int:
+        """Bytes of program workspace that steps of up to ``max_tokens`` tokens of up to ``max_seqs`` requests need:
+        the most over a ladder of step sizes, each as one portion of a prompt, as a portion beside single tokens
+        and (where it fits) as single tokens only, plus a tenth."""
+        prog = self.program
+        G = len(self.manager.groups)
+        sizes = sorted({n for n in (1, 2, 8, 16, 17, 64, 65, 128, 129, 256, 257, 512, 1024, 2048, 4096, max_tokens // 2,
+                                    max_tokens) if 1 <= n <= max_tokens})
+        need = 0
+        for n in sizes:
+            shapes = {(1, 1), (min(max_seqs, max(1, n // 2)), min(max_seqs, max(1, n // 2)))}
+            if n <= max_seqs:
+                shapes.add((n, n))
+            for segs, rows in shapes:
+                if segs <= n:
+                    need = max(need, prog.workspace_need(n, segs, rows, self.max_model_len, G))
+        return int(need * 1.1) + (1 << 20)
 
     # ------------------------------------------------------------------ the step
 
@@ -66,6 +100,10 @@ class ModelExecutor:
         entries that name one of them (``StepEntry.prev_row``) instead of a token the host knows."""
         entries = [e for e in entries if len(e.tokens) > 0]
         self._validate(entries)
+        if self.program is not None and self.program.stale():
+            # somebody moved the kernels' switch points (tests, tuning): record again before anything of this step
+            # is built for the old program, and forget what was captured
+            self._record_program()
         from_prev = any(e.prev_row >= 0 for e in entries)
         if from_prev and prev_tokens is None:
             raise StepError("an entry names a token of the step before, which was not given")
@@ -88,37 +126,32 @@ class ModelExecutor:
         return logits
 
     def _forward(self, ctx: StepContext, logits_out: Optional[torch.Tensor] = None) -> torch.Tensor:
-        """The model over the step: through the recorded program where there is one and it takes the step, else
-        part by part."""
+        """The model over the step: through the recorded program where there is one, else part by part."""
         prog = self.program
-        if prog is not None and prog.stale():
-            # somebody moved the kernels' switch points (tests, tuning): record again, and forget what was captured
-            from ..ops.program import record_program
-            prog = self.program = record_program(self.model, self.rt.ops)
-            self._static.clear()
-        if prog is not None:
+        plan = ctx.aux.get("program_plan")
+        if prog is not None and (ctx.all_single or plan is not None):
             from ..ops.hip_ops import _current_device, _raw_stream
             R = ctx.n_logit_rows
             out = logits_out
             if out is None and R:
                 out = torch.empty((R, self.vocab_size), dtype=torch.float32, device=self.rt.device)
-            plan_ptr = ctx.aux.get("program_plan")
-            if ctx.all_single or plan_ptr is not None:
-                stream = _raw_stream(_current_device())
-                capturing = torch.cuda.is_current_stream_capturing()
-                nbytes = max(prog.workspace.numel() if prog.workspace is not None else 0, self.program_workspace_bytes)
-                while True:
-                    if not capturing:
-                        prog.ensure_workspace(nbytes)
-                    if prog.run(ctx, out, plan_ptr, stream):
-                        self.program_steps += 1
-                        if out is None:
-                            return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.rt.device)
-                        return out
-                    if capturing or "too small" not in getattr(prog, "last_refusal", "") or nbytes >= (32 << 30):
-                        break
-                    nbytes *= 2
-                    self._static.clear()     # captured steps point into the workspace that is about to go
+            stream = _raw_stream(_current_device())
+            capturing = torch.cuda.is_current_stream_capturing()
+            while True:
+                if prog.run(ctx, out, plan, stream):
+                    self.program_steps += 1
+                    if out is None:
+                        return torch.empty((0, self.vocab_size), dtype=torch.float32, device=self.rt.device)
+                    return out
+                # a step larger than the workspace was sized for: a larger one (never while a step is captured, and
+                # what has been captured points into the one that goes)
+                if capturing or self.program_workspace_bytes >= (64 << 30):
+                    break
+                self.program_workspace_bytes *= 2
+                kept = [k for k, sb in self._static.items() if sb.graph is None]
+                for k in [k for k in self._static if k not in kept]:
+                    del self._static[k]
+                prog.ensure_workspace(self.program_workspace_bytes)
         if logits_out is not None:
             return self.model.forward(ctx, logits_out=logits_out)
         return self.model.forward(ctx)
@@ -199,7 +232,7 @@ class ModelExecutor:
             src_at, total = total, total + _pad4(n_all)
         # a step that the recorded program may run carries its attention plan behind that
         plan_at = plan_cap = 0
-        if self.program is not None and static is None and N != S and (N, R) not in self.program._refused:
+        if self.program is not None and static is None and N != S:
             plan_at, plan_cap = total, self.program.plan_capacity(N)
             total += plan_cap
         if self._pinned is None or self._pinned.numel() < total:
@@ -247,8 +280,9 @@ class ModelExecutor:
             for gi in range(G):
                 section("slots%d" % gi)[N:] = -1
                 section("tables%d" % gi)[N * widths[gi]:] = 0
+        plan_info = None
         if plan_cap:
-            used = self.program.write_plan(lens, starts, host_np[plan_at:plan_at + plan_cap], plan_cap)
+            used, plan_info = self.program.write_plan(lens, starts, host_np[plan_at:plan_at + plan_cap], plan_cap)
             total = plan_at + _pad4(max(used, 1))
             host = self._pinned[:total]
         # the copy is synchronous: the staging buffer is free again when the next step fills it
@@ -282,7 +316,8 @@ class ModelExecutor:
         groups = [GroupView(slots=view("slots%d" % gi),
                             block_tables=view("tables%d" % gi).view(S_all, widths[gi]),
                             page_size=mgr.groups[gi].page_size) for gi in range(G)]
-        aux = {"program_plan": dev.data_ptr() + 4 * plan_at} if plan_cap else {}
+        # (where the plan lies on the device and how it is laid out travel with the step, not with the program)
+        aux = {"program_plan": (dev.data_ptr() + 4 * plan_at, plan_info)} if plan_cap else {}
         return StepContext(
             aux=aux, n_tokens=n_all, n_segments=S_all, token_ids=view("token_ids"), positions=view("positions"),
             seg_of_token=view("seg_of"), seg_starts=view("seg_starts"), seg_first_pos=view("seg_first"),

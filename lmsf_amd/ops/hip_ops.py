@@ -10,6 +10,7 @@ from typing import Optional
 
 import torch
 
+from . import dispatch as D
 from . import library
 from .handles import DeferredLinear, PendingProduct, ScaledRows
 
@@ -57,22 +58,51 @@ class HipOps:
             raise library.KernelLibraryError(
                 "the kernels are built for gfx950 only; this device reports %r" % self.device_arch)
         self._bad_flag = None
+        # The switch points between the kernels live in one structure that the C++ side reads (csrc/dispatch.h says
+        # what each means); they are attributes of this object all the same (see __setattr__).
         self.use_library_gemm = True   # bfloat16 matrix products of many rows go to the BLAS library
-        self.prefill_attention_variant = 0   # 0: keys and values staged in LDS; 1: fetched by every wave for itself; 2: as 0 with a short window of the block table in LDS (for tests)
-        self.decode_attention_order = 0      # 0: chosen from the number of workgroups; 1: the tokens of a head start together; 2: the heads of a token
-        self.decode_attention_splits = 0     # 0: chosen from the batch and the context; n: at most n splits of the keys
-        self.fuse_norm_rows = 16             # with up to this many rows (beyond fuse_stream_rows) the products around a norm do its work (0: never)
-        self.fuse_stream_rows = 1            # with up to this many rows the residual addition and the norm run inside the products (0: never)
-        self.gemv_max_rows = 2               # products of up to this many rows stream W without the matrix cores (0: never)
-        self.skinny_variant = 0        # tiling of the few-rows kernel (0: default; others for tuning)
+        self.prefill_attention_variant = 0
+        self.decode_attention_order = 0
+        self.decode_attention_splits = 0
+        self.fuse_norm_rows = 16
+        self.fuse_stream_rows = 1
+        self.gemv_max_rows = 2
+        self.skinny_variant = 0
         self.mid_wide_max_cols = 8192  # beyond 64 rows only products of up to this many columns: the library is good at the wide ones (measured)
         self.mid_max_rows = 128        # rows up to which the 17-and-more-rows kernel beats the library (64 with the gated activation)
         self.skinny_max_rows = 16      # rows up to which the few-rows kernel beats the library (measured)
         self.large_max_rows = 256      # rows up to which the many-rows kernel beats the library (measured; 0: never)
-        self.weight_row_pad_bytes = 512  # bytes left between two rows of a linear layer's weight (see weight_row_pad)
         self.large_deep_min_rows = 64    # products whose K is at least three times N go to the many-rows kernel from beyond this many rows already (down at 128 rows: 42.8 -> 38.0 us; decode at batch 128: 6.63 -> 6.53 ms a step, at 96: 5.83 -> 5.74)
         self.mid_scaled_rows = 16        # rows up to which the gated product after a norm runs in the 17-and-more-rows kernel where that kernel's workgroups fit on the chip at once (0: never)
         self.large_deep_max_rows = 1024  # the same for products whose K is at least three times N (down: 57 against 76 us at 320 rows, 74 against 94 at 512, 102 against 108 at 768, level at 1,024)
+        self.weight_row_pad_bytes = 512  # bytes left between two rows of a linear layer's weight (see weight_row_pad)
+        # the BLAS library's products are called from C++ (csrc/blas.hip); its handle and workspace are made here
+        if self.lib.lmsf_blas_init(self.blas_workspace_bytes) != 0:
+            raise library.KernelLibraryError("the BLAS library cannot be used: " + library.last_error(self.lib))
+
+    blas_workspace_bytes = 128 << 20
+
+    def __setattr__(self, name, value):
+        if name in D.TUNABLE_NAMES:
+            setattr(self.__dict__.setdefault("_tun", D.Tunables()), name, int(value))
+        else:
+            object.__setattr__(self, name, value)
+
+    def __getattr__(self, name):
+        # (called only for names that are no ordinary attributes: the switch points)
+        if name in D.TUNABLE_NAMES and "_tun" in self.__dict__:
+            return int(getattr(self.__dict__["_tun"], name))
+        raise AttributeError(name)
+
+    def tunables(self) -> tuple:
+        """The switch points as they are now, in the order of ``dispatch.TUNABLE_NAMES``."""
+        return self._tun.as_tuple()
+
+    def _shape(self, x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype) -> D.ProductShape:
+        """What the C++ side wants to know of a product x weight^T before it names the kernel."""
+        return D.ProductShape(x.shape[0], weight.shape[0], x.shape[1], _code(x.dtype), _code(weight.dtype),
+                              _code(out_dtype), x.stride(0), weight.stride(0), 1 if x.data_ptr() % 16 == 0 else 0,
+                              1 if weight.data_ptr() % 16 == 0 else 0)
 
     # ------------------------------------------------------------------ helpers
 
@@ -188,9 +218,11 @@ class HipOps:
                 and residual.is_contiguous() and tuple(residual.shape) == branch.shape)
         prepares = (fits and defer_ok and out_dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
                     and weight.is_contiguous() and weight.shape == (N,))
-        one_or_two = fits and M <= min(self.fuse_stream_rows, self.gemv_max_rows) and self._gemv_ok(M, K)
+        rt = D.Route()
+        self.lib.lmsf_route_deferred_norm(ctypes.byref(self._tun), M, N, K, 1 if fits else 0, 1 if prepares else 0,
+                                          ctypes.byref(rt))
         operands = (_ptr(branch.x), branch.x.stride(0), _ptr(branch.weight), branch.weight.stride(0), _ptr(branch.bias))
-        if prepares and one_or_two and self._gemv_ok(M, N):
+        if rt.route == D.GEMV_ADD_NORM:
             # adds into the stream, leaves stream * w and its workgroups' sums of squares
             self._dev(branch.x, branch.weight, branch.bias, residual, weight)
             parts = self.lib.lmsf_gemv_partials(N)
@@ -200,7 +232,7 @@ class HipOps:
                                                     float(weight_offset), _ptr(xw), xw.stride(0), _ptr(sumsq), M, N, K,
                                                     self._stream()))
             return ScaledRows(xw, sumsq, parts, M, residual, weight, float(eps), float(weight_offset), out_dtype), None
-        if prepares and M <= min(self.fuse_norm_rows, self.skinny_max_rows, 16) and not one_or_two:
+        if rt.route == D.SKINNY_ADD_NORM:
             # the same from the few-rows kernel: sums of squares per 16 columns
             self._dev(branch.x, branch.weight, branch.bias, residual, weight)
             tiles = -(-N // 16)
@@ -210,7 +242,7 @@ class HipOps:
                                                            float(weight_offset), _ptr(xw), xw.stride(0), _ptr(sumsq), M,
                                                            N, K, self.skinny_variant, self._stream()))
             return ScaledRows(xw, sumsq, tiles, 16, residual, weight, float(eps), float(weight_offset), out_dtype), None
-        if one_or_two:
+        if rt.route == D.GEMV_ADD:
             # adds into the stream; the norm kernel follows
             self._dev(branch.x, branch.weight, branch.bias, residual)
             self._check(self.lib.lmsf_gemv_add(*operands, _ptr(residual), residual.stride(0), M, N, K, self._stream()))
@@ -317,48 +349,38 @@ class HipOps:
         be a ``ScaledRows``."""
         M, K = x.shape
         N = (nh + 2 * nkv) * d
-        if isinstance(x, ScaledRows):
-            if not (table is not None and slots is not None and neox and rot_dim == d and d % 32 == 0
-                    and weight.dtype == torch.bfloat16 and tuple(weight.shape) == (N, K) and weight.stride(1) == 1
-                    and self._skinny_ok(x.xw, weight) and k_pages is not None and k_pages.dtype == torch.bfloat16
-                    and (x.rows_per_tile == 16 or self._gemv_ok(M, K))):
-                return self.qkv_rope_cache(self.materialize(x), weight, bias, nh, nkv, d, positions, table, rot_dim,
-                                           neox, slots, k_pages, v_pages)
-            self._dev(x.xw, x.sumsq, weight, bias, positions, table, slots, k_pages, v_pages)
+        scaled = isinstance(x, ScaledRows)
+        xt = x.xw if scaled else x
+        fused_shape = (table is not None and slots is not None and neox and rot_dim == d and d % 32 == 0
+                       and weight.dtype == torch.bfloat16 and tuple(weight.shape) == (N, K) and xt.stride(1) == 1
+                       and weight.stride(1) == 1 and k_pages is not None and k_pages.dtype == torch.bfloat16)
+        rt = D.Route()
+        self.lib.lmsf_route_qkv(ctypes.byref(self._tun), ctypes.byref(self._shape(xt, weight, xt.dtype)),
+                                1 if fused_shape else 0, x.rows_per_tile if scaled else 0, ctypes.byref(rt))
+        if rt.route == D.MATERIALIZE:
+            return self.qkv_rope_cache(self.materialize(x), weight, bias, nh, nkv, d, positions, table, rot_dim,
+                                       neox, slots, k_pages, v_pages)
+        if rt.route != D.SEPARATE:
+            self._dev(xt, weight, bias, positions, table, slots, k_pages, v_pages)
             num_pages, ps = self._check_qkv_fused(bias, weight, N, table, d, positions, slots, M, k_pages, v_pages, nkv)
             y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
-            if x.rows_per_tile != 16:
-                self._check(self.lib.lmsf_gemv_scaled_qkv_rope_cache(
-                    _ptr(x.xw), x.xw.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(y), y.stride(0), M, K,
+            head = (_ptr(xt), xt.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(y), y.stride(0), M, K,
                     _ptr(positions), _ptr(table), table.shape[0], _ptr(slots), _ptr(k_pages), _ptr(v_pages), num_pages,
-                    nh, nkv, d, ps, _ptr(x.sumsq), x.tiles, x.eps, self._stream()))
-                return y
-            self._check(self.lib.lmsf_gemm_qkv_rope_cache_scaled(
-                _ptr(x.xw), x.xw.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(y), y.stride(0), M, K,
-                _ptr(positions), _ptr(table), table.shape[0], _ptr(slots), _ptr(k_pages), _ptr(v_pages), num_pages,
-                nh, nkv, d, ps, _ptr(x.sumsq), x.tiles, x.eps, self._stream()))
+                    nh, nkv, d, ps)
+            if rt.route == D.GEMV_SCALED:
+                self._dev(x.sumsq)
+                self._check(self.lib.lmsf_gemv_scaled_qkv_rope_cache(*head, _ptr(x.sumsq), x.tiles, x.eps, self._stream()))
+            elif rt.route == D.SKINNY_SCALED:
+                self._dev(x.sumsq)
+                self._check(self.lib.lmsf_gemm_qkv_rope_cache_scaled(*head, _ptr(x.sumsq), x.tiles, x.eps, self._stream()))
+            elif rt.route == D.GEMV:
+                self._check(self.lib.lmsf_gemv_qkv_rope_cache(*head, self._stream()))
+            else:
+                self._check(self.lib.lmsf_gemm_qkv_rope_cache(*head, self.skinny_variant, self._stream()))
             return y
-        if (table is not None and slots is not None and neox and rot_dim == d and d % 32 == 0
-                and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and 0 < M <= self.skinny_max_rows
-                and tuple(weight.shape) == (N, K) and x.stride(1) == 1 and weight.stride(1) == 1
-                and self._skinny_ok(x, weight) and k_pages is not None and k_pages.dtype == torch.bfloat16):
-            self._dev(x, weight, bias, positions, table, slots, k_pages, v_pages)
-            num_pages, ps = self._check_qkv_fused(bias, weight, N, table, d, positions, slots, M, k_pages, v_pages, nkv)
-            y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
-            if M <= self.gemv_max_rows and self._gemv_ok(M, K):
-                self._check(self.lib.lmsf_gemv_qkv_rope_cache(
-                    _ptr(x), x.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(y), y.stride(0), M, K,
-                    _ptr(positions), _ptr(table), table.shape[0], _ptr(slots), _ptr(k_pages), _ptr(v_pages), num_pages,
-                    nh, nkv, d, ps, self._stream()))
-                return y
-            self._check(self.lib.lmsf_gemm_qkv_rope_cache(
-                _ptr(x), x.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(y), y.stride(0), M, K,
-                _ptr(positions), _ptr(table), table.shape[0], _ptr(slots), _ptr(k_pages), _ptr(v_pages), num_pages,
-                nh, nkv, d, ps, self.skinny_variant, self._stream()))
-            return y
-        y = self.linear(x, weight, bias, pending_ok=M > max(self.fuse_stream_rows, self.fuse_norm_rows, self.skinny_max_rows))
+        y = self.linear(x, weight, bias, pending_ok=bool(rt.pending))
         if isinstance(y, PendingProduct):
-            # 17 to 64 rows with K split: the rotation and the cache write add up the partial sums themselves
+            # 17 and more rows with K split: the rotation and the cache write add up the partial sums themselves
             if (table is None and slots is None) or tuple(weight.shape) != (N, K):
                 return self.materialize(y)
             return self._rope_cache_write_pending(y, nh, nkv, d, positions, table, rot_dim, neox, slots, k_pages,
@@ -458,25 +480,10 @@ class HipOps:
                 _ptr(seg), _ptr(pos), nh, nkv, d, ps, float(scale), int(window or 0), self.prefill_attention_variant,
                 self._stream()))
         if plan.n_single:
-            n_hb = -(-(nh // nkv) // 16)
-            most = -(-plan.max_context // 128)
-            # Measured: about 512 workgroups fill the chip; beyond that a split only adds partial results,
-            # and with two short halves the reduction kernel costs more than the second half saves.
-            # With contexts of tens of thousands of keys twice as many do better (8 tokens of 100,000 keys: a step of
-            # 21.2 -> 19.2 ms, 16 of 50,000: 21.6 -> 18.9, 4 of 100,000: 12.3 -> 11.8; 8 and 32 of 32,000: the same),
-            # unless a single token's heads would be cut into more than 64 parts (one token of 120,000: 5.54 -> 5.64).
-            # From 49,152 keys on, four times as many, from 16 pairs of token and kv head on (2 tokens of 100,000 keys:
-            # 8.28 -> 7.33 ms; 4: 12.3 -> 11.9; 16 of 50,000: 18.9 either way).
-            pairs = plan.n_single * nkv * n_hb
-            fill = 2048 if plan.max_context >= 49152 and pairs >= 16 else \
-                1024 if plan.max_context >= 32768 and pairs >= 32 else 512
-            want = max(1, min(most, fill // (plan.n_single * nkv * n_hb)))
-            if want == 2 and plan.max_context <= 512:
-                want = 1
-            if self.decode_attention_splits:
-                want = min(most, self.decode_attention_splits)
-            chunk = -(-(-(-plan.max_context // want)) // 128) * 128
-            n_splits = -(-plan.max_context // chunk)
+            c_chunk, c_splits = ctypes.c_int(0), ctypes.c_int(0)
+            self.lib.lmsf_route_decode_attention(ctypes.byref(self._tun), plan.n_single, nh, nkv, plan.max_context,
+                                                 ctypes.byref(c_chunk), ctypes.byref(c_splits))
+            chunk, n_splits = c_chunk.value, c_splits.value
             floats = self.lib.lmsf_attention_decode_scratch_floats(plan.n_single, nh, d, n_splits)
             scratch = torch.empty(floats if n_splits > 1 else 1, dtype=torch.float32, device=q.device)
             self._check(self.lib.lmsf_paged_attention_decode_mfma(
@@ -593,12 +600,13 @@ class HipOps:
                out: Optional[torch.Tensor] = None):
         """y = x weight^T (+ bias); x [M, K], weight [N, K]; y [M, N] in ``out_dtype`` (default x's).
         With ``pending_ok`` the caller takes a ``PendingProduct`` as well, which comes back where the
-        product splits K over workgroups (17 to 64 rows, few columns). ``out``: a contiguous [M, N] tensor of
-        ``out_dtype`` that takes the result instead of a new one (not together with ``pending_ok``).
+        product splits K over workgroups, or a ``DeferredLinear`` (few rows). ``out``: a contiguous [M, N]
+        tensor of ``out_dtype`` that takes the result instead of a new one (not together with ``pending_ok``).
 
-        float32 operands always run the float32 multiply-add kernel. bfloat16 products with bfloat16
-        output and many rows go to the BLAS library, as the reference's do
-        (core/src/model_executor/layers/linear.rs:44-106 calls cuBLASLt); the rest run here.
+        Which kernel runs is decided by ``lmsf_route_linear`` (csrc/dispatch.hip), as for the step program:
+        float32 operands always run the float32 multiply-add kernel; bfloat16 products with bfloat16 output
+        and many rows go to the BLAS library, as the reference's do (core/src/model_executor/layers/linear.rs:44-106
+        calls cuBLASLt), through csrc/blas.hip; the rest run in this package's kernels.
         """
         self._dev(x, weight, bias)
         if x.dim() != 2 or weight.dim() != 2 or x.shape[1] != weight.shape[1]:
@@ -614,149 +622,101 @@ class HipOps:
             if pending_ok or tuple(out.shape) != (M, N) or out.dtype != out_dtype or not out.is_contiguous() \
                     or out.device != x.device:
                 raise ValueError("linear: out must be a contiguous [%d, %d] %s tensor on x's device" % (M, N, out_dtype))
-
-        def new():
-            return out if out is not None else torch.empty((M, N), dtype=out_dtype, device=x.device)
-
-        both_bf16 = x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
-        deep = K >= 3 * N and out_dtype == torch.bfloat16
-        if (both_bf16 and self.skinny_max_rows < M <= self.mid_max_rows and self._mid_ok(x, weight)
-                and (M <= 64 or N <= self.mid_wide_max_cols or out_dtype == torch.float32)
-                and not (deep and M > self.large_deep_min_rows)):
-            return self._linear_mid(x, weight, bias, 0, out_dtype, pending_ok and out_dtype == torch.bfloat16, out=out)
-        if (both_bf16 and out_dtype == torch.bfloat16 and self._mid_ok(x, weight)
-                and (self.mid_max_rows < M <= self.large_max_rows
-                     or (deep and self.large_deep_min_rows < M <= self.large_deep_max_rows))):
-            # 129 to 256 rows: the library is weak there (0.12 to 0.5 PFLOP/s at these widths)
-            return self._linear_large(x, weight, bias, 0, pending_ok, out=out)
-        if pending_ok and both_bf16 and out_dtype == torch.bfloat16 and self._skinny_ok(x, weight) and M > 0:
-            if (M <= min(self.fuse_stream_rows, self.gemv_max_rows) and self._gemv_ok(M, K)) \
-                    or M <= min(self.fuse_norm_rows, self.skinny_max_rows, 16):
-                return DeferredLinear(x, weight, bias, out_dtype)
-        if both_bf16 and 0 < M <= min(1, self.gemv_max_rows) and self._skinny_ok(x, weight) and self._gemv_ok(M, K) \
-                and N * K <= 2 ** 28:
-            # one row: a pure stream of W (with two rows only the fused forms gain; the LM head's matrix is large
-            # enough for the few-rows kernel to reach the same rate, so it stays there)
-            y = new()
+        rt = D.Route()
+        self.lib.lmsf_route_linear(ctypes.byref(self._tun), ctypes.byref(self._shape(x, weight, out_dtype)),
+                                   1 if pending_ok else 0, ctypes.byref(rt))
+        if rt.route == D.MID:
+            return self._linear_mid(x, weight, bias, 0, out_dtype, rt, out=out)
+        if rt.route == D.LARGE:
+            return self._linear_large(x, weight, bias, 0, bool(rt.pending), out=out, plan=rt.plan)
+        if rt.route == D.DEFERRED:
+            return DeferredLinear(x, weight, bias, out_dtype)
+        y = out if out is not None else torch.empty((M, N), dtype=out_dtype, device=x.device)
+        if rt.route == D.GEMV:
             self._check(self.lib.lmsf_gemv(_ptr(x), x.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(y),
                                            _code(out_dtype), y.stride(0), M, N, K, 0, self._stream()))
-            return y
-        if both_bf16 and out_dtype == torch.float32 and M > self.mid_max_rows and self._mid_ok(x, weight):
-            # float32 output (logits) for many rows, which the library does not offer: as many rows at a time
-            # as the kernel above takes
-            y = new()
-            for r0 in range(0, M, self.mid_max_rows):
-                rows = min(self.mid_max_rows, M - r0)
-                y[r0:r0 + rows] = self.linear(x[r0:r0 + rows], weight, bias, out_dtype=out_dtype)
-            return y
-        if both_bf16 and self._skinny_ok(x, weight):
-            # few rows: the weight-streaming kernel. It also serves float32 output where the kernels above
-            # do not take the operands, for any number of rows, 64 at a time.
-            limit = self.skinny_max_rows if out_dtype == torch.bfloat16 else 64
-            if M <= limit or out_dtype == torch.float32:
-                y = new()
-                for r0 in range(0, M, 64):
-                    rows = min(64, M - r0)
-                    xs, ys = x[r0:r0 + rows], y[r0:r0 + rows]
-                    self._check(self.lib.lmsf_gemm_skinny(
-                        _ptr(xs), xs.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(ys),
-                        _code(out_dtype), ys.stride(0), rows, N, K, self.skinny_variant, 0, self._stream()))
-                return y
-        if self.use_library_gemm and both_bf16 and M > self.skinny_max_rows and out_dtype == torch.bfloat16:
-            # (float32 output that no kernel above takes, a K that is no multiple of 8, goes to the plain kernel below:
-            # the library would round it to bfloat16 first)
-            y = torch.nn.functional.linear(x, weight, bias)
-            if out is not None:
-                return out.copy_(y)
-            return y
-        y = new()
-        self._check(self.lib.lmsf_gemm_plain(_ptr(x), _code(x.dtype), x.stride(0), _ptr(weight), _code(weight.dtype),
-                                             weight.stride(0), _ptr(bias), _ptr(y), _code(out_dtype), y.stride(0),
-                                             M, N, K, self._stream()))
+        elif rt.route == D.CHUNKS:
+            for r0 in range(0, M, rt.chunk_rows):
+                rows = min(rt.chunk_rows, M - r0)
+                self.linear(x[r0:r0 + rows], weight, bias, out_dtype=out_dtype, out=y[r0:r0 + rows])
+        elif rt.route == D.SKINNY:
+            for r0 in range(0, M, 64):
+                rows = min(64, M - r0)
+                xs, ys = x[r0:r0 + rows], y[r0:r0 + rows]
+                self._check(self.lib.lmsf_gemm_skinny(
+                    _ptr(xs), xs.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(ys),
+                    _code(out_dtype), ys.stride(0), rows, N, K, self.skinny_variant, 0, self._stream()))
+        elif rt.route == D.BLAS:
+            self._check(self.lib.lmsf_blas_linear(_ptr(x), x.stride(0), _ptr(weight), weight.stride(0), _ptr(bias),
+                                                  _ptr(y), y.stride(0), M, N, K, self._stream()))
+        else:
+            self._check(self.lib.lmsf_gemm_plain(_ptr(x), _code(x.dtype), x.stride(0), _ptr(weight),
+                                                 _code(weight.dtype), weight.stride(0), _ptr(bias), _ptr(y),
+                                                 _code(out_dtype), y.stride(0), M, N, K, self._stream()))
         return y
 
     def linear_gated(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
                      kind: str = "silu") -> torch.Tensor:
         """act(x Wg^T + bg) * (x Wu^T + bu) for the fused weight [2 I, K] = [Wg; Wu] (bias [2 I] likewise);
-        [M, I] in x's dtype. With up to 64 bfloat16 rows the activation is the epilogue of the weight-streaming
+        [M, I] in x's dtype. Where ``lmsf_route_linear_gated`` says so the activation is the epilogue of the
         product; otherwise the product and the activation kernel run one after the other. Both ways round
         the two products to the storage type before the activation, so they give the same bits wherever
         they add up K in the same order (the default tilings of the fused and the plain product do not: they
-        split K over 8 and over 16 waves)."""
+        split K over 8 and over 16 waves). ``x`` may be a ``ScaledRows``."""
         if weight.dim() != 2 or weight.shape[0] % 2 != 0:
             raise ValueError("linear_gated: weight must be [2 I, K]")
         kinds = {"silu": 1, "gelu": 2}
         if kind not in kinds:
             raise ValueError("unknown activation %r (known: %s)" % (kind, ", ".join(kinds)))
         M, I = x.shape[0], weight.shape[0] // 2
-        if isinstance(x, ScaledRows):
-            K = x.shape[1]
-            if not (weight.dtype == torch.bfloat16 and weight.shape[1] == K and weight.stride(1) == 1
-                    and self._skinny_ok(x.xw, weight) and (x.rows_per_tile == 16 or self._gemv_ok(M, K))):
-                return self.linear_gated(self.materialize(x), weight, bias, kind)
-            self._dev(x.xw, x.sumsq, weight, bias)
-            if bias is not None and (bias.shape != (2 * I,) or bias.dtype != weight.dtype or not bias.is_contiguous()):
-                raise ValueError("linear_gated: bias must be [%d] of the weight's dtype" % (2 * I))
-            y = torch.empty((M, I), dtype=torch.bfloat16, device=x.device)
-            if (x.rows_per_tile == 16 and M <= self.mid_scaled_rows and self._mid_ok(x.xw, weight)
-                    and self.lib.lmsf_gemm_mid_scaled_fits(M, I, K, x.tiles)):
-                self._check(self.lib.lmsf_gemm_mid_scaled(
-                    _ptr(x.xw), x.xw.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(y), y.stride(0), M, I, K,
-                    kinds[kind], _ptr(x.sumsq), x.tiles, x.eps, self._stream()))
-                return y
-            if x.rows_per_tile != 16:
-                self._check(self.lib.lmsf_gemv_scaled(
-                    _ptr(x.xw), x.xw.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(y), y.stride(0), M, I, K,
-                    kinds[kind], _ptr(x.sumsq), x.tiles, x.eps, self._stream()))
-                return y
-            self._check(self.lib.lmsf_gemm_skinny_scaled(
-                _ptr(x.xw), x.xw.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(y), y.stride(0), M, I, K,
-                kinds[kind], _ptr(x.sumsq), x.tiles, x.eps, self.skinny_variant, self._stream()))
-            return y
-        if (x.dim() == 2 and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and 0 < M <= self.skinny_max_rows
-                and x.shape[1] == weight.shape[1] and x.stride(1) == 1 and weight.stride(1) == 1
-                and self._skinny_ok(x, weight)):
-            self._dev(x, weight, bias)
-            if bias is not None and (bias.shape != (2 * I,) or bias.dtype != weight.dtype or not bias.is_contiguous()):
-                raise ValueError("linear_gated: bias must be [%d] of the weight's dtype" % (2 * I))
-            y = torch.empty((M, I), dtype=x.dtype, device=x.device)
-            if M <= self.gemv_max_rows and self._gemv_ok(M, x.shape[1]):
-                self._check(self.lib.lmsf_gemv(_ptr(x), x.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(y),
-                                               BF16, y.stride(0), M, I, x.shape[1], kinds[kind], self._stream()))
-                return y
-            self._check(self.lib.lmsf_gemm_skinny(
-                _ptr(x), x.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(y), BF16, y.stride(0), M, I,
-                x.shape[1], self.skinny_variant, kinds[kind], self._stream()))
-            return y
-        if (x.dim() == 2 and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
-                and self.skinny_max_rows < M <= 64 and x.shape[1] == weight.shape[1] and self._mid_ok(x, weight)):
-            return self._linear_mid(x, weight, bias, kinds[kind])
-        if (x.dim() == 2 and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16
-                and 64 < M <= self.large_max_rows and x.shape[1] == weight.shape[1] and self._mid_ok(x, weight)
-                and I % 8 == 0):    # (that kernel writes its outputs eight at a time)
-            return self._linear_large(x, weight, bias, kinds[kind])
-        return self.gated_act(self.linear(x, weight, bias), kind)
-
-    @staticmethod
-    def _mid_ok(x: torch.Tensor, weight: torch.Tensor) -> bool:
-        """What the kernel for 17 to 64 rows asks: K a multiple of 64, N of 4, unit column strides, row strides
-        that are multiples of 8, 16-byte bases."""
-        K = x.shape[1]
-        return (K % 64 == 0 and weight.shape[0] % 8 == 0 and x.stride(1) == 1 and weight.stride(1) == 1
-                and x.stride(0) % 8 == 0 and weight.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
-                and weight.data_ptr() % 16 == 0)
+        scaled = isinstance(x, ScaledRows)
+        xt = x.xw if scaled else x
+        if xt.dim() != 2 or xt.shape[1] != weight.shape[1] or xt.stride(1) != 1 or weight.stride(1) != 1:
+            raise ValueError("linear_gated: x %s and weight %s do not match" % (tuple(xt.shape), tuple(weight.shape)))
+        K = xt.shape[1]
+        rt = D.Route()
+        self.lib.lmsf_route_linear_gated(ctypes.byref(self._tun), ctypes.byref(self._shape(xt, weight, xt.dtype)),
+                                         x.rows_per_tile if scaled else 0, x.tiles if scaled else 0, ctypes.byref(rt))
+        if rt.route == D.MATERIALIZE:
+            return self.linear_gated(self.materialize(x), weight, bias, kind)
+        if rt.route == D.SEPARATE:
+            return self.gated_act(self.linear(x, weight, bias), kind)
+        self._dev(xt, weight, bias)
+        if bias is not None and (bias.shape != (2 * I,) or bias.dtype != weight.dtype or not bias.is_contiguous()):
+            raise ValueError("linear_gated: bias must be [%d] of the weight's dtype" % (2 * I))
+        if rt.route == D.MID:
+            return self._linear_mid(x, weight, bias, kinds[kind], torch.bfloat16, rt)
+        if rt.route == D.LARGE:
+            return self._linear_large(x, weight, bias, kinds[kind], plan=rt.plan)
+        y = torch.empty((M, I), dtype=torch.bfloat16, device=x.device)
+        head = (_ptr(xt), xt.stride(0), _ptr(weight), weight.stride(0), _ptr(bias), _ptr(y))
+        if rt.route == D.MID_SCALED:
+            self._check(self.lib.lmsf_gemm_mid_scaled(*head, y.stride(0), M, I, K, kinds[kind], _ptr(x.sumsq), x.tiles,
+                                                      x.eps, self._stream()))
+        elif rt.route == D.GEMV_SCALED:
+            self._check(self.lib.lmsf_gemv_scaled(*head, y.stride(0), M, I, K, kinds[kind], _ptr(x.sumsq), x.tiles,
+                                                  x.eps, self._stream()))
+        elif rt.route == D.SKINNY_SCALED:
+            self._check(self.lib.lmsf_gemm_skinny_scaled(*head, y.stride(0), M, I, K, kinds[kind], _ptr(x.sumsq),
+                                                         x.tiles, x.eps, self.skinny_variant, self._stream()))
+        elif rt.route == D.GEMV:
+            self._check(self.lib.lmsf_gemv(*head, BF16, y.stride(0), M, I, K, kinds[kind], self._stream()))
+        else:
+            self._check(self.lib.lmsf_gemm_skinny(*head, BF16, y.stride(0), M, I, K, self.skinny_variant, kinds[kind],
+                                                  self._stream()))
+        return y
 
     def _linear_mid(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], act: int,
-                    out_dtype: torch.dtype = torch.bfloat16, pending_ok: bool = False,
-                    out: Optional[torch.Tensor] = None):
+                    out_dtype: torch.dtype, rt: D.Route, out: Optional[torch.Tensor] = None):
+        """The 17-and-more-rows product (csrc/gemm_mid.hip) as ``rt`` says."""
         self._dev(x, weight, bias)
         M, K = x.shape
         N = weight.shape[0] // 2 if act else weight.shape[0]
         if bias is not None and (bias.shape != (weight.shape[0],) or bias.dtype != weight.dtype
                                  or not bias.is_contiguous()):
             raise ValueError("linear: bias must be [%d] of the weight's dtype" % weight.shape[0])
-        splits = self.lib.lmsf_gemm_mid_splits(M, N, K, act)
-        if pending_ok and act == 0 and splits > 1:
+        splits = rt.splits
+        if rt.pending:
             partials = torch.empty((splits, M, N), dtype=torch.float32, device=x.device)
             self._check(self.lib.lmsf_gemm_mid_partial(_ptr(x), x.stride(0), _ptr(weight), weight.stride(0), M, N, K,
                                                        splits, _ptr(partials), self._stream()))
@@ -771,7 +731,8 @@ class HipOps:
 
     def _linear_large(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], act: int,
                       pending_ok: bool = False, out: Optional[torch.Tensor] = None, plan: Optional[int] = None):
-        """The many-rows product (csrc/gemm_large.hip); operands as ``_mid_ok`` asks them."""
+        """The many-rows product (csrc/gemm_large.hip); K a multiple of 64, W's rows of 8, row strides of 8,
+        16-byte aligned bases. ``plan``: tiling and split (``lmsf_gemm_large_plan`` proposes one)."""
         self._dev(x, weight, bias)
         M, K = x.shape
         N = weight.shape[0] // 2 if act else weight.shape[0]
@@ -793,17 +754,25 @@ class HipOps:
                                              y.stride(0), M, N, K, act, plan, _ptr(scratch), 1, self._stream()))
         return y
 
-    @staticmethod
-    def _gemv_ok(M: int, K: int) -> bool:
-        """The one-or-two-rows kernel keeps x in LDS."""
-        return M * K * 2 <= 128 * 1024
-
-    @staticmethod
-    def _skinny_ok(x: torch.Tensor, weight: torch.Tensor) -> bool:
-        """What the few-rows kernel asks of its operands: K and the row strides multiples of 8, 16-byte bases."""
-        K = x.shape[1]
-        return (K % 8 == 0 and x.stride(0) % 8 == 0 and weight.stride(0) % 8 == 0
-                and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
+    def tune_products(self, x: torch.Tensor, weights, bias: Optional[torch.Tensor] = None, candidates: int = 16,
+                      reps: int = 5):
+        """Lets the BLAS library's candidates for the product of ``x`` [M, K] with matrices like ``weights`` (a list of
+        [N, K] tensors of one shape and row distance: the same product of several layers, so that no run finds its
+        weights in cache) race, and keeps the fastest for later products of that shape
+        (tops/src/cublas.rs:121-223 profiles cuBLASLt's tactics likewise). Returns (first choice's us, fastest's us)."""
+        w0 = weights[0]
+        self._dev(x, bias, *weights)
+        if any(w.shape != w0.shape or w.stride(0) != w0.stride(0) or w.dtype != torch.bfloat16 or w.stride(1) != 1
+               for w in weights) or x.dtype != torch.bfloat16 or x.shape[1] != w0.shape[1] or x.stride(1) != 1:
+            raise ValueError("tune_products: bfloat16 operands of one shape are needed")
+        M, K = x.shape
+        N = w0.shape[0]
+        y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+        ptrs = (ctypes.c_void_p * len(weights))(*[w.data_ptr() for w in weights])
+        times = (ctypes.c_float * 2)()
+        self._check(self.lib.lmsf_blas_tune(_ptr(x), x.stride(0), ptrs, len(weights), w0.stride(0), _ptr(bias), _ptr(y),
+                                            y.stride(0), M, N, K, int(candidates), int(reps), times, self._stream()))
+        return float(times[0]), float(times[1])
 
     # ------------------------------------------------------------------ sampling
 

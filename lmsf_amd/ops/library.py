@@ -4,12 +4,13 @@ There is no fallback: if the library cannot be built or loaded, or reports anoth
 version, importing the kernels fails with the reason.
 """
 import ctypes
-from ctypes import c_char_p, c_double, c_float, c_int, c_long, c_void_p
+from ctypes import POINTER, c_char_p, c_double, c_float, c_int, c_long, c_void_p
 from typing import Optional
 
 from ..csrc import build as _build
+from .dispatch import ProductShape, Route, Tunables
 
-ABI_VERSION = 21
+ABI_VERSION = 22
 
 _lib: Optional[ctypes.CDLL] = None
 _lib_path: Optional[str] = None
@@ -81,6 +82,17 @@ _SIGNATURES = {
     "lmsf_measure_copy": (c_int, [_P, _P, c_long, _P]),
     "lmsf_measure_mfma": (c_double, [_P, c_int, c_int, _P]),
     "lmsf_apply_penalties": (c_int, [_P, c_long, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, _P]),
+    "lmsf_blas_init": (c_int, [c_long]),
+    "lmsf_blas_ready": (c_int, []),
+    "lmsf_blas_linear": (c_int, [_P, c_long, _P, c_long, _P, _P, c_long, c_int, c_int, c_int, _P]),
+    "lmsf_blas_tune": (c_int, [_P, c_long, _P, c_int, c_long, _P, _P, c_long, c_int, c_int, c_int, c_int, c_int, _P, _P]),
+    "lmsf_blas_plans": (c_long, []),
+    "lmsf_route_linear": (None, [POINTER(Tunables), POINTER(ProductShape), c_int, POINTER(Route)]),
+    "lmsf_route_linear_gated": (None, [POINTER(Tunables), POINTER(ProductShape), c_int, c_int, POINTER(Route)]),
+    "lmsf_route_qkv": (None, [POINTER(Tunables), POINTER(ProductShape), c_int, c_int, POINTER(Route)]),
+    "lmsf_route_deferred_norm": (None, [POINTER(Tunables), c_int, c_int, c_int, c_int, c_int, POINTER(Route)]),
+    "lmsf_route_decode_attention": (None, [POINTER(Tunables), c_int, c_int, c_int, c_int, POINTER(c_int),
+                                           POINTER(c_int)]),
 }
 
 
