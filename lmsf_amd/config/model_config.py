@@ -2,51 +2,53 @@
 
 The reference parses config.json into a serde struct per architecture
 (core/src/model_executor/models/llama/config.rs:6-27) behind an accessor trait
-(core/src/model_executor/models/model.rs:8-37). Here a configuration is a frozen
-dataclass with explicit defaults and validation; every size and constant that the model
-code uses comes from one of its fields.
+(core/src/model_executor/models/model.rs:8-37). Here the struct, its defaults and its validation are
+C++ (csrc/host/llama_config.{h,cc}: one message per fault, naming the key); ``LlamaConfig`` and
+``RopeScaling`` below are its face, frozen dataclasses whose fields are what the C++ side read. Every
+size and constant that the model code uses comes from one of these fields.
 """
+import ctypes
 import dataclasses
 import json
 import os
+from ctypes import Structure, c_char, c_double, c_int, c_int64
 from dataclasses import dataclass
 from typing import Any, Dict, Optional, Tuple
+
+MAX_EOS_IDS = 16
+
+
+class _NativeRopeScaling(Structure):
+    _fields_ = [("present", c_int), ("rope_type", c_char * 16), ("factor", c_double), ("low_freq_factor", c_double),
+                ("high_freq_factor", c_double), ("original_max_position_embeddings", c_int64)]
+
+
+class _NativeLlamaConfig(Structure):
+    _fields_ = ([(n, c_int64) for n in ("vocab_size", "max_position_embeddings", "hidden_size", "intermediate_size",
+                                        "num_hidden_layers", "num_attention_heads", "num_key_value_heads", "head_dim")]
+                + [("rms_norm_eps", c_double), ("rope_theta", c_double), ("rope_scaling", _NativeRopeScaling)]
+                + [(n, c_int) for n in ("tie_word_embeddings", "attention_bias", "mlp_bias")]
+                + [("hidden_act", c_char * 32), ("torch_dtype", c_char * 16), ("has_bos_token_id", c_int),
+                   ("bos_token_id", c_int64), ("n_eos_token_ids", c_int), ("eos_token_ids", c_int64 * MAX_EOS_IDS)])
+
+
+def _native(call: str, *args) -> None:
+    """Calls the host library's ``call``; a refusal becomes a ConfigError with the library's message."""
+    from ..host.library import last_error, load_host_library
+    lib = load_host_library()
+    if getattr(lib, call)(*args) != 0:
+        raise ConfigError(last_error(lib))
+
+
+def _as_json(d: Any, what: str) -> bytes:
+    try:
+        return json.dumps(d, allow_nan=False).encode()
+    except (TypeError, ValueError) as e:
+        raise ConfigError("%s cannot be written as JSON: %s" % (what, e))
 
 
 class ConfigError(ValueError):
     """A config.json that cannot be used; the message names the key."""
-
-
-_MISSING = object()
-
-
-def _take(d: Dict[str, Any], key: str, kind, default=_MISSING):
-    """d[key] converted to ``kind``; a missing key without default is an error."""
-    if key not in d or d[key] is None:
-        if default is _MISSING:
-            raise ConfigError("config.json: required key '%s' is missing" % key)
-        return default
-    v = d[key]
-    try:
-        if kind is bool:
-            if not isinstance(v, bool):
-                raise TypeError
-            return v
-        if kind is int:
-            if isinstance(v, bool) or (isinstance(v, float) and v != int(v)):
-                raise TypeError
-            return int(v)
-        if kind is float:
-            if isinstance(v, bool):
-                raise TypeError
-            return float(v)
-        if kind is str:
-            if not isinstance(v, str):
-                raise TypeError
-            return v
-    except (TypeError, ValueError):
-        raise ConfigError("config.json: key '%s' has value %r, expected %s" % (key, v, kind.__name__))
-    raise AssertionError(kind)
 
 
 @dataclass(frozen=True)
@@ -60,32 +62,20 @@ class RopeScaling:
     high_freq_factor: float = 4.0
     original_max_position_embeddings: int = 8192
 
-    KNOWN_TYPES = ("default", "llama3")
-
     @classmethod
     def from_dict(cls, d: Optional[Dict[str, Any]]) -> Optional["RopeScaling"]:
         if d is None:
             return None
-        if not isinstance(d, dict):
-            raise ConfigError("config.json: 'rope_scaling' must be an object or null, got %r" % (d,))
-        kind = d.get("rope_type", d.get("type", "default"))
-        if kind not in cls.KNOWN_TYPES:
-            raise ConfigError("config.json: rope_scaling.rope_type %r is not supported (known: %s)"
-                              % (kind, ", ".join(cls.KNOWN_TYPES)))
-        if kind == "default":
-            return cls()
-        rs = cls(
-            rope_type=kind,
-            factor=_take(d, "factor", float),
-            low_freq_factor=_take(d, "low_freq_factor", float),
-            high_freq_factor=_take(d, "high_freq_factor", float),
-            original_max_position_embeddings=_take(d, "original_max_position_embeddings", int),
-        )
-        if rs.factor <= 0 or rs.original_max_position_embeddings <= 0:
-            raise ConfigError("config.json: rope_scaling factor and original_max_position_embeddings must be > 0")
-        if rs.high_freq_factor <= rs.low_freq_factor:
-            raise ConfigError("config.json: rope_scaling.high_freq_factor must exceed low_freq_factor")
-        return rs
+        native = _NativeRopeScaling()
+        _native("lmsf_rope_scaling_parse", _as_json(d, "rope_scaling"), ctypes.byref(native))
+        return cls._from_native(native) or cls()
+
+    @classmethod
+    def _from_native(cls, n: _NativeRopeScaling) -> Optional["RopeScaling"]:
+        if not n.present:
+            return None
+        return cls(n.rope_type.decode(), n.factor, n.low_freq_factor, n.high_freq_factor,
+                   int(n.original_max_position_embeddings))
 
     def to_dict(self) -> Dict[str, Any]:
         if self.rope_type == "default":
@@ -97,9 +87,6 @@ class RopeScaling:
             "high_freq_factor": self.high_freq_factor,
             "original_max_position_embeddings": self.original_max_position_embeddings,
         }
-
-
-_TORCH_DTYPES = ("float32", "bfloat16", "float16", "half", "float")
 
 
 @dataclass(frozen=True)
@@ -150,72 +137,63 @@ class LlamaConfig(ArchConfig):
 
     @classmethod
     def from_dict(cls, d: Dict[str, Any]) -> "LlamaConfig":
-        hidden = _take(d, "hidden_size", int)
-        heads = _take(d, "num_attention_heads", int)
-        if heads <= 0:
-            raise ConfigError("config.json: num_attention_heads must be > 0")
-        head_dim = _take(d, "head_dim", int, None)
-        if head_dim is None:
-            if hidden % heads != 0:
-                raise ConfigError("config.json: hidden_size %d is not a multiple of num_attention_heads %d "
-                                  "and no head_dim is given" % (hidden, heads))
-            head_dim = hidden // heads
-        eos = d.get("eos_token_id")
-        if eos is None:
-            eos_ids: Tuple[int, ...] = ()
-        elif isinstance(eos, list):
-            eos_ids = tuple(int(e) for e in eos)
-        else:
-            eos_ids = (int(eos),)
-        dtype = _take(d, "torch_dtype", str, _take(d, "dtype", str, "bfloat16"))
-        cfg = cls(
+        """Parsed, completed with defaults and validated by the host library."""
+        n = _NativeLlamaConfig()
+        _native("lmsf_llama_config_parse", _as_json(d, "the configuration"), ctypes.byref(n))
+        return cls(
             architecture=cls.ARCHITECTURE,
-            vocab_size=_take(d, "vocab_size", int),
-            max_position_embeddings=_take(d, "max_position_embeddings", int),
-            torch_dtype=dtype,
-            eos_token_ids=eos_ids,
-            bos_token_id=_take(d, "bos_token_id", int, None),
-            hidden_size=hidden,
-            intermediate_size=_take(d, "intermediate_size", int),
-            num_hidden_layers=_take(d, "num_hidden_layers", int),
-            num_attention_heads=heads,
-            num_key_value_heads=_take(d, "num_key_value_heads", int, heads),
-            head_dim=head_dim,
-            rms_norm_eps=_take(d, "rms_norm_eps", float),
-            rope_theta=_take(d, "rope_theta", float, 10000.0),
-            rope_scaling=RopeScaling.from_dict(d.get("rope_scaling")),
-            tie_word_embeddings=_take(d, "tie_word_embeddings", bool, False),
-            attention_bias=_take(d, "attention_bias", bool, False),
-            mlp_bias=_take(d, "mlp_bias", bool, False),
-            hidden_act=_take(d, "hidden_act", str, "silu"),
+            vocab_size=int(n.vocab_size),
+            max_position_embeddings=int(n.max_position_embeddings),
+            torch_dtype=n.torch_dtype.decode(),
+            eos_token_ids=tuple(int(n.eos_token_ids[i]) for i in range(n.n_eos_token_ids)),
+            bos_token_id=int(n.bos_token_id) if n.has_bos_token_id else None,
+            hidden_size=int(n.hidden_size),
+            intermediate_size=int(n.intermediate_size),
+            num_hidden_layers=int(n.num_hidden_layers),
+            num_attention_heads=int(n.num_attention_heads),
+            num_key_value_heads=int(n.num_key_value_heads),
+            head_dim=int(n.head_dim),
+            rms_norm_eps=n.rms_norm_eps,
+            rope_theta=n.rope_theta,
+            rope_scaling=RopeScaling._from_native(n.rope_scaling),
+            tie_word_embeddings=bool(n.tie_word_embeddings),
+            attention_bias=bool(n.attention_bias),
+            mlp_bias=bool(n.mlp_bias),
+            hidden_act=n.hidden_act.decode(),
         )
-        cfg.validate()
-        return cfg
+
+    def _to_native(self) -> _NativeLlamaConfig:
+        n = _NativeLlamaConfig()
+        for name in ("vocab_size", "max_position_embeddings", "hidden_size", "intermediate_size", "num_hidden_layers",
+                     "num_attention_heads", "num_key_value_heads", "head_dim", "rms_norm_eps", "rope_theta"):
+            setattr(n, name, getattr(self, name))
+        for name in ("tie_word_embeddings", "attention_bias", "mlp_bias"):
+            setattr(n, name, 1 if getattr(self, name) else 0)
+        for name, cap in (("hidden_act", 32), ("torch_dtype", 16)):
+            text = str(getattr(self, name)).encode()
+            if len(text) >= cap:
+                raise ConfigError("config.json: %s %r is too long" % (name, getattr(self, name)))
+            setattr(n, name, text)
+        if self.bos_token_id is not None:
+            n.has_bos_token_id, n.bos_token_id = 1, self.bos_token_id
+        if len(self.eos_token_ids) > MAX_EOS_IDS:
+            raise ConfigError("config.json: eos_token_id lists %d ids, at most %d are taken"
+                              % (len(self.eos_token_ids), MAX_EOS_IDS))
+        n.n_eos_token_ids = len(self.eos_token_ids)
+        for i, e in enumerate(self.eos_token_ids):
+            n.eos_token_ids[i] = e
+        rs = self.rope_scaling
+        if rs is not None and rs.rope_type != "default":
+            n.rope_scaling.present = 1
+            n.rope_scaling.rope_type = rs.rope_type.encode()
+            n.rope_scaling.factor, n.rope_scaling.low_freq_factor = rs.factor, rs.low_freq_factor
+            n.rope_scaling.high_freq_factor = rs.high_freq_factor
+            n.rope_scaling.original_max_position_embeddings = rs.original_max_position_embeddings
+        return n
 
     def validate(self) -> None:
-        for name in ("vocab_size", "hidden_size", "intermediate_size", "num_hidden_layers",
-                     "num_attention_heads", "num_key_value_heads", "head_dim",
-                     "max_position_embeddings"):
-            if getattr(self, name) <= 0:
-                raise ConfigError("config.json: %s must be > 0, got %r" % (name, getattr(self, name)))
-        if self.num_attention_heads % self.num_key_value_heads != 0:
-            raise ConfigError("config.json: num_attention_heads %d is not a multiple of num_key_value_heads %d"
-                              % (self.num_attention_heads, self.num_key_value_heads))
-        if self.head_dim % 2 != 0:
-            raise ConfigError("config.json: head_dim %d must be even for rotary embedding" % self.head_dim)
-        if not (self.rms_norm_eps > 0):
-            raise ConfigError("config.json: rms_norm_eps must be > 0")
-        if not (self.rope_theta > 0):
-            raise ConfigError("config.json: rope_theta must be > 0")
-        if self.hidden_act != "silu":
-            raise ConfigError("config.json: hidden_act %r is not supported by LlamaForCausalLM (silu)"
-                              % self.hidden_act)
-        if self.torch_dtype not in _TORCH_DTYPES:
-            raise ConfigError("config.json: torch_dtype %r is not one of %s"
-                              % (self.torch_dtype, ", ".join(_TORCH_DTYPES)))
-        for e in self.eos_token_ids:
-            if not (0 <= e < self.vocab_size):
-                raise ConfigError("config.json: eos_token_id %d outside vocabulary of %d" % (e, self.vocab_size))
+        """The host library's checks on the fields as they are (after ``replace``)."""
+        _native("lmsf_llama_config_validate", ctypes.byref(self._to_native()))
 
     def to_dict(self) -> Dict[str, Any]:
         d: Dict[str, Any] = {

@@ -6,9 +6,16 @@
 #include <string>
 
 #include "cache_manager.h"
+#include "llama_config.h"
 #include "scheduler.h"
 
 using namespace lmsf;
+
+namespace lmsf {
+void llama_config_parse(const std::string& text, LmsfLlamaConfig* out);
+void llama_config_validate(const LmsfLlamaConfig& c);
+void rope_scaling_parse(const std::string& text, LmsfRopeScaling* out);
+}  // namespace lmsf
 
 static thread_local std::string g_error;
 
@@ -27,7 +34,7 @@ static thread_local std::string g_error;
 
 extern "C" {
 
-int lmsf_host_abi_version() { return 2; }
+int lmsf_host_abi_version() { return 3; }
 const char* lmsf_host_last_error() { return g_error.c_str(); }
 
 // ---------------------------------------------------------------- a page pool alone
@@ -305,5 +312,26 @@ int lmsf_sched_queue(void* s, int which, int64_t* out, int cap, int* count) {
   LMSF_API_END
 }
 int64_t lmsf_sched_num_preemptions(void* s) { return static_cast<Scheduler*>(s)->num_preemptions(); }
+
+// ---------------------------------------------------------------- configuration
+
+int lmsf_llama_config_parse(const char* config_json, LmsfLlamaConfig* out) {
+  LMSF_API_BEGIN
+  if (!config_json || !out) fail(kValueError, "bad arguments");
+  llama_config_parse(config_json, out);
+  LMSF_API_END
+}
+int lmsf_llama_config_validate(const LmsfLlamaConfig* config) {
+  LMSF_API_BEGIN
+  if (!config) fail(kValueError, "bad arguments");
+  llama_config_validate(*config);
+  LMSF_API_END
+}
+int lmsf_rope_scaling_parse(const char* rope_scaling_json, LmsfRopeScaling* out) {
+  LMSF_API_BEGIN
+  if (!rope_scaling_json || !out) fail(kValueError, "bad arguments");
+  rope_scaling_parse(rope_scaling_json, out);
+  LMSF_API_END
+}
 
 }  // extern "C"

@@ -55,7 +55,7 @@ def _default_ops():
 
 
 def build_model(arch: Architecture, config: ArchConfig, rt: Runtime, model_dir: Optional[str],
-                load_format: str = "auto", seed: int = 0) -> DecoderModel:
+                load_format: str = "auto", seed: int = 0, keep_float32_weights: bool = False) -> DecoderModel:
     model = DecoderModel(arch.build_spec(config), rt)
     if load_format == "random":
         std = 0.02
@@ -66,7 +66,8 @@ def build_model(arch: Architecture, config: ArchConfig, rt: Runtime, model_dir: 
     elif load_format == "auto":
         if model_dir is None:
             raise ValueError("a model folder is needed unless load_format is 'random'")
-        load_weights(model.parts(), model_dir, rt.device, rt.dtype, tolerated=arch.tolerated_tensors)
+        load_weights(model.parts(), model_dir, rt.device, rt.dtype, tolerated=arch.tolerated_tensors,
+                     keep_float32=keep_float32_weights)
     else:
         raise ValueError("load_format %r unknown (auto, random)" % load_format)
     return model
@@ -125,8 +126,9 @@ def load_engine_core(model_dir: Optional[str], dtype: Optional[str] = None, bloc
                      max_num_batched_tokens: Optional[int] = None, device: str = "cuda:0",
                      ops: Any = None, load_format: str = "auto", seed: int = 0,
                      config: Optional[ArchConfig] = None, enforce_eager: bool = False,
-                     use_program: bool = True) -> EngineCore:
-    """``num_pages``: pages of every cache group (tests, replay); None sizes the pools from free memory."""
+                     use_program: bool = True, keep_float32_weights: bool = False) -> EngineCore:
+    """``num_pages``: pages of every cache group (tests, replay); None sizes the pools from free memory.
+    ``keep_float32_weights``: matrices stored in 32 bits stay so in a bfloat16 run instead of being cast."""
     if config is None:
         if model_dir is None:
             raise ValueError("need a model folder or a configuration")
@@ -149,7 +151,7 @@ def load_engine_core(model_dir: Optional[str], dtype: Optional[str] = None, bloc
     if ops is None:
         ops = _default_ops()
     rt = Runtime(ops=ops, device=dev, dtype=run_dtype, max_positions=max_model_len)
-    model = build_model(arch, config, rt, model_dir, load_format, seed)
+    model = build_model(arch, config, rt, model_dir, load_format, seed, keep_float32_weights)
     groups, _ = plan_groups(model.cache_requirements(), block_size)
     if max_num_batched_tokens is None:
         max_num_batched_tokens = max(max_model_len, 2048)   # config.rs:301-307

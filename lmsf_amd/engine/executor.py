@@ -156,6 +156,31 @@ class ModelExecutor:
             return self.model.forward(ctx, logits_out=logits_out)
         return self.model.forward(ctx)
 
+    def tune_products(self, rows: Sequence[int], candidates: int = 16, reps: int = 5) -> dict:
+        """For steps of these numbers of tokens, lets the BLAS library's candidates race for every shape of matrix
+        product the model has and keeps the winners (``HipOps.tune_products``; tops/src/cublas.rs:121-223 profiles
+        cuBLASLt's tactics per weight shape and bucket of rows likewise). Only products that go to the library at
+        that many rows are looked at. Returns {(rows, N, K): (first choice's us, fastest's us)}."""
+        from ..ops import dispatch as D
+        from ..parts.linear import FusedLinear
+        import ctypes
+        ops = self.rt.ops
+        shapes = {}
+        for p in self.model.parts():
+            w = getattr(p, "weight", None)
+            if isinstance(p, FusedLinear) and w is not None and w.dtype == torch.bfloat16 and w.is_cuda:
+                shapes.setdefault((w.shape[0], w.shape[1], w.stride(0), p.bias is not None), []).append(p)
+        found = {}
+        for M in sorted(set(int(m) for m in rows)):
+            for (N, K, ld, has_bias), parts in shapes.items():
+                x = torch.randn((M, K), device=self.rt.device, dtype=torch.float32).to(torch.bfloat16)
+                rt = D.Route()
+                ops.lib.lmsf_route_linear(ctypes.byref(ops._tun), ctypes.byref(ops._shape(x, parts[0].weight, x.dtype)),
+                                          0, ctypes.byref(rt))
+                if rt.route == D.BLAS:
+                    found[(M, N, K)] = ops.tune_products(x, [p.weight for p in parts], parts[0].bias, candidates, reps)
+        return found
+
     def release(self, request_id: Hashable) -> None:
         """The request is finished: its pages and state slot go back."""
         if self.manager.has_request(request_id):

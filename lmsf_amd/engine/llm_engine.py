@@ -56,7 +56,8 @@ class LLMEngine:
             args.model or None, dtype=args.dtype, block_size=args.block_size, max_model_len=args.max_model_len,
             num_pages=args.num_gpu_blocks_override, gpu_memory_utilization=args.gpu_memory_utilization,
             max_num_seqs=args.max_num_seqs, max_num_batched_tokens=args.max_num_batched_tokens, device=args.device,
-            ops=ops, load_format=args.load_format, seed=args.seed, enforce_eager=args.enforce_eager)
+            ops=ops, load_format=args.load_format, seed=args.seed, enforce_eager=args.enforce_eager,
+            keep_float32_weights=args.keep_float32_weights)
         max_len = self.core.max_model_len
         budget = args.max_num_batched_tokens or max(max_len, 2048)      # core/src/common/config.rs:301-307
         self.scheduler = Scheduler(SchedulerConfig(budget, args.max_num_seqs, max_len, args.prefill_chunk_size),

@@ -7,7 +7,7 @@ from typing import Optional
 
 from ..csrc import build as _build
 
-HOST_ABI_VERSION = 2
+HOST_ABI_VERSION = 3
 
 OK, CACHE_ERROR, OUT_OF_PAGES, VALUE_ERROR = 0, 1, 2, 3
 
@@ -63,6 +63,9 @@ _SIGNATURES = {
     "lmsf_sched_plan": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P]),
     "lmsf_sched_queue": (c_int, [_P, c_int, _P, c_int, POINTER(c_int)]),
     "lmsf_sched_num_preemptions": (c_int64, [_P]),
+    "lmsf_llama_config_parse": (c_int, [c_char_p, _P]),
+    "lmsf_llama_config_validate": (c_int, [_P]),
+    "lmsf_rope_scaling_parse": (c_int, [c_char_p, _P]),
 }
 
 

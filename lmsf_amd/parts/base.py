@@ -82,13 +82,16 @@ class ModelSpec:
 
 @dataclass(frozen=True)
 class TensorDecl:
-    """A checkpoint tensor a part expects. kind "float": loaded in the runtime dtype unless stored
-    in 32 bits, which it then keeps; "int": loaded as int32. ``init`` says how the random-weights
-    mode fills it: "normal" (mean 0, the mode's standard deviation), "ones" or "zeros"."""
+    """A checkpoint tensor a part expects. kind "float": loaded in the runtime dtype; "int": loaded as int32.
+    ``keeps_float32``: a tensor stored in 32 bits stays so in a bfloat16 run (the norms' weights: their kernels
+    compute in float32 anyway and take the weight as it is); the matrices of the products are cast as the
+    reference casts everything (core/src/model_executor/models/model_factory.rs:124-139). ``init`` says how
+    the random-weights mode fills it: "normal" (mean 0, the mode's standard deviation), "ones" or "zeros"."""
 
     shape: Tuple[int, ...]
     kind: str = "float"
     init: str = "normal"
+    keeps_float32: bool = False
 
 
 @dataclass(frozen=True)

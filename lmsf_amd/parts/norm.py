@@ -29,7 +29,7 @@ class RMSNorm(Norm):
 
     def checkpoint_tensors(self) -> Dict[str, TensorDecl]:
         init = "ones" if self.weight_offset == 0.0 else "zeros"
-        return {self.weight_name: TensorDecl((self.size,), init=init)}
+        return {self.weight_name: TensorDecl((self.size,), init=init, keeps_float32=True)}
 
     def load_weights(self, fetch: Callable[[str], torch.Tensor]) -> None:
         self.weight = fetch(self.weight_name).contiguous()

@@ -6,9 +6,12 @@ core/src/model_executor/layers/linear.rs:285-290; names in models/llama/llama.rs
 its checkpoint tensors first; the file set is compared with the declarations once, and a single
 error lists every missing tensor, every unexpected tensor and every wrong shape.
 
-Element types: a tensor declared "float" is kept in bfloat16 in a bfloat16 run (float16 storage is
-converted) and converted to float32 in a float32 run; a tensor stored in 32 bits stays in 32 bits
-in either run. A tensor declared "int" becomes int32.
+Element types: a tensor declared "float" is cast to the run's type as the reference casts at load
+(core/src/model_executor/models/model_factory.rs:124-139, core/src/common/config.rs:181-186): bfloat16 in
+a bfloat16 run (float16 and float32 storage are converted), float32 in a float32 run. A tensor stored in
+32 bits stays in 32 bits in a bfloat16 run where its declaration says so (``TensorDecl.keeps_float32``: the
+norms' weights) or where the caller asks for it for all of them (``keep_float32``: the matrices' products
+then run in float32 arithmetic, at twice the memory). A tensor declared "int" becomes int32.
 """
 import warnings
 from typing import Callable, Dict, Iterable, List, Optional, Sequence, Tuple
@@ -68,7 +71,7 @@ def check_against_declarations(decls: Dict[str, TensorDecl], found: Dict[str, Tu
     raise WeightsError("\n".join(lines), missing, unexpected, wrong)
 
 
-def _convert(t: torch.Tensor, decl: TensorDecl, run_dtype: torch.dtype) -> torch.Tensor:
+def _convert(t: torch.Tensor, decl: TensorDecl, run_dtype: torch.dtype, keep_float32: bool = False) -> torch.Tensor:
     if decl.kind == "int":
         if t.dtype.is_floating_point or t.dtype == torch.bool:
             raise WeightsError("tensor declared as integer table is stored as %s" % t.dtype)
@@ -77,8 +80,8 @@ def _convert(t: torch.Tensor, decl: TensorDecl, run_dtype: torch.dtype) -> torch
         raise WeightsError("tensor declared as float is stored as %s" % t.dtype)
     if run_dtype == torch.float32:
         return t.to(torch.float32)
-    if t.dtype in (torch.float32, torch.float64):
-        return t.to(torch.float32)          # stored in 32 bits (or more): stays 32-bit
+    if t.dtype in (torch.float32, torch.float64) and (decl.keeps_float32 or keep_float32):
+        return t.to(torch.float32)          # stored in 32 bits (or more) and meant to stay so
     return t.to(run_dtype)
 
 
@@ -95,9 +98,10 @@ def _return_freed_memory(device) -> None:
 
 
 def load_weights(parts: Sequence[Part], folder: str, device: torch.device, run_dtype: torch.dtype,
-                 tolerated: Sequence[str] = ()) -> None:
+                 tolerated: Sequence[str] = (), keep_float32: bool = False) -> None:
     """Check the checkpoint in ``folder`` against the parts' declarations, then hand every part its
-    tensors on ``device``. A name declared by two parts (tied weights) is loaded once and shared."""
+    tensors on ``device``. A name declared by two parts (tied weights) is loaded once and shared.
+    ``keep_float32``: every tensor stored in 32 bits stays so in a bfloat16 run (see the module's text)."""
     parts = list(parts)
     shared: set = set()
     decls = collect_declarations(parts, shared)
@@ -124,7 +128,7 @@ def load_weights(parts: Sequence[Part], folder: str, device: torch.device, run_d
                 return cache[name]
             f, _ = entries[name]
             try:
-                t = _convert(f.read(name), decls[name], run_dtype)
+                t = _convert(f.read(name), decls[name], run_dtype, keep_float32)
             except WeightsError as e:
                 raise WeightsError("%s: %s" % (name, e))
             if t.dtype == torch.float32 and run_dtype != torch.float32 and t.dim() >= 2:

@@ -6,7 +6,10 @@
 #include <cstdio>
 #include <cstdlib>
 #include <map>
+#include <string>
 #include <vector>
+
+#include "llama_config.h"
 
 extern "C" {
 int lmsf_host_abi_version();
@@ -80,6 +83,40 @@ static uint32_t rnd(uint32_t n) {
 int main(int argc, char** argv) {
   if (argc > 1) rng_state = std::strtoull(argv[1], nullptr, 10);
   if (lmsf_host_abi_version() < 1) return 1;
+
+  // the configuration reader: good text, every kind of broken text, and random cuts and flips of good text
+  {
+    const std::string good =
+        "{\"architectures\": [\"LlamaForCausalLM\"], \"hidden_size\": 64, \"num_attention_heads\": 4, "
+        "\"num_key_value_heads\": 2, \"intermediate_size\": 176, \"num_hidden_layers\": 2, \"vocab_size\": 256, "
+        "\"max_position_embeddings\": 128, \"rms_norm_eps\": 1e-5, \"rope_theta\": 10000.0, \"eos_token_id\": [2, 3], "
+        "\"tie_word_embeddings\": true, \"hidden_act\": \"si\\u006cu\", \"torch_dtype\": \"bfloat16\", "
+        "\"rope_scaling\": {\"rope_type\": \"llama3\", \"factor\": 8.0, \"low_freq_factor\": 1.0, "
+        "\"high_freq_factor\": 4.0, \"original_max_position_embeddings\": 64}}";
+    LmsfLlamaConfig cfg;
+    MUST(lmsf_llama_config_parse(good.c_str(), &cfg));
+    if (cfg.head_dim != 16 || cfg.n_eos_token_ids != 2 || !cfg.rope_scaling.present || std::string(cfg.hidden_act) != "silu")
+      return 1;
+    MUST(lmsf_llama_config_validate(&cfg));
+    cfg.head_dim = 15;
+    MUST_FAIL(lmsf_llama_config_validate(&cfg), 3);
+    for (const char* bad : {"", "{", "[1, 2", "{\"a\": }", "{\"hidden_size\": 1e999}", "\"text\"", "{\"a\": \"\\u12\"}",
+                            "{\"hidden_size\": 64} trailing", "nul", "{\"a\" 1}"})
+      MUST_FAIL(lmsf_llama_config_parse(bad, &cfg), 3);
+    std::string deep(200, '[');
+    MUST_FAIL(lmsf_llama_config_parse(deep.c_str(), &cfg), 3);
+    for (int it = 0; it < 400; ++it) {
+      std::string t = good;
+      if (rnd(2)) t.resize(rnd((uint32_t)t.size()));
+      for (int k = (int)rnd(4); k > 0 && !t.empty(); --k) t[rnd((uint32_t)t.size())] = (char)(32 + rnd(95));
+      const int rc = lmsf_llama_config_parse(t.c_str(), &cfg);
+      if (rc != 0 && rc != 3) return 1;
+    }
+    LmsfRopeScaling rs;
+    MUST(lmsf_rope_scaling_parse("{\"type\": \"default\"}", &rs));
+    if (rs.present) return 1;
+    MUST_FAIL(lmsf_rope_scaling_parse("{\"rope_type\": \"yarn\"}", &rs), 3);
+  }
 
   // the pool alone, with its error paths
   void* pool = nullptr;

@@ -114,3 +114,26 @@ def test_registering_another_architecture_needs_one_call():
     finally:
         unregister_architecture("ToyForCausalLM")
     assert "ToyForCausalLM" not in registered_architectures()
+
+
+def test_the_configuration_is_read_and_checked_by_the_host_library(tmp_path):
+    """from_dict hands the keys to the C++ reader (csrc/host/llama_config.cc) and takes back what it read: null
+    counts as absent, an integer written as 2.0 is one, text is read with its escapes, and what ``replace`` makes is
+    checked by the same code."""
+    from lmsf_amd.config.model_config import replace
+    d = dict(TINY_A, num_hidden_layers=2.0, rope_theta=None, hidden_act="silu")
+    c = LlamaConfig.from_dict(d)
+    assert c.num_hidden_layers == 2 and isinstance(c.num_hidden_layers, int) and c.rope_theta == 10000.0
+    folder = str(tmp_path)
+    with open(os.path.join(folder, "config.json"), "w") as f:
+        f.write(json.dumps(dict(TINY_B, hidden_act="silu")).replace('"silu"', '"si\\u006cu"').replace(", ", " ,\n\t"))
+    assert load_model_config(folder)[1] == LlamaConfig.from_dict(TINY_B)
+    with pytest.raises(ConfigError, match="at most 16"):
+        LlamaConfig.from_dict(dict(TINY_A, eos_token_id=list(range(17))))
+    with pytest.raises(ConfigError, match="eos_token_id"):
+        LlamaConfig.from_dict(dict(TINY_A, eos_token_id=[1, "two"]))
+    with pytest.raises(ConfigError, match="multiple of num_key_value_heads"):
+        replace(c, num_key_value_heads=3)
+    with pytest.raises(ConfigError, match="JSON"):
+        LlamaConfig.from_dict(dict(TINY_A, hidden_size=float("inf")))
+    assert replace(c, num_key_value_heads=4).num_key_value_heads == 4

@@ -253,9 +253,23 @@ def _is_model_tensor(model, t):
                for p in model.parts() for a in ("weight", "bias"))
 
 
-def test_matrices_stored_in_32_bits_are_reported(tmp_path):
+def test_matrices_stored_in_32_bits_are_cast_to_the_run_type_at_load(tmp_path):
+    """A float32 checkpoint in a bfloat16 run: the matrices are cast as the reference casts at load
+    (core/src/model_executor/models/model_factory.rs:124-139), the norms' weights keep their 32 bits; on request
+    the matrices stay as stored, and that is reported."""
+    import warnings
     folder, cfg = make_model_folder(tmp_path, "A", dtype="float32")
     m = cpu_model(cfg, torch.bfloat16)
-    with pytest.warns(UserWarning, match="stored in 32 bits"):
+    with warnings.catch_warnings():
+        warnings.simplefilter("error")
         load_weights(m.parts(), folder, torch.device("cpu"), torch.bfloat16)
-    assert m.blocks[0].mixer.qkv.weight.dtype == torch.float32
+    for part in m.parts():
+        w = getattr(part, "weight", None)
+        if w is not None:
+            assert w.dtype == (torch.float32 if w.dim() == 1 else torch.bfloat16), part.prefix
+    raw = load_file(os.path.join(folder, "model.safetensors"))
+    assert torch.equal(m.blocks[0].feed_forward.down.weight, raw["model.layers.0.mlp.down_proj.weight"].to(torch.bfloat16))
+    kept = cpu_model(cfg, torch.bfloat16)
+    with pytest.warns(UserWarning, match="stored in 32 bits"):
+        load_weights(kept.parts(), folder, torch.device("cpu"), torch.bfloat16, keep_float32=True)
+    assert kept.blocks[0].mixer.qkv.weight.dtype == torch.float32
