@@ -51,13 +51,12 @@ def weight_bytes(engine):
     """Bytes of every weight a decode step reads once: all matrices and norm weights, the LM head, not
     the embedding table (one row per token)."""
     seen, total = set(), 0
-    emb = engine.core.model.embedding.weight
-    head = engine.core.model.head.weight
-    for p in engine.core.model.parts():
+    model = engine.core.model
+    head = {t.data_ptr() for t in model.head.tensors()}
+    gathered = {t.data_ptr() for t in model.embedding.tensors()} - head     # (tied: the head reads the table whole)
+    for p in model.parts():
         for t in p.tensors():
-            if t.data_ptr() in seen:
-                continue
-            if t.data_ptr() == emb.data_ptr() and emb.data_ptr() != head.data_ptr():
+            if t.data_ptr() in seen or t.data_ptr() in gathered:
                 continue
             seen.add(t.data_ptr())
             total += t.numel() * t.element_size()

@@ -215,6 +215,14 @@ class CacheManager:
             first_live.append(fl)
         return RequestCache(rid, int(info[0]), int(info[1]), int(info[2]), tables, first_live)
 
+    def state_slot(self, rid: Hashable) -> int:
+        """The state slot that the live request ``rid`` holds."""
+        info = np.zeros(3, dtype=np.int64)
+        rc = self._lib.lmsf_cm_request_info(self._h, self._must(rid), _ptr(info))
+        if rc:
+            _raise(self._lib, rc, "request %r" % (rid,))
+        return int(info[0])
+
     def _table(self, h: int, group: int):
         n, fl = ctypes.c_int(), ctypes.c_int()
         rc = self._lib.lmsf_cm_block_table(self._h, h, group, None, 0, ctypes.byref(n), ctypes.byref(fl))

@@ -3,7 +3,8 @@
 The reference allocates per layer K [blocks, kv_heads, d/x, block, x] and V [blocks, kv_heads, d, block]
 (core/src/worker/cache_engine.rs:107-160) and sizes the pool from free device memory
 (core/src/worker/model_worker.rs:128-162, block bytes :cache_engine.rs:88-105). Here K is
-[pages, kv_heads, page_size, head_dim] and V [pages, kv_heads, head_dim, page_size]; runs of layers whose mixers declare equal needs form
+[pages, kv_heads, page_size, head_dim] and V [pages, kv_heads, v_head_dim, page_size] (a value as wide as a key
+unless the mixer says otherwise); runs of layers whose mixers declare equal needs form
 a group that shares page ids, so one block table serves all of them.
 """
 from dataclasses import dataclass
@@ -23,7 +24,8 @@ class GroupLayout:
     num_pages: int = 0
 
     def bytes_per_page(self, elem_size: int) -> int:
-        return len(self.entries) * 2 * self.spec.num_kv_heads * self.page_size * self.spec.head_dim * elem_size
+        return len(self.entries) * self.spec.num_kv_heads * self.page_size * (self.spec.head_dim + self.spec.value_dim) \
+            * elem_size
 
 
 def plan_groups(requirements: Sequence[Tuple[Optional[CacheSpec], Optional[StateSpec], Optional[int]]],
@@ -76,7 +78,7 @@ class CacheStorage:
                     n = max(1, g.num_pages)
                     b.k_pages = torch.zeros((n, cspec.num_kv_heads, g.page_size, cspec.head_dim), dtype=rt.dtype,
                                             device=rt.device)
-                    b.v_pages = torch.zeros((n, cspec.num_kv_heads, cspec.head_dim, g.page_size), dtype=rt.dtype,
+                    b.v_pages = torch.zeros((n, cspec.num_kv_heads, cspec.value_dim, g.page_size), dtype=rt.dtype,
                                             device=rt.device)
                 else:
                     b.k_pages, b.v_pages = bindings[src].k_pages, bindings[src].v_pages
@@ -88,7 +90,19 @@ class CacheStorage:
                                       device=rt.device)
             bindings.append(b)
         self.bindings = bindings
+        self.has_state = any(b.state is not None for b in bindings)
         model.bind_cache(bindings)
+
+    def clear_state_slots(self, slots: Sequence[int]) -> None:
+        """Zeroes these slots of every state tensor: a request that takes a slot finds no trace of the one that
+        held it before (the reference has no per-request state; its block manager hands out blocks as they are,
+        core/src/sched/block_manager.rs:29-43, which is right for keys that are written before they are read)."""
+        states = {b.state.data_ptr(): b.state for b in self.bindings if b.state is not None}
+        if not states or not len(slots):
+            return
+        idx = torch.as_tensor(list(slots), dtype=torch.long, device=self.rt.device)
+        for st in states.values():
+            st.index_fill_(0, idx, 0)
 
     def bytes_allocated(self) -> int:
         total = 0

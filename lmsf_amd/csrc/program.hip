@@ -668,7 +668,7 @@ int run_pass(const Program& prog, const LmsfStepDesc& st, hipStream_t stream, bo
   r.stream = stream;
   r.dry = dry;
   r.regs.assign(prog.n_regs, Value());
-  r.far_at = r.limit = (size_t)st.workspace_bytes;
+  r.far_at = r.limit = (size_t)st.workspace_bytes & ~(size_t)255;   // (everything handed out is 256-byte aligned)
   const int N = st.n_tokens, R = st.n_logit_rows;
   for (size_t i = 0; i < prog.ops.size(); ++i) {
     const LmsfOpDesc& op = prog.ops[i];

@@ -88,7 +88,9 @@ def profile_num_pages(model: DecoderModel, rt: Runtime, block_size: int, gpu_mem
     torch.cuda.empty_cache()
     free, total = torch.cuda.mem_get_info(rt.device)
     spec = model.spec
-    mats = [t for p in model.parts() for t in p.tensors() if t.dim() == 2 and t.shape[0] != spec.vocab_size]
+    # (the embedding's table and the head's matrix apart: the first is gathered from, the second meets wanted rows only)
+    ends = {t.data_ptr() for p in (model.embedding, model.head) for t in p.tensors()}
+    mats = [t for p in model.parts() for t in p.tensors() if t.dim() == 2 and t.data_ptr() not in ends]
     widest = max((t.shape[0] for t in mats), default=spec.hidden_size)
     wes = max((t.element_size() for t in mats), default=es)       # matrices kept in 32 bits have 32-bit products
     # one step's activations (float32 stream twice, three buffers of the widest product), the logits of every

@@ -55,6 +55,7 @@ class ModelExecutor:
         self.max_step_tokens = int(max_step_tokens) if max_step_tokens else None
         self.max_step_seqs = int(max_step_seqs) if max_step_seqs else None
         self.program_steps = 0          # steps that the program ran
+        self.python_parts = None        # (part, method name) -> True: that call runs in Python inside the program (tests, debugging)
         self.program_workspace_bytes = 32 << 20    # the workspace's size; it doubles if a step finds no room all the same
         if self.use_program:
             self._record_program()
@@ -64,7 +65,7 @@ class ModelExecutor:
         step the engine will build needs (found by walking such steps without launching), so that no step in
         the middle of serving has to allocate."""
         from ..ops.program import record_program
-        self.program = record_program(self.model, self.rt.ops)
+        self.program = record_program(self.model, self.rt.ops, self.python_parts)
         self._static.clear()            # captured steps belong to the program that launched them
         if self.program is None:
             return
@@ -115,6 +116,9 @@ class ModelExecutor:
         lens = [len(e.tokens) for e in entries]
         handles, starts, added = mgr.begin_step(rids, lens)      # OutOfPages: nothing was taken
         try:
+            if self.storage.has_state and added.any():
+                # a request that has just taken a state slot finds it cleared
+                self.storage.clear_state_slots([mgr.state_slot(rids[i]) for i in np.nonzero(added)[0]])
             if self.pad_decode and all(n == 1 for n in lens) and len(entries) <= self.max_graph_batch:
                 logits = self._decode_step(entries, handles, starts)
             else:

@@ -41,7 +41,8 @@ class DecoderModel:
                                      % (i, e.cache_from))
                 a = self.blocks[e.layer].mixer.cache_spec()
                 b = self.blocks[self.schedule[e.cache_from].layer].mixer.cache_spec()
-                if a is None or b is None or (a.num_kv_heads, a.head_dim) != (b.num_kv_heads, b.head_dim):
+                if a is None or b is None or (a.num_kv_heads, a.head_dim, a.value_dim) != (b.num_kv_heads, b.head_dim,
+                                                                                          b.value_dim):
                     raise ValueError("schedule entry %d cannot read the cache of entry %d: cache shapes differ"
                                      % (i, e.cache_from))
         self.bindings: List[CacheBinding] = [CacheBinding() for _ in self.schedule]

@@ -167,6 +167,7 @@ class Recorder:
         self.callbacks: List[_Callback] = []
         self.step_ctx = None                    # the placeholder StepContext of the recording
         self.roles = {}                         # id(part) -> "embedding" / "head"
+        self.in_python = None                   # (part, method name) -> True: record this call as a callback anyway
 
     # -- helpers
     def _new(self, cols: Optional[int] = None, dtype: Optional[torch.dtype] = None) -> Sym:
@@ -340,6 +341,8 @@ class Recorder:
         placeholder, what it recorded is taken back and the whole call becomes one callback operation."""
 
         def call(*args, **kwargs):
+            if self.in_python is not None and self.in_python(part, name):
+                return self._callback(part, name, fn, args, kwargs, "asked for")
             mark = self.mark()
             try:
                 return fn(*args, **kwargs)
@@ -462,7 +465,7 @@ class StepProgram:
     def ensure_workspace(self, nbytes: int) -> None:
         if self.workspace is None or self.workspace.numel() < nbytes:
             self.workspace = None
-            self.workspace = torch.empty(int(nbytes), dtype=torch.uint8, device=self.device)
+            self.workspace = torch.empty((int(nbytes) + 255) // 256 * 256, dtype=torch.uint8, device=self.device)
 
     # -- sizing
     def workspace_need(self, n_tokens: int, n_segments: int, n_logit_rows: int, max_context: int,
@@ -598,8 +601,10 @@ def _step_array(ctx, code: int):
 last_failure: Optional[str] = None
 
 
-def record_program(model, hip_ops) -> Optional[StepProgram]:
-    """The model's forward as a step program, or None if the model cannot be recorded (``last_failure`` says why)."""
+def record_program(model, hip_ops, in_python: Optional[Callable[[Any, str], bool]] = None) -> Optional[StepProgram]:
+    """The model's forward as a step program, or None if the model cannot be recorded (``last_failure`` says why).
+    ``in_python(part, method name)``: True for calls that are to run in Python as callbacks although the recorder
+    could follow them (to watch a part's operands in the middle of a step, say)."""
     global last_failure
     from ..engine.batch import GroupView, StepContext
     rt = model.rt
@@ -612,6 +617,7 @@ def record_program(model, hip_ops) -> Optional[StepProgram]:
         return None
     rec = Recorder(rt.dtype, model.spec.hidden_size, model.spec.vocab_size)
     rec.roles = {id(model.embedding): "embedding", id(model.head): "head"}
+    rec.in_python = in_python
     groups = [GroupView(slots=CtxRef(CTX_SLOTS + g), block_tables=CtxRef(CTX_TABLES + g), page_size=0)
               for g in range(n_groups)]
     ctx = StepContext(

@@ -98,16 +98,24 @@ class TensorDecl:
 class CacheSpec:
     """Paged key/value needs of a mixer. Runs with equal specs share a page pool and block tables.
     window None: all keys are kept; window W: only the last W positions are ever read, pages that
-    the window has passed are given back."""
+    the window has passed are given back. ``head_dim`` is the width of a key; a value has ``v_head_dim``
+    (None: the same). The attention kernels of this package take equal widths; a mixer with unequal ones
+    reads and writes its pages itself."""
 
     num_kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    v_head_dim: Optional[int] = None
+
+    @property
+    def value_dim(self) -> int:
+        return self.head_dim if self.v_head_dim is None else self.v_head_dim
 
 
 @dataclass(frozen=True)
 class StateSpec:
-    """Fixed-size per-request state of a mixer: one tensor of ``shape`` and ``dtype`` per live request."""
+    """Fixed-size per-request state of a mixer: one tensor of ``shape`` and ``dtype`` per live request. A slot
+    is all zeros when a request's first tokens run: the engine clears it when the request takes it."""
 
     shape: Tuple[int, ...]
     dtype: torch.dtype = torch.float32
@@ -119,7 +127,7 @@ class CacheBinding:
 
     group: Optional[int] = None            # index of the cache group (page pool + block tables)
     k_pages: Optional[torch.Tensor] = None  # [pages, kv_heads, page_size, head_dim]
-    v_pages: Optional[torch.Tensor] = None  # [pages, kv_heads, head_dim, page_size]
+    v_pages: Optional[torch.Tensor] = None  # [pages, kv_heads, v_head_dim, page_size]
     writes_cache: bool = True              # False: reads another run's pages
     state: Optional[torch.Tensor] = None   # [slots, *StateSpec.shape]
 

@@ -43,8 +43,8 @@ def test_llama3_8b_layer_sizes_every_product_path(full_model):
     from lmsf_amd.engine import load_engine_core
     folder, cfg, w = full_model
     V = cfg["vocab_size"]
-    # lengths chosen for the paths: 100 tokens at once (library products), portions of 24 and 40 (17 to 64 rows,
-    # partial sums), single tokens of up to four requests together (few rows)
+    # lengths chosen for the paths: 100 and 70 tokens at once (the 17-and-more-rows and the many-rows products),
+    # portions of 24 and 40 (17 to 64 rows, partial sums), single tokens of up to four requests together (few rows)
     reqs = {"a": random_tokens(100, V, 1), "b": random_tokens(70, V, 2), "c": random_tokens(41, V, 3),
             "d": random_tokens(9, V, 4)}
     refs = {rid: plain_llama_forward(cfg, w, toks) for rid, toks in reqs.items()}
@@ -60,6 +60,29 @@ def test_llama3_8b_layer_sizes_every_product_path(full_model):
     # greedy tokens of the engine's sampler against the plain logits (ties aside: random weights have none)
     logits = torch.stack([refs[r][-1] for r in reqs])
     assert core.rt.ops.sample(logits.cuda()).tolist() == logits.argmax(dim=-1).tolist()
+
+
+@pytest.mark.parametrize("n_prompt", [200, 300, 700, 2048])
+def test_llama3_8b_layer_sizes_whole_prompts_of_hundreds_of_tokens(full_model, n_prompt):
+    """Whole prompts of 200 tokens (the many-rows product inside the step program), of 300 and 700 (the BLAS
+    library's products called from the program, the many-rows product for down) and of 2,048 (the many-tile prefill
+    attention, the tiled rotary and cache kernel, the vectorised activation), then four tokens decoded one by one
+    from the cache that the prompt left: the last prompt position and the four after it against the plain
+    implementation."""
+    from lmsf_amd.engine import StepEntry, load_engine_core
+    folder, cfg, w = full_model
+    toks = random_tokens(n_prompt + 4, cfg["vocab_size"], 100 + n_prompt)
+    ref = plain_llama_forward(cfg, w, toks, last=5)
+    core = load_engine_core(folder, dtype="bfloat16", block_size=16, num_pages=-(-(n_prompt + 4) // 16) + 1, max_num_seqs=2,
+                            max_num_batched_tokens=2048)
+    ex = core.executor
+    rows = [ex.step([StepEntry("p", toks[:n_prompt], [n_prompt - 1])]).float().cpu()]
+    for t in toks[n_prompt:]:
+        rows.append(ex.step([StepEntry("p", [t], [0])]).float().cpu())
+    ex.release("p")
+    assert ex.program is not None and ex.program_steps >= 2      # (the prompt, then single tokens until their kind is a graph)
+    check({"p": torch.cat(rows[:5])}, {"p": ref}, "bfloat16", "a whole prompt of %d tokens and four more" % n_prompt, BOUND)
+    core.storage.manager.check_invariants()
 
 
 def test_llama3_8b_layer_sizes_in_true_float32(full_model):
@@ -144,6 +167,38 @@ def test_loading_leaves_no_holes_in_device_memory():
     slack = torch.cuda.memory_reserved() - torch.cuda.memory_allocated() - base
     weights = sum(t.numel() * t.element_size() for p in core.model.parts() for t in p.tensors())
     assert weights > 5e9 and slack < (200 << 20), (slack, weights)
+
+
+@pytest.mark.parametrize("library", [1, 0])
+def test_recorded_program_at_these_sizes_steps_of_300_to_2048_tokens(full_model, library):
+    """Steps of 300, 700 and 2,048 tokens (and of 100 beside them) through the program and part by part: the same
+    kernels for the same routes, so the same bits. With the BLAS library (its products called from C++ by both) and
+    without it (use_library_gemm 0: the deep product of down stays with the many-rows kernel up to 1,024 rows, the
+    others fall to the float32 multiply-add kernel; 2,048 tokens are left out there, for the time they would take)."""
+    from lmsf_amd.engine import load_engine_core
+    from lmsf_amd.ops import get_ops
+    folder, cfg, w = full_model
+    V = cfg["vocab_size"]
+    lens = {"e": 300, "f": 700, "g": 100}
+    if library:
+        lens["h"] = 2048
+    reqs = {r: random_tokens(n, V, 60 + n) for r, n in lens.items()}
+    steps = trace_whole(reqs) + trace_portions({"i": random_tokens(900, V, 35)}, seed=4)
+    ops = get_ops()
+    was = ops.use_library_gemm
+    ops.use_library_gemm = library
+    try:
+        outs = []
+        for use_program in (True, False):
+            core = load_engine_core(folder, dtype="bfloat16", block_size=16, num_pages=132, max_num_seqs=4,
+                                    max_num_batched_tokens=2048, use_program=use_program, enforce_eager=True)
+            outs.append(replay_in_process(core.executor, steps))
+            if use_program:
+                assert core.executor.program_steps >= len(steps)
+        for rid in outs[0]:
+            assert torch.equal(outs[0][rid], outs[1][rid]), rid
+    finally:
+        ops.use_library_gemm = was
 
 
 def test_recorded_program_at_these_sizes_with_the_smallest_workspace(full_model):

@@ -77,7 +77,7 @@ def test_rms_norm_part(dtype):
     rt = runtime(dtype)
     H, eps = 80, 3e-6
     norm = build_part("norm", PartSpec("rms_norm", {"size": H, "eps": eps}), "n", rt)
-    assert norm.checkpoint_tensors() == {"n.weight": TensorDecl((H,), init="ones")}
+    assert norm.checkpoint_tensors() == {"n.weight": TensorDecl((H,), init="ones", keeps_float32=True)}
     w = rnd(H, seed=1) + 1.0
     give(norm, {"n.weight": w}, dtype)
     x = rnd(7, H, seed=2)
@@ -329,9 +329,7 @@ class RunningMeanMixer(Mixer):
         out = torch.empty_like(h)
         for s, (start, n, first, slot) in enumerate(zip(ctx.host_seg_starts, ctx.host_seg_lens, ctx.host_seg_first_pos,
                                                         ctx.host_state_slots)):
-            st = binding.state[slot]
-            if first == 0:
-                st.zero_()                                        # a slot keeps the last request's state
+            st = binding.state[slot]                              # (all zeros when a request begins: the engine clears it)
             x = h[start:start + n].float()
             sums = st[:self.H] + torch.cumsum(x, 0)
             counts = st[self.H] + torch.arange(1, n + 1, device=h.device, dtype=torch.float32)
@@ -488,13 +486,151 @@ def test_toy_parts_are_registered_built_and_stepped(toy_architecture, tmp_path):
     assert states[0].data_ptr() != states[2].data_ptr() and tuple(states[0].shape) == (3 + 1, cfg.hidden_size + 1)
     assert core.storage.entry_group == [None, 0, None]
     assert not core.executor.use_graphs                          # a part that does not declare itself graph-safe: eager
+    # the step is a recorded program all the same: the parts the recorder cannot follow (the two runs of the mean
+    # mixer and of the routed feed-forward, the learned positions) are five callbacks in it, the rest is native
+    prog = core.executor.program
+    assert prog is not None and len(prog.callbacks) == 5, [c.what for c in prog.callbacks] if prog else None
     from test_replay_gpu import check
     for name, steps in (("whole", trace_whole(reqs)), ("bulk then single", trace_bulk_then_single(reqs)),
                         ("portions", trace_portions(reqs, seed=7)),
                         ("mixed", trace_mixed(reqs, 192, seed=3, max_live=3))):      # 5 requests through 3 state slots
         check(replay_in_process(core.executor, steps), refs, "float32", name)
         assert core.storage.manager.num_free_state_slots() == 3
+    assert core.executor.program_steps > 50
+    # part by part, without the program: the same bits
+    plain = load_engine_core(folder, dtype="float32", block_size=8, num_pages=24, max_num_seqs=3, use_program=False)
+    steps = trace_mixed(reqs, 192, seed=3, max_live=3)
+    a, b = replay_in_process(core.executor, steps), replay_in_process(plain.executor, steps)
+    assert plain.executor.program is None and all(torch.equal(a[r], b[r]) for r in a)
     # bfloat16 builds and steps too
     core16 = load_engine_core(folder, dtype="bfloat16", block_size=8, num_pages=24, max_num_seqs=3)
     out = core16.executor.step([StepEntry("x", reqs["b"], [len(reqs["b"]) - 1])])
     check({"x": out.float().cpu()}, {"x": refs["b"][-1:]}, "bfloat16", "toy parts in bfloat16")
+
+
+# --------------------------------------------------------------------------- a mixer whose values are wider than its keys
+
+class WideValueAttention(Mixer):
+    """Causal attention with keys of width d and values of width dv, written with torch: it stores into its pages
+    and reads from them through the block tables itself (the package's kernels take equal widths)."""
+
+    def __init__(self, prefix, rt, hidden_size, num_heads, num_kv_heads, head_dim, v_head_dim):
+        super().__init__(prefix, rt)
+        self.H, self.nh, self.nkv, self.d, self.dv = hidden_size, num_heads, num_kv_heads, head_dim, v_head_dim
+
+    def _shapes(self):
+        return {"q": (self.nh * self.d, self.H), "k": (self.nkv * self.d, self.H), "v": (self.nkv * self.dv, self.H),
+                "o": (self.H, self.nh * self.dv)}
+
+    def checkpoint_tensors(self):
+        return {"%s.%s.weight" % (self.prefix, n): TensorDecl(s) for n, s in self._shapes().items()}
+
+    def load_weights(self, fetch):
+        self.w = {n: fetch("%s.%s.weight" % (self.prefix, n)) for n in self._shapes()}
+
+    def tensors(self):
+        return list(self.w.values())
+
+    def cache_spec(self):
+        from lmsf_amd.parts import CacheSpec
+        return CacheSpec(num_kv_heads=self.nkv, head_dim=self.d, v_head_dim=self.dv)
+
+    def forward(self, h, ctx, binding):
+        N = h.shape[0]
+        x = h.float()
+        q = (x @ self.w["q"].float().t()).view(N, self.nh, self.d)
+        k = (x @ self.w["k"].float().t()).view(N, self.nkv, self.d)
+        v = (x @ self.w["v"].float().t()).view(N, self.nkv, self.dv)
+        group = ctx.groups[binding.group]
+        ps = group.page_size
+        slots = group.slots.long()
+        binding.k_pages[slots // ps, :, slots % ps, :] = k.to(binding.k_pages.dtype)
+        binding.v_pages[slots // ps, :, :, slots % ps] = v.to(binding.v_pages.dtype)
+        out = torch.empty(N, self.nh, self.dv, dtype=torch.float32, device=h.device)
+        rep = self.nh // self.nkv
+        for s, (start, n, first) in enumerate(zip(ctx.host_seg_starts, ctx.host_seg_lens, ctx.host_seg_first_pos)):
+            T = first + n
+            pages = group.block_tables[s, :-(-T // ps)].long()
+            K = binding.k_pages[pages].float().permute(1, 0, 2, 3).reshape(self.nkv, -1, self.d)[:, :T]
+            V = binding.v_pages[pages].float().permute(1, 0, 3, 2).reshape(self.nkv, -1, self.dv)[:, :T]
+            qs = q[start:start + n]
+            scores = torch.einsum("thd,hjd->thj", qs, K.repeat_interleave(rep, 0)) / self.d ** 0.5
+            dead = torch.arange(T, device=h.device)[None, :] > (first + torch.arange(n, device=h.device))[:, None]
+            probs = torch.softmax(scores.masked_fill(dead[:, None, :], float("-inf")), -1)
+            out[start:start + n] = torch.einsum("thj,hjd->thd", probs, V.repeat_interleave(rep, 0))
+        return (out.reshape(N, self.nh * self.dv) @ self.w["o"].float().t()).to(h.dtype)
+
+
+class WideConfig(LlamaConfig):
+    ARCHITECTURE = "WideValueForCausalLM"
+    MODEL_TYPE = "wide_value"
+
+
+WIDE_DV = 24      # values of 24 numbers beside keys of 16
+
+
+def build_wide_spec(cfg):
+    H = cfg.hidden_size
+
+    def norm(prefix):
+        return PartSpec("rms_norm", {"prefix": prefix, "size": H, "eps": cfg.rms_norm_eps})
+
+    layers = tuple(LayerSpec("wide.layers.%d" % i, PartSpec("prenorm_residual"),
+                             PartSpec("toy_wide_value", {"prefix": "attn", "hidden_size": H, "num_heads": cfg.num_attention_heads,
+                                                         "num_kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
+                                                         "v_head_dim": WIDE_DV}),
+                             PartSpec("gated_mlp", {"prefix": "mlp", "hidden_size": H, "intermediate_size": cfg.intermediate_size}),
+                             {"input": norm("ln1"), "post_mixer": norm("ln2")}) for i in range(cfg.num_hidden_layers))
+    return ModelSpec(
+        embedding=PartSpec("token_embedding", {"prefix": "wide.embed", "vocab_size": cfg.vocab_size, "hidden_size": H}),
+        layers=layers, schedule=tuple(ScheduleEntry(i) for i in range(cfg.num_hidden_layers)),
+        final_norm=norm("wide.norm"), head=PartSpec("lm_head", {"prefix": "wide.head", "vocab_size": cfg.vocab_size,
+                                                                "hidden_size": H}),
+        vocab_size=cfg.vocab_size, hidden_size=H)
+
+
+def plain_wide_forward(cfg, w, toks):
+    H, nh, nkv, d, eps = cfg.hidden_size, cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim, cfg.rms_norm_eps
+    T = len(toks)
+    s = P.plain_embedding(w["wide.embed.weight"], toks)
+    for i in range(cfg.num_hidden_layers):
+        p = "wide.layers.%d." % i
+        h = P.plain_rms_norm(s, w[p + "ln1.weight"], eps)
+        q = P.plain_linear(h, w[p + "attn.q.weight"]).view(T, nh, d)
+        k = P.plain_linear(h, w[p + "attn.k.weight"]).view(T, nkv, d)
+        v = P.plain_linear(h, w[p + "attn.v.weight"]).view(T, nkv, WIDE_DV)
+        s = s + P.plain_linear(P.plain_attention(q, k, v).reshape(T, nh * WIDE_DV), w[p + "attn.o.weight"])
+        h = P.plain_rms_norm(s, w[p + "ln2.weight"], eps)
+        s = s + P.plain_swiglu_mlp(h, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+    return P.plain_linear(P.plain_rms_norm(s, w["wide.norm.weight"], eps), w["wide.head.weight"])
+
+
+def test_a_mixer_with_values_wider_than_its_keys(tmp_path):
+    """A cache group may hold values of another width than its keys (CacheSpec.v_head_dim): the pages are made so,
+    a page's bytes count both widths, and a toy mixer that reads and writes such pages itself goes through the
+    four ways of cutting, with pages used again, as a callback inside the recorded program."""
+    register_part("mixer", "toy_wide_value")(WideValueAttention)
+    register_architecture("WideValueForCausalLM", "wide_value", WideConfig, build_wide_spec)
+    try:
+        cfg = WideConfig.from_dict(dict(TINY["A"][0], tie_word_embeddings=False, max_position_embeddings=96))
+        folder = write_random_model(str(tmp_path / "wide"), cfg, seed=4, std=0.2)
+        _, w = P.read_model_folder(folder)
+        core = load_engine_core(folder, dtype="float32", block_size=8, num_pages=24, max_num_seqs=4)
+        b = core.storage.bindings[0]
+        assert tuple(b.k_pages.shape) == (24, cfg.num_key_value_heads, 8, cfg.head_dim)
+        assert tuple(b.v_pages.shape) == (24, cfg.num_key_value_heads, WIDE_DV, 8)
+        assert core.storage.groups[0].bytes_per_page(4) == 2 * cfg.num_key_value_heads * 8 * (cfg.head_dim + WIDE_DV) * 4
+        prog = core.executor.program
+        assert prog is not None and len(prog.callbacks) == cfg.num_hidden_layers
+        reqs = {"a": random_tokens(50, cfg.vocab_size, 1), "b": random_tokens(9, cfg.vocab_size, 2),
+                "c": random_tokens(33, cfg.vocab_size, 3), "d": random_tokens(64, cfg.vocab_size, 4),
+                "e": random_tokens(21, cfg.vocab_size, 5)}
+        refs = {r: plain_wide_forward(cfg, w, toks) for r, toks in reqs.items()}
+        from test_replay_gpu import check
+        for name, steps in (("whole", trace_whole(reqs)), ("bulk then single", trace_bulk_then_single(reqs)),
+                            ("portions", trace_portions(reqs, seed=7)), ("mixed", trace_mixed(reqs, 192, seed=3))):
+            check(replay_in_process(core.executor, steps), refs, "float32", "wide values, " + name)
+            assert core.storage.manager.num_free_pages(0) == 24
+    finally:
+        unregister_architecture("WideValueForCausalLM")
+        unregister_part("mixer", "toy_wide_value")

@@ -132,6 +132,33 @@ def test_rope_llama3_scaling():
     assert torch.equal(P.plain_rope_inv_freq(64, 500000.0, {"rope_type": "default"}), base)
 
 
+def test_rope_llama3_blend_is_linear_in_frequency_and_meets_both_ends():
+    """The band between the two wavelengths pinned by arithmetic alone: at the band's short end (wavelength
+    orig / high) the blend is the frequency itself, at its long end (orig / low) the frequency over the factor,
+    and at the frequency midway between the two ends the ratio is (1 + 1 / factor) / 2: the blend is linear in the
+    frequency (a blend linear in the wavelength gives (1 + 1 / factor) / 2 midway between the wavelengths instead,
+    and 0.4 here). With rotary_dim 4 the second frequency is theta^(-1/2), so theta places it anywhere. The same
+    for the product's table builder."""
+    from lmsf_amd.parts.rotary import inverse_frequencies
+    orig, low, high, factor = 64.0, 1.0, 4.0, 8.0
+    sc = dict(rope_type="llama3", factor=factor, low_freq_factor=low, high_freq_factor=high,
+              original_max_position_embeddings=int(orig))
+    f_short, f_long = 2 * math.pi * high / orig, 2 * math.pi * low / orig
+    cases = [(f_short, 1.0), (f_long, 1.0 / factor), ((f_short + f_long) / 2, (1 + 1 / factor) / 2),
+             (f_long + 0.25 * (f_short - f_long), 0.25 + 0.75 / factor),
+             (f_short * 1.5, 1.0), (f_long / 1.5, 1.0 / factor)]
+    for f, want in cases:
+        theta = 1.0 / (f * f)
+        for build in (P.plain_rope_inv_freq, inverse_frequencies):
+            got = build(4, theta, sc)
+            assert got[0].item() == 1.0                              # wavelength 2 pi: short, kept
+            assert abs(got[1].item() / f - want) < 2e-6, (build.__name__, f, got[1].item() / f, want)
+    # what a blend linear in the wavelength would give midway between the frequencies: far from the above
+    lam = 2 * math.pi / ((f_short + f_long) / 2)
+    s_wave = (orig / low - lam) / (orig / low - orig / high)
+    assert abs(((1 - s_wave) / factor + s_wave) - (1 + 1 / factor) / 2) > 0.05
+
+
 # --------------------------------------------------------------------------- attention
 
 @pytest.mark.parametrize("nh,nkv", [(4, 4), (4, 2), (6, 1)])

@@ -11,6 +11,8 @@ from helpers import (TINY, make_model_folder, random_tokens, replay_in_process, 
                      trace_mixed, trace_portions, trace_whole)
 from plain_llama import plain_llama_forward, read_model_folder
 
+from lmsf_amd.engine import StepEntry
+
 pytestmark = pytest.mark.gpu
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -310,15 +312,29 @@ def test_decode_steps_of_many_requests_of_different_lengths(models, dtype):
     core.storage.manager.check_invariants()
 
 
-def test_float32_checkpoint_in_a_bfloat16_run(models):
-    """A checkpoint stored in 32 bits keeps its 32 bits in a bfloat16 run (with a warning): activations and cache
-    are bfloat16, the products run in float32 arithmetic, and the logits are the plain implementation's within
-    the bfloat16 bound, under portions and single tokens alike."""
+@pytest.mark.parametrize("keep", [False, True])
+def test_float32_checkpoint_in_a_bfloat16_run(models, keep):
+    """A checkpoint stored in 32 bits in a bfloat16 run: its matrices are cast to bfloat16 at load, as the reference
+    casts (core/src/model_executor/models/model_factory.rs:124-139); the norms' weights keep their 32 bits. On
+    request (keep_float32_weights) the matrices stay as stored, with a warning: activations and cache are bfloat16,
+    the products run in float32 arithmetic. Either way the logits are the plain implementation's within the
+    bfloat16 bound, under portions and single tokens alike."""
+    import warnings
     folder, cfg, w = models[("B", "float32")]
     from lmsf_amd.engine import load_engine_core
-    with pytest.warns(UserWarning, match="stored in 32 bits"):
-        core = load_engine_core(folder, dtype="bfloat16", block_size=16, num_pages=24, max_num_seqs=4)
-    assert core.model.blocks[0].mixer.qkv.weight.dtype == torch.float32
+    if keep:
+        with pytest.warns(UserWarning, match="stored in 32 bits"):
+            core = load_engine_core(folder, dtype="bfloat16", block_size=16, num_pages=24, max_num_seqs=4,
+                                    keep_float32_weights=True)
+    else:
+        with warnings.catch_warnings():
+            warnings.simplefilter("error")
+            core = load_engine_core(folder, dtype="bfloat16", block_size=16, num_pages=24, max_num_seqs=4)
+    for part in core.model.parts():
+        wt = getattr(part, "weight", None)
+        if wt is not None and wt.dim() == 2:
+            assert wt.dtype == (torch.float32 if keep else torch.bfloat16), part.prefix
+    assert core.model.final_norm.weight.dtype == torch.float32
     assert core.model.bindings[0].k_pages.dtype == torch.bfloat16
     reqs = {"a": random_tokens(150, cfg["vocab_size"], 31), "b": random_tokens(40, cfg["vocab_size"], 32)}
     refs = {rid: plain_llama_forward(cfg, w, toks) for rid, toks in reqs.items()}
@@ -371,6 +387,82 @@ def test_recorded_program_gives_the_bits_of_the_parts(models, which, dtype):
             assert torch.equal(a[rid], b[rid]), rid
     refs = {rid: plain_llama_forward(cfg, w, toks) for rid, toks in reqs.items()}
     check(outs[0][1], refs, dtype, "recorded program, mixed")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_any_part_may_run_in_python_inside_the_program(models, dtype):
+    """The program's callback operation with Llama's own parts: one kind of part after the other is made to run in
+    Python in the middle of the recorded program (its operands are then finished tensors in the workspace, what it
+    returns is copied to its place), the rest stays native. In float32 every variant gives the bits of the model run
+    part by part; in bfloat16 a part that runs in Python takes finished tensors where its native form takes the
+    unfinished products of its neighbours (other kernels, other roundings), so there the plain implementation is
+    the yardstick. Under mixed steps with page reuse."""
+    from lmsf_amd.engine import load_engine_core
+    folder, cfg, w = models[("B", dtype)]
+    reqs = requests_for(cfg, "B")
+    longest = -(-max(len(t) for t in reqs.values()) // 64) * 64
+    steps = trace_mixed(reqs, longest + 128, seed=11)
+    bs = TINY["B"][2]
+
+    def run(python_parts):
+        core = load_engine_core(folder, dtype=dtype, block_size=bs, num_pages=(longest + 128) // bs, max_num_seqs=8,
+                                use_program=python_parts is not None, enforce_eager=True)
+        if python_parts:
+            core.executor.python_parts = python_parts
+            core.executor._record_program()
+            assert len(core.executor.program.callbacks) > 0
+        return replay_in_process(core.executor, steps), core.executor.program_steps
+
+    want, _ = run(None)
+    kinds = {"block": lambda p, n: type(p).__name__ == "PreNormResidualBlock" and p.prefix.endswith(".1"),
+             "mixer": lambda p, n: type(p).__name__ == "PagedAttention",
+             "feed-forward": lambda p, n: type(p).__name__ == "GatedMLP",
+             "norms": lambda p, n: type(p).__name__ == "RMSNorm" and n == "forward_add",
+             "embedding and head": lambda p, n: type(p).__name__ in ("TokenEmbedding", "LMHead"),
+             "a layer's linear parts": lambda p, n: type(p).__name__ in ("Linear", "FusedLinear") and ".layers.0." in p.prefix}
+    refs = {rid: plain_llama_forward(cfg, w, toks) for rid, toks in reqs.items()}
+    for name, pred in kinds.items():
+        got, steps_run = run(pred)
+        assert steps_run >= len(steps), name
+        if dtype == "float32":
+            for rid in reqs:
+                assert torch.equal(got[rid], want[rid]), (name, rid)
+        check(got, refs, dtype, "in Python: " + name)
+
+
+def test_a_switch_point_moved_between_two_mixed_steps(models):
+    """Somebody moves one of the kernels' switch points between two steps that hold a prompt's portion beside single
+    tokens: the program is recorded again before anything of the next step is built, and that step's attention
+    plan belongs to it (the plan's layout travels with the step, not with the program object). Against the model
+    run part by part under the same settings, bit for bit."""
+    from lmsf_amd.engine import load_engine_core
+    folder, cfg, w = models[("B", "bfloat16")]
+    V = cfg["vocab_size"]
+    toks = {r: random_tokens(70, V, 90 + i) for i, r in enumerate("abc")}
+
+    def run(use_program):
+        core = load_engine_core(folder, dtype="bfloat16", block_size=16, num_pages=24, max_num_seqs=4,
+                                use_program=use_program, enforce_eager=True)
+        ex, ops, outs = core.executor, core.rt.ops, []
+        was = ops.skinny_max_rows
+        try:
+            ex.step([StepEntry("a", toks["a"][:30], []), StepEntry("b", toks["b"][:50], [])])
+            first = ex.program
+            outs.append(ex.step([StepEntry("a", toks["a"][30:31], [0]), StepEntry("b", toks["b"][50:51], [0]),
+                                 StepEntry("c", toks["c"][:40], [39])]))
+            ops.skinny_max_rows = 8                       # 9 to 16 rows now go to the 17-and-more-rows kernel
+            outs.append(ex.step([StepEntry("a", toks["a"][31:32], [0]), StepEntry("b", toks["b"][51:52], [0]),
+                                 StepEntry("c", toks["c"][40:50], [9])]))
+            if use_program:
+                assert ex.program is not first and ex.program is not None
+        finally:
+            ops.skinny_max_rows = was
+        return [o.float().cpu() for o in outs]
+
+    a, b = run(True), run(False)
+    assert all(torch.equal(x, y) for x, y in zip(a, b))
+    ref = plain_llama_forward(cfg, w, toks["c"][:50])
+    check({"c": torch.stack([a[0][2], a[1][2]])}, {"c": ref[[39, 49]]}, "bfloat16", "after a switch point moved")
 
 
 @pytest.mark.parametrize("which", ["A", "B", "C", "W"])
