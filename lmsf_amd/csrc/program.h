@@ -116,6 +116,19 @@ typedef struct {
 // launches before it and after it; whatever it launches belongs on the step's stream.
 typedef int (*LmsfCallbackFn)(const LmsfCallbackArgs* args);
 
+// What the last step that ran launched, by kind (lmsf_program_stats): the routes of dispatch.h for the products
+// (plain, gated and QKV alike), then the kernels that take an unfinished product, then attention and callbacks.
+enum {
+  LMSF_STAT_NORM_OVER_PARTIALS = 16,
+  LMSF_STAT_ROPE_OVER_PARTIALS,
+  LMSF_STAT_REDUCE_PARTIALS,
+  LMSF_STAT_PREFILL_ATTENTION,
+  LMSF_STAT_DECODE_ATTENTION,
+  LMSF_STAT_GENERIC_ATTENTION,
+  LMSF_STAT_CALLBACK,
+  LMSF_STAT_COUNT
+};
+
 void* lmsf_program_create(const LmsfTunables* tunables);
 void lmsf_program_destroy(void* program);
 int lmsf_program_add(void* program, const LmsfOpDesc* op);
@@ -125,6 +138,7 @@ long lmsf_program_plan(void* program, int S, const int* seg_lens, const int* seg
                        LmsfPlanInfo* info);
 long lmsf_program_plan_capacity(void* program, int N);
 int lmsf_program_run(void* program, const LmsfStepDesc* step, int check_only, hipStream_t stream);
+int lmsf_program_stats(void* program, long* out, int capacity);
 
 #ifdef __cplusplus
 }

@@ -72,6 +72,7 @@ struct Program {
   LmsfTunables tun;
   std::vector<int> tile_sizes;      // the distinct tile sizes of the attention operations
   LmsfCallbackFn callback = nullptr;
+  mutable long stats[LMSF_STAT_COUNT] = {0};   // what the last step that ran launched
 };
 
 const int kLongLife = 12;   // a register read this many operations after it was written lives at the far end
@@ -88,6 +89,9 @@ struct Run {
   bool cur_long = false;
 
   char* base() const { return (char*)st->workspace; }
+  void count(int what) const {
+    if (!dry && what >= 0 && what < LMSF_STAT_COUNT) ++prog->stats[what];
+  }
 
   void release_dead() {
     while (!ring.empty() && (ring.front().reg < 0 || prog->last_use[ring.front().reg] < op_index)) ring.pop_front();
@@ -260,6 +264,7 @@ int op_linear(Run& r, const Value& x, const void* W, int wdtype, long ldw, int N
   const LmsfProductShape shape = shape_of(x.p, x.dtype, x.ld, M, K, W, wdtype, ldw, N, out_dtype);
   LmsfRoute rt;
   lmsf_route_linear(&t, &shape, pending_ok ? 1 : 0, &rt);
+  if (rt.route != LMSF_ROUTE_CHUNKS) r.count(rt.route);
   if (rt.route == LMSF_ROUTE_MID) return linear_mid(r, x, W, ldw, N, bias, 0, out_dtype, rt, out, res);
   if (rt.route == LMSF_ROUTE_LARGE) return linear_large(r, x, W, ldw, N, bias, 0, rt, out, res);
   if (rt.route == LMSF_ROUTE_DEFERRED) {
@@ -335,6 +340,7 @@ int materialize(Run& r, const Value& v, Value* res) {
   }
   if (v.kind == V_PENDING) {
     TAKE(y, void*, (size_t)v.M * v.N * esize(v.dtype));
+    r.count(LMSF_STAT_REDUCE_PARTIALS);
     LAUNCH(lmsf_gemm_mid_reduce(v.partials, v.bias, y, v.dtype, v.N, v.M, v.N, v.n_split, r.stream));
     *res = tensor(y, v.dtype, v.M, v.N);
     return 0;
@@ -355,6 +361,7 @@ int op_add_rms_norm(Run& r, const Value& branch_in, float* residual, int M, int 
     const bool fits = H % 4 == 0 && H <= 16384 && lmsf_aligned16(weight) && (residual == nullptr || lmsf_aligned16(residual));
     if (fits && branch.N == H) {
       TAKE(out, void*, (size_t)n_out * H * esize(out_dtype));
+      r.count(LMSF_STAT_NORM_OVER_PARTIALS);
       LAUNCH(lmsf_add_rms_norm_partial(branch.partials, branch.bias, branch.n_split, branch.M, residual, weight, wdtype,
                                        out, out_dtype, rows, n_out, H, eps, weight_offset, r.stream));
       *res = tensor(out, out_dtype, n_out, H);
@@ -370,6 +377,7 @@ int op_add_rms_norm(Run& r, const Value& branch_in, float* residual, int M, int 
     const bool prepares = fits && defer_ok && out_dtype == LMSF_BF16 && wdtype == LMSF_BF16;
     LmsfRoute rt;
     lmsf_route_deferred_norm(&t, Mb, N, K, fits ? 1 : 0, prepares ? 1 : 0, &rt);
+    if (rt.route != LMSF_ROUTE_MATERIALIZE) r.count(rt.route);
     if (rt.route == LMSF_ROUTE_GEMV_ADD_NORM || rt.route == LMSF_ROUTE_SKINNY_ADD_NORM) {
       const bool one_or_two = rt.route == LMSF_ROUTE_GEMV_ADD_NORM;
       const int tiles = one_or_two ? lmsf_gemv_partials(N) : (N + 15) / 16;
@@ -435,6 +443,7 @@ int op_linear_gated(Run& r, const Value& x_in, const void* W, int wdtype, long l
     const LmsfProductShape shape = shape_of(x.p, x.dtype, x.ld, x.M, x.N, W, wdtype, ldw, w_rows, LMSF_BF16);
     lmsf_route_linear_gated(&t, &shape, x.rows_per_tile, x.tiles, &rt);
     if (rt.route != LMSF_ROUTE_MATERIALIZE) {
+      r.count(rt.route);
       const int M = x.M, K = x.N;
       TAKE(y, void*, (size_t)M * I * 2);
       if (rt.route == LMSF_ROUTE_MID_SCALED)
@@ -456,6 +465,7 @@ int op_linear_gated(Run& r, const Value& x_in, const void* W, int wdtype, long l
   const int M = x.M, K = x.N;
   const LmsfProductShape shape = shape_of(x.p, x.dtype, x.ld, M, K, W, wdtype, ldw, w_rows, x.dtype);
   lmsf_route_linear_gated(&t, &shape, 0, 0, &rt);
+  if (rt.route != LMSF_ROUTE_SEPARATE) r.count(rt.route);
   if (rt.route == LMSF_ROUTE_GEMV || rt.route == LMSF_ROUTE_SKINNY) {
     TAKE(y, void*, (size_t)M * I * 2);
     if (rt.route == LMSF_ROUTE_GEMV)
@@ -504,6 +514,7 @@ int op_qkv_rope_cache(Run& r, const Value& x_in, const LmsfOpDesc& op, const int
     const LmsfProductShape shape = shape_of(x.p, x.dtype, x.ld, M, K, op.w, op.wdtype, op.ldw, op.N, LMSF_BF16);
     lmsf_route_qkv(&t, &shape, fused_shape(K) ? 1 : 0, x.rows_per_tile, &rt);
     if (rt.route != LMSF_ROUTE_MATERIALIZE) {
+      r.count(rt.route);
       TAKE(y, void*, (size_t)M * N * 2);
       if (rt.route == LMSF_ROUTE_GEMV_SCALED)
         LAUNCH(lmsf_gemv_scaled_qkv_rope_cache(x.p, x.ld, op.w, op.ldw, op.bias, y, N, M, K, positions, table,
@@ -525,6 +536,7 @@ int op_qkv_rope_cache(Run& r, const Value& x_in, const LmsfOpDesc& op, const int
   const int M = x.M, K = x.N;
   const LmsfProductShape shape = shape_of(x.p, x.dtype, x.ld, M, K, op.w, op.wdtype, op.ldw, op.N, x.dtype);
   lmsf_route_qkv(&t, &shape, fused_shape(K) ? 1 : 0, 0, &rt);
+  if (rt.route != LMSF_ROUTE_SEPARATE) r.count(rt.route);
   if (rt.route == LMSF_ROUTE_GEMV || rt.route == LMSF_ROUTE_SKINNY) {
     TAKE(y, void*, (size_t)M * N * 2);
     if (rt.route == LMSF_ROUTE_GEMV)
@@ -552,6 +564,7 @@ int op_qkv_rope_cache(Run& r, const Value& x_in, const LmsfOpDesc& op, const int
     }
     TAKE(out, void*, (size_t)M * N * 2);
     const bool rot = table != nullptr;
+    r.count(LMSF_STAT_ROPE_OVER_PARTIALS);
     LAUNCH(lmsf_rope_cache_write_partial(y.partials, y.bias, y.n_split, out, N, M, rot ? positions : nullptr, table,
                                          rot ? op.rot : 0, op.neox, rot ? op.max_pos : 0, slots,
                                          slots ? op.k_pages : nullptr, slots ? op.v_pages : nullptr,
@@ -598,6 +611,7 @@ int op_attention(Run& r, const Value& q, const LmsfOpDesc& op, const int* tables
   const bool fast_ok = q.dtype == LMSF_BF16 && d % 16 == 0 && 16 <= d && d <= 256 && ps % 4 == 0 && q.ld % 8 == 0 &&
                        lmsf_aligned16(q.p) && op.scale > 0.f;
   if (!fast_ok) {
+    r.count(LMSF_STAT_GENERIC_ATTENTION);
     LAUNCH(lmsf_paged_attention_generic(q.p, q.ld, out, (long)nh * d, op.k_pages, op.v_pages, op.num_pages, tables, width,
                                         st.seg_of, st.positions, N, nh, nkv, d, ps, op.scale, op.window, q.dtype,
                                         r.stream));
@@ -627,6 +641,8 @@ int op_attention(Run& r, const Value& q, const LmsfOpDesc& op, const int* tables
     tiles = n_tiles ? st.plan + info.tiles_at[at] : nullptr;
     single = n_single ? st.plan + info.single_at[at] : nullptr;
   }
+  if (n_tiles) r.count(LMSF_STAT_PREFILL_ATTENTION);
+  if (n_single) r.count(LMSF_STAT_DECODE_ATTENTION);
   if (n_tiles)
     LAUNCH(lmsf_paged_attention_prefill_mfma(q.p, q.ld, out, (long)nh * d, op.k_pages, op.v_pages, op.num_pages, tables,
                                              width, tiles, n_tiles, st.seg_of, st.positions, nh, nkv, d, ps, op.scale,
@@ -803,6 +819,7 @@ int run_pass(const Program& prog, const LmsfStepDesc& st, hipStream_t stream, bo
           res = tensor(y, op.out_dtype, rows, op.N);
         }
         args.out = ref(res);
+        r.count(LMSF_STAT_CALLBACK);
         if (!r.dry && prog.callback(&args) != 0) {
           lmsf_set_error("program: callback %d failed", op.callback_id);
           return 1;
@@ -954,5 +971,15 @@ extern "C" int lmsf_program_run(void* program, const LmsfStepDesc* step, int che
   LMSF_CHECK(!step->all_single || step->longest_first, "program_run: a step of single tokens carries their order");
   const int rc = run_pass(*p, *step, stream, true);
   if (rc != 0 || check_only) return rc;
+  std::fill(p->stats, p->stats + LMSF_STAT_COUNT, 0L);
   return run_pass(*p, *step, stream, false);
+}
+
+// What the last step that ran launched, by kind (the indices of program.h); returns how many were written.
+extern "C" int lmsf_program_stats(void* program, long* out, int capacity) {
+  const Program* p = static_cast<const Program*>(program);
+  if (!p || !out) return 0;
+  const int n = std::min(capacity, (int)LMSF_STAT_COUNT);
+  std::copy(p->stats, p->stats + n, out);
+  return n;
 }

@@ -23,27 +23,13 @@ from .scheduler import Scheduler, SchedulerConfig, StepPlan
 from .sequence import Sequence, SequenceState
 
 
-class _SeqSet:
-    """Sequences by identity."""
-
-    def __init__(self, ids):
-        self._ids = set(ids)
-
-    def __contains__(self, seq) -> bool:
-        return id(seq) in self._ids
-
-    def __bool__(self) -> bool:
-        return bool(self._ids)
-
-
 class _InFlight:
     """A step that has been launched: its plan, the requests it samples for and where their tokens will be."""
 
-    __slots__ = ("plan", "sampled", "tokens_dev", "t_start", "pending_of", "host_tokens", "event")
+    __slots__ = ("plan", "sampled", "tokens_dev", "t_start", "host_tokens", "event")
 
-    def __init__(self, plan, sampled, tokens_dev, t_start, pending_of):
+    def __init__(self, plan, sampled, tokens_dev, t_start):
         self.plan, self.sampled, self.tokens_dev, self.t_start = plan, sampled, tokens_dev, t_start
-        self.pending_of = pending_of      # requests whose token of the step before this step took from the device
         self.host_tokens = None
         self.event = None
 
@@ -76,6 +62,7 @@ class LLMEngine:
         # one step may be in flight on the GPU while the host prepares the next (see ``step``)
         self.run_ahead = bool(getattr(args, "run_ahead", True))
         self._inflight: Optional[_InFlight] = None
+        self._undelivered: List[RequestOutput] = []          # outputs finished by a step() that then raised
         self._token_slots = [[None, None], [None, None]]     # pinned buffer and event, two steps in turn
         self._token_turn = 0
 
@@ -138,7 +125,7 @@ class LLMEngine:
         self._requests.pop(request_id, None)
 
     def has_unfinished_requests(self) -> bool:
-        return self.scheduler.has_unfinished()
+        return self.scheduler.has_unfinished() or bool(self._undelivered)
 
     def get_num_unfinished_requests(self) -> int:
         return self.scheduler.num_unfinished()
@@ -157,7 +144,9 @@ class LLMEngine:
         an end-of-sequence token or a stop string has one more token computed for nothing, which is dropped.
         A step is not launched ahead when a request of the step before reaches its length limit with the token
         being sampled, or uses penalties (which count the tokens on the host)."""
-        outputs: List[RequestOutput] = []
+        # (what a step that failed half-way had already finished comes first)
+        outputs: List[RequestOutput] = self._undelivered
+        self._undelivered = []
         if self._inflight is None:
             self._inflight = self._launch(outputs, None)
             if self._inflight is None:
@@ -170,8 +159,13 @@ class LLMEngine:
             try:
                 ahead = self._launch(outputs, cur)
             except BaseException:
+                # the step ahead failed; the one in flight is sound: its tokens are read and its outputs kept for
+                # the caller's next step(), with whatever the failed launch had already finished (ignored prompts)
                 for seq in cur.sampled:
                     seq.pending = 0
+                self._inflight = None
+                self._finish(cur, outputs)
+                self._undelivered = outputs
                 raise
         self._finish(cur, outputs)
         self._inflight = ahead if self.scheduler.has_unfinished() else None
@@ -229,7 +223,7 @@ class LLMEngine:
         rows = [SamplingRow(seq.params, seq.seed, len(seq.output_token_ids) + seq.pending, seq.prompt_token_ids,
                             seq.output_token_ids) for seq in sampled]
         tokens_dev = self.sampler.sample_on_device(logits, rows)
-        rec = _InFlight(plan, sampled, tokens_dev, t_start, _SeqSet(pending_of))
+        rec = _InFlight(plan, sampled, tokens_dev, t_start)
         if tokens_dev is not None and tokens_dev.is_cuda:
             # the tokens travel to pinned memory behind the sampler, ahead of whatever is launched next; the
             # event says when they are there

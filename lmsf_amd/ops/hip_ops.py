@@ -539,14 +539,14 @@ class HipOps:
         if len(single) == len(lens):
             plan = _AttentionPlan(None, 0, None, len(single), max_context)
         else:
-            both = self._upload_ints(tiles + single, dev)
+            both = self.upload_ints(tiles + single, dev)
             plan = _AttentionPlan(both[:len(tiles)], len(tiles) // 2,
                                   both[len(tiles):] if single else None, len(single), max_context)
         if aux is not None:
             aux[key] = plan
         return plan
 
-    def _upload_ints(self, values, dev: torch.device) -> torch.Tensor:
+    def upload_ints(self, values, dev: torch.device) -> torch.Tensor:
         """int32 values to the device through pinned memory, without waiting for the copy. Four buffers take
         turns; before a buffer is written again its last copy's event is waited for (long past, as a rule)."""
         n = len(values)

@@ -85,6 +85,7 @@ _SIGNATURES = {
     "lmsf_program_plan": (c_long, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_long, POINTER(PlanInfo)]),
     "lmsf_program_plan_capacity": (c_long, [c_void_p, c_int]),
     "lmsf_program_run": (c_int, [c_void_p, POINTER(StepDesc), c_int, c_void_p]),
+    "lmsf_program_stats": (c_int, [c_void_p, POINTER(c_long), c_int]),
 }
 
 
@@ -446,6 +447,18 @@ class StepProgram:
     def stale(self) -> bool:
         """True once somebody has changed the kernels' switch points since the recording (tests, tuning)."""
         return self.tunables != self.hip_ops.tunables()
+
+    STAT_NAMES = ("plain", "mid", "large", "deferred", "gemv", "chunks", "skinny", "blas", "materialize", "mid_scaled",
+                  "gemv_scaled", "skinny_scaled", "separate", "gemv_add_norm", "skinny_add_norm", "gemv_add",
+                  "norm_over_partials", "rope_over_partials", "reduce_partials", "prefill_attention",
+                  "decode_attention", "generic_attention", "callback")
+
+    def last_step_stats(self) -> dict:
+        """What the last step that ran launched, by kind: the products by their routes (csrc/dispatch.h), the
+        kernels that took an unfinished product, the attention kernels, the callbacks."""
+        out = (c_long * len(self.STAT_NAMES))()
+        n = self.lib.lmsf_program_stats(self.handle, out, len(self.STAT_NAMES))
+        return {name: int(out[i]) for i, name in enumerate(self.STAT_NAMES[:n]) if out[i]}
 
     def plan_capacity(self, n_tokens: int) -> int:
         return int(self.lib.lmsf_program_plan_capacity(self.handle, n_tokens))

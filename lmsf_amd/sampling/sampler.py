@@ -34,7 +34,12 @@ class Sampler:
         self.device = device
 
     def _upload(self, words: "np.ndarray") -> torch.Tensor:
-        """One copy to the device for everything a call needs: int32 words, float32 values as their bits."""
+        """One copy to the device for everything a call needs: int32 words, float32 values as their bits. Through
+        the kernels' pinned buffers where there are any (they take turns behind events), so that the host does not
+        wait for the step that is computing."""
+        upload = getattr(self.ops, "upload_ints", None)
+        if upload is not None and self.device.type == "cuda":
+            return upload(words, self.device)
         return torch.from_numpy(words).to(self.device, non_blocking=False)
 
     def sample(self, logits: torch.Tensor, rows: Sequence[SamplingRow]) -> List[int]:

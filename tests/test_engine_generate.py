@@ -177,3 +177,50 @@ def test_a_prompt_that_is_too_long_is_ignored_with_a_warning(tmp_path, capsys):
     assert len(done["fits"].outputs[0].token_ids) == 4
     err = capsys.readouterr().err
     assert "'long'" in err and "40 tokens" in err and "too long" in err and "'fits'" not in err
+
+
+def test_a_step_ahead_that_fails_loses_no_token_and_no_output(tmp_path):
+    """The step launched ahead raises (here: the step function refuses it). The step in flight is sound: its tokens
+    are appended, its outputs come with the caller's next step(), nothing is counted twice, and the run ends with the
+    tokens of an undisturbed run and every page back."""
+    from lmsf_amd.engine.executor import StepError
+    engine, folder, cfg = make_engine(tmp_path, "A", prefill_chunk_size=16)
+    calm, _, _ = make_engine(tmp_path, "A", prefill_chunk_size=16)
+    prompts = [random_tokens(n, cfg.vocab_size, 80 + n) for n in (9, 21)]
+    for e in (engine, calm):
+        for i, p in enumerate(prompts):
+            e.add_request(i, p, SamplingParams(temperature=0.0, max_tokens=6, ignore_eos=True))
+    want = {i: o.outputs[0].token_ids for i, o in run(calm).items()}
+    real_step, calls, failed = engine.core.executor.step, [0], [0]
+
+    def flaky(entries, prev_tokens=None):
+        calls[0] += 1
+        if calls[0] in (3, 5):                                   # steps launched ahead of the one in flight
+            failed[0] += 1
+            raise StepError("refused for the test")
+        return real_step(entries, prev_tokens=prev_tokens)
+
+    engine.core.executor.step = flaky
+    done, seen = {}, {0: [], 1: [], "too long": []}
+    while engine.has_unfinished_requests():
+        if calls[0] == 2 and "too long" not in engine._requests and "too long" not in done:
+            # a prompt that the scheduler ignores, in the very step whose launch then fails: its output was collected
+            # before the failure and must not be lost with it
+            engine.add_request("too long", random_tokens(cfg.max_position_embeddings + 5, cfg.vocab_size, 3),
+                               SamplingParams(temperature=0.0, max_tokens=2))
+        try:
+            outs = engine.step()
+        except StepError:
+            engine.core.storage.manager.check_invariants()
+            continue
+        for out in outs:
+            seen[out.request_id].append(out.outputs[0].latest_token)
+            if out.finished:
+                done[out.request_id] = out
+    assert failed[0] == 2
+    assert done.pop("too long").outputs[0].finish_reason == "length" and seen.pop("too long") == [None]
+    assert {i: o.outputs[0].token_ids for i, o in done.items()} == want
+    # every token of every request was reported exactly once, in order: no output lost, none twice
+    assert seen == want
+    engine.core.storage.manager.check_invariants()
+    assert engine.core.storage.manager.num_free_pages(0) == 64

@@ -43,7 +43,7 @@ def test_llm_generate_bfloat16_follows_plain_argmax(tmp_path):
         assert len(gen) == 12
         logits = plain_llama_forward(cfg_dict, w, p + gen[:-1])[len(p) - 1:]
         for i, tok in enumerate(gen):
-            assert logits[i, tok] >= logits[i].max() - 0.05 * logits[i].abs().max(), (len(p), i)
+            assert logits[i, tok] >= logits[i].max() - 1.5e-2 * max(0.25, logits[i].abs().max().item()), (len(p), i)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

@@ -128,6 +128,17 @@ def test_wide_model_leaves_products_unfinished(models, monkeypatch):
     got2 = replay_in_process(core.executor, steps)
     assert seen == {"norm": 2 * L, "rope": L}
     check({"a": torch.cat([got["a"], got2["a"]])}, {"a": ref}, "bfloat16", "wide")
+    # the recorded program says what it launched itself: the same choices
+    core = engine(folder, "W", "bfloat16", num_pages=8)
+    prog = core.executor.program
+    core.executor.step([StepEntry("a", toks[:40], list(range(40)))])
+    stats = prog.last_step_stats()
+    assert stats["norm_over_partials"] == 2 * L and stats["rope_over_partials"] == L and stats["prefill_attention"] == L
+    assert stats["mid"] >= 3 * L and "blas" not in stats and "callback" not in stats
+    core.executor.step([StepEntry("a", toks[40:], list(range(8)))])
+    stats = prog.last_step_stats()
+    # (8 rows: the norms run inside the products around them, but for the last, which picks the wanted rows)
+    assert "norm_over_partials" not in stats and "rope_over_partials" not in stats and stats["skinny_add_norm"] == 2 * L - 1
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
