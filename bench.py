@@ -44,7 +44,7 @@ def make_engine(cfg, args, max_num_seqs, dtype, prefill_chunk_size=None):
     return LLMEngine(EngineArgs(model=folder, dtype=dtype, block_size=getattr(args, "block_size", 16), load_format="random", seed=0,
                                 max_num_seqs=max_num_seqs, max_num_batched_tokens=args.max_num_batched_tokens,
                                 gpu_memory_utilization=args.gpu_memory_utilization,
-                                prefill_chunk_size=prefill_chunk_size))
+                                prefill_chunk_size=prefill_chunk_size, tune_products=not getattr(args, "no_tune", False)))
 
 
 def weight_bytes(engine):
@@ -107,6 +107,9 @@ def prefill_run(engine, n_tokens, reps, seed):
     rng = random.Random(seed)
     V = engine.core.config.vocab_size
     times = []
+    if getattr(engine.args, "tune_products", False):
+        # the library's candidates for this step's products race first, as the engine does at load for its full step
+        engine.core.executor.tune_products([n_tokens])
     for r in range(reps + 1):
         toks = [rng.randrange(V) for _ in range(n_tokens)]
         torch.cuda.synchronize()
@@ -341,6 +344,9 @@ def main():
                     help="set an attribute of ops.HipOps (a number of rows at which kernels change, a variant) first")
     ap.add_argument("--points", default="1,64,128", help="decode: further batch sizes, comma separated")
     ap.add_argument("--block-size", type=int, default=16, help="tokens a page of the cache")
+    ap.add_argument("--no-tune", action="store_true",
+                    help="leave the BLAS library's choice of algorithm as it is (default: its candidates race for the "
+                         "shapes of the prefill steps, as EngineArgs.tune_products does at load)")
     ap.add_argument("--max-context", type=int, default=None,
                     help="decode: positions the model allows, for --prompt-len beyond the shape's own "
                          "(--batch 1 --prompt-len 120000 --max-context 131072 --skip-points)")

@@ -37,6 +37,7 @@ class EngineArgs:
     num_gpu_blocks_override: Optional[int] = None
     enforce_eager: bool = False                    # True: never capture decode steps as HIP graphs
     run_ahead: bool = True                         # False: never launch a step before the tokens of the one before are read
+    tune_products: bool = False                    # True: at load, the BLAS library's candidates race for the products of a full step
     keep_float32_weights: bool = False             # True: matrices stored in 32 bits are not cast to a bfloat16 run's type
     skip_tokenizer_init: bool = False              # True: work on token ids even if the folder has a tokenizer.json
     device: str = "cuda:0"
@@ -83,6 +84,10 @@ class EngineArgs:
         a("--no-run-ahead", dest="run_ahead", action="store_false",
           help="launch a step only after the tokens of the step before it have been read")
         a("--skip-tokenizer-init", action="store_true", help="do not load the folder's tokenizer.json")
+        a("--tune-products", action="store_true",
+          help="at load, time the BLAS library's candidate algorithms for the matrix products of a step of "
+               "--max-num-batched-tokens tokens (and of --prefill-chunk-size) on the model's own weights and keep the "
+               "fastest of each")
         a("--keep-float32-weights", action="store_true",
           help="with --dtype bfloat16, leave matrices that the checkpoint stores in 32 bits as they are (their "
                "products then run in float32 arithmetic, at twice the memory) instead of casting them at load")

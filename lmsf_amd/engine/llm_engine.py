@@ -50,6 +50,11 @@ class LLMEngine:
                                    self.core.storage.manager)
         self.sampler = Sampler(self.core.rt.ops, self.core.rt.device)
         self.eos_token_ids = set(self.core.config.eos_token_ids)
+        if args.tune_products and self.core.rt.device.type == "cuda":
+            # the shapes of a full step's products, as the reference profiles cuBLASLt's tactics per weight shape
+            # and bucket of rows (tops/src/cublas.rs:121-223)
+            self.tuned_products = self.core.executor.tune_products(
+                sorted({budget, min(budget, args.prefill_chunk_size or budget)}))
         self.tokenizer = None if args.skip_tokenizer_init else load_tokenizer(args.model)
         self._arrivals = 0
         self._requests: Dict[Hashable, Sequence] = {}
