@@ -8,8 +8,9 @@ then exactly K decode steps are timed between device synchronisations; every ste
 itself with HIP events and the median is reported. The same line carries the prefill of 2,048 tokens,
 the decode step's share of the HBM roofline with the machine's measured rates beside the published
 peaks, and ``points``: decode at batch 1, 64 and 128, at 8,000 tokens of context, a 512-token prompt,
-a mixed step (8 decoding requests beside a 32-token portion of a prompt) and continuous batching of
-64 requests at Llama-2-7B shape. Weights are random (N(0, 0.02), bfloat16, made on the device),
+a mixed step (8 decoding requests beside a 32-token portion of a prompt), continuous batching of
+64 requests at Llama-2-7B shape, decode at 32,000 tokens of context, a small model (Llama-3.2-1B sizes) and
+the Llama-3.1-70B sizes at all 80 layers (each from an engine of its own, built and dropped in turn). Weights are random (N(0, 0.02), bfloat16, made on the device),
 token ids are seeded uniform-random. The reference publishes no numbers, so vs_baseline is null.
 """
 import argparse
@@ -28,6 +29,8 @@ if ROOT not in sys.path:
 HBM_BYTES_PER_S = 8.0e12
 PEAK_FLOPS = {"bf16": 2.5e15, "fp16": 2.5e15, "fp8": 5.0e15, "fp32": 157.3e12}
 
+TUNE_PRODUCTS = True      # --no-tune: the BLAS library's own choice of algorithm for the prefill steps' products
+
 LLAMA3_8B = dict(
     architectures=["LlamaForCausalLM"], model_type="llama", vocab_size=128256, hidden_size=4096,
     intermediate_size=14336, num_hidden_layers=32, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
@@ -44,7 +47,7 @@ def make_engine(cfg, args, max_num_seqs, dtype, prefill_chunk_size=None):
     return LLMEngine(EngineArgs(model=folder, dtype=dtype, block_size=getattr(args, "block_size", 16), load_format="random", seed=0,
                                 max_num_seqs=max_num_seqs, max_num_batched_tokens=args.max_num_batched_tokens,
                                 gpu_memory_utilization=args.gpu_memory_utilization,
-                                prefill_chunk_size=prefill_chunk_size, tune_products=not getattr(args, "no_tune", False)))
+                                prefill_chunk_size=prefill_chunk_size))
 
 
 def weight_bytes(engine):
@@ -107,8 +110,9 @@ def prefill_run(engine, n_tokens, reps, seed):
     rng = random.Random(seed)
     V = engine.core.config.vocab_size
     times = []
-    if getattr(engine.args, "tune_products", False):
-        # the library's candidates for this step's products race first, as the engine does at load for its full step
+    if TUNE_PRODUCTS:
+        # the library's candidates for this step's products race first, as the engine does at load for its full
+        # step with EngineArgs.tune_products
         engine.core.executor.tune_products([n_tokens])
     for r in range(reps + 1):
         toks = [rng.randrange(V) for _ in range(n_tokens)]
@@ -309,6 +313,67 @@ def products_run(args):
             del a, b
 
 
+def further_shape_points(args, points, peak):
+    """Points at other sizes than the headline's, each from an engine of its own that is built and dropped in
+    turn: decode at 32,000 tokens of context (batch 8, the headline shape with room for such contexts), a small
+    model (Llama-3.2-1B sizes: launches count) at batch 1 and 64, and the Llama-3.1-70B sizes at all 80 layers
+    (141 GB of weights) at batch 1 and 8 with a 2,048-token prefill. Every rate comes with its share of the roofline."""
+    import gc
+    import torch
+
+    def with_engine(cfg, max_seqs, fn, utilization=None):
+        a = argparse.Namespace(**vars(args))
+        if utilization:
+            a.gpu_memory_utilization = utilization
+        try:
+            engine = make_engine(cfg, a, max_num_seqs=max_seqs, dtype=args.dtype)
+        except Exception as e:  # noqa: BLE001 - a point that cannot be measured is named, the line is still printed
+            return "%s: %s" % (type(e).__name__, str(e)[:160])
+        try:
+            fn(engine)
+        finally:
+            del engine
+            gc.collect()
+            torch.cuda.synchronize()
+            torch.cuda.empty_cache()
+        return None
+
+    es = 2 if args.dtype == "bfloat16" else 4
+
+    def decode_point(engine, cfg, name, batch, prompt_len, steps, warmup, seed):
+        kv = 2 * cfg["num_key_value_heads"] * cfg["head_dim"] * cfg["num_hidden_layers"] * es
+        d, ctx = decode_run(engine, batch, prompt_len, steps, warmup, seed=seed)
+        points[name] = round(batch * steps / d, 1)
+        points[name + "_hbm_frac"] = round((weight_bytes(engine) + batch * ctx * kv) / (d / steps) / HBM_BYTES_PER_S, 4)
+
+    long_cfg = dict(LLAMA3_8B, max_position_embeddings=32768 + 64)
+    err = with_engine(long_cfg, 8, lambda e: decode_point(e, long_cfg, "decode_b8_ctx32000", 8, 32000, 16, 4, 71))
+    if err:
+        points["decode_b8_ctx32000_error"] = err
+
+    small = dict(LLAMA32_1B)
+
+    def small_points(e):
+        decode_point(e, small, "llama1b_decode_b1", 1, 512, 32, 8, 72)
+        decode_point(e, small, "llama1b_decode_b64", 64, 512, 32, 8, 73)
+    err = with_engine(small, 64, small_points)
+    if err:
+        points["llama1b_error"] = err
+
+    big = dict(LLAMA31_70B)
+
+    def big_points(e):
+        points["llama70b_layers"] = big["num_hidden_layers"]
+        decode_point(e, big, "llama70b_decode_b1", 1, 512, 12, 3, 74)
+        decode_point(e, big, "llama70b_decode_b8", 8, 512, 12, 3, 75)
+        t = prefill_run(e, 2048, reps=3, seed=76)
+        points["llama70b_prefill_2048_tok_s"] = round(2048 / t, 1)
+        points["llama70b_prefill_2048_frac"] = round(prefill_flops(big, 2048) / t / peak, 4)
+    err = with_engine(big, 8, big_points, utilization=0.9)
+    if err:
+        points["llama70b_error"] = err
+
+
 def prefill_flops(cfg, T):
     """Multiply-adds times two of a causal prefill of T tokens: the linear layers on every token, the
     attention scores and values over the causal half, the LM head on one row."""
@@ -355,6 +420,8 @@ def main():
         print("bench.py: this engine runs on one GPU; --gpus %d is not supported" % args.gpus)
         sys.exit(2)
 
+    global TUNE_PRODUCTS
+    TUNE_PRODUCTS = not args.no_tune
     if args.tunable:
         from lmsf_amd.ops import get_ops
         ops = get_ops()
@@ -439,6 +506,7 @@ def main():
             points["serve_total_tok_s"] = serve["config"]["total_tok_per_s"]
             points["serve_ms_per_step"] = serve["ms_per_step"]
             points["serve_preemptions"] = serve["config"]["preemptions"]
+            further_shape_points(args, points, peak)
 
     line = {
         "metric": "decode tok/s at batch %d (%s %s)" % (args.batch, shape_name, "bf16" if args.dtype == "bfloat16" else "fp32"),
