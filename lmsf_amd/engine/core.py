@@ -168,7 +168,10 @@ def load_engine_core(model_dir: Optional[str], dtype: Optional[str] = None, bloc
     else:
         counts = [int(num_pages)] * len(groups)
     storage = CacheStorage(model, rt, block_size, counts, num_state_slots=max_num_seqs)
+    # (a step never holds more tokens than the pools that keep every key have room for: the program's workspace is
+    # sized for that many at most)
+    room = [c * block_size for c, g in zip(counts, groups) if g.spec.window is None]
     executor = ModelExecutor(model, storage, rt, max_model_len, use_graphs=not enforce_eager,
-                             use_program=use_program, max_step_tokens=max_num_batched_tokens,
+                             use_program=use_program, max_step_tokens=min([max_num_batched_tokens] + room),
                              max_step_seqs=max_num_seqs)
     return EngineCore(arch, config, rt, model, storage, executor, max_model_len, block_size)
