@@ -326,3 +326,19 @@ def test_top_k_top_p_min_p():
     p = P.plain_sampling_distribution(x, temperature=0.5, top_k=3)
     want = torch.tensor([0.25, 0.0625, 0.015625, 0, 0])
     assert torch.allclose(p, want / want.sum(), atol=1e-6)
+
+
+def test_the_noise_generator_is_philox4x32_10():
+    """The counter-based generator behind the sampler's noise (tests/torch_ops.py, which the kernel's draws are
+    compared with bit for bit on the GPU) against the algorithm's published known answers: the first output word
+    for three (counter, key) pairs (all zeros; all ones; digits of pi). A wrong multiplier, key schedule, round
+    count or word order fails all three."""
+    import numpy as np
+    from torch_ops import _philox_first
+
+    def first(c, k):
+        return int(_philox_first(np.array([c[0]], dtype=np.uint64), c[1], k[0], k[1], c[2], c[3])[0])
+
+    assert first((0, 0, 0, 0), (0, 0)) == 0x6627E8D5
+    assert first((0xFFFFFFFF,) * 4, (0xFFFFFFFF,) * 2) == 0x408F276D
+    assert first((0x243F6A88, 0x85A308D3, 0x13198A2E, 0x03707344), (0xA4093822, 0x299F31D0)) == 0xD16CFE09

@@ -16,14 +16,14 @@ import torch
 
 # ---------------------------------------------------------------- counter-based noise (same as sampling.hip)
 
-def _philox_first(c0, c1, k0, k1):
-    """First output word of Philox4x32-10 for counters (c0, c1, 0, 0) and key (k0, k1); numpy uint64 maths."""
+def _philox_first(c0, c1, k0, k1, c2=0, c3=0):
+    """First output word of Philox4x32-10 for counters (c0, c1, c2, c3) and key (k0, k1); numpy uint64 maths."""
     M0, M1 = np.uint64(0xD2511F53), np.uint64(0xCD9E8D57)
     mask = np.uint64(0xFFFFFFFF)
     c0 = c0.astype(np.uint64)
     c1 = np.full_like(c0, c1, dtype=np.uint64)
-    c2 = np.zeros_like(c0)
-    c3 = np.zeros_like(c0)
+    c2 = np.full_like(c0, c2, dtype=np.uint64)
+    c3 = np.full_like(c0, c3, dtype=np.uint64)
     k0 = np.uint64(k0)
     k1 = np.uint64(k1)
     for _ in range(10):
