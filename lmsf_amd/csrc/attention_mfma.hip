@@ -693,7 +693,15 @@ static int launch_prefill_dma(dim3 grid, hipStream_t stream, const bf16_t* q, lo
 // tokens of 1,150 keys with 32 kv heads. Nor two sets of fragments a wave, the next step's keys and values asked for
 // before this step is multiplied (the table's entries for the step after asked for first, since loads come back in
 // the order they were asked for): the same times at 64 and 128 tokens and at 8,000 keys, so it is not a wave's
-// waiting for its own loads that bounds the kernel at 4.4 to 4.9 TB/s there.)
+// waiting for its own loads that bounds the kernel at 4.4 to 4.9 TB/s there. Nor a form for steps of single tokens
+// that takes the unrotated QKV product (finished, or as the partial sums of a product that splits K), rotates its
+// queries itself and has the one wave whose keys include the token's own make, store and use that key and value
+// from its registers, so that no rotation kernel runs between product and attention: the same bits, but at 64
+// tokens of 585 keys 38.6 us from partial sums and 33.4 from a finished product against 27.2 + 5.4 for the two
+// kernels, at 128 tokens 77 and 66 against 51.6 + 6.3. With the chip's queues full of keys and values a trip to
+// memory takes about 5 us, and the trips that position -> table and product -> rotation add before the first
+// score, and slot -> key and value for the owning wave, cost more than the launch they save: 4 us for the queries
+// alone, 7 for the token's own key and value, nothing for the stores.)
 // FULL: the head size is DPAD itself (a multiple of 32); the loads and products of a step then run without a test
 // each for the part of DPAD beyond the head size (8 tokens of 585 keys: 12.3 -> 11.6 us with the reduction).
 // ROW8: a step's 32 keys are dealt so that a lane's eight scores are eight keys in a row (row c of score block b is
