@@ -9,7 +9,8 @@ itself with HIP events and the median is reported. The same line carries the pre
 the decode step's share of the HBM roofline with the machine's measured rates beside the published
 peaks, and ``points``: decode at batch 1, 64 and 128, at 8,000 tokens of context, a 512-token prompt,
 a mixed step (8 decoding requests beside a 32-token portion of a prompt), continuous batching of
-64 requests at Llama-2-7B shape, decode at 32,000 tokens of context, a small model (Llama-3.2-1B sizes) and
+64 requests at Llama-2-7B shape, decode at 32,000 tokens of context, 2,000 short requests with 512 running at a
+time, a small model (Llama-3.2-1B sizes) and
 the Llama-3.1-70B sizes at all 80 layers (each from an engine of its own, built and dropped in turn). Weights are random (N(0, 0.02), bfloat16, made on the device),
 token ids are seeded uniform-random. The reference publishes no numbers, so vs_baseline is null.
 """
@@ -350,6 +351,36 @@ def further_shape_points(args, points, peak):
     err = with_engine(long_cfg, 8, lambda e: decode_point(e, long_cfg, "decode_b8_ctx32000", 8, 32000, 16, 4, 71))
     if err:
         points["decode_b8_ctx32000_error"] = err
+
+    def short_requests(e):
+        """Thousands of short requests at once at the headline shape: 2,000 requests of 32 to 96 prompt tokens and
+        16 to 32 generated, 512 running at a time; every step holds the decoding requests beside the prompts of
+        those just admitted, about 1,500 tokens."""
+        from lmsf_amd.sampling import SamplingParams
+        rng = random.Random(5)
+        V = LLAMA3_8B["vocab_size"]
+
+        def load(n_req, tag):
+            for i in range(n_req):
+                prompt = [rng.randrange(V) for _ in range(rng.randint(32, 96))]
+                e.add_request("%s%d" % (tag, i), prompt,
+                              SamplingParams(temperature=0.0, max_tokens=rng.randint(16, 32), ignore_eos=True))
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            steps = generated = 0
+            while e.has_unfinished_requests():
+                generated += len(e.step())
+                steps += 1
+            torch.cuda.synchronize()
+            return time.perf_counter() - t0, steps, generated
+        load(16, "w")
+        dt, steps, generated = load(2000, "q")
+        points["short_requests_tok_s"] = round(generated / dt, 1)
+        points["short_requests_running"] = 512
+        points["short_requests_ms_per_step"] = round(dt / steps * 1e3, 3)
+    err = with_engine(dict(LLAMA3_8B), 512, short_requests)
+    if err:
+        points["short_requests_error"] = err
 
     small = dict(LLAMA32_1B)
 
