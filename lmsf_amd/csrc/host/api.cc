@@ -7,6 +7,7 @@
 
 #include "cache_manager.h"
 #include "llama_config.h"
+#include "safetensors.h"
 #include "scheduler.h"
 
 using namespace lmsf;
@@ -34,7 +35,7 @@ static thread_local std::string g_error;
 
 extern "C" {
 
-int lmsf_host_abi_version() { return 3; }
+int lmsf_host_abi_version() { return 4; }
 const char* lmsf_host_last_error() { return g_error.c_str(); }
 
 // ---------------------------------------------------------------- a page pool alone
@@ -332,6 +333,47 @@ int lmsf_rope_scaling_parse(const char* rope_scaling_json, LmsfRopeScaling* out)
   if (!rope_scaling_json || !out) fail(kValueError, "bad arguments");
   rope_scaling_parse(rope_scaling_json, out);
   LMSF_API_END
+}
+
+// ---------------------------------------------------------------- checkpoint files
+
+// One tensor of a safetensors file. ``name`` points into the file object and lives as long as it does.
+typedef struct {
+  const char* name;
+  char dtype[8];
+  int ndim;
+  int64_t shape[8];
+  int64_t begin, end;   // bytes from the start of the data section
+} LmsfTensorRecord;
+
+int lmsf_safetensors_open(const char* path, void** out) {
+  LMSF_API_BEGIN
+  if (!path || !out) fail(kValueError, "bad arguments");
+  *out = new SafetensorsFile(path);
+  LMSF_API_END
+}
+void lmsf_safetensors_close(void* file) { delete static_cast<SafetensorsFile*>(file); }
+int64_t lmsf_safetensors_count(void* file) { return (int64_t) static_cast<SafetensorsFile*>(file)->tensors().size(); }
+int lmsf_safetensors_record(void* file, int64_t index, LmsfTensorRecord* out) {
+  LMSF_API_BEGIN
+  const auto& all = static_cast<SafetensorsFile*>(file)->tensors();
+  if (!out || index < 0 || index >= (int64_t)all.size()) fail(kValueError, "bad arguments");
+  const TensorRecord& r = all[(size_t)index];
+  if (r.shape.size() > 8) fail(kValueError, "tensor '%s' has %zu dimensions (at most 8)", r.name.c_str(), r.shape.size());
+  out->name = r.name.c_str();
+  std::memset(out->dtype, 0, sizeof(out->dtype));
+  std::strncpy(out->dtype, r.dtype.c_str(), sizeof(out->dtype) - 1);
+  out->ndim = (int)r.shape.size();
+  for (size_t i = 0; i < 8; ++i) out->shape[i] = i < r.shape.size() ? r.shape[i] : 0;
+  out->begin = r.begin;
+  out->end = r.end;
+  LMSF_API_END
+}
+// Address of the data section in this process (valid until the file is closed) and its size.
+const void* lmsf_safetensors_data(void* file, int64_t* size) {
+  auto* f = static_cast<SafetensorsFile*>(file);
+  if (size) *size = f->data_size();
+  return f->data();
 }
 
 }  // extern "C"

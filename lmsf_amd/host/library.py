@@ -7,7 +7,7 @@ from typing import Optional
 
 from ..csrc import build as _build
 
-HOST_ABI_VERSION = 3
+HOST_ABI_VERSION = 4
 
 OK, CACHE_ERROR, OUT_OF_PAGES, VALUE_ERROR = 0, 1, 2, 3
 
@@ -66,6 +66,11 @@ _SIGNATURES = {
     "lmsf_llama_config_parse": (c_int, [c_char_p, _P]),
     "lmsf_llama_config_validate": (c_int, [_P]),
     "lmsf_rope_scaling_parse": (c_int, [c_char_p, _P]),
+    "lmsf_safetensors_open": (c_int, [c_char_p, _PP]),
+    "lmsf_safetensors_close": (None, [_P]),
+    "lmsf_safetensors_count": (c_int64, [_P]),
+    "lmsf_safetensors_record": (c_int, [_P, c_int64, _P]),
+    "lmsf_safetensors_data": (c_void_p, [_P, POINTER(c_int64)]),
 }
 
 

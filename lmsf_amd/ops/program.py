@@ -29,7 +29,6 @@ import torch
 
 from . import library
 from .dispatch import Tunables
-from .handles import DeferredLinear, PendingProduct, ScaledRows  # noqa: F401  (what the placeholders stand for)
 
 MAX_GROUPS = 8
 MAX_PLANS = 4

@@ -3,18 +3,20 @@ header {name: {dtype, shape, data_offsets}}, then the raw little-endian data.
 
 The reference memory-maps the files through candle's VarBuilder
 (core/src/model_executor/models/model_factory.rs:133-139) and lists them from
-model.safetensors.index.json (:64-77). Here the file is memory-mapped and a tensor's bytes are
-touched only when that tensor is fetched, so a checkpoint larger than host memory can be loaded
-tensor by tensor.
+model.safetensors.index.json (:64-77). Here the file is memory-mapped (in C++, csrc/host/safetensors.cc)
+and a tensor's bytes are touched only when that tensor is fetched, so a checkpoint larger than host
+memory can be loaded tensor by tensor.
 """
+import ctypes
 import json
-import mmap
 import os
 import struct
 from dataclasses import dataclass
 from typing import Dict, Iterable, List, Tuple
 
 import torch
+
+from ..host.library import last_error, load_host_library
 
 
 class SafetensorsError(ValueError):
@@ -47,48 +49,38 @@ class TensorEntry:
     end: int
 
 
+class _NativeRecord(ctypes.Structure):
+    # LmsfTensorRecord of csrc/host/api.cc
+    _fields_ = [("name", ctypes.c_char_p), ("dtype", ctypes.c_char * 8), ("ndim", ctypes.c_int),
+                ("shape", ctypes.c_int64 * 8), ("begin", ctypes.c_int64), ("end", ctypes.c_int64)]
+
+
 class SafetensorsFile:
-    """One memory-mapped .safetensors file."""
+    """One memory-mapped .safetensors file. The file is opened, mapped and its header read and checked in C++
+    (``csrc/host/safetensors.cc``: every tensor's dtype, byte count against its shape, place inside the file, no
+    two overlapping or of one name); this class is the face of that object and turns a tensor's bytes into a
+    torch tensor."""
 
     def __init__(self, path: str):
         self.path = path
-        size = os.path.getsize(path)
-        if size < 8:
-            raise SafetensorsError("%s: too short to be a safetensors file (%d bytes)" % (path, size))
-        self._f = open(path, "rb")
-        (hlen,) = struct.unpack("<Q", self._f.read(8))
-        if hlen <= 0 or 8 + hlen > size:
-            raise SafetensorsError("%s: header length %d does not fit the file of %d bytes" % (path, hlen, size))
-        try:
-            header = json.loads(self._f.read(hlen).decode("utf-8"))
-        except (UnicodeDecodeError, json.JSONDecodeError) as e:
-            raise SafetensorsError("%s: header is not valid JSON: %s" % (path, e))
-        if not isinstance(header, dict):
-            raise SafetensorsError("%s: header is not a JSON object" % path)
-        self.data_start = 8 + hlen
-        self.data_size = size - self.data_start
+        self._lib = lib = load_host_library()
+        handle = ctypes.c_void_p()
+        if lib.lmsf_safetensors_open(os.fsencode(path), ctypes.byref(handle)) != 0:
+            raise SafetensorsError(last_error(lib))
+        self._handle = handle
+        size = ctypes.c_int64()
+        self._data = lib.lmsf_safetensors_data(handle, ctypes.byref(size))
+        self.data_size = size.value
         self.entries: Dict[str, TensorEntry] = {}
-        for name, info in header.items():
-            if name == "__metadata__":
-                continue
-            try:
-                dtype = info["dtype"]
-                shape = tuple(int(s) for s in info["shape"])
-                begin, end = (int(x) for x in info["data_offsets"])
-            except (KeyError, TypeError, ValueError):
-                raise SafetensorsError("%s: malformed header entry for %r" % (path, name))
-            if dtype not in _DTYPES:
-                raise SafetensorsError("%s: tensor %r has unsupported dtype %s" % (path, name, dtype))
-            n = 1
-            for s in shape:
-                n *= s
-            if end - begin != n * _DTYPES[dtype][1]:
-                raise SafetensorsError("%s: tensor %r: %d bytes for shape %s of %s" % (path, name, end - begin,
-                                                                                      list(shape), dtype))
-            if begin < 0 or end > self.data_size:
-                raise SafetensorsError("%s: tensor %r lies outside the file (truncated?)" % (path, name))
-            self.entries[name] = TensorEntry(name, path, dtype, shape, begin, end)
-        self._mm = mmap.mmap(self._f.fileno(), 0, access=mmap.ACCESS_READ) if size > 0 else None
+        rec = _NativeRecord()
+        for i in range(lib.lmsf_safetensors_count(handle)):
+            if lib.lmsf_safetensors_record(handle, i, ctypes.byref(rec)) != 0:
+                msg = last_error(lib)
+                self.close()
+                raise SafetensorsError("%s: %s" % (path, msg))
+            name = rec.name.decode("utf-8")
+            self.entries[name] = TensorEntry(name, path, rec.dtype.decode("ascii"),
+                                             tuple(int(rec.shape[k]) for k in range(rec.ndim)), rec.begin, rec.end)
 
     def read(self, name: str) -> torch.Tensor:
         """The tensor as a CPU tensor that owns its memory."""
@@ -97,14 +89,22 @@ class SafetensorsFile:
         nbytes = e.end - e.begin
         if nbytes == 0:
             return torch.empty(e.shape, dtype=tdtype)
-        buf = bytearray(self._mm[self.data_start + e.begin:self.data_start + e.end])
-        return torch.frombuffer(buf, dtype=tdtype).reshape(e.shape)
+        if self._handle is None:
+            raise SafetensorsError("%s is closed" % self.path)
+        mapped = (ctypes.c_ubyte * nbytes).from_address(self._data + e.begin)
+        # (bytes -> a tensor over the mapping -> a copy that outlives it)
+        return torch.frombuffer(mapped, dtype=tdtype).reshape(e.shape).clone()
 
     def close(self):
-        if self._mm is not None:
-            self._mm.close()
-            self._mm = None
-        self._f.close()
+        if self._handle is not None:
+            self._lib.lmsf_safetensors_close(self._handle)
+            self._handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:  # noqa: BLE001 - nothing to do about it at this point
+            pass
 
 
 def list_weight_files(folder: str) -> List[str]:

@@ -9,9 +9,23 @@
 #include <string>
 #include <vector>
 
+#include <unistd.h>
+
 #include "llama_config.h"
 
 extern "C" {
+typedef struct {
+  const char* name;
+  char dtype[8];
+  int ndim;
+  int64_t shape[8];
+  int64_t begin, end;
+} LmsfTensorRecord;
+int lmsf_safetensors_open(const char* path, void** out);
+void lmsf_safetensors_close(void* file);
+int64_t lmsf_safetensors_count(void* file);
+int lmsf_safetensors_record(void* file, int64_t index, LmsfTensorRecord* out);
+const void* lmsf_safetensors_data(void* file, int64_t* size);
 int lmsf_host_abi_version();
 const char* lmsf_host_last_error();
 int lmsf_pool_create(int num_pages, void** out);
@@ -116,6 +130,79 @@ int main(int argc, char** argv) {
     MUST(lmsf_rope_scaling_parse("{\"type\": \"default\"}", &rs));
     if (rs.present) return 1;
     MUST_FAIL(lmsf_rope_scaling_parse("{\"rope_type\": \"yarn\"}", &rs), 3);
+  }
+
+  // the checkpoint reader: a good file, then cuts and flips of its header and a shortened data section; whatever it
+  // accepts is read to the last byte of every tensor (the sanitizer sees a read outside the mapping)
+  {
+    const std::string good =
+        "{\"__metadata__\": {\"format\": \"pt\"}, \"b\": {\"dtype\": \"BF16\", \"shape\": [3, 4], \"data_offsets\": [16, 40]}, "
+        "\"a\": {\"dtype\": \"F32\", \"shape\": [2, 2], \"data_offsets\": [0, 16]}, "
+        "\"e\": {\"dtype\": \"I32\", \"shape\": [0], \"data_offsets\": [40, 40]}}";
+    char path[] = "/tmp/lmsf_san_XXXXXX";
+    const int fd = mkstemp(path);
+    if (fd < 0) return 1;
+    close(fd);
+    const auto write_file = [&](const std::string& header, size_t data_bytes, uint64_t claimed) {
+      FILE* f = std::fopen(path, "wb");
+      if (!f) std::exit(1);
+      unsigned char len[8];
+      for (int i = 0; i < 8; ++i) len[i] = (unsigned char)(claimed >> (8 * i));
+      std::fwrite(len, 1, 8, f);
+      std::fwrite(header.data(), 1, header.size(), f);
+      for (size_t i = 0; i < data_bytes; ++i) std::fputc((int)(i & 0xff), f);
+      std::fclose(f);
+    };
+    const auto open_and_read = [&](long* sum) {
+      void* file = nullptr;
+      const int rc = lmsf_safetensors_open(path, &file);
+      if (rc != 0) return rc;
+      int64_t size = 0;
+      const unsigned char* data = (const unsigned char*)lmsf_safetensors_data(file, &size);
+      for (int64_t i = 0; i < lmsf_safetensors_count(file); ++i) {
+        LmsfTensorRecord r;
+        if (lmsf_safetensors_record(file, i, &r) != 0) continue;
+        if (r.begin < 0 || r.end > size || r.begin > r.end) std::exit(1);
+        for (int64_t b = r.begin; b < r.end; ++b) *sum += data[b];
+      }
+      lmsf_safetensors_close(file);
+      return 0;
+    };
+    long sum = 0;
+    write_file(good, 40, good.size());
+    MUST(open_and_read(&sum));
+    if (sum != 40 * 39 / 2) return 1;
+    write_file(good, 39, good.size());                   // a byte short
+    MUST_FAIL(open_and_read(&sum), 3);
+    write_file(good, 40, (uint64_t)1 << 40);             // a header longer than the file
+    MUST_FAIL(open_and_read(&sum), 3);
+    write_file(good, 0, 0);
+    MUST_FAIL(open_and_read(&sum), 3);
+    for (const char* bad :
+         {"{\"a\": {\"dtype\": \"F32\", \"shape\": [2, 2], \"data_offsets\": [0, 12]}}",          // bytes against shape
+          "{\"a\": {\"dtype\": \"F8\", \"shape\": [4], \"data_offsets\": [0, 4]}}",              // unknown dtype
+          "{\"a\": {\"dtype\": \"U8\", \"shape\": [8], \"data_offsets\": [0, 8]}, "
+          "\"b\": {\"dtype\": \"U8\", \"shape\": [8], \"data_offsets\": [4, 12]}}",               // overlap
+          "{\"a\": {\"dtype\": \"U8\", \"shape\": [4], \"data_offsets\": [0, 4]}, "
+          "\"a\": {\"dtype\": \"U8\", \"shape\": [4], \"data_offsets\": [4, 8]}}",                // one name twice
+          "{\"a\": {\"dtype\": \"U8\", \"shape\": [-4], \"data_offsets\": [0, 4]}}",
+          "{\"a\": {\"dtype\": \"U8\", \"shape\": [4.0], \"data_offsets\": [0, 4]}}",
+          "{\"a\": {\"dtype\": \"I64\", \"shape\": [4294967296, 4294967296], \"data_offsets\": [0, 0]}}",
+          "{\"a\": [1, 2]}", "[]", "{\"a\": {\"dtype\": \"U8\", \"shape\": [4]}}"}) {
+      write_file(bad, 40, std::string(bad).size());
+      MUST_FAIL(open_and_read(&sum), 3);
+    }
+    for (int it = 0; it < 300; ++it) {
+      std::string t = good;
+      if (rnd(3) == 0) t.resize(rnd((uint32_t)t.size()));
+      for (int k = (int)rnd(4); k > 0 && !t.empty(); --k) t[rnd((uint32_t)t.size())] = (char)(32 + rnd(95));
+      write_file(t, rnd(48), rnd(8) ? t.size() : rnd(200));
+      const int rc = open_and_read(&sum);
+      if (rc != 0 && rc != 3) return 1;
+    }
+    unlink(path);
+    void* none = nullptr;
+    MUST_FAIL(lmsf_safetensors_open(path, &none), 3);   // no such file
   }
 
   // the pool alone, with its error paths

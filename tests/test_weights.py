@@ -68,6 +68,62 @@ def test_written_folder_is_read_by_the_safetensors_package_and_back(tmp_path):
     assert abs(w.std().item() - 0.02) < 0.002 and abs(w.mean().item()) < 0.002
 
 
+def test_reader_takes_every_storage_type_and_refuses_a_header_that_lies(tmp_path):
+    """The reader is C++ (csrc/host/safetensors.cc): a file of every dtype written by the safetensors package is
+    read back to the bit, also tensors of no elements and of no dimensions; headers whose entries overlap, repeat a
+    name, claim more bytes than their shape holds or more than the file has are refused, each by name."""
+    from safetensors.torch import save_file
+    g = torch.Generator().manual_seed(3)
+    tensors = {
+        "f32": torch.randn(3, 5, generator=g), "bf16": torch.randn(7, generator=g).bfloat16(),
+        "f16": torch.randn(2, 3, 4, generator=g).half(), "f64": torch.randn(2, generator=g).double(),
+        "i64": torch.arange(5), "i32": torch.arange(6, dtype=torch.int32).reshape(2, 3),
+        "i16": torch.arange(4, dtype=torch.int16), "i8": torch.arange(3, dtype=torch.int8),
+        "u8": torch.arange(9, dtype=torch.uint8), "flag": torch.tensor([True, False, True]),
+        "none": torch.zeros(0, 4), "scalar": torch.tensor(2.5),
+    }
+    path = str(tmp_path / "all.safetensors")
+    save_file(tensors, path)
+    f = SafetensorsFile(path)
+    assert set(f.entries) == set(tensors)
+    for name, t in tensors.items():
+        got = f.read(name)
+        assert got.dtype == t.dtype and got.shape == t.shape and torch.equal(got, t), name
+    kept = f.read("f32")
+    f.close()
+    assert torch.equal(kept, tensors["f32"])          # (a tensor read owns its memory)
+
+    def file_with(header: dict, data: bytes = bytes(64)) -> str:
+        text = json.dumps(header).encode()
+        bad = str(tmp_path / "bad.safetensors")
+        with open(bad, "wb") as out:
+            out.write(struct.pack("<Q", len(text)) + text + data)
+        return bad
+    entry = lambda dtype, shape, a, b: {"dtype": dtype, "shape": shape, "data_offsets": [a, b]}   # noqa: E731
+    for header, what in (
+            ({"a": entry("U8", [8], 0, 8), "b": entry("U8", [8], 4, 12)}, "overlap"),
+            ({"a": entry("F32", [2, 2], 0, 12)}, "12 bytes for shape"),
+            ({"a": entry("F32", [2, 2], 56, 72)}, "outside the file"),
+            ({"a": entry("F8_E4M3", [4], 0, 4)}, "unsupported dtype"),
+            ({"a": entry("U8", [-4], 0, 4)}, "malformed header entry"),
+            ({"a": {"dtype": "U8", "shape": [4]}}, "malformed header entry"),
+            ({"a": [1, 2]}, "malformed header entry"),
+            ({"a": entry("U8", [1] * 9, 0, 1)}, "9 dimensions")):
+        with pytest.raises(SafetensorsError, match=what):
+            SafetensorsFile(file_with(header))
+    twice = b'{"a": {"dtype": "U8", "shape": [4], "data_offsets": [0, 4]}, "a": {"dtype": "U8", "shape": [4], "data_offsets": [4, 8]}}'
+    with open(str(tmp_path / "twice.safetensors"), "wb") as out:
+        out.write(struct.pack("<Q", len(twice)) + twice + bytes(8))
+    with pytest.raises(SafetensorsError, match="listed twice"):
+        SafetensorsFile(str(tmp_path / "twice.safetensors"))
+    with open(str(tmp_path / "text.safetensors"), "wb") as out:
+        out.write(struct.pack("<Q", 5) + b"{nope")
+    with pytest.raises(SafetensorsError, match="not valid JSON"):
+        SafetensorsFile(str(tmp_path / "text.safetensors"))
+    with pytest.raises(SafetensorsError, match="cannot be opened"):
+        SafetensorsFile(str(tmp_path / "absent.safetensors"))
+
+
 def test_fused_rows_and_tied_head(tmp_path):
     folder, cfg = make_model_folder(tmp_path, "B")
     model = cpu_model(cfg)
