@@ -85,6 +85,29 @@ def test_llama3_8b_layer_sizes_whole_prompts_of_hundreds_of_tokens(full_model, n
     core.storage.manager.check_invariants()
 
 
+def test_llama3_8b_layer_sizes_with_the_library_products_raced_at_load(full_model):
+    """``tune_products``: at load the library's candidates race for the products of a full step (1,024 tokens here)
+    and of a portion of ``prefill_chunk_size`` tokens on the model's own weights. Prompts of 600 and 1,024 tokens and
+    a portion of 512 against the plain implementation."""
+    from lmsf_amd.engine import EngineArgs, LLMEngine, StepEntry
+    folder, cfg, w = full_model
+    engine = LLMEngine(EngineArgs(model=folder, dtype="bfloat16", block_size=16, num_gpu_blocks_override=160,
+                                  max_num_seqs=4, max_num_batched_tokens=1024, prefill_chunk_size=512,
+                                  tune_products=True, skip_tokenizer_init=True))
+    tuned = engine.tuned_products
+    assert {m for (m, _n, _k) in tuned} == {512, 1024} and len(tuned) >= 6       # QKV, o, gate_up at either; down stays with this package's product
+    assert all(0 < best <= first for first, best in tuned.values())
+    ex = engine.core.executor
+    reqs = {"a": random_tokens(600, cfg["vocab_size"], 31), "b": random_tokens(1024, cfg["vocab_size"], 32),
+            "c": random_tokens(512, cfg["vocab_size"], 33)}
+    got = {}
+    for rid, toks in reqs.items():
+        got[rid] = ex.step([StepEntry(rid, toks, [len(toks) - 2, len(toks) - 1])]).float().cpu()
+        ex.release(rid)
+    refs = {rid: plain_llama_forward(cfg, w, toks, last=2) for rid, toks in reqs.items()}
+    check(got, refs, "bfloat16", "prompts after the race", BOUND)
+
+
 def test_llama3_8b_layer_sizes_in_true_float32(full_model):
     """The 32-bit path at these sizes (float32 multiply-add products over K = 4,096 and 14,336, the general
     attention kernel), on the same weights: a prompt in two portions and a few single tokens."""

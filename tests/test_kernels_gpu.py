@@ -901,6 +901,34 @@ def test_linear_many_rows_every_tiling_and_split(ops, ref, M, N, K):
         assert torch.equal(a, c) and torch.equal(r1, r2)
 
 
+@pytest.mark.parametrize("bias", [False, True])
+def test_library_products_race_for_a_shape(ops, bias):
+    """The BLAS library's candidates for one shape race on three copies of the weight and the winner is kept for that
+    shape (one plan more, none for its neighbours). Whatever algorithm runs, the product is the product: the raced
+    shape and others of the same weight against float32."""
+    g = torch.Generator().manual_seed(9)
+    N, K = 1536, 1024
+    pad = ops.weight_row_pad(K, torch.bfloat16)
+    weights = []
+    for _ in range(3):
+        buf = dev(torch.zeros(N, K + pad).bfloat16())
+        buf[:, :K].copy_(dev((torch.randn(N, K, generator=g) * K ** -0.5).bfloat16()))
+        weights.append(buf[:, :K])
+    b = dev(torch.randn(N, generator=g).bfloat16()) if bias else None
+    x = dev(torch.randn(2048, K, generator=g).bfloat16())
+    plans = ops.lib.lmsf_blas_plans()
+    first, best = ops.tune_products(x[:1024], weights, b, candidates=8, reps=3)
+    assert 0 < best <= first < 1e5
+    assert ops.lib.lmsf_blas_plans() == plans + 1
+    for M in (1024, 1000, 513, 2048, 300):
+        got = ops.linear(x[:M], weights[1], b)
+        want = x[:M].float() @ weights[1].float().t() + (b.float() if bias else 0.0)
+        assert (got.float() - want).abs().max().item() <= 2e-2 * max(1.0, want.abs().max().item()), M
+    # a race needs operands of one shape
+    with pytest.raises(ValueError, match="one shape"):
+        ops.tune_products(x[:512], [weights[0], weights[1][:8]], b)
+
+
 def test_linear_mixed_storage(ops, ref):
     """A weight stored in 32 bits stays so and still multiplies bfloat16 activations."""
     g = torch.Generator().manual_seed(5)
