@@ -19,7 +19,14 @@
 // the same prefetch within steps of 64 k with the barrier in the middle of a step (0.74); tiles of 256 x 256 with two
 // stages, which is all LDS holds of them (0.6, the compiler spills around 256 accumulators); the same tiles with the
 // 32 x 32 x 16 instruction, wave tiles of 128 x 128 and no spills (0.85 to 1.0: two stages do not cover the way from
-// memory).
+// memory); and those tiles again with four or five stages of 32 k (rows of 64 bytes), the accumulators in the 256
+// accumulation registers and the next step's operands read from LDS under the current step's multiplications: 0.91
+// PFLOP/s on gate_up at 2,048 rows against the library's 1.38 to 1.44, 0.55 on o (128 tiles: half the chip). The
+// same loop without its transfers reaches 1.20, without transfers and barriers 1.31 (1.7 a compute unit on o), the
+// same whether the transfers bring new data or the same lines again: what costs is the transfers' instructions
+// themselves, six to eight each with their addresses, issued in a burst during which the matrix pipe runs dry, and
+// the barrier of four waves every 1,024 cycles. The library stages through registers and places every instruction
+// by hand; with 3.5 rounds of tiles over the chip (896 tiles) the ceiling here would be 1.2 to 1.25.
 //
 // Counters of this kernel and of the library's on the same product (2,048 x 14,336 x 4,096, the weight in cache):
 // the same 1.47e7 matrix instructions; beside each of them 0.71 other vector instructions here and 0.06 there; the
