@@ -128,7 +128,12 @@ def load_weights(parts: Sequence[Part], folder: str, device: torch.device, run_d
                 return cache[name]
             f, _ = entries[name]
             try:
-                t = _convert(f.read(name), decls[name], run_dtype, keep_float32)
+                if torch.device(device).type == "cuda":
+                    # from the mapped file to the device as stored, converted there: the bytes are passed over once
+                    # on the host, and a 32-bit checkpoint is cast by the GPU
+                    t = _convert(f.read(name, copy=False).to(device), decls[name], run_dtype, keep_float32)
+                else:
+                    t = _convert(f.read(name), decls[name], run_dtype, keep_float32)
             except WeightsError as e:
                 raise WeightsError("%s: %s" % (name, e))
             if t.dtype == torch.float32 and run_dtype != torch.float32 and t.dim() >= 2:

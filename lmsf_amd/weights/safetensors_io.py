@@ -82,8 +82,10 @@ class SafetensorsFile:
             self.entries[name] = TensorEntry(name, path, rec.dtype.decode("ascii"),
                                              tuple(int(rec.shape[k]) for k in range(rec.ndim)), rec.begin, rec.end)
 
-    def read(self, name: str) -> torch.Tensor:
-        """The tensor as a CPU tensor that owns its memory."""
+    def read(self, name: str, copy: bool = True) -> torch.Tensor:
+        """The tensor as a CPU tensor that owns its memory. ``copy=False``: a tensor over the mapped file itself,
+        which must be gone before the file is closed (the loader copies it to the device at once and drops it: one
+        pass over the bytes fewer)."""
         e = self.entries[name]
         tdtype, _ = _DTYPES[e.dtype]
         nbytes = e.end - e.begin
@@ -93,7 +95,8 @@ class SafetensorsFile:
             raise SafetensorsError("%s is closed" % self.path)
         mapped = (ctypes.c_ubyte * nbytes).from_address(self._data + e.begin)
         # (bytes -> a tensor over the mapping -> a copy that outlives it)
-        return torch.frombuffer(mapped, dtype=tdtype).reshape(e.shape).clone()
+        view = torch.frombuffer(mapped, dtype=tdtype).reshape(e.shape)
+        return view.clone() if copy else view
 
     def close(self):
         if self._handle is not None:

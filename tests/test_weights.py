@@ -90,6 +90,9 @@ def test_reader_takes_every_storage_type_and_refuses_a_header_that_lies(tmp_path
         got = f.read(name)
         assert got.dtype == t.dtype and got.shape == t.shape and torch.equal(got, t), name
     kept = f.read("f32")
+    over_the_file = f.read("bf16", copy=False)       # (a tensor over the mapping: gone before the file closes)
+    assert torch.equal(over_the_file, tensors["bf16"])
+    del over_the_file
     f.close()
     assert torch.equal(kept, tensors["f32"])          # (a tensor read owns its memory)
 
