@@ -30,6 +30,7 @@ typedef struct {
   int large_deep_min_rows;        // products with K >= 3 N go to the many-rows kernel from beyond this many rows
   int mid_scaled_rows;            // rows up to which the gated product after a norm runs in the 17-and-more-rows kernel (0: never)
   int large_deep_max_rows;        // rows up to which products with K >= 3 N stay with the many-rows kernel
+  int qkv_fused_max_rows;         // rows up to which the QKV product with rotation and cache write runs in the few-rows kernel
 } LmsfTunables;
 
 enum {

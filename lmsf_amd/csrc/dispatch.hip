@@ -136,7 +136,8 @@ extern "C" void lmsf_route_qkv(const LmsfTunables* t, const LmsfProductShape* sp
       *out = route(LMSF_ROUTE_MATERIALIZE);
     return;
   }
-  if (fused_shape && s.x_dtype == LMSF_BF16 && 0 < M && M <= t->skinny_max_rows && skinny_ok(s)) {
+  if (fused_shape && s.x_dtype == LMSF_BF16 && 0 < M && M <= std::min(64, std::max(t->skinny_max_rows, t->qkv_fused_max_rows)) &&
+      skinny_ok(s)) {
     *out = route(M <= t->gemv_max_rows && gemv_ok(M, K) ? LMSF_ROUTE_GEMV : LMSF_ROUTE_SKINNY);
     return;
   }

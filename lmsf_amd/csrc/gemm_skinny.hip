@@ -457,7 +457,7 @@ extern "C" int lmsf_gemm_qkv_rope_cache(const void* x, long ldx, const void* W, 
                                         const int* slots, void* k_pages, void* v_pages, long num_pages, int nh,
                                         int nkv, int d, int ps, int variant, hipStream_t stream) {
   LMSF_CHECK(x && W && y && positions && table && slots && k_pages && v_pages, "gemm_qkv_rope_cache: null pointer");
-  LMSF_CHECK(M >= 0 && M <= 16, "gemm_qkv_rope_cache: M=%d outside [0, 16]", M);
+  LMSF_CHECK(M >= 0 && M <= 64, "gemm_qkv_rope_cache: M=%d outside [0, 64]", M);
   LMSF_CHECK(nh > 0 && nkv > 0 && d >= 32 && d % 32 == 0, "gemm_qkv_rope_cache: head size %d must be a multiple of 32", d);
   const long N = (long)(nh + 2 * nkv) * d;
   LMSF_CHECK(N / 32 <= 2147483647L, "gemm_qkv_rope_cache: too many rows");
@@ -472,7 +472,13 @@ extern "C" int lmsf_gemm_qkv_rope_cache(const void* x, long ldx, const void* W, 
   rc.k_pages = (bf16_t*)k_pages; rc.v_pages = (bf16_t*)v_pages;
   rc.nh = nh; rc.nkv = nkv; rc.d = d; rc.ps = ps;
   int r;
-  if (variant == 1)
+  if (M > 48)       // (eight waves: the stages of sixteen would not fit LDS beside three and four tiles of x)
+    r = launch_skinny<4, 64, 8, bf16_t, 3>(x, ldx, W, ldw, bias, y, ldy, M, (int)N, K, stream, rc);
+  else if (M > 32)
+    r = launch_skinny<3, 64, 8, bf16_t, 3>(x, ldx, W, ldw, bias, y, ldy, M, (int)N, K, stream, rc);
+  else if (M > 16)
+    r = launch_skinny<2, 64, 16, bf16_t, 3>(x, ldx, W, ldw, bias, y, ldy, M, (int)N, K, stream, rc);
+  else if (variant == 1)
     r = launch_skinny<1, 64, 8, bf16_t, 3>(x, ldx, W, ldw, bias, y, ldy, M, (int)N, K, stream, rc);
   else
     r = launch_skinny<1, 64, 16, bf16_t, 3>(x, ldx, W, ldw, bias, y, ldy, M, (int)N, K, stream, rc);

@@ -16,7 +16,7 @@ void lmsf_set_error(const char* fmt, ...) {
 extern "C" const char* lmsf_last_error() { return g_last_error; }
 
 // ABI version of the entry points; the Python side refuses a library that reports another.
-extern "C" int lmsf_abi_version() { return 22; }
+extern "C" int lmsf_abi_version() { return 23; }
 
 // Compute units of the current device (asked once per device; 0 if the device cannot be asked).
 int lmsf_compute_units() {

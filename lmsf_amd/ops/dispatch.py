@@ -8,7 +8,8 @@ from ctypes import Structure, c_int, c_long
 TUNABLE_NAMES = (
     "fuse_norm_rows", "fuse_stream_rows", "gemv_max_rows", "skinny_variant", "mid_wide_max_cols", "mid_max_rows",
     "skinny_max_rows", "prefill_attention_variant", "decode_attention_order", "decode_attention_splits",
-    "use_library_gemm", "large_max_rows", "large_deep_min_rows", "mid_scaled_rows", "large_deep_max_rows")
+    "use_library_gemm", "large_max_rows", "large_deep_min_rows", "mid_scaled_rows", "large_deep_max_rows",
+    "qkv_fused_max_rows")
 
 
 class Tunables(Structure):

@@ -75,6 +75,7 @@ class HipOps:
         self.large_deep_min_rows = 64    # products whose K is at least three times N go to the many-rows kernel from beyond this many rows already (down at 128 rows: 42.8 -> 38.0 us; decode at batch 128: 6.63 -> 6.53 ms a step, at 96: 5.83 -> 5.74)
         self.mid_scaled_rows = 16        # rows up to which the gated product after a norm runs in the 17-and-more-rows kernel where that kernel's workgroups fit on the chip at once (0: never)
         self.large_deep_max_rows = 1024  # the same for products whose K is at least three times N (down: 57 against 76 us at 320 rows, 74 against 94 at 512, 102 against 108 at 768, level at 1,024)
+        self.qkv_fused_max_rows = 32     # rows up to which the QKV product with rotation and cache write runs in the few-rows kernel, beyond skinny_max_rows (one kernel against the 17-and-more-rows product and the rotary kernel over its partial sums: decode at batch 24 3.99 -> 3.92 ms a step, at 32 4.11 -> 3.99; level at 48, behind at 64: 4.80 -> 4.87)
         self.weight_row_pad_bytes = 512  # bytes left between two rows of a linear layer's weight (see weight_row_pad)
         # the BLAS library's products are called from C++ (csrc/blas.hip); its handle and workspace are made here
         if self.lib.lmsf_blas_init(self.blas_workspace_bytes) != 0:

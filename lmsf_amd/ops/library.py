@@ -10,7 +10,7 @@ from typing import Optional
 from ..csrc import build as _build
 from .dispatch import ProductShape, Route, Tunables
 
-ABI_VERSION = 22
+ABI_VERSION = 23
 
 _lib: Optional[ctypes.CDLL] = None
 _lib_path: Optional[str] = None

@@ -22,7 +22,7 @@ def defaults():
     return D.Tunables(fuse_norm_rows=16, fuse_stream_rows=1, gemv_max_rows=2, skinny_variant=0, mid_wide_max_cols=8192,
                       mid_max_rows=128, skinny_max_rows=16, prefill_attention_variant=0, decode_attention_order=0,
                       decode_attention_splits=0, use_library_gemm=1, large_max_rows=256, large_deep_min_rows=64,
-                      mid_scaled_rows=16, large_deep_max_rows=1024)
+                      mid_scaled_rows=16, large_deep_max_rows=1024, qkv_fused_max_rows=32)
 
 
 def shape(M, N, K, x=BF16, w=BF16, out=BF16, ld_pad=256, ok16=1):
@@ -97,8 +97,11 @@ def test_gated_and_qkv_products(lib):
         lib.lmsf_route_qkv(ctypes.byref(t), ctypes.byref(shape(M, QKV, H)), fused, scaled, ctypes.byref(r))
         return r
 
-    assert [qkv(M).route for M in (1, 2, 3, 16, 17, 2048)] == [D.GEMV, D.GEMV, D.SKINNY, D.SKINNY, D.SEPARATE, D.SEPARATE]
-    assert qkv(17).pending == 1 and qkv(8, fused=0).route == D.SEPARATE and qkv(8, fused=0).pending == 0
+    # (with its rotation and cache write as epilogue the few-rows kernel keeps the QKV product up to 32 rows)
+    assert [qkv(M).route for M in (1, 2, 3, 16, 17, 32, 33, 2048)] == [D.GEMV, D.GEMV, D.SKINNY, D.SKINNY, D.SKINNY,
+                                                                     D.SKINNY, D.SEPARATE, D.SEPARATE]
+    assert qkv(33).pending == 1 and qkv(8, fused=0).route == D.SEPARATE and qkv(8, fused=0).pending == 0
+    assert qkv(17, fused=0).route == D.SEPARATE and qkv(17, fused=0).pending == 1
     assert qkv(8, scaled=16).route == D.SKINNY_SCALED and qkv(2, scaled=2).route == D.GEMV_SCALED
     assert qkv(8, fused=0, scaled=16).route == D.MATERIALIZE
 

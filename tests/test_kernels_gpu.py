@@ -604,6 +604,43 @@ def test_qkv_rope_cache_fused_equals_the_three_steps(ops, ref, M, H, nh, nkv, d,
     assert (a.float() - c.float()).abs().max().item() <= 2e-2 * scale and (k4.float() - k5.float()).abs().max().item() <= 2e-2 * scale
 
 
+@pytest.mark.parametrize("M", [17, 24, 32, 33, 48, 49, 64])
+@pytest.mark.parametrize("H,nh,nkv,d,ps", [(4096, 32, 8, 128, 16), (1024, 6, 3, 64, 8), (320, 5, 5, 32, 4)])
+@pytest.mark.parametrize("bias", [False, True])
+def test_qkv_rope_cache_in_the_few_rows_kernel_beyond_16_rows(ops, ref, M, H, nh, nkv, d, ps, bias):
+    """The QKV product with rotation and cache write as epilogue takes up to 64 rows in the few-rows kernel (two to
+    four tiles of rows; the switch point ``qkv_fused_max_rows`` says up to where it is used): against the plain
+    formulas, and within a rounding of the 17-and-more-rows product followed by the rotary kernel, which adds up K in
+    another order."""
+    g = torch.Generator().manual_seed(M + H + d)
+    N = (nh + 2 * nkv) * d
+    x = dev(torch.randn(M, H, generator=g).bfloat16())
+    w = dev((torch.randn(N, H, generator=g) * H ** -0.5).bfloat16())
+    b = dev(torch.randn(N, generator=g).bfloat16()) if bias else None
+    max_pos, pages = 70, -(-M // ps) + 3
+    pos = dev(torch.randint(0, max_pos, (M,), generator=g, dtype=torch.int32))
+    ang = torch.arange(max_pos, dtype=torch.float32)[:, None] * torch.rand(d // 2, generator=g)[None, :]
+    table = dev(torch.cat([ang.cos(), ang.sin()], dim=1).contiguous())
+    slots = torch.randperm(pages * ps, generator=g)[:M].to(torch.int32)
+    slots[M - 1] = -1
+    slots = dev(slots)
+    k1, v1 = dev(torch.zeros(pages, nkv, ps, d).bfloat16()), dev(torch.zeros(pages, nkv, d, ps).bfloat16())
+    k2, v2, k3, v3 = k1.clone(), v1.clone(), k1.clone(), v1.clone()
+    before = ops.qkv_fused_max_rows
+    try:
+        ops.qkv_fused_max_rows = 64
+        fused = ops.qkv_rope_cache(x, w, b, nh, nkv, d, pos, table, d, True, slots, k1, v1)
+        ops.qkv_fused_max_rows = 0
+        apart = ops.qkv_rope_cache(x, w, b, nh, nkv, d, pos, table, d, True, slots, k2, v2)
+    finally:
+        ops.qkv_fused_max_rows = before
+    plain = ref.qkv_rope_cache(x, w, b, nh, nkv, d, pos, table, d, True, slots, k3, v3)
+    scale = max(1.0, plain.float().abs().max().item())
+    for got, want in ((fused, plain), (k1, k3), (v1, v3), (fused, apart), (k1, k2), (v1, v2)):
+        assert (got.float() - want.float()).abs().max().item() <= 2e-2 * scale
+    assert not torch.equal(k1, torch.zeros_like(k1))
+
+
 @pytest.mark.parametrize("M,N,K", [(17, 256, 1024), (40, 4096, 4096), (64, 80, 1280), (33, 1000, 2048), (65, 256, 1024),
                                    (100, 4096, 4096), (128, 80, 1280)])
 @pytest.mark.parametrize("bias", [False, True])
